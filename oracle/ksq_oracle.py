@@ -1,0 +1,329 @@
+"""ctypes/numpy front end of the CPU oracle (oracle/ksq_oracle.c).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by ``__graft_entry__.smoke()`` and by the
+``cpu_baseline`` leg of ``bench.py``.  The product package never imports this module.
+
+All arrays are numpy; 16-bit floats travel as ``uint16`` bit patterns so that the oracle
+sees exactly the bits the GPU sees.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "libksq_oracle.so")
+
+F16, BF16, F32 = 0, 1, 2
+
+
+def build(force=False):
+    """Compile the oracle with gcc (a few seconds)."""
+    if force or not os.path.exists(_SO) or os.path.getmtime(_SO) < os.path.getmtime(os.path.join(_HERE, "ksq_oracle.c")):
+        subprocess.check_call(["make", "-C", _HERE, "-B"], stdout=subprocess.DEVNULL)
+    return _SO
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_SO):
+            build()
+        _lib = ctypes.CDLL(_SO)
+        _lib.ksqo_f16_to_f32.restype = ctypes.c_float
+        _lib.ksqo_f16_to_f32.argtypes = [ctypes.c_uint16]
+        _lib.ksqo_f32_to_f16.restype = ctypes.c_uint16
+        _lib.ksqo_f32_to_f16.argtypes = [ctypes.c_float]
+        _lib.ksqo_f32_to_e4m3.restype = ctypes.c_uint8
+        _lib.ksqo_f32_to_e4m3.argtypes = [ctypes.c_float]
+        _lib.ksqo_e4m3_to_f32.restype = ctypes.c_float
+        _lib.ksqo_e4m3_to_f32.argtypes = [ctypes.c_uint8]
+    return _lib
+
+
+def _p(a):
+    return a.ctypes.data_as(ctypes.c_void_p)
+
+
+def _c(a, dtype):
+    return np.ascontiguousarray(a, dtype=dtype)
+
+
+def _sz(v):
+    return ctypes.c_size_t(int(v))
+
+
+# ---------------------------------------------------------------- scalar formats
+def _bulk(fn, src, src_dt, dst_dt):
+    src = _c(src, src_dt)
+    dst = np.empty(src.shape, dtype=dst_dt)
+    getattr(lib(), fn)(_p(src), _p(dst), _sz(src.size))
+    return dst
+
+
+def f16_to_f32(h):
+    return _bulk("ksqo_f16_to_f32_n", h, np.uint16, np.float32)
+
+
+def f32_to_f16(f):
+    return _bulk("ksqo_f32_to_f16_n", f, np.float32, np.uint16)
+
+
+def bf16_to_f32(h):
+    return _bulk("ksqo_bf16_to_f32_n", h, np.uint16, np.float32)
+
+
+def f32_to_bf16(f):
+    return _bulk("ksqo_f32_to_bf16_n", f, np.float32, np.uint16)
+
+
+def e4m3_to_f32(c):
+    return _bulk("ksqo_e4m3_to_f32_n", c, np.uint8, np.float32)
+
+
+def f32_to_e4m3(f):
+    return _bulk("ksqo_f32_to_e4m3_n", f, np.float32, np.uint8)
+
+
+def to_bits(f, dtype):
+    """float32 array -> storage array of ``dtype`` (uint16 bits for f16/bf16)."""
+    if dtype == F16:
+        return f32_to_f16(f)
+    if dtype == BF16:
+        return f32_to_bf16(f)
+    return _c(f, np.float32)
+
+
+def from_bits(b, dtype):
+    if dtype == F16:
+        return f16_to_f32(b)
+    if dtype == BF16:
+        return bf16_to_f32(b)
+    return _c(b, np.float32)
+
+
+def _store_dt(dtype):
+    return np.float32 if dtype == F32 else np.uint16
+
+
+# ---------------------------------------------------------------- checkpoint layouts
+def gptq_unpack(qweight):
+    q = _c(qweight, np.uint32)
+    K, N = q.shape[0] * 8, q.shape[1]
+    out = np.empty((K, N), np.uint8)
+    lib().ksqo_gptq_unpack(_p(q), _p(out), _sz(K), _sz(N))
+    return out
+
+
+def gptq_pack(codes):
+    c = _c(codes, np.uint8)
+    K, N = c.shape
+    out = np.empty((K // 8, N), np.uint32)
+    lib().ksqo_gptq_pack(_p(c), _p(out), _sz(K), _sz(N))
+    return out
+
+
+def awq_unpack(q):
+    q = _c(q, np.uint32)
+    R, N = q.shape[0], q.shape[1] * 8
+    out = np.empty((R, N), np.uint8)
+    lib().ksqo_awq_unpack(_p(q), _p(out), _sz(R), _sz(N))
+    return out
+
+
+def awq_pack(codes):
+    c = _c(codes, np.uint8)
+    R, N = c.shape
+    out = np.empty((R, N // 8), np.uint32)
+    lib().ksqo_awq_pack(_p(c), _p(out), _sz(R), _sz(N))
+    return out
+
+
+def pack_int8_to_int4x2(w):
+    w = _c(w, np.int8)
+    K, N = w.shape
+    out = np.empty((K, N // 2), np.int8)
+    lib().ksqo_pack_int8_to_int4x2(_p(w), _p(out), _sz(K), _sz(N))
+    return out
+
+
+def moe_unpack(w):
+    """[E, N, K/2] u8 -> codes [E, K, N] u8."""
+    w = _c(w, np.uint8)
+    E, N, K2 = w.shape
+    out = np.empty((E, K2 * 2, N), np.uint8)
+    lib().ksqo_moe_unpack(_p(w), _p(out), _sz(E), _sz(N), _sz(K2 * 2))
+    return out
+
+
+def moe_pack(codes):
+    """codes [E, K, N] u8 -> [E, N, K/2] u8."""
+    c = _c(codes, np.uint8)
+    E, K, N = c.shape
+    out = np.empty((E, N, K // 2), np.uint8)
+    lib().ksqo_moe_pack(_p(c), _p(out), _sz(E), _sz(N), _sz(K))
+    return out
+
+
+def marlin_gptq_repack(qweight):
+    q = _c(qweight, np.uint32)
+    K, N = q.shape[0] * 8, q.shape[1]
+    out = np.empty((K // 16, 2 * N), np.uint32)
+    assert lib().ksqo_marlin_gptq_repack(_p(q), _p(out), _sz(K), _sz(N)) == 0
+    return out
+
+
+def marlin_awq_repack(qweight):
+    q = _c(qweight, np.uint32)
+    K, N = q.shape[0], q.shape[1] * 8
+    out = np.empty((K // 16, 2 * N), np.uint32)
+    assert lib().ksqo_marlin_awq_repack(_p(q), _p(out), _sz(K), _sz(N)) == 0
+    return out
+
+
+def marlin_awq_zero_points(qz):
+    q = _c(qz, np.uint32)
+    R, N = q.shape[0], q.shape[1] * 8
+    out = np.empty((R, N // 8), np.uint32)
+    assert lib().ksqo_marlin_awq_zero_points(_p(q), _p(out), _sz(R), _sz(N)) == 0
+    return out
+
+
+# ---------------------------------------------------------------- W4A16
+def w4a16_dequant(codes, scales_bits, zeros, group, dtype):
+    c = _c(codes, np.uint8)
+    K, N = c.shape
+    s = _c(scales_bits, _store_dt(dtype))
+    z = None if zeros is None else _c(zeros, np.uint8)
+    w = np.empty((K, N), np.float32)
+    lib().ksqo_w4a16_dequant(_p(c), _p(s), _p(z) if z is not None else None, _p(w), _sz(K), _sz(N), _sz(group),
+                             ctypes.c_int(dtype))
+    return w
+
+
+def gemm_xw_f32(x_bits, w, dtype):
+    x = _c(x_bits, _store_dt(dtype))
+    w = _c(w, np.float32)
+    M, K = x.shape
+    N = w.shape[1]
+    y = np.empty((M, N), np.float32)
+    lib().ksqo_gemm_xw_f32(_p(x), _p(w), _p(y), _sz(M), _sz(N), _sz(K), ctypes.c_int(dtype))
+    return y
+
+
+def gemm_xw_f64(x_bits, w, dtype):
+    x = _c(x_bits, _store_dt(dtype))
+    w = _c(w, np.float32)
+    M, K = x.shape
+    N = w.shape[1]
+    y = np.empty((M, N), np.float64)
+    lib().ksqo_gemm_xw_f64(_p(x), _p(w), _p(y), _sz(M), _sz(N), _sz(K), ctypes.c_int(dtype))
+    return y
+
+
+def w4a16_gemm(x_bits, codes, scales_bits, zeros, group, dtype):
+    """Dequantize-then-GEMM, fp32 result (not rounded to dtype)."""
+    x = _c(x_bits, _store_dt(dtype))
+    c = _c(codes, np.uint8)
+    s = _c(scales_bits, _store_dt(dtype))
+    z = None if zeros is None else _c(zeros, np.uint8)
+    M, K = x.shape
+    N = c.shape[1]
+    y = np.empty((M, N), np.float32)
+    rc = lib().ksqo_w4a16_gemm(_p(x), _p(c), _p(s), _p(z) if z is not None else None, _p(y), _sz(M), _sz(N), _sz(K),
+                               _sz(group), ctypes.c_int(dtype))
+    assert rc == 0
+    return y
+
+
+# ---------------------------------------------------------------- FP8
+def fp8_group_quant(x_bits, k, group, column_major, fuse_silu_mul, dtype):
+    x = _c(x_bits, _store_dt(dtype))
+    m = x.shape[0]
+    q = np.empty((m, k), np.uint8)
+    ng = k // group
+    s = np.empty((ng, m) if column_major else (m, ng), np.float32)
+    lib().ksqo_fp8_group_quant(_p(x), _p(q), _p(s), _sz(m), _sz(k), _sz(group), ctypes.c_int(int(column_major)),
+                               ctypes.c_int(int(fuse_silu_mul)), ctypes.c_int(dtype))
+    return q, s
+
+
+def fp8_blockwise_gemm(a, a_s, b, b_s, a_s_column_major=True):
+    a = _c(a, np.uint8)
+    b = _c(b, np.uint8)
+    a_s = _c(a_s, np.float32)
+    b_s = _c(b_s, np.float32)
+    m, k = a.shape
+    n = b.shape[0]
+    out = np.empty((m, n), np.float32)
+    lib().ksqo_fp8_blockwise_gemm(_p(a), _p(a_s), _p(b), _p(b_s), _p(out), _sz(m), _sz(n), _sz(k),
+                                  ctypes.c_int(int(a_s_column_major)))
+    return out
+
+
+def fp8_block_quant_weight(w):
+    w = _c(w, np.float32)
+    n, k = w.shape
+    q = np.empty((n, k), np.uint8)
+    s = np.empty(((n + 127) // 128, (k + 127) // 128), np.float32)
+    lib().ksqo_fp8_block_quant_weight(_p(w), _p(q), _p(s), _sz(n), _sz(k))
+    return q, s
+
+
+# ---------------------------------------------------------------- MoE
+def moe_align(topk_ids, E, block_size):
+    ids = _c(topk_ids, np.int32).reshape(-1)
+    numel = ids.size
+    cap = numel + E * (block_size - 1)
+    sorted_ids = np.empty(cap, np.int32)
+    expert_ids = np.full((cap + block_size - 1) // block_size, -1, np.int32)
+    npp = np.zeros(1, np.int32)
+    assert lib().ksqo_moe_align(_p(ids), _sz(numel), ctypes.c_int(E), ctypes.c_int(block_size), _p(sorted_ids),
+                                _p(expert_ids), _p(npp)) == 0
+    return sorted_ids, expert_ids, int(npp[0])
+
+
+def moe_w4a16_gemm(x_bits, w, scales_bits, topk_ids, topk_w, top_k_div, group, mul_routed, dtype):
+    x = _c(x_bits, _store_dt(dtype))
+    w = _c(w, np.uint8)
+    s = _c(scales_bits, _store_dt(dtype))
+    ids = _c(topk_ids, np.int32).reshape(-1)
+    tw = _c(topk_w, np.float32).reshape(-1)
+    E, N, K2 = w.shape
+    K = K2 * 2
+    out = np.empty((ids.size, N), np.float32)
+    lib().ksqo_moe_w4a16_gemm(_p(x), _p(w), _p(s), _p(ids), _p(tw), _p(out), _sz(ids.size), ctypes.c_int(top_k_div),
+                              _sz(N), _sz(K), _sz(group), ctypes.c_int(int(mul_routed)), ctypes.c_int(dtype))
+    return out
+
+
+def silu_mul(x_bits, dtype):
+    x = _c(x_bits, _store_dt(dtype))
+    rows, two_i = x.shape
+    out = np.empty((rows, two_i // 2), _store_dt(dtype))
+    lib().ksqo_silu_mul(_p(x), _p(out), _sz(rows), _sz(two_i // 2), ctypes.c_int(dtype))
+    return out
+
+
+def moe_sum(x_bits, dtype):
+    x = _c(x_bits, _store_dt(dtype))
+    T, topk, d = x.shape
+    out = np.empty((T, d), _store_dt(dtype))
+    lib().ksqo_moe_sum(_p(x), _p(out), _sz(T), _sz(topk), _sz(d), ctypes.c_int(dtype))
+    return out
+
+
+def moe_forward(x_bits, w13, s13, w2, s2, topk_ids, topk_w, group, dtype):
+    """Whole int4 MoE block as S/kernels/nvidia/moe_kernel_wrapper.cpp:616-652 sequences it:
+    GEMM1 (no routed weight) -> T, silu*mul -> T, GEMM2 (* routed weight) -> T, sum over top-k in T."""
+    T, topk = np.asarray(topk_ids).shape
+    c1 = moe_w4a16_gemm(x_bits, w13, s13, topk_ids, topk_w, topk, group, False, dtype)
+    c1b = to_bits(c1, dtype)
+    c2b = silu_mul(c1b, dtype)
+    c3 = moe_w4a16_gemm(c2b, w2, s2, topk_ids, topk_w, 1, group, True, dtype)
+    c3b = to_bits(c3, dtype).reshape(T, topk, -1)
+    return moe_sum(c3b, dtype)

@@ -1,0 +1,328 @@
+"""Pins the CPU oracle against the known-answer vectors the reference's own tests hold, and against what the
+mathematics fixes.  No GPU."""
+import numpy as np
+import pytest
+import torch
+
+
+# ----------------------------------------------------------------------------- scalar formats
+def test_f16_roundtrip_all_codes(oracle):
+    bits = np.arange(65536, dtype=np.uint16)
+    f = oracle.f16_to_f32(bits)
+    ref = torch.from_numpy(bits.view(np.int16)).view(torch.float16).float().numpy()
+    ok = ~np.isnan(ref)  # NaN payloads may be quietened by the library
+    np.testing.assert_array_equal(f.view(np.uint32)[ok], ref.view(np.uint32)[ok])
+    assert np.all(np.isnan(f[~ok]))
+    finite = np.isfinite(f)
+    back = oracle.f32_to_f16(f[finite])
+    np.testing.assert_array_equal(back, bits[finite])
+
+
+def test_f32_to_f16_bf16_rne_matches_library(oracle):
+    rng = np.random.default_rng(1)
+    x = np.concatenate([
+        rng.standard_normal(200000).astype(np.float32) * 10,
+        (rng.standard_normal(50000) * 1e-6).astype(np.float32),
+        np.float32([65504, 65519.99, 65520, 1e9, -1e9, 2.0**-24, 2.0**-25, 1.5 * 2.0**-24, 0.0, -0.0]),
+    ])
+    # ties: value exactly halfway between two halfs / bfloat16s
+    ties = (np.arange(1, 4000, dtype=np.float32) * 2 + 1) * np.float32(2.0**-11)
+    x = np.concatenate([x, ties, ties * 8])
+    t = torch.from_numpy(x)
+    np.testing.assert_array_equal(oracle.f32_to_f16(x), t.half().view(torch.int16).numpy().view(np.uint16))
+    np.testing.assert_array_equal(oracle.f32_to_bf16(x), t.bfloat16().view(torch.int16).numpy().view(np.uint16))
+
+
+def test_e4m3_decode_table(oracle):
+    codes = np.arange(256, dtype=np.uint8)
+    f = oracle.e4m3_to_f32(codes)
+    ref = torch.from_numpy(codes).view(torch.float8_e4m3fn).float().numpy()
+    ok = ~np.isnan(ref)
+    np.testing.assert_array_equal(f[ok], ref[ok])
+    assert np.isnan(f[0x7F]) and np.isnan(f[0xFF])
+    assert f[0x7E] == 448.0 and f[0x01] == 2.0**-9 and f[0x08] == 2.0**-6
+
+
+def test_e4m3_encode_rne_satfinite(oracle):
+    # every code re-encodes to itself
+    codes = np.array([c for c in range(256) if c & 0x7F != 0x7F], dtype=np.uint8)
+    vals = oracle.e4m3_to_f32(codes)
+    back = oracle.f32_to_e4m3(vals)
+    # -0.0 keeps its sign bit
+    np.testing.assert_array_equal(back, codes)
+    # halfway points go to the even mantissa; values just off the tie go to the nearer neighbour
+    pos = oracle.e4m3_to_f32(np.arange(0, 0x7F, dtype=np.uint8))
+    mid = (pos[:-1].astype(np.float64) + pos[1:].astype(np.float64)) / 2
+    enc = oracle.f32_to_e4m3(mid.astype(np.float32))
+    lo = np.arange(0, 0x7E, dtype=np.uint8)
+    expect = np.where(lo % 2 == 0, lo, lo + 1)
+    np.testing.assert_array_equal(enc, expect)
+    np.testing.assert_array_equal(oracle.f32_to_e4m3(np.nextafter(mid.astype(np.float32), np.float32(0))), lo)
+    np.testing.assert_array_equal(oracle.f32_to_e4m3(np.nextafter(mid.astype(np.float32), np.float32(1e9))), lo + 1)
+    # SURVEY-noted library cross-check: 17->16, 19->20, 2^-10 -> 0, 1.5*2^-9 -> code 2
+    got = oracle.e4m3_to_f32(oracle.f32_to_e4m3(np.float32([17, 19, 2.0**-10, 1.5 * 2.0**-9])))
+    np.testing.assert_array_equal(got, np.float32([16, 20, 0, 2 * 2.0**-9]))
+    # saturation instead of NaN, both signs; inf saturates, NaN stays NaN
+    sat = oracle.f32_to_e4m3(np.float32([448, 449, 464, 465, 1e30, np.inf, -500, -np.inf]))
+    np.testing.assert_array_equal(sat, np.uint8([0x7E] * 6 + [0xFE] * 2))
+    assert oracle.f32_to_e4m3(np.float32([np.nan]))[0] & 0x7F == 0x7F
+    # random cross-check against torch's cast inside the finite range
+    rng = np.random.default_rng(2)
+    x = (rng.standard_normal(300000) * rng.choice([1e-3, 0.1, 1, 30, 200], 300000)).astype(np.float32)
+    x = np.clip(x, -448, 448)
+    ref = torch.from_numpy(x).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    np.testing.assert_array_equal(oracle.f32_to_e4m3(x), ref)
+
+
+# ----------------------------------------------------------------------------- checkpoint layouts
+def test_unpack_known_answer_0x66666666(oracle):
+    """S/models/quant/cutlass_utils_test.cpp:80-108: int32 1717986918 everywhere -> every packed byte == -18."""
+    q = np.full((64, 128), 1717986918, dtype=np.uint32)
+    for unpack in (oracle.gptq_unpack, oracle.awq_unpack):
+        codes = unpack(q)
+        signed = (codes.astype(np.int16) - 8).astype(np.int8)
+        packed = oracle.pack_int8_to_int4x2(signed)
+        assert np.all(packed == -18)
+
+
+def test_gptq_awq_unpack_positions(oracle):
+    # one distinct nibble per position fixes the order
+    word = sum(i << (4 * i) for i in range(8))  # nibble i holds value i
+    g = oracle.gptq_unpack(np.full((1, 1), word, np.uint32))
+    np.testing.assert_array_equal(g[:, 0], np.arange(8))
+    a = oracle.awq_unpack(np.full((1, 1), word, np.uint32))
+    # column 8j+i is read from nibble {0,4,1,5,2,6,3,7}[i]
+    np.testing.assert_array_equal(a[0], [0, 4, 1, 5, 2, 6, 3, 7])
+    rng = np.random.default_rng(0)
+    codes = rng.integers(0, 16, (64, 48), dtype=np.uint8)
+    np.testing.assert_array_equal(oracle.gptq_unpack(oracle.gptq_pack(codes)), codes)
+    np.testing.assert_array_equal(oracle.awq_unpack(oracle.awq_pack(codes)), codes)
+
+
+def test_marlin_repack_golden(oracle):
+    """S/models/quant/marlin_utils_test.cpp:29-91: arange(1024*1024) int32 viewed [1024,1024]."""
+    t = np.arange(1024 * 1024, dtype=np.uint32).reshape(1024, 1024)
+    awq = oracle.marlin_awq_repack(t)    # k=1024, n=8192
+    gptq = oracle.marlin_gptq_repack(t)  # k=8192, n=1024
+    assert gptq.shape == (512, 2048) and awq.shape == (64, 16384)
+    g, a = gptq.reshape(-1).view(np.int32), awq.reshape(-1).view(np.int32)
+    np.testing.assert_array_equal(g[:10], [34816, 286361600, 572688384, 859015168, 16448, 16448, 16448, 16448, 0, 0])
+    np.testing.assert_array_equal(a[:10], [285217024, 857879330, 1430541636, 2003203942, 285217024, 857879330,
+                                           1430541636, 2003203942, 285217024, 857879330])
+    np.testing.assert_array_equal(g[-10:], [-1029, -1029, 65535, 65535, 65535, 65535, 0, 0, 0, 0])
+    np.testing.assert_array_equal(a[-10:], [0] * 10)
+
+
+def test_marlin_awq_zero_points_golden(oracle):
+    """S/models/quant/marlin_utils_test.cpp:149-173."""
+    t = np.arange(1024 * 128, dtype=np.uint32).reshape(1024, 128)
+    zp = oracle.marlin_awq_zero_points(t)
+    assert zp.shape == (1024, 128)
+    z = zp.reshape(-1).view(np.int32)
+    np.testing.assert_array_equal(z[:10], [1966171168, 0, 0, 0, 0, 0, 0, 0, -38146904, 0])
+    np.testing.assert_array_equal(z[-10:], [-1, 0, -38146904, 286331153, -1, 0, -1, 0, -1, 0])
+
+
+def test_moe_layout_roundtrip_and_nibble_order(oracle):
+    w = np.zeros((1, 2, 4), np.uint8)
+    w[0, 1, 2] = 0xA3  # n=1, k=4 -> 3 ; k=5 -> 10
+    codes = oracle.moe_unpack(w)
+    assert codes[0, 4, 1] == 3 and codes[0, 5, 1] == 10 and codes.sum() == 13
+    rng = np.random.default_rng(0)
+    c = rng.integers(0, 16, (3, 32, 16), dtype=np.uint8)
+    np.testing.assert_array_equal(oracle.moe_unpack(oracle.moe_pack(c)), c)
+
+
+# ----------------------------------------------------------------------------- W4A16 numerics
+def test_dequant_all_zero_codes_is_minus_8(oracle):
+    """S/models/quant/quant_int4_weight_test.cpp:259-287 (CommonDeQuantTest)."""
+    codes = np.zeros((256, 32), np.uint8)
+    s = oracle.to_bits(np.ones((2, 32), np.float32), oracle.F16)
+    w = oracle.w4a16_dequant(codes, s, None, 128, oracle.F16)
+    assert np.all(w == -8.0)
+
+
+@pytest.mark.parametrize("dtype", [0, 1])
+def test_w4a16_gemm_vs_float64(oracle, dtype):
+    rng = np.random.default_rng(3)
+    M, N, K, G = 5, 96, 512, 128
+    codes = rng.integers(0, 16, (K, N), dtype=np.uint8)
+    zeros = rng.integers(6, 10, (K // G, N), dtype=np.uint8)
+    s_bits = oracle.to_bits(rng.uniform(0.003, 0.015, (K // G, N)).astype(np.float32), dtype)
+    x_bits = oracle.to_bits(rng.standard_normal((M, K)).astype(np.float32), dtype)
+    s = oracle.from_bits(s_bits, dtype).astype(np.float64)
+    x = oracle.from_bits(x_bits, dtype).astype(np.float64)
+    for z in (None, zeros):
+        zp = 8.0 if z is None else np.repeat(z, G, axis=0).astype(np.float64)
+        wref = (codes.astype(np.float64) - zp) * np.repeat(s, G, axis=0)
+        yref = x @ wref
+        y = oracle.w4a16_gemm(x_bits, codes, s_bits, z, G, dtype)
+        assert np.abs(y - yref).max() < 2e-5 * np.abs(yref).max() + 1e-5
+        w = oracle.w4a16_dequant(codes, s_bits, z, G, dtype)
+        np.testing.assert_array_equal(w, wref.astype(np.float32))
+        y64 = oracle.gemm_xw_f64(x_bits, w, dtype)
+        np.testing.assert_allclose(y64, yref, rtol=1e-12, atol=1e-12)
+
+
+# ----------------------------------------------------------------------------- fp8 quantizer
+TARGET_Q = [
+    0, 70, 78, 83, 86, 89, 91, 92, 94, 96, 97, 98, 99, 99, 100, 101, 102, 103, 104, 104, 105, 105,
+    106, 106, 107, 107, 107, 108, 108, 109, 109, 110, 110, 111, 111, 111, 112, 112, 112, 113, 113, 113, 113, 113,
+    114, 114, 114, 114, 115, 115, 115, 115, 115, 116, 116, 116, 116, 117, 117, 117, 117, 117, 118, 118, 118, 118,
+    119, 119, 119, 119, 119, 119, 120, 120, 120, 120, 120, 120, 121, 121, 121, 121, 121, 121, 121, 121, 121, 122,
+    122, 122, 122, 122, 122, 122, 122, 122, 123, 123, 123, 123, 123, 123, 123, 123, 123, 124, 124, 124, 124, 124,
+    124, 124, 124, 124, 125, 125, 125, 125, 125, 125, 125, 125, 125, 126, 126, 126, 126, 126, 118, 118, 118, 118,
+    118, 119, 119, 119, 119, 119, 119, 119, 119, 119, 120, 120, 120, 120, 120, 120, 120, 120, 120, 120, 120, 120,
+    120, 121, 121, 121, 121, 121, 121, 121, 121, 121, 121, 121, 121, 121, 121, 121, 121, 121, 121, 121, 122, 122,
+    122, 122, 122, 122, 122, 122, 122, 122, 122, 122, 122, 122, 122, 122, 122, 122, 123, 123, 123, 123, 123, 123,
+    123, 123, 123, 123, 123, 123, 123, 123, 123, 123, 123, 123, 123, 124, 124, 124, 124, 124, 124, 124, 124, 124,
+    124, 124, 124, 124, 124, 124, 124, 124, 124, 125, 125, 125, 125, 125, 125, 125, 125, 125, 125, 125, 125, 125,
+    125, 125, 125, 125, 125, 126, 126, 126, 126, 126, 126, 126, 126, 126]
+
+
+@pytest.mark.parametrize("dtype", [0, 1])
+@pytest.mark.parametrize("n", [128, 256])
+@pytest.mark.parametrize("colmajor", [False, True])
+def test_fp8_group_quant_known_answer(oracle, dtype, n, colmajor):
+    """K/others/sglang/main/quantization/fp8/per_token_group_quant_test.cu:77-98: x[i] = i/100, m = 1;
+    scales {0.0028, 0.0057} within 1e-4, codes within +-1 of the table (the table is shared by fp16 and bf16)."""
+    x = (np.arange(n, dtype=np.float32) / np.float32(100.0)).reshape(1, n)
+    xb = oracle.to_bits(x, dtype)
+    q, s = oracle.fp8_group_quant(xb, n, 128, colmajor, False, dtype)
+    s = s.reshape(-1)
+    np.testing.assert_allclose(s, [0.0028, 0.0057][: n // 128], atol=1e-4)
+    diff = np.abs(q.reshape(-1).astype(int) - np.array(TARGET_Q[:n]))
+    assert diff.max() <= 1
+    assert (diff == 0).mean() > 0.95
+
+
+def test_fp8_group_quant_closed_form(oracle):
+    rng = np.random.default_rng(5)
+    m, k = 7, 384
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    x[rng.random((m, k)) < 0.01] *= 20
+    x[3, 128:256] = 0  # an all-zero group hits the 1e-10 floor
+    for dtype in (0, 1):
+        xb = oracle.to_bits(x, dtype)
+        xr = oracle.from_bits(xb, dtype)
+        q, s = oracle.fp8_group_quant(xb, k, 128, False, False, dtype)
+        q2, s2 = oracle.fp8_group_quant(xb, k, 128, True, False, dtype)
+        np.testing.assert_array_equal(q, q2)
+        np.testing.assert_array_equal(s, s2.T)
+        amax = np.maximum(np.abs(xr).reshape(m, 3, 128).max(-1), np.float32(1e-10))
+        np.testing.assert_array_equal(s, amax / np.float32(448.0))
+        assert s[3, 1] == np.float32(1e-10) / np.float32(448.0) and np.all(q[3, 128:256] == 0)
+        # library cross-check: IEEE divide then torch's RNE cast (inputs never exceed 448 in magnitude)
+        r = xr.reshape(m, 3, 128) / s[:, :, None]
+        ref = torch.from_numpy(np.clip(r, -448, 448).reshape(m, k)).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+        np.testing.assert_array_equal(q, ref)
+        # the group's largest element always lands on +-448
+        assert np.all(np.abs(oracle.e4m3_to_f32(q)).reshape(m, 3, 128).max(-1)[amax > 1e-10] == 448.0)
+
+
+def test_fp8_group_quant_fused_silu_close_to_unfused(oracle):
+    rng = np.random.default_rng(6)
+    m, k = 4, 256
+    gu = rng.standard_normal((m, 2 * k)).astype(np.float32)
+    for dtype in (0, 1):
+        b = oracle.to_bits(gu, dtype)
+        f = oracle.from_bits(b, dtype)
+        act = oracle.to_bits(f[:, :k] / (1 + np.exp(-f[:, :k])) * f[:, k:], dtype)
+        q0, s0 = oracle.fp8_group_quant(act, k, 128, True, False, dtype)
+        q1, s1 = oracle.fp8_group_quant(b, k, 128, True, True, dtype)
+        np.testing.assert_allclose(s1, s0, rtol=2e-2)
+        assert (np.abs(q1.astype(int) - q0.astype(int)) <= 1).mean() > 0.99
+
+
+# ----------------------------------------------------------------------------- blockwise fp8 GEMM
+def test_fp8_blockwise_gemm_vs_float64(oracle):
+    rng = np.random.default_rng(7)
+    m, n, k = 5, 200, 384  # n not a multiple of 128: last scale row is partial
+    w = (rng.standard_normal((n, k)) * 0.02).astype(np.float32)
+    bq, bs = oracle.fp8_block_quant_weight(w)
+    assert bs.shape == (2, 3)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    aq, a_s = oracle.fp8_group_quant(oracle.to_bits(x, 1), k, 128, True, False, 1)
+    out = oracle.fp8_blockwise_gemm(aq, a_s, bq, bs, True)
+    out_rm = oracle.fp8_blockwise_gemm(aq, np.ascontiguousarray(a_s.T), bq, bs, False)
+    np.testing.assert_array_equal(out, out_rm)
+    A = oracle.e4m3_to_f32(aq).astype(np.float64) * np.repeat(a_s.T.astype(np.float64), 128, axis=1)
+    B = oracle.e4m3_to_f32(bq).astype(np.float64) * np.repeat(np.repeat(bs.astype(np.float64), 128, 0)[:n], 128, 1)
+    ref = A @ B.T
+    assert np.abs(out - ref).max() < 1e-5 * np.abs(ref).max()
+    # quantization itself stays close to the unquantized product
+    full = x.astype(np.float64) @ w.astype(np.float64).T
+    assert np.linalg.norm(ref - full) / np.linalg.norm(full) < 0.06
+    # weight block scale = amax/448 and block maxima land on 448
+    blk = np.abs(w[:128, :128]).max()
+    assert bs[0, 0] == np.float32(blk) / np.float32(448.0)
+
+
+# ----------------------------------------------------------------------------- MoE
+def test_moe_align_worked_example(oracle):
+    """K/moe_utils/moe_utils.cu:150-156."""
+    ids = [0, 1, 2, 1, 2, 3, 0, 3, 4]
+    sorted_ids, expert_ids, npp = oracle.moe_align(ids, 5, 4)
+    P = 9
+    np.testing.assert_array_equal(sorted_ids[:20], [0, 6, P, P, 1, 3, P, P, 2, 4, P, P, 5, 7, P, P, 8, P, P, P])
+    assert npp == 20
+    np.testing.assert_array_equal(expert_ids[:5], [0, 1, 2, 3, 4])
+
+
+def test_moe_align_invariants(oracle):
+    rng = np.random.default_rng(8)
+    for E, bm, numel in [(256, 16, 8), (256, 64, 4096), (8, 4, 0), (3, 1, 50)]:
+        ids = rng.integers(0, E, numel).astype(np.int32)
+        s, e, npp = oracle.moe_align(ids, E, bm)
+        counts = np.bincount(ids, minlength=E)
+        assert npp == int((np.ceil(counts / bm) * bm).sum())
+        assert np.all(s[npp:] == numel)
+        real = s[:npp][s[:npp] < numel]
+        assert sorted(real.tolist()) == list(range(numel))
+        for b in range(npp // bm):
+            seg = s[b * bm:(b + 1) * bm]
+            seg = seg[seg < numel]
+            assert np.all(ids[seg] == e[b]) and np.all(np.diff(seg) > 0)
+        # stable: inside an expert ids ascend across blocks too
+        for ex in np.unique(ids):
+            pos = real[ids[real] == ex]
+            assert np.all(np.diff(pos) > 0)
+
+
+def test_moe_gemm_matches_dense_dequant(oracle):
+    rng = np.random.default_rng(9)
+    E, N, K, G, T, topk = 6, 32, 256, 128, 5, 2
+    codes = rng.integers(0, 16, (E, K, N), dtype=np.uint8)
+    w = oracle.moe_pack(codes)
+    dtype = 1
+    s_bits = oracle.to_bits(rng.uniform(0.002, 0.01, (E, N, K // G)).astype(np.float32), dtype)
+    x_bits = oracle.to_bits(rng.standard_normal((T, K)).astype(np.float32), dtype)
+    ids = np.stack([rng.choice(E, topk, replace=False) for _ in range(T)]).astype(np.int32)
+    tw = rng.random((T, topk)).astype(np.float32)
+    out = oracle.moe_w4a16_gemm(x_bits, w, s_bits, ids, tw, topk, G, True, dtype)
+    x = oracle.from_bits(x_bits, dtype).astype(np.float64)
+    s = oracle.from_bits(s_bits, dtype).astype(np.float64)
+    for t in range(T):
+        for j in range(topk):
+            e = ids[t, j]
+            wd = (codes[e].astype(np.float64) - 8) * np.repeat(s[e].T, G, axis=0)  # [K, N]
+            ref = x[t] @ wd * tw[t, j]
+            np.testing.assert_allclose(out[t * topk + j], ref, rtol=1e-4, atol=1e-5)
+
+
+def test_silu_mul_and_moe_sum(oracle):
+    rng = np.random.default_rng(10)
+    x = rng.standard_normal((3, 64)).astype(np.float32)
+    for dtype in (0, 1):
+        xb = oracle.to_bits(x, dtype)
+        xf = oracle.from_bits(xb, dtype)
+        out = oracle.from_bits(oracle.silu_mul(xb, dtype), dtype)
+        ref = oracle.from_bits(oracle.to_bits(xf[:, :32] / (1 + np.exp(-xf[:, :32])) * xf[:, 32:], dtype), dtype)
+        assert np.abs(out - ref).max() <= np.abs(ref).max() * 2.0**-7
+        y = rng.standard_normal((2, 8, 16)).astype(np.float32)
+        yb = oracle.to_bits(y, dtype)
+        tt = torch.from_numpy(oracle.from_bits(yb, dtype)).to(torch.float16 if dtype == 0 else torch.bfloat16)
+        acc = torch.zeros_like(tt[:, 0])
+        for j in range(8):
+            acc = acc + tt[:, j]
+        np.testing.assert_array_equal(oracle.from_bits(oracle.moe_sum(yb, dtype), dtype), acc.float().numpy())
