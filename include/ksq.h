@@ -1,0 +1,190 @@
+/*
+ * ksq.h - C-ABI of libksq_hip.so, the MI355X (gfx950) quantized-GEMM kernel library that sits under
+ * KsanaLLM's matmul / MoE layer classes.
+ *
+ * Conventions
+ *   - plain pointers and sizes only; every device pointer is caller-owned HBM;
+ *   - `stream` is a hipStream_t passed as void* (NULL = default stream);
+ *   - every function that launches work returns an int status (KSQ_OK == 0), never allocates device memory,
+ *     never synchronizes; ksq_last_error_string() explains the last non-zero status of the calling thread;
+ *   - `dtype` is the activation/output/scale type T of the reference's templates (KSQ_F16 or KSQ_BF16);
+ *   - 16-byte alignment is required of every device pointer.
+ *
+ * Citations name the reference interface each entry point replaces:
+ *   S/ = src/ksana_llm/      K/ = 3rdparty/LLM_kernels/csrc/kernels/nvidia/
+ */
+#ifndef KSQ_H_
+#define KSQ_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define KSQ_VERSION 1
+
+/* status codes */
+enum {
+  KSQ_OK = 0,
+  KSQ_ERR_INVALID_ARGUMENT = 1, /* null pointer, misaligned pointer, zero / non-conforming size */
+  KSQ_ERR_UNSUPPORTED = 2,      /* valid request the library has no kernel for (dtype, group size ...) */
+  KSQ_ERR_WORKSPACE = 3,        /* workspace smaller than ksq_*_workspace_size() reported */
+  KSQ_ERR_LAUNCH = 4            /* hipGetLastError() after the launch was not hipSuccess */
+};
+
+/* element type tags */
+enum { KSQ_F16 = 0, KSQ_BF16 = 1, KSQ_F32 = 2 };
+
+/* checkpoint-side int4 weight layouts accepted by the repack (what the loader holds after slicing) */
+enum {
+  KSQ_SRC_GPTQ = 0,    /* [E][K/8, N] int32, nibble i of a word = row 8*(k/8)+i     (S/models/quant/cutlass_utils.cpp:41-50) */
+  KSQ_SRC_AWQ = 1,     /* [E][K, N/8] int32, AWQ column order {0,2,4,6,1,3,5,7}     (S/models/quant/cutlass_utils.cpp:12-38) */
+  KSQ_SRC_MOE_NK = 2,  /* [E, N, K/2] uint8, low nibble = even k                    (S/models/quant/quant_weight.cpp:182-319) */
+  KSQ_SRC_INT4X2_KN = 3 /* [E][K, N/2] int8, two signed nibbles (code-8), low = even n (S/models/quant/cutlass_utils.cpp:53-59) */
+};
+
+/* scale / zero-point source layouts */
+enum {
+  KSQ_SCALE_GN = 0, /* [E][K/group, N]   dense GPTQ / AWQ checkpoints */
+  KSQ_SCALE_NG = 1  /* [E, N, K/group]   MoE expert stacks (S/models/quant/quant_weight.cpp:182-319) */
+};
+enum {
+  KSQ_ZERO_AWQ_PACKED = 0, /* [K/group, N/8] int32 in AWQ column order (qzeros as stored in the checkpoint) */
+  KSQ_ZERO_U8_GN = 1       /* [K/group, N] uint8 codes 0..15 */
+};
+
+int ksq_version(void);
+
+/* Replaces the cudaGetErrorString / KLLM_KERNEL_CHECK text paths.  Thread-local, never NULL. */
+const char* ksq_last_error_string(void);
+
+/* ------------------------------------------------------------------------------------------------------------------
+ * Load-time repack: checkpoint layout <-> CDNA4 tile layout.
+ *
+ * The packed weight is a sequence of 1 KiB tiles, tile (e, n/16, k/128) at ((e*N/16 + n/16)*(K/128) + k/128).
+ * Inside a tile, wavefront lane l = 16*((k%32)/8) + n%16 owns 16 bytes; dword d = (k%128)/32 of those bytes holds
+ * the eight codes k%8 = {0,2,4,6,1,3,5,7} from nibble 0 upward, so `(w >> 4i) & 0x000F000F` is the MFMA operand
+ * pair (k=2i, k=2i+1).  Scales are [e][n/16][K/group][16] in T, zero points the same shape in uint8.
+ * K must be a multiple of 128, N of 16, group one of 32/64/128.
+ *
+ * Replaces fast_preprocess_weights_for_mixed_gemm (K/asymmetric_gemm/cutlass_preprocessors_fast.cu:370),
+ * gptq_marlin_repack / awq_marlin_repack (K/gptq_marlin/gptq_marlin_repack.cu:276-295, awq_marlin_repack.cu:208-222),
+ * machete_prepack_weight (K/machete/machete_wrapper.h:38-109), permute_scales (K/gptq_marlin/gptq_marlin.cu:641-682)
+ * and the AWQ zero-point conversions (S/models/quant/quant_weight.cpp:716-753, S/models/quant/marlin_utils.cpp:36-104).
+ * ------------------------------------------------------------------------------------------------------------------ */
+size_t ksq_w4a16_packed_weight_bytes(size_t E, size_t K, size_t N);
+size_t ksq_w4a16_packed_scales_bytes(size_t E, size_t K, size_t N, size_t group, int dtype);
+size_t ksq_w4a16_packed_zeros_bytes(size_t E, size_t K, size_t N, size_t group);
+
+int ksq_w4a16_repack(const void* src, int src_layout, void* dst_packed, size_t E, size_t K, size_t N, void* stream);
+/* exact inverse of ksq_w4a16_repack for every src_layout */
+int ksq_w4a16_unpack(const void* packed, int dst_layout, void* dst, size_t E, size_t K, size_t N, void* stream);
+
+int ksq_w4a16_repack_scales(const void* src, int src_layout, void* dst_packed, size_t E, size_t K, size_t N,
+                            size_t group, int dtype, void* stream);
+int ksq_w4a16_unpack_scales(const void* packed, int dst_layout, void* dst, size_t E, size_t K, size_t N, size_t group,
+                            int dtype, void* stream);
+int ksq_w4a16_repack_zeros(const void* src, int src_layout, void* dst_packed, size_t K, size_t N, size_t group,
+                           void* stream);
+int ksq_w4a16_unpack_zeros(const void* packed, int dst_layout, void* dst, size_t K, size_t N, size_t group,
+                           void* stream);
+
+/* ------------------------------------------------------------------------------------------------------------------
+ * W4A16 group-wise GEMM: y[m,n] = x[m,k] . ((code - zp) * scale), zp = 8 when zeros_packed == NULL (GPTQ symmetric),
+ * else the per-(group,n) zero point (AWQ).  x, y row-major T; weights / scales / zeros in the packed layout above.
+ * The kernel variant (decode split-K vs MFMA tile, tile sizes) is chosen internally by ksq_select_tile.
+ *
+ * Replaces InvokeFpAIntBGroupCudaGemm / InvokeFpAIntBGroupCutlassGemm / InvokeMarlinGemm / InvokeMacheteGemm
+ * (S/kernels/nvidia/basic_kernel_wrapper.h:32-115) and their workspace probes
+ * (GetFpAIntBGroupCutlassGemmWorkspaceSize, GetMarlinWorkspace K/gptq_marlin/gptq_marlin.cu:610-638).
+ * ------------------------------------------------------------------------------------------------------------------ */
+size_t ksq_w4a16_workspace_size(size_t max_m, size_t n, size_t k, size_t group, int dtype);
+int ksq_w4a16_gemm(void* y, const void* x, const void* w_packed, const void* scales_packed, const void* zeros_packed,
+                   void* workspace, size_t workspace_bytes, size_t m, size_t n, size_t k, size_t group, int dtype,
+                   void* stream);
+
+/* ------------------------------------------------------------------------------------------------------------------
+ * FP8 (OCP e4m3) per-token, per-`group`-channel activation quantizer.
+ *   amax = max(1e-10, max|x|); s = amax / 448; q = e4m3_rne_satfinite(x / s)   (IEEE fp32 divisions)
+ * x [m, k] T (or [m, 2k] when fuse_silu_mul: x = T(silu(x[:, :k]) * x[:, k:])), q [m, k] bytes,
+ * s fp32 [m, k/group] or, when column_major, [k/group, m].
+ * Replaces InvokePerTokenGroupQuantFp8E4m3 (S/kernels/nvidia/basic_kernel_wrapper.cpp:1222-1232;
+ * K/others/sglang/main/quantization/fp8/per_token_group_quant.cu:275-329).
+ * ------------------------------------------------------------------------------------------------------------------ */
+int ksq_fp8_group_quant(const void* x, void* q, void* s, size_t m, size_t k, size_t group, int column_major,
+                        int fuse_silu_mul, int dtype, void* stream);
+
+/* ------------------------------------------------------------------------------------------------------------------
+ * Blockwise FP8 GEMM: out[m,n] = sum_kb (a_q[m,kb] . b[n,kb]) * a_s[kb,m] * b_s[n/128,kb], fp32 accumulate.
+ * a_q [m,k] e4m3 row-major, a_s fp32 column-major [k/128, m], b [n,k] e4m3 row-major (checkpoint layout, no repack),
+ * b_s fp32 [ceil(n/128), k/128], out [m,n] in out_dtype.  k must be a multiple of 128, n of 16.
+ * Replaces InvokeBlockGemm / InvokeGetBlockGemmWorkspaceSize (K/blockwise_gemm/blockwise_gemm.cu:17-33) and
+ * DeepGEMMWrapper::Gemm / GemmSwapAB (K/gemm/deepgemm/deepgemm_wrapper.cu:33-103).
+ * ------------------------------------------------------------------------------------------------------------------ */
+size_t ksq_fp8_blockwise_workspace_size(size_t max_m, size_t n, size_t k);
+int ksq_fp8_blockwise_gemm(const void* a_q, const void* a_s, const void* b, const void* b_s, void* out, size_t m,
+                           size_t n, size_t k, int out_dtype, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------------------------------------------------
+ * MoE: expert-offset / permutation build, grouped W4A16 GEMM, silu*mul, top-k sum.
+ * ------------------------------------------------------------------------------------------------------------------ */
+
+/* Counting sort of topk_ids[numel] (int32, ids outside [0,E) are dropped) by expert, every expert's segment padded
+ * to a multiple of block_m with the value `numel`; order inside an expert is ascending flat index (deterministic,
+ * unlike the atomic rank of sgl_moe_token_sort_kernel).  sorted_ids has ksq_moe_align_capacity() entries and is
+ * completely written; expert_ids has capacity/block_m entries, num_post_pad one.  `scratch` is
+ * ksq_moe_align_scratch_bytes() of device memory.
+ * Replaces InvokeSglMoeAlignBlockSize / InvokeMoeAlignBlockSize / InvokeFillIntToBuffer
+ * (K/moe_utils/moe_utils.cu:660-755). */
+size_t ksq_moe_align_capacity(size_t numel, size_t E, size_t block_m);
+size_t ksq_moe_align_scratch_bytes(size_t numel, size_t E);
+int ksq_moe_align(const void* topk_ids, size_t numel, size_t E, size_t block_m, void* sorted_ids, void* expert_ids,
+                  void* num_post_pad, void* scratch, void* stream);
+
+/* Grouped GEMM over the aligned blocks: for every valid sorted slot id s (< numel)
+ *   out[s, :] = x[s / top_k, :] . dequant(W[expert of s's block]) * (topk_w ? topk_w[s] : 1)
+ * x [rows, k] T, out [numel, n] T, W/scales packed per expert as by ksq_w4a16_repack(E = experts),
+ * zeros_packed NULL for symmetric (code-8).  top_k = 1 reads x rows by slot (second MoE GEMM).
+ * Replaces InvokeMoeWna16Gemm (K/moe/moe_wna16/moe_wna16.cu:263-288) and the Triton
+ * InvokeFusedMoeGptqAwqKernel (S/kernels/nvidia/triton_wrapper.h:68-75). */
+int ksq_moe_w4a16_gemm(void* out, const void* x, const void* w_packed, const void* scales_packed,
+                       const void* zeros_packed, const void* topk_w, const void* sorted_ids, const void* expert_ids,
+                       const void* num_post_pad, size_t numel, size_t top_k, size_t E, size_t n, size_t k,
+                       size_t group, size_t block_m, int dtype, void* stream);
+
+/* out[r, i] = T(silu(x[r, i]) * x[r, inter + i]), fp32 math a / (1 + expf(-a)) * b.
+ * Replaces InvokeSiluAndMul (K/moe_utils/moe_utils.cu:893-905). */
+int ksq_moe_silu_mul(const void* x, void* out, size_t rows, size_t inter, int dtype, void* stream);
+
+/* out[t, :] = sum_j in[t, j, :], accumulated in T precision in ascending j.
+ * Replaces InvokeMoeSum (K/moe_utils/moe_utils.cu:789-835). */
+int ksq_moe_sum(const void* in, void* out, size_t tokens, size_t topk, size_t d, int dtype, void* stream);
+
+/* ------------------------------------------------------------------------------------------------------------------
+ * Per-shape tile selection: a pure host function of (kind, m, n, k, dtype); no timing, no device access.
+ * Replaces GetBestConfigIndex (K/asymmetric_gemm/asymmetric_gemm_wrapper.cu:101-146), machete_best_schedule
+ * (K/machete/machete_wrapper.h:38-109), get_best_gemm_config (K/others/tensorrt-llm/dev/deep_gemm/jit_utils.cuh:143-222)
+ * and the threshold sweep of BlockwiseMatMulLayer::Preprocess (S/layers/nvidia/blockwise_matmul_layer.cpp:71-181).
+ * ------------------------------------------------------------------------------------------------------------------ */
+enum { KSQ_KIND_W4A16 = 0, KSQ_KIND_FP8_BLOCKWISE = 1, KSQ_KIND_MOE_W4A16 = 2 };
+enum { KSQ_KERNEL_SPLITK_WAVE = 0, KSQ_KERNEL_MFMA_TILE = 1 };
+
+typedef struct ksq_tile_desc {
+  int32_t kernel;   /* KSQ_KERNEL_* */
+  int32_t block_m;  /* rows of x / tokens per workgroup */
+  int32_t block_n;  /* output columns per workgroup */
+  int32_t block_k;  /* k extent of one main-loop stage */
+  int32_t waves;    /* wavefronts (64 lanes) per workgroup */
+  int32_t split_k;  /* k slices reduced inside the kernel (across wavefronts and/or workgroups) */
+  int32_t grid;     /* workgroups launched */
+  int32_t reserved;
+} ksq_tile_desc;
+
+int ksq_select_tile(int kind, size_t m, size_t n, size_t k, int dtype, ksq_tile_desc* out_desc);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KSQ_H_ */

@@ -1,0 +1,97 @@
+// Shared host/device helpers of libksq_hip (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <cstdarg>
+#include <cstdio>
+
+#include "ksq.h"
+
+#define KSQ_EXPORT extern "C" __attribute__((visibility("default")))
+
+namespace ksq {
+
+// ---------------------------------------------------------------------------------------------- errors
+void set_error(const char* fmt, ...);
+int fail(int code, const char* fmt, ...);
+int check_launch(const char* what);
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
+
+// ---------------------------------------------------------------------------------------------- vector types
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+
+struct F16 {
+  static constexpr int kTag = KSQ_F16;
+  // 0x6400 | code is the half 1024 + code
+  static constexpr uint32_t kMagic2 = 0x64006400u;
+  static constexpr float kMagic = 1024.0f;
+  typedef f16x8 frag;
+  static __device__ __forceinline__ f32x4 mfma(frag a, frag b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ float to_float(uint16_t b) {
+    return static_cast<float>(__builtin_bit_cast(_Float16, b));
+  }
+  static __device__ __forceinline__ uint16_t from_float(float f) {
+    return __builtin_bit_cast(uint16_t, static_cast<_Float16>(f));
+  }
+  static constexpr uint32_t kOne2 = 0x3c003c00u;  // (1.0, 1.0)
+};
+
+struct BF16 {
+  static constexpr int kTag = KSQ_BF16;
+  // 0x4300 | code is the bfloat16 128 + code
+  static constexpr uint32_t kMagic2 = 0x43004300u;
+  static constexpr float kMagic = 128.0f;
+  typedef bf16x8 frag;
+  static __device__ __forceinline__ f32x4 mfma(frag a, frag b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ float to_float(uint16_t b) {
+    return __builtin_bit_cast(float, static_cast<uint32_t>(b) << 16);
+  }
+  // round-to-nearest-even, NaN kept quiet
+  static __device__ __forceinline__ uint16_t from_float(float f) {
+    uint32_t x = __builtin_bit_cast(uint32_t, f);
+    if ((x & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((x >> 16) | 0x40u);
+    x += 0x7fffu + ((x >> 16) & 1u);
+    return static_cast<uint16_t>(x >> 16);
+  }
+  static constexpr uint32_t kOne2 = 0x3f803f80u;
+};
+
+template <typename T>
+__device__ __forceinline__ typename T::frag as_frag(u32x4 v) {
+  return __builtin_bit_cast(typename T::frag, v);
+}
+
+// Eight int4 codes of one packed dword -> the MFMA operand (k pairs in ascending order), each element holding
+// magic + code.  Nibble i and nibble i+4 are the pair (k = 2i, k = 2i+1).
+template <typename T>
+__device__ __forceinline__ typename T::frag dequant_magic(uint32_t w) {
+  u32x4 v;
+  v.x = (w & 0x000f000fu) | T::kMagic2;
+  v.y = ((w >> 4) & 0x000f000fu) | T::kMagic2;
+  v.z = ((w >> 8) & 0x000f000fu) | T::kMagic2;
+  v.w = ((w >> 12) & 0x000f000fu) | T::kMagic2;
+  return as_frag<T>(v);
+}
+
+__device__ __forceinline__ uint32_t pack2(uint16_t lo, uint16_t hi) {
+  return static_cast<uint32_t>(lo) | (static_cast<uint32_t>(hi) << 16);
+}
+
+inline size_t div_up(size_t a, size_t b) { return (a + b - 1) / b; }
+
+}  // namespace ksq

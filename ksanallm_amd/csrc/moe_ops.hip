@@ -1,0 +1,212 @@
+// MoE helpers around the grouped GEMM: expert-offset / permutation build, silu*mul, top-k sum.
+#include "ksq_common.h"
+
+namespace ksq {
+namespace {
+
+constexpr int kAlignThreads = 1024;
+
+// Stable counting sort by expert in one workgroup.
+//   chunk c (one thread) owns ids [c*per, (c+1)*per); cnt[c+1][e] = #ids == e in chunk c  (global scratch)
+//   column scan over chunks turns cnt[c][e] into "ids == e before chunk c";  padded totals are scanned over experts
+//   in LDS; every chunk then places its ids in order, so positions inside an expert ascend with the flat index.
+__global__ void __launch_bounds__(kAlignThreads) moe_align_kernel(const int32_t* __restrict__ ids, uint32_t numel,
+                                                                  uint32_t E, uint32_t block_m, uint32_t capacity,
+                                                                  int32_t* __restrict__ sorted, int32_t* __restrict__ expert_ids,
+                                                                  int32_t* __restrict__ num_post_pad,
+                                                                  int32_t* __restrict__ cnt, uint32_t chunks,
+                                                                  uint32_t per) {
+  extern __shared__ int32_t lds[];  // [2][E_pad + 1] ping-pong scan buffers
+  const uint32_t tid = threadIdx.x;
+  const uint32_t EP = E + 1;
+  int32_t* scan_a = lds;
+  int32_t* scan_b = lds + EP;
+
+  // fill: every slot starts as padding
+  for (uint32_t i = tid; i < capacity; i += kAlignThreads) sorted[i] = static_cast<int32_t>(numel);
+  // clear counters
+  for (uint32_t i = tid; i < (chunks + 1) * E; i += kAlignThreads) cnt[i] = 0;
+  __syncthreads();
+
+  const uint32_t begin = tid * per;
+  const uint32_t end = (begin + per < numel) ? begin + per : numel;
+  if (tid < chunks) {
+    for (uint32_t i = begin; i < end; ++i) {
+      uint32_t e = static_cast<uint32_t>(ids[i]);
+      if (e < E) cnt[(tid + 1) * E + e] += 1;
+    }
+  }
+  __syncthreads();
+
+  // per expert: running sum over chunks
+  for (uint32_t e = tid; e < E; e += kAlignThreads) {
+    int32_t run = 0;
+    for (uint32_t c = 1; c <= chunks; ++c) {
+      run += cnt[c * E + e];
+      cnt[c * E + e] = run;
+    }
+    // cnt[chunks][e] == total of expert e ; padded size goes into the scan buffer (shifted by one: exclusive scan)
+    scan_a[e + 1] = (run + static_cast<int32_t>(block_m) - 1) / static_cast<int32_t>(block_m) * static_cast<int32_t>(block_m);
+  }
+  if (tid == 0) scan_a[0] = 0;
+  __syncthreads();
+
+  // inclusive Hillis-Steele scan over EP entries -> scan[e] = first slot of expert e, scan[E] = padded total
+  int32_t* src = scan_a;
+  int32_t* dst = scan_b;
+  for (uint32_t off = 1; off < EP; off <<= 1) {
+    for (uint32_t i = tid; i < EP; i += kAlignThreads) dst[i] = src[i] + (i >= off ? src[i - off] : 0);
+    __syncthreads();
+    int32_t* t = src;
+    src = dst;
+    dst = t;
+  }
+  const int32_t* first = src;
+
+  if (tid == 0) num_post_pad[0] = first[E];
+  for (uint32_t e = tid; e < E; e += kAlignThreads)
+    for (int32_t s = first[e]; s < first[e + 1]; s += static_cast<int32_t>(block_m)) expert_ids[s / static_cast<int32_t>(block_m)] = static_cast<int32_t>(e);
+
+  if (tid < chunks) {
+    for (uint32_t i = begin; i < end; ++i) {
+      uint32_t e = static_cast<uint32_t>(ids[i]);
+      if (e < E) {
+        int32_t r = cnt[tid * E + e];
+        cnt[tid * E + e] = r + 1;
+        sorted[first[e] + r] = static_cast<int32_t>(i);
+      }
+    }
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) silu_mul_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ out,
+                                                       size_t rows, uint32_t inter) {
+  // 8 elements per thread
+  const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  const size_t per_row = inter / 8;
+  if (i >= rows * per_row) return;
+  const size_t r = i / per_row;
+  const uint32_t c = static_cast<uint32_t>(i % per_row) * 8;
+  const uint16_t* a = x + r * 2 * inter + c;
+  u32x4 ra = *reinterpret_cast<const u32x4*>(a);
+  u32x4 rb = *reinterpret_cast<const u32x4*>(a + inter);
+  u32x4 o;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    float a0 = T::to_float(static_cast<uint16_t>(ra[j] & 0xffffu)), a1 = T::to_float(static_cast<uint16_t>(ra[j] >> 16));
+    float b0 = T::to_float(static_cast<uint16_t>(rb[j] & 0xffffu)), b1 = T::to_float(static_cast<uint16_t>(rb[j] >> 16));
+    float y0 = a0 / (1.0f + expf(-a0)) * b0;
+    float y1 = a1 / (1.0f + expf(-a1)) * b1;
+    o[j] = pack2(T::from_float(y0), T::from_float(y1));
+  }
+  *reinterpret_cast<u32x4*>(out + r * inter + c) = o;
+}
+
+// sum over top-k in T precision, ascending j (each partial sum is rounded to T like the reference's `scalar_t x`)
+template <typename T>
+__global__ void __launch_bounds__(256) moe_sum_kernel(const uint16_t* __restrict__ in, uint16_t* __restrict__ out,
+                                                      size_t tokens, uint32_t topk, uint32_t d) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  const size_t per_row = d / 8;
+  if (i >= tokens * per_row) return;
+  const size_t t = i / per_row;
+  const uint32_t c = static_cast<uint32_t>(i % per_row) * 8;
+  float acc[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) acc[j] = 0.f;
+  for (uint32_t s = 0; s < topk; ++s) {
+    u32x4 r = *reinterpret_cast<const u32x4*>(in + (t * topk + s) * d + c);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      acc[2 * j] = T::to_float(T::from_float(acc[2 * j] + T::to_float(static_cast<uint16_t>(r[j] & 0xffffu))));
+      acc[2 * j + 1] = T::to_float(T::from_float(acc[2 * j + 1] + T::to_float(static_cast<uint16_t>(r[j] >> 16))));
+    }
+  }
+  u32x4 o;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) o[j] = pack2(T::from_float(acc[2 * j]), T::from_float(acc[2 * j + 1]));
+  *reinterpret_cast<u32x4*>(out + t * d + c) = o;
+}
+
+void align_geometry(size_t numel, uint32_t* chunks, uint32_t* per) {
+  size_t c = div_up(numel, 8);
+  if (c < 1) c = 1;
+  if (c > kAlignThreads) c = kAlignThreads;
+  *chunks = static_cast<uint32_t>(c);
+  *per = static_cast<uint32_t>(div_up(numel, c));
+}
+
+}  // namespace
+}  // namespace ksq
+
+using namespace ksq;
+
+KSQ_EXPORT size_t ksq_moe_align_capacity(size_t numel, size_t E, size_t block_m) {
+  if (block_m == 0) return 0;
+  return numel + E * (block_m - 1);
+}
+
+KSQ_EXPORT size_t ksq_moe_align_scratch_bytes(size_t numel, size_t E) {
+  uint32_t chunks, per;
+  align_geometry(numel, &chunks, &per);
+  return (static_cast<size_t>(chunks) + 1) * E * sizeof(int32_t);
+}
+
+KSQ_EXPORT int ksq_moe_align(const void* topk_ids, size_t numel, size_t E, size_t block_m, void* sorted_ids,
+                             void* expert_ids, void* num_post_pad, void* scratch, void* stream) {
+  const char* fn = "ksq_moe_align";
+  if (!sorted_ids || !expert_ids || !num_post_pad || !scratch || (!topk_ids && numel))
+    return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: null pointer", fn);
+  if (E == 0 || E > 4096) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: expert count %zu outside 1..4096", fn, E);
+  if (block_m == 0 || block_m > 1024) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: block_m %zu outside 1..1024", fn, block_m);
+  const size_t cap = ksq_moe_align_capacity(numel, E, block_m);
+  if (cap > 0x7fffffffull) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: too many ids", fn);
+  uint32_t chunks, per;
+  align_geometry(numel, &chunks, &per);
+  const size_t lds = 2 * (E + 1) * sizeof(int32_t);
+  moe_align_kernel<<<1, kAlignThreads, lds, as_stream(stream)>>>(
+      static_cast<const int32_t*>(topk_ids), static_cast<uint32_t>(numel), static_cast<uint32_t>(E),
+      static_cast<uint32_t>(block_m), static_cast<uint32_t>(cap), static_cast<int32_t*>(sorted_ids),
+      static_cast<int32_t*>(expert_ids), static_cast<int32_t*>(num_post_pad), static_cast<int32_t*>(scratch), chunks,
+      per);
+  return check_launch(fn);
+}
+
+KSQ_EXPORT int ksq_moe_silu_mul(const void* x, void* out, size_t rows, size_t inter, int dtype, void* stream) {
+  const char* fn = "ksq_moe_silu_mul";
+  if (!x || !out) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: null pointer", fn);
+  if (!aligned16(x) || !aligned16(out)) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: pointers must be 16-byte aligned", fn);
+  if (inter == 0 || inter % 8 != 0 || inter > 0x7fffffffull)
+    return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: inter must be a positive multiple of 8", fn);
+  if (dtype != KSQ_F16 && dtype != KSQ_BF16) return fail(KSQ_ERR_UNSUPPORTED, "%s: dtype must be f16 or bf16", fn);
+  if (rows == 0) return KSQ_OK;
+  const size_t blocks = div_up(rows * (inter / 8), 256);
+  if (blocks > 0x7fffffffull) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: tensor too large", fn);
+  const uint16_t* xp = static_cast<const uint16_t*>(x);
+  uint16_t* op = static_cast<uint16_t*>(out);
+  if (dtype == KSQ_F16)
+    silu_mul_kernel<F16><<<static_cast<unsigned>(blocks), 256, 0, as_stream(stream)>>>(xp, op, rows, static_cast<uint32_t>(inter));
+  else
+    silu_mul_kernel<BF16><<<static_cast<unsigned>(blocks), 256, 0, as_stream(stream)>>>(xp, op, rows, static_cast<uint32_t>(inter));
+  return check_launch(fn);
+}
+
+KSQ_EXPORT int ksq_moe_sum(const void* in, void* out, size_t tokens, size_t topk, size_t d, int dtype, void* stream) {
+  const char* fn = "ksq_moe_sum";
+  if (!in || !out) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: null pointer", fn);
+  if (!aligned16(in) || !aligned16(out)) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: pointers must be 16-byte aligned", fn);
+  if (d == 0 || d % 8 != 0 || d > 0x7fffffffull || topk == 0 || topk > 0x7fffffffull)
+    return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: d must be a positive multiple of 8 and topk positive", fn);
+  if (dtype != KSQ_F16 && dtype != KSQ_BF16) return fail(KSQ_ERR_UNSUPPORTED, "%s: dtype must be f16 or bf16", fn);
+  if (tokens == 0) return KSQ_OK;
+  const size_t blocks = div_up(tokens * (d / 8), 256);
+  if (blocks > 0x7fffffffull) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: tensor too large", fn);
+  const uint16_t* ip = static_cast<const uint16_t*>(in);
+  uint16_t* op = static_cast<uint16_t*>(out);
+  if (dtype == KSQ_F16)
+    moe_sum_kernel<F16><<<static_cast<unsigned>(blocks), 256, 0, as_stream(stream)>>>(ip, op, tokens, static_cast<uint32_t>(topk), static_cast<uint32_t>(d));
+  else
+    moe_sum_kernel<BF16><<<static_cast<unsigned>(blocks), 256, 0, as_stream(stream)>>>(ip, op, tokens, static_cast<uint32_t>(topk), static_cast<uint32_t>(d));
+  return check_launch(fn);
+}

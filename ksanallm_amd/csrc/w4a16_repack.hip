@@ -1,0 +1,314 @@
+// Load-time repack between checkpoint int4 layouts and the CDNA4 tile layout described in ksq.h.
+// Pure nibble permutations: bit-exact and exactly invertible.
+#include "ksq_common.h"
+
+namespace ksq {
+namespace {
+
+// AWQ: logical column 8j+i sits in nibble kAwqNib[i] of word j (S/models/quant/cutlass_utils.cpp:12-38)
+__device__ __forceinline__ int awq_nibble(int i) {
+  // {0,4,1,5,2,6,3,7}
+  return ((i & 1) << 2) | (i >> 1);
+}
+// position of code (k % 8 == j) inside a packed dword: even j in nibbles 0..3, odd j in nibbles 4..7
+__device__ __forceinline__ int packed_nibble(int j) { return ((j & 1) << 2) | (j >> 1); }
+
+struct Geometry {
+  size_t E, K, N;
+  size_t k_tiles, n_tiles;
+};
+
+// packed dword index of element (e, k, n)
+__device__ __forceinline__ size_t packed_dword(const Geometry& g, size_t e, size_t k, size_t n) {
+  size_t tile = (e * g.n_tiles + n / 16) * g.k_tiles + k / 128;
+  size_t lane = ((k % 32) / 8) * 16 + (n % 16);
+  size_t d = (k % 128) / 32;
+  return tile * 256 + lane * 4 + d;
+}
+
+template <int SRC>
+__global__ void __launch_bounds__(256) repack_weight_kernel(const void* __restrict__ src_v,
+                                                            uint32_t* __restrict__ dst, Geometry g) {
+  size_t o = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  size_t total = g.E * g.K * g.N / 8;
+  if (o >= total) return;
+  size_t tile = o / 256;
+  int within = static_cast<int>(o % 256);
+  int lane = within / 4, d = within % 4;
+  size_t kt = tile % g.k_tiles;
+  size_t nt = (tile / g.k_tiles) % g.n_tiles;
+  size_t e = tile / (g.k_tiles * g.n_tiles);
+  size_t n = nt * 16 + (lane % 16);
+  size_t kbase = kt * 128 + d * 32 + (lane / 16) * 8;
+
+  uint32_t codes[8];
+  if (SRC == KSQ_SRC_GPTQ) {
+    const uint32_t* src = static_cast<const uint32_t*>(src_v);
+    uint32_t w = src[(e * (g.K / 8) + kbase / 8) * g.N + n];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) codes[j] = (w >> (4 * j)) & 15u;
+  } else if (SRC == KSQ_SRC_MOE_NK) {
+    const uint8_t* src = static_cast<const uint8_t*>(src_v);
+    uint32_t w = *reinterpret_cast<const uint32_t*>(src + (e * g.N + n) * (g.K / 2) + kbase / 2);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) codes[j] = (w >> (4 * j)) & 15u;
+  } else if (SRC == KSQ_SRC_AWQ) {
+    const uint32_t* src = static_cast<const uint32_t*>(src_v);
+    int sh = 4 * awq_nibble(static_cast<int>(n % 8));
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      uint32_t w = src[(e * g.K + kbase + j) * (g.N / 8) + n / 8];
+      codes[j] = (w >> sh) & 15u;
+    }
+  } else {  // KSQ_SRC_INT4X2_KN
+    const uint8_t* src = static_cast<const uint8_t*>(src_v);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      uint32_t b = src[(e * g.K + kbase + j) * (g.N / 2) + n / 2];
+      codes[j] = (((n & 1) ? (b >> 4) : b) & 15u) ^ 8u;
+    }
+  }
+  uint32_t out = 0;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) out |= codes[j] << (4 * packed_nibble(j));
+  dst[o] = out;
+}
+
+// one thread per 8 codes of the destination
+template <int DST>
+__global__ void __launch_bounds__(256) unpack_weight_kernel(const uint32_t* __restrict__ packed,
+                                                            void* __restrict__ dst_v, Geometry g) {
+  size_t o = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  size_t total = g.E * g.K * g.N / 8;
+  if (o >= total) return;
+  if (DST == KSQ_SRC_GPTQ || DST == KSQ_SRC_MOE_NK) {
+    size_t e, kp, n;
+    if (DST == KSQ_SRC_GPTQ) {  // dst word (e, kp, n)
+      n = o % g.N;
+      kp = (o / g.N) % (g.K / 8);
+      e = o / (g.N * (g.K / 8));
+    } else {  // dst u32 (e, n, kp)
+      kp = o % (g.K / 8);
+      n = (o / (g.K / 8)) % g.N;
+      e = o / (g.N * (g.K / 8));
+    }
+    uint32_t w = packed[packed_dword(g, e, kp * 8, n)];
+    uint32_t out = 0;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) out |= ((w >> (4 * packed_nibble(j))) & 15u) << (4 * j);
+    static_cast<uint32_t*>(dst_v)[o] = out;
+  } else {  // AWQ word (e, k, n/8) or four INT4X2 bytes (e, k, n/2 .. +3)
+    size_t j8 = o % (g.N / 8);
+    size_t k = (o / (g.N / 8)) % g.K;
+    size_t e = o / ((g.N / 8) * g.K);
+    int sh = 4 * packed_nibble(static_cast<int>(k % 8));
+    uint32_t out = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      uint32_t c = (packed[packed_dword(g, e, k, j8 * 8 + i)] >> sh) & 15u;
+      if (DST == KSQ_SRC_AWQ)
+        out |= c << (4 * awq_nibble(i));
+      else
+        out |= (c ^ 8u) << (4 * i);
+    }
+    static_cast<uint32_t*>(dst_v)[o] = out;
+  }
+}
+
+// scales: 16-bit elements.  packed index = ((e*n_tiles + n/16)*G + g)*16 + n%16
+template <int LAYOUT, bool TO_PACKED>
+__global__ void __launch_bounds__(256) scales_kernel(const uint16_t* __restrict__ src, uint16_t* __restrict__ dst,
+                                                     size_t E, size_t G, size_t N) {
+  size_t o = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (o >= E * G * N) return;
+  size_t nn = o % 16;
+  size_t gi = (o / 16) % G;
+  size_t nt = (o / (16 * G)) % (N / 16);
+  size_t e = o / (16 * G * (N / 16));
+  size_t n = nt * 16 + nn;
+  size_t lin = (LAYOUT == KSQ_SCALE_GN) ? (e * G + gi) * N + n : (e * N + n) * G + gi;
+  if (TO_PACKED)
+    dst[o] = src[lin];
+  else
+    dst[lin] = src[o];
+}
+
+template <int LAYOUT>
+__global__ void __launch_bounds__(256) zeros_pack_kernel(const void* __restrict__ src_v, uint8_t* __restrict__ dst,
+                                                         size_t G, size_t N) {
+  size_t o = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (o >= G * N) return;
+  size_t nn = o % 16;
+  size_t gi = (o / 16) % G;
+  size_t nt = o / (16 * G);
+  size_t n = nt * 16 + nn;
+  if (LAYOUT == KSQ_ZERO_AWQ_PACKED) {
+    uint32_t w = static_cast<const uint32_t*>(src_v)[gi * (N / 8) + n / 8];
+    dst[o] = static_cast<uint8_t>((w >> (4 * awq_nibble(static_cast<int>(n % 8)))) & 15u);
+  } else {
+    dst[o] = static_cast<const uint8_t*>(src_v)[gi * N + n];
+  }
+}
+
+// one thread per 8 zero points of the destination
+template <int LAYOUT>
+__global__ void __launch_bounds__(256) zeros_unpack_kernel(const uint8_t* __restrict__ packed,
+                                                           void* __restrict__ dst_v, size_t G, size_t N) {
+  size_t o = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (o >= G * N / 8) return;
+  size_t j8 = o % (N / 8);
+  size_t gi = o / (N / 8);
+  uint32_t out = 0;
+  for (int i = 0; i < 8; ++i) {
+    size_t n = j8 * 8 + i;
+    uint32_t z = packed[((n / 16) * G + gi) * 16 + n % 16];
+    if (LAYOUT == KSQ_ZERO_AWQ_PACKED)
+      out |= (z & 15u) << (4 * awq_nibble(i));
+    else
+      static_cast<uint8_t*>(dst_v)[gi * N + n] = static_cast<uint8_t>(z);
+  }
+  if (LAYOUT == KSQ_ZERO_AWQ_PACKED) static_cast<uint32_t*>(dst_v)[o] = out;
+}
+
+int check_weight_args(const void* a, const void* b, size_t E, size_t K, size_t N, const char* fn) {
+  if (!a || !b) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: null pointer", fn);
+  if (!aligned16(a) || !aligned16(b)) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: pointers must be 16-byte aligned", fn);
+  if (E == 0 || K == 0 || N == 0 || K % 128 != 0 || N % 16 != 0)
+    return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: need E>0, K %% 128 == 0, N %% 16 == 0 (E=%zu K=%zu N=%zu)", fn, E, K, N);
+  if (E * K * N / 8 / 256 + 1 > 0x7fffffffull) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: tensor too large", fn);
+  return KSQ_OK;
+}
+
+int check_group(size_t K, size_t group, const char* fn) {
+  if (group != 32 && group != 64 && group != 128)
+    return fail(KSQ_ERR_UNSUPPORTED, "%s: group size %zu not in {32,64,128}", fn, group);
+  if (K % group) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: K not a multiple of group", fn);
+  return KSQ_OK;
+}
+
+}  // namespace
+}  // namespace ksq
+
+using namespace ksq;
+
+KSQ_EXPORT int ksq_w4a16_repack(const void* src, int src_layout, void* dst, size_t E, size_t K, size_t N,
+                                void* stream) {
+  if (int rc = check_weight_args(src, dst, E, K, N, "ksq_w4a16_repack")) return rc;
+  Geometry g{E, K, N, K / 128, N / 16};
+  unsigned blocks = static_cast<unsigned>(div_up(E * K * N / 8, 256));
+  hipStream_t s = as_stream(stream);
+  uint32_t* d = static_cast<uint32_t*>(dst);
+  switch (src_layout) {
+    case KSQ_SRC_GPTQ:
+      repack_weight_kernel<KSQ_SRC_GPTQ><<<blocks, 256, 0, s>>>(src, d, g);
+      break;
+    case KSQ_SRC_AWQ:
+      repack_weight_kernel<KSQ_SRC_AWQ><<<blocks, 256, 0, s>>>(src, d, g);
+      break;
+    case KSQ_SRC_MOE_NK:
+      repack_weight_kernel<KSQ_SRC_MOE_NK><<<blocks, 256, 0, s>>>(src, d, g);
+      break;
+    case KSQ_SRC_INT4X2_KN:
+      repack_weight_kernel<KSQ_SRC_INT4X2_KN><<<blocks, 256, 0, s>>>(src, d, g);
+      break;
+    default:
+      return fail(KSQ_ERR_INVALID_ARGUMENT, "ksq_w4a16_repack: unknown source layout %d", src_layout);
+  }
+  return check_launch("ksq_w4a16_repack");
+}
+
+KSQ_EXPORT int ksq_w4a16_unpack(const void* packed, int dst_layout, void* dst, size_t E, size_t K, size_t N,
+                                void* stream) {
+  if (int rc = check_weight_args(packed, dst, E, K, N, "ksq_w4a16_unpack")) return rc;
+  Geometry g{E, K, N, K / 128, N / 16};
+  unsigned blocks = static_cast<unsigned>(div_up(E * K * N / 8, 256));
+  hipStream_t s = as_stream(stream);
+  const uint32_t* p = static_cast<const uint32_t*>(packed);
+  switch (dst_layout) {
+    case KSQ_SRC_GPTQ:
+      unpack_weight_kernel<KSQ_SRC_GPTQ><<<blocks, 256, 0, s>>>(p, dst, g);
+      break;
+    case KSQ_SRC_AWQ:
+      unpack_weight_kernel<KSQ_SRC_AWQ><<<blocks, 256, 0, s>>>(p, dst, g);
+      break;
+    case KSQ_SRC_MOE_NK:
+      unpack_weight_kernel<KSQ_SRC_MOE_NK><<<blocks, 256, 0, s>>>(p, dst, g);
+      break;
+    case KSQ_SRC_INT4X2_KN:
+      unpack_weight_kernel<KSQ_SRC_INT4X2_KN><<<blocks, 256, 0, s>>>(p, dst, g);
+      break;
+    default:
+      return fail(KSQ_ERR_INVALID_ARGUMENT, "ksq_w4a16_unpack: unknown destination layout %d", dst_layout);
+  }
+  return check_launch("ksq_w4a16_unpack");
+}
+
+static int scales_common(const void* src, int layout, void* dst, size_t E, size_t K, size_t N, size_t group, int dtype,
+                         void* stream, bool to_packed, const char* fn) {
+  if (int rc = check_weight_args(src, dst, E, K, N, fn)) return rc;
+  if (int rc = check_group(K, group, fn)) return rc;
+  if (dtype != KSQ_F16 && dtype != KSQ_BF16) return fail(KSQ_ERR_UNSUPPORTED, "%s: dtype must be f16 or bf16", fn);
+  size_t G = K / group;
+  unsigned blocks = static_cast<unsigned>(div_up(E * G * N, 256));
+  hipStream_t s = as_stream(stream);
+  const uint16_t* a = static_cast<const uint16_t*>(src);
+  uint16_t* b = static_cast<uint16_t*>(dst);
+  if (layout == KSQ_SCALE_GN) {
+    if (to_packed)
+      scales_kernel<KSQ_SCALE_GN, true><<<blocks, 256, 0, s>>>(a, b, E, G, N);
+    else
+      scales_kernel<KSQ_SCALE_GN, false><<<blocks, 256, 0, s>>>(a, b, E, G, N);
+  } else if (layout == KSQ_SCALE_NG) {
+    if (to_packed)
+      scales_kernel<KSQ_SCALE_NG, true><<<blocks, 256, 0, s>>>(a, b, E, G, N);
+    else
+      scales_kernel<KSQ_SCALE_NG, false><<<blocks, 256, 0, s>>>(a, b, E, G, N);
+  } else {
+    return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: unknown scale layout %d", fn, layout);
+  }
+  return check_launch(fn);
+}
+
+KSQ_EXPORT int ksq_w4a16_repack_scales(const void* src, int src_layout, void* dst, size_t E, size_t K, size_t N,
+                                       size_t group, int dtype, void* stream) {
+  return scales_common(src, src_layout, dst, E, K, N, group, dtype, stream, true, "ksq_w4a16_repack_scales");
+}
+
+KSQ_EXPORT int ksq_w4a16_unpack_scales(const void* packed, int dst_layout, void* dst, size_t E, size_t K, size_t N,
+                                       size_t group, int dtype, void* stream) {
+  return scales_common(packed, dst_layout, dst, E, K, N, group, dtype, stream, false, "ksq_w4a16_unpack_scales");
+}
+
+KSQ_EXPORT int ksq_w4a16_repack_zeros(const void* src, int src_layout, void* dst, size_t K, size_t N, size_t group,
+                                      void* stream) {
+  const char* fn = "ksq_w4a16_repack_zeros";
+  if (int rc = check_weight_args(src, dst, 1, K, N, fn)) return rc;
+  if (int rc = check_group(K, group, fn)) return rc;
+  size_t G = K / group;
+  unsigned blocks = static_cast<unsigned>(div_up(G * N, 256));
+  hipStream_t s = as_stream(stream);
+  if (src_layout == KSQ_ZERO_AWQ_PACKED)
+    zeros_pack_kernel<KSQ_ZERO_AWQ_PACKED><<<blocks, 256, 0, s>>>(src, static_cast<uint8_t*>(dst), G, N);
+  else if (src_layout == KSQ_ZERO_U8_GN)
+    zeros_pack_kernel<KSQ_ZERO_U8_GN><<<blocks, 256, 0, s>>>(src, static_cast<uint8_t*>(dst), G, N);
+  else
+    return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: unknown zero-point layout %d", fn, src_layout);
+  return check_launch(fn);
+}
+
+KSQ_EXPORT int ksq_w4a16_unpack_zeros(const void* packed, int dst_layout, void* dst, size_t K, size_t N, size_t group,
+                                      void* stream) {
+  const char* fn = "ksq_w4a16_unpack_zeros";
+  if (int rc = check_weight_args(packed, dst, 1, K, N, fn)) return rc;
+  if (int rc = check_group(K, group, fn)) return rc;
+  size_t G = K / group;
+  unsigned blocks = static_cast<unsigned>(div_up(G * N / 8, 256));
+  hipStream_t s = as_stream(stream);
+  if (dst_layout == KSQ_ZERO_AWQ_PACKED)
+    zeros_unpack_kernel<KSQ_ZERO_AWQ_PACKED><<<blocks, 256, 0, s>>>(static_cast<const uint8_t*>(packed), dst, G, N);
+  else if (dst_layout == KSQ_ZERO_U8_GN)
+    zeros_unpack_kernel<KSQ_ZERO_U8_GN><<<blocks, 256, 0, s>>>(static_cast<const uint8_t*>(packed), dst, G, N);
+  else
+    return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: unknown zero-point layout %d", fn, dst_layout);
+  return check_launch(fn);
+}

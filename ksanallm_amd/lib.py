@@ -1,0 +1,84 @@
+"""ctypes binding of libksq_hip.so; signatures follow include/ksq.h one to one."""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libksq_hip.so")
+
+F16, BF16, F32 = 0, 1, 2
+SRC_GPTQ, SRC_AWQ, SRC_MOE_NK, SRC_INT4X2_KN = 0, 1, 2, 3
+SCALE_GN, SCALE_NG = 0, 1
+ZERO_AWQ_PACKED, ZERO_U8_GN = 0, 1
+KIND_W4A16, KIND_FP8_BLOCKWISE, KIND_MOE_W4A16 = 0, 1, 2
+
+c_sz = ctypes.c_size_t
+c_p = ctypes.c_void_p
+c_i = ctypes.c_int
+
+
+class TileDesc(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int32) for n in
+                ("kernel", "block_m", "block_n", "block_k", "waves", "split_k", "grid", "reserved")]
+
+
+# name -> (restype, argtypes); also the list the ABI test checks against the header
+SIGNATURES = {
+    "ksq_version": (c_i, []),
+    "ksq_last_error_string": (ctypes.c_char_p, []),
+    "ksq_w4a16_packed_weight_bytes": (c_sz, [c_sz, c_sz, c_sz]),
+    "ksq_w4a16_packed_scales_bytes": (c_sz, [c_sz, c_sz, c_sz, c_sz, c_i]),
+    "ksq_w4a16_packed_zeros_bytes": (c_sz, [c_sz, c_sz, c_sz, c_sz]),
+    "ksq_w4a16_repack": (c_i, [c_p, c_i, c_p, c_sz, c_sz, c_sz, c_p]),
+    "ksq_w4a16_unpack": (c_i, [c_p, c_i, c_p, c_sz, c_sz, c_sz, c_p]),
+    "ksq_w4a16_repack_scales": (c_i, [c_p, c_i, c_p, c_sz, c_sz, c_sz, c_sz, c_i, c_p]),
+    "ksq_w4a16_unpack_scales": (c_i, [c_p, c_i, c_p, c_sz, c_sz, c_sz, c_sz, c_i, c_p]),
+    "ksq_w4a16_repack_zeros": (c_i, [c_p, c_i, c_p, c_sz, c_sz, c_sz, c_p]),
+    "ksq_w4a16_unpack_zeros": (c_i, [c_p, c_i, c_p, c_sz, c_sz, c_sz, c_p]),
+    "ksq_w4a16_workspace_size": (c_sz, [c_sz, c_sz, c_sz, c_sz, c_i]),
+    "ksq_w4a16_gemm": (c_i, [c_p, c_p, c_p, c_p, c_p, c_p, c_sz, c_sz, c_sz, c_sz, c_sz, c_i, c_p]),
+    "ksq_fp8_group_quant": (c_i, [c_p, c_p, c_p, c_sz, c_sz, c_sz, c_i, c_i, c_i, c_p]),
+    "ksq_fp8_blockwise_workspace_size": (c_sz, [c_sz, c_sz, c_sz]),
+    "ksq_fp8_blockwise_gemm": (c_i, [c_p, c_p, c_p, c_p, c_p, c_sz, c_sz, c_sz, c_i, c_p, c_sz, c_p]),
+    "ksq_moe_align_capacity": (c_sz, [c_sz, c_sz, c_sz]),
+    "ksq_moe_align_scratch_bytes": (c_sz, [c_sz, c_sz]),
+    "ksq_moe_align": (c_i, [c_p, c_sz, c_sz, c_sz, c_p, c_p, c_p, c_p, c_p]),
+    "ksq_moe_w4a16_gemm": (c_i, [c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_sz, c_sz, c_sz, c_sz, c_sz, c_sz,
+                                 c_sz, c_i, c_p]),
+    "ksq_moe_silu_mul": (c_i, [c_p, c_p, c_sz, c_sz, c_i, c_p]),
+    "ksq_moe_sum": (c_i, [c_p, c_p, c_sz, c_sz, c_sz, c_i, c_p]),
+    "ksq_select_tile": (c_i, [c_i, c_sz, c_sz, c_sz, c_i, ctypes.POINTER(TileDesc)]),
+}
+
+_lib = None
+
+
+class KsqError(RuntimeError):
+    def __init__(self, code, message):
+        super().__init__("ksq status %d: %s" % (code, message))
+        self.code = code
+
+
+def load():
+    """Load the built library; raises if it is missing (there is no fallback path)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError("libksq_hip.so is not built: run `python -m ksanallm_amd.build` (needs hipcc)")
+        lib = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+    return _lib
+
+
+def check(rc):
+    if rc != 0:
+        raise KsqError(rc, load().ksq_last_error_string().decode())
+
+
+def select_tile(kind, m, n, k, dtype):
+    d = TileDesc()
+    check(load().ksq_select_tile(kind, m, n, k, dtype, ctypes.byref(d)))
+    return {n: getattr(d, n) for n, _ in TileDesc._fields_ if n != "reserved"}

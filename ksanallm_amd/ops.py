@@ -1,0 +1,192 @@
+"""Host-side mirror of the reference's kernel-wrapper surface for the quantized-GEMM path, on torch device tensors.
+
+Each function names the ``Invoke*`` wrapper of the reference it stands for
+(src/ksana_llm/kernels/nvidia/basic_kernel_wrapper.h:32-115,295-336 and moe_kernel_wrapper.h:28-88) and forwards to
+the C-ABI of libksq_hip.so on the tensor's current stream.  Torch is used for device memory and streams only.
+"""
+import torch
+
+from . import lib as _l
+
+_lib = _l.load()
+
+F16, BF16 = _l.F16, _l.BF16
+
+
+def _dt(t):
+    if t.dtype == torch.float16:
+        return F16
+    if t.dtype == torch.bfloat16:
+        return BF16
+    raise TypeError("activation dtype must be float16 or bfloat16, got %s" % t.dtype)
+
+
+def _torch_dt(tag):
+    return torch.float16 if tag == F16 else torch.bfloat16
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t):
+    if t is None:
+        return None
+    assert t.is_cuda and t.is_contiguous(), "device-resident contiguous tensor required"
+    return t.data_ptr()
+
+
+# ----------------------------------------------------------------------------------------------- load-time repack
+def repack_weight(src, layout, E, K, N):
+    """Checkpoint int4 weight -> CDNA4 tile layout (uint8 tensor of E*K*N/2 bytes)."""
+    dst = torch.empty(_lib.ksq_w4a16_packed_weight_bytes(E, K, N), dtype=torch.uint8, device=src.device)
+    _l.check(_lib.ksq_w4a16_repack(_ptr(src), layout, _ptr(dst), E, K, N, _stream()))
+    return dst
+
+
+def unpack_weight(packed, layout, E, K, N):
+    """Inverse of :func:`repack_weight`; returns the checkpoint layout as int32 (GPTQ/AWQ) or uint8/int8 bytes."""
+    if layout == _l.SRC_GPTQ:
+        dst = torch.empty((E, K // 8, N) if E > 1 else (K // 8, N), dtype=torch.int32, device=packed.device)
+    elif layout == _l.SRC_AWQ:
+        dst = torch.empty((E, K, N // 8) if E > 1 else (K, N // 8), dtype=torch.int32, device=packed.device)
+    elif layout == _l.SRC_MOE_NK:
+        dst = torch.empty((E, N, K // 2), dtype=torch.uint8, device=packed.device)
+    else:
+        dst = torch.empty((E, K, N // 2) if E > 1 else (K, N // 2), dtype=torch.int8, device=packed.device)
+    _l.check(_lib.ksq_w4a16_unpack(_ptr(packed), layout, _ptr(dst), E, K, N, _stream()))
+    return dst
+
+
+def repack_scales(src, layout, E, K, N, group):
+    dst = torch.empty(E * (K // group) * N, dtype=src.dtype, device=src.device)
+    _l.check(_lib.ksq_w4a16_repack_scales(_ptr(src), layout, _ptr(dst), E, K, N, group, _dt(src), _stream()))
+    return dst
+
+
+def unpack_scales(packed, layout, E, K, N, group):
+    G = K // group
+    shape = ((E, G, N) if E > 1 else (G, N)) if layout == _l.SCALE_GN else (E, N, G)
+    dst = torch.empty(shape, dtype=packed.dtype, device=packed.device)
+    _l.check(_lib.ksq_w4a16_unpack_scales(_ptr(packed), layout, _ptr(dst), E, K, N, group, _dt(packed), _stream()))
+    return dst
+
+
+def repack_zeros(src, layout, K, N, group):
+    dst = torch.empty((K // group) * N, dtype=torch.uint8, device=src.device)
+    _l.check(_lib.ksq_w4a16_repack_zeros(_ptr(src), layout, _ptr(dst), K, N, group, _stream()))
+    return dst
+
+
+def unpack_zeros(packed, layout, K, N, group):
+    G = K // group
+    if layout == _l.ZERO_AWQ_PACKED:
+        dst = torch.empty((G, N // 8), dtype=torch.int32, device=packed.device)
+    else:
+        dst = torch.empty((G, N), dtype=torch.uint8, device=packed.device)
+    _l.check(_lib.ksq_w4a16_unpack_zeros(_ptr(packed), layout, _ptr(dst), K, N, group, _stream()))
+    return dst
+
+
+# ----------------------------------------------------------------------------------------------- W4A16 GEMM
+def w4a16_workspace_size(max_m, n, k, group, dtype):
+    return _lib.ksq_w4a16_workspace_size(max_m, n, k, group, dtype)
+
+
+def w4a16_gemm(x, w_packed, scales_packed, zeros_packed, n, k, group, out=None, workspace=None):
+    """InvokeFpAIntBGroupCudaGemm / InvokeFpAIntBGroupCutlassGemm / InvokeMarlinGemm / InvokeMacheteGemm."""
+    m = x.shape[0]
+    if out is None:
+        out = torch.empty((m, n), dtype=x.dtype, device=x.device)
+    ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    _l.check(_lib.ksq_w4a16_gemm(_ptr(out), _ptr(x), _ptr(w_packed), _ptr(scales_packed), _ptr(zeros_packed),
+                                 _ptr(workspace), ws_bytes, m, n, k, group, _dt(x), _stream()))
+    return out
+
+
+# ----------------------------------------------------------------------------------------------- FP8
+def per_token_group_quant_fp8(x, k, group=128, column_major=True, fuse_silu_mul=False, q=None, s=None):
+    """InvokePerTokenGroupQuantFp8E4m3: returns (codes uint8 [m,k], scales fp32 [k/group,m] or [m,k/group])."""
+    m = x.shape[0]
+    if q is None:
+        q = torch.empty((m, k), dtype=torch.uint8, device=x.device)
+    if s is None:
+        s = torch.empty((k // group, m) if column_major else (m, k // group), dtype=torch.float32, device=x.device)
+    _l.check(_lib.ksq_fp8_group_quant(_ptr(x), _ptr(q), _ptr(s), m, k, group, int(column_major), int(fuse_silu_mul),
+                                      _dt(x), _stream()))
+    return q, s
+
+
+def fp8_blockwise_gemm(a_q, a_s, b, b_s, out_dtype=torch.bfloat16, out=None, workspace=None):
+    """InvokeBlockGemm / DeepGEMMWrapper::Gemm: a_q [m,k] e4m3 bytes, a_s [k/128,m], b [n,k], b_s [n/128,k/128]."""
+    m, k = a_q.shape
+    n = b.shape[0]
+    if out is None:
+        out = torch.empty((m, n), dtype=out_dtype, device=a_q.device)
+    ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    _l.check(_lib.ksq_fp8_blockwise_gemm(_ptr(a_q), _ptr(a_s), _ptr(b), _ptr(b_s), _ptr(out), m, n, k, _dt(out),
+                                         _ptr(workspace), ws_bytes, _stream()))
+    return out
+
+
+# ----------------------------------------------------------------------------------------------- MoE
+def moe_align_block_size(topk_ids, num_experts, block_m):
+    """InvokeSglMoeAlignBlockSize / InvokeMoeAlignBlockSize: (sorted_ids, expert_ids, num_post_pad) int32 tensors."""
+    ids = topk_ids.reshape(-1)
+    numel = ids.numel()
+    cap = _lib.ksq_moe_align_capacity(numel, num_experts, block_m)
+    dev = topk_ids.device
+    sorted_ids = torch.empty(cap, dtype=torch.int32, device=dev)
+    expert_ids = torch.empty((cap + block_m - 1) // block_m, dtype=torch.int32, device=dev)
+    num_post_pad = torch.empty(1, dtype=torch.int32, device=dev)
+    scratch = torch.empty(_lib.ksq_moe_align_scratch_bytes(numel, num_experts), dtype=torch.uint8, device=dev)
+    _l.check(_lib.ksq_moe_align(_ptr(ids), numel, num_experts, block_m, _ptr(sorted_ids), _ptr(expert_ids),
+                                _ptr(num_post_pad), _ptr(scratch), _stream()))
+    return sorted_ids, expert_ids, num_post_pad
+
+
+def moe_w4a16_gemm(x, w_packed, scales_packed, topk_w, sorted_ids, expert_ids, num_post_pad, numel, top_k, E, n, k,
+                   group, block_m, out=None):
+    """InvokeMoeWna16Gemm / InvokeFusedMoeGptqAwqKernel: out [numel, n]."""
+    if out is None:
+        out = torch.empty((numel, n), dtype=x.dtype, device=x.device)
+    _l.check(_lib.ksq_moe_w4a16_gemm(_ptr(out), _ptr(x), _ptr(w_packed), _ptr(scales_packed), None, _ptr(topk_w),
+                                     _ptr(sorted_ids), _ptr(expert_ids), _ptr(num_post_pad), numel, top_k, E, n, k,
+                                     group, block_m, _dt(x), _stream()))
+    return out
+
+
+def silu_and_mul(x, out=None):
+    """InvokeSiluAndMul: x [rows, 2*inter] -> [rows, inter]."""
+    rows, two = x.shape
+    if out is None:
+        out = torch.empty((rows, two // 2), dtype=x.dtype, device=x.device)
+    _l.check(_lib.ksq_moe_silu_mul(_ptr(x), _ptr(out), rows, two // 2, _dt(x), _stream()))
+    return out
+
+
+def moe_sum(x, out=None):
+    """InvokeMoeSum: x [tokens, topk, d] -> [tokens, d]."""
+    tokens, topk, d = x.shape
+    if out is None:
+        out = torch.empty((tokens, d), dtype=x.dtype, device=x.device)
+    _l.check(_lib.ksq_moe_sum(_ptr(x), _ptr(out), tokens, topk, d, _dt(x), _stream()))
+    return out
+
+
+def fused_moe_w4a16(x, w13_packed, s13_packed, w2_packed, s2_packed, topk_ids, topk_w, E, hidden, inter, group,
+                    block_m=None):
+    """InvokeFusedMoe<T,false> for int4 weights (S/kernels/nvidia/moe_kernel_wrapper.cpp:463-654):
+    align -> GEMM1 -> silu*mul -> GEMM2 (* routed weight) -> sum over top-k."""
+    T, topk = topk_ids.shape
+    numel = T * topk
+    if block_m is None:
+        block_m = 16 if numel // E < 16 else 32
+    sorted_ids, expert_ids, npp = moe_align_block_size(topk_ids, E, block_m)
+    tw = topk_w.reshape(-1).to(torch.float32).contiguous()
+    c1 = moe_w4a16_gemm(x, w13_packed, s13_packed, None, sorted_ids, expert_ids, npp, numel, topk, E, 2 * inter,
+                        hidden, group, block_m)
+    c2 = silu_and_mul(c1)
+    c3 = moe_w4a16_gemm(c2, w2_packed, s2_packed, tw, sorted_ids, expert_ids, npp, numel, 1, E, hidden, inter, group,
+                        block_m)
+    return moe_sum(c3.view(T, topk, hidden))

@@ -1,0 +1,71 @@
+"""Synthetic inputs of the benchmark configurations and the comparison rules shared by the GPU parity tests."""
+import numpy as np
+import torch
+
+from oracle import ksq_oracle as orc
+
+F16, BF16 = 0, 1
+TORCH_DT = {F16: torch.float16, BF16: torch.bfloat16}
+
+
+def gen(seed):
+    g = torch.Generator(device="cpu")
+    g.manual_seed(seed)
+    return g
+
+
+def bits_of(t):
+    """torch 16-bit float tensor (cpu) -> numpy uint16 bit patterns."""
+    return t.contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+def uniform(g, shape, lo, hi, dtype):
+    return (torch.rand(shape, generator=g) * (hi - lo) + lo).to(TORCH_DT[dtype])
+
+
+def make_w4a16(seed, M, N, K, group, dtype, awq, x_std=1.0, s_lo=0.004, s_hi=0.02, z_lo=6, z_hi=9):
+    """Returns a dict with checkpoint-format tensors (torch, cpu) and the numpy views the oracle needs."""
+    g = gen(seed)
+    codes = torch.randint(0, 16, (K, N), generator=g, dtype=torch.uint8)
+    scales = uniform(g, (K // group, N), s_lo, s_hi, dtype)
+    x = (torch.randn((M, K), generator=g) * x_std).to(TORCH_DT[dtype])
+    d = {"codes": codes.numpy(), "scales": scales, "x": x, "M": M, "N": N, "K": K, "group": group, "dtype": dtype}
+    if awq:
+        zeros = torch.randint(z_lo, z_hi + 1, (K // group, N), generator=g, dtype=torch.uint8)
+        d["zeros"] = zeros.numpy()
+        d["qweight"] = torch.from_numpy(orc.awq_pack(d["codes"]).view(np.int32))
+        d["qzeros"] = torch.from_numpy(orc.awq_pack(d["zeros"]).view(np.int32))
+    else:
+        d["zeros"] = None
+        d["qweight"] = torch.from_numpy(orc.gptq_pack(d["codes"]).view(np.int32))
+    return d
+
+
+def w4a16_oracle(d):
+    return orc.w4a16_gemm(bits_of(d["x"]), d["codes"], bits_of(d["scales"]), d["zeros"], d["group"], d["dtype"])
+
+
+def ulp(ref, dtype):
+    """Spacing of the output type at |ref| (fp16: 10 mantissa bits, bf16: 7)."""
+    mant = 10 if dtype == F16 else 7
+    a = np.maximum(np.abs(ref.astype(np.float64)), 2.0 ** -14)
+    return 2.0 ** (np.floor(np.log2(a)) - mant)
+
+
+def check_gemm(y_gpu, ref_f32, dtype, what=""):
+    """rel-L2 <= 5e-3 and max-abs <= 2e-2 against the fp32-accumulated dequant reference.
+
+    The absolute bound is applied to the error that is left after allowing for the output type's own rounding
+    (half a unit in the last place of the reference value): once |y| >= 8 in bf16, half an ulp alone is 0.031, so the
+    raw difference cannot meet 2e-2 for any kernel.  The raw maximum is returned for reporting.
+    """
+    y = y_gpu.float().cpu().numpy().astype(np.float64)
+    ref = ref_f32.astype(np.float64)
+    assert y.shape == ref.shape
+    assert np.all(np.isfinite(y)), what
+    rel_l2 = np.linalg.norm(y - ref) / max(np.linalg.norm(ref), 1e-30)
+    err = np.abs(y - ref)
+    excess = np.maximum(err - 0.5 * ulp(ref, dtype), 0.0).max()
+    assert rel_l2 <= 5e-3, "%s rel-L2 %.3e" % (what, rel_l2)
+    assert excess <= 2e-2, "%s max-abs beyond output rounding %.3e (raw %.3e)" % (what, excess, err.max())
+    return rel_l2, err.max()

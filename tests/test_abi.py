@@ -1,0 +1,39 @@
+"""The C-ABI library loads on a machine without a GPU and exports exactly what include/ksq.h declares."""
+import os
+import re
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "ksq.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ksq_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from ksanallm_amd import lib as L
+    lib = L.load()
+    names = declared_functions()
+    assert len(names) >= 20
+    for n in names:
+        assert hasattr(lib, n), n
+    assert sorted(L.SIGNATURES) == names
+    assert lib.ksq_version() == 1
+    assert lib.ksq_last_error_string() is not None
+
+
+def test_size_queries_and_tile_selection_are_host_only():
+    from ksanallm_amd import lib as L
+    lib = L.load()
+    assert lib.ksq_w4a16_packed_weight_bytes(1, 4096, 4096) == 4096 * 4096 // 2
+    assert lib.ksq_w4a16_packed_scales_bytes(1, 4096, 4096, 128, L.F16) == 32 * 4096 * 2
+    assert lib.ksq_w4a16_packed_zeros_bytes(1, 4096, 14336, 128) == 32 * 14336
+    assert lib.ksq_moe_align_capacity(64, 256, 16) == 64 + 256 * 15
+    d = L.select_tile(L.KIND_W4A16, 1, 4096, 4096, L.F16)
+    assert d["kernel"] == 0 and d["grid"] >= 256
+    # deterministic: same answer every time, no timing involved
+    assert d == L.select_tile(L.KIND_W4A16, 1, 4096, 4096, L.F16)
+    import pytest
+    with pytest.raises(L.KsqError):
+        L.select_tile(99, 1, 16, 128, 0)

@@ -1,0 +1,93 @@
+"""W4A16 group-wise GEMM (GPTQ symmetric / AWQ zero-point) against the fp32 dequant-then-GEMM oracle on identical
+seeded inputs.  Tolerance: rel-L2 <= 5e-3, max-abs <= 2e-2 (see tests/helpers.check_gemm)."""
+import numpy as np
+import pytest
+import torch
+
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from ksanallm_amd import ops
+    return ops
+
+
+def run_case(ops, d):
+    from ksanallm_amd import lib as L
+    K, N, group = d["K"], d["N"], d["group"]
+    awq = d["zeros"] is not None
+    qw = d["qweight"].cuda()
+    wp = ops.repack_weight(qw, L.SRC_AWQ if awq else L.SRC_GPTQ, 1, K, N)
+    sp = ops.repack_scales(d["scales"].cuda(), L.SCALE_GN, 1, K, N, group)
+    zp = ops.repack_zeros(d["qzeros"].cuda(), L.ZERO_AWQ_PACKED, K, N, group) if awq else None
+    y = ops.w4a16_gemm(d["x"].cuda(), wp, sp, zp, N, K, group)
+    torch.cuda.synchronize()
+    return y
+
+
+# config 1: GPTQ fp16, N=K=4096, M in {1,16}
+@pytest.mark.parametrize("M", [1, 16])
+def test_cfg1_gptq_fp16(ops, M):
+    d = H.make_w4a16(1000 + M, M, 4096, 4096, 128, H.F16, awq=False)
+    y = run_case(ops, d)
+    H.check_gemm(y, H.w4a16_oracle(d), H.F16, "cfg1 M=%d" % M)
+
+
+# config 2: AWQ bf16 on the Llama-3-8B MLP shapes
+@pytest.mark.parametrize("N,K", [(14336, 4096), (4096, 14336)])
+@pytest.mark.parametrize("M", [1, 8, 32, 128])
+def test_cfg2_awq_bf16(ops, M, N, K):
+    d = H.make_w4a16(2000 + M + N, M, N, K, 128, H.BF16, awq=True, s_lo=0.003, s_hi=0.015)
+    y = run_case(ops, d)
+    H.check_gemm(y, H.w4a16_oracle(d), H.BF16, "cfg2 M=%d N=%d K=%d" % (M, N, K))
+
+
+@pytest.mark.parametrize("dtype", [H.F16, H.BF16])
+@pytest.mark.parametrize("group", [32, 64, 128])
+@pytest.mark.parametrize("awq", [False, True])
+@pytest.mark.parametrize("M", [1, 3, 16, 17, 33])
+def test_small_shapes_all_groups(ops, dtype, group, awq, M):
+    d = H.make_w4a16(77 + M + group, M, 48, 384, group, dtype, awq=awq, z_lo=0, z_hi=15)
+    y = run_case(ops, d)
+    H.check_gemm(y, H.w4a16_oracle(d), dtype, "small")
+
+
+def test_extreme_codes_and_zero_points(ops):
+    """All codes 0 / 15 with zero points 15 / 0: the largest dequantized magnitudes the format can hold."""
+    for code, z in ((0, 15), (15, 0)):
+        d = H.make_w4a16(5, 4, 64, 256, 128, H.BF16, awq=True)
+        d["codes"][:] = code
+        d["zeros"][:] = z
+        from oracle import ksq_oracle as orc
+        d["qweight"] = torch.from_numpy(orc.awq_pack(d["codes"]).view(np.int32))
+        d["qzeros"] = torch.from_numpy(orc.awq_pack(d["zeros"]).view(np.int32))
+        y = run_case(ops, d)
+        H.check_gemm(y, H.w4a16_oracle(d), H.BF16, "extreme")
+
+
+def test_linearity_full_size(ops):
+    """Size-independent property at a full benchmark shape: GEMM(x1 + x2) == GEMM(x1) + GEMM(x2) up to rounding, and
+    a zero activation row gives an exactly zero output row."""
+    d = H.make_w4a16(9, 8, 14336, 4096, 128, H.BF16, awq=True, s_lo=0.003, s_hi=0.015)
+    d["x"][3] = 0
+    x1 = d["x"].clone()
+    y1 = run_case(ops, d).float()
+    assert torch.all(y1[3] == 0)
+    d["x"] = (x1.float() * 2).to(torch.bfloat16)  # exact doubling
+    y2 = run_case(ops, d).float()
+    assert torch.equal(y2, y1 * 2)
+
+
+def test_bad_arguments(ops):
+    from ksanallm_amd import lib as L
+    x = torch.zeros((1, 100), dtype=torch.float16, device="cuda")
+    w = torch.zeros(4096, dtype=torch.uint8, device="cuda")
+    with pytest.raises(L.KsqError) as e:
+        ops.w4a16_gemm(x, w, w, None, 16, 100, 128)
+    assert e.value.code == 1 and "k % 128" in str(e.value)
+    with pytest.raises(L.KsqError) as e:
+        ops.w4a16_gemm(x, w, w, None, 16, 128, 100)
+    assert e.value.code == 2
