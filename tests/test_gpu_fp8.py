@@ -87,7 +87,7 @@ def test_quant_full_size_properties(ops, oracle):
     assert torch.all(deq.abs().amax(-1) == 448.0)
     rec = deq * s.t().contiguous().view(m, k // 128, 1)
     err = (rec - x.cuda().float().view(m, k // 128, 128)).abs()
-    assert torch.all(err <= s.t().contiguous().view(m, k // 128, 1) * 16.0 + 1e-12)  # half of the largest step (32)
+    assert torch.all(err <= s.t().contiguous().view(m, k // 128, 1) * 16.001 + 1e-12)  # half of the largest step (32), plus fp32 rounding of x/s
     rows = [0, 1, 777, 4095]
     qo, so = oracle.fp8_group_quant(H.bits_of(x[rows]), k, 128, True, False, H.BF16)
     np.testing.assert_array_equal(q[rows].cpu().numpy(), qo)
