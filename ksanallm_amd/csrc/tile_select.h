@@ -7,9 +7,12 @@ namespace ksq {
 struct SplitKChoice {
   int mt;     // 16-row tiles of x per workgroup
   int nt;     // 16-column tiles per workgroup
-  int waves;  // wavefronts per workgroup, each taking every waves-th k-tile
+  int waves;  // wavefronts per workgroup; wavefront w takes every waves-th k-tile
 };
 
+// m rows in one dense GEMM
 SplitKChoice select_splitk(size_t m, size_t n, size_t k);
+// same rule for a grid of m_blocks row blocks of 16*mt rows each (MoE: one block per aligned expert segment)
+SplitKChoice select_splitk_blocks(int mt, size_t m_blocks, size_t n, size_t k);
 
 }  // namespace ksq

@@ -7,18 +7,30 @@ namespace ksq {
 
 static constexpr int kNumCU = 256;
 
-// Split-K wavefront kernel: every workgroup streams NT column tiles over the whole K.
-// - WAVES: enough k-tiles per wavefront to keep a prefetch stage in flight, at most 16 wavefronts (1024 threads).
-// - NT: two column tiles per workgroup halve the x-operand traffic out of L2, but only when that still leaves at
-//   least two workgroups per CU.
+// Split-K wavefront kernel (decode regime, HBM-bound).  Measured on MI355X the kernel runs fastest with few, long
+// lived wavefronts, each streaming a deep ring of loads, and with every workgroup resident from the first cycle:
+// - 4 wavefronts per workgroup, wavefront w taking every 4th k-tile;
+// - NT, the column tiles a wavefront streams per k-tile, as wide as the register file allows (8 for one 16-row tile
+//   of x, 4 for two) while the grid still has about one workgroup per CU: the x fragments and the sum-of-x MFMA are
+//   shared by the NT tiles, which also divides the x traffic out of L2 by NT.
 SplitKChoice select_splitk(size_t m, size_t n, size_t k) {
+  const int mt = m <= 16 ? 1 : 2;
+  return select_splitk_blocks(mt, div_up(m, 16 * mt), n, k);
+}
+
+SplitKChoice select_splitk_blocks(int mt, size_t m_blocks, size_t n, size_t k) {
   SplitKChoice c;
-  c.mt = m <= 16 ? 1 : 2;
-  const size_t kt = k / 128;
-  c.waves = kt >= 32 ? 16 : 8;
+  c.mt = mt;
+  c.waves = 4;
+  c.nt = 1;
   const size_t n_tiles = n / 16;
-  c.nt = (n_tiles % 2 == 0 && n_tiles / 2 >= 2 * static_cast<size_t>(kNumCU)) ? 2 : 1;
-  if (c.mt == 2 && c.nt == 2) c.waves = 8;  // 16 wavefronts leave 128 VGPRs each, too few for a 2x2 tile
+  for (int nt = (mt == 1 ? 8 : 4); nt > 1; nt >>= 1) {
+    if (n_tiles % nt == 0 && n_tiles / nt * m_blocks >= static_cast<size_t>(kNumCU) * 3 / 4) {
+      c.nt = nt;
+      break;
+    }
+  }
+  (void)k;
   return c;
 }
 

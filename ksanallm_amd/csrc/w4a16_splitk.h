@@ -1,16 +1,26 @@
-// Decode-regime W4A16 kernel (small M, HBM-bound): split-K across the wavefronts of a workgroup.
+// Decode-regime W4A16 kernel (small M, HBM-bound).
 //
-// A workgroup owns NT tiles of 16 output columns and MT tiles of 16 rows of x.  Wavefront w walks the 128-wide
-// k-tiles w, w+WAVES, ... ; per k-tile each lane loads 16 bytes of packed codes per column tile (one coalesced 1 KiB
-// wavefront load), turns every dword into an MFMA operand holding magic+code with four and-or instructions, and
-// feeds v_mfma_f32_16x16x32 with the weights as the row operand and x as the column operand.  The group's zero point
-// and scale are applied to the fp32 partial afterwards:
+// Work decomposition
+//   grid.x : groups of NT column tiles (16 output columns each)
+//   grid.y : blocks of MT*16 rows of x (MoE: aligned blocks of sorted slots, one expert each)
+// Wavefront w of a workgroup takes the 128-wide k-tiles w, w+WAVES, ...
+// Per k-tile a wavefront loads the x operand once (MT*4 fragments of 16 bytes per lane) and streams the NT weight
+// tiles of that k-tile, one coalesced 1 KiB wavefront load each.  Every packed dword becomes an MFMA operand holding
+// magic+code with seven bit operations, x is the row operand and the weights the column operand of
+// v_mfma_f32_16x16x32, so a lane's four results share one output column, hence one scale and one zero point:
 //     acc += s * (sum_k x*(magic+code) - (magic+zp) * sum_k x)
-// where sum_k x comes from one more MFMA against an all-ones operand, so nothing but and-or work runs on the VALU
-// per weight.  The wavefronts' partials meet in LDS and are summed in wavefront order (deterministic).
+// with sum_k x from one more MFMA against an all-ones operand, shared by the NT tiles.
 //
-// The same kernel serves the MoE grouped GEMM: rows come from sorted slot ids, the expert of the block selects the
-// weight slab, and the routed weight is applied on the way out.
+// What bounds the kernel is HBM latency x bandwidth, so the loads of a wavefront form one ring in issue order
+// (vmcnt retires loads in order: a second, shallower ring would drain the first each time it is waited for).  The
+// ring holds LOOK k-tiles ahead, NT weight tiles plus the x fragments each, sized so that a CU keeps 64 KiB or more
+// in flight; buffer loads with a scalar offset keep address arithmetic off the VALU.
+//
+// The wavefronts' partials meet in LDS and are summed in wavefront order: the summation order is fixed, so the
+// output does not depend on timing.
+//
+// Rows of x beyond M are read from the last valid row instead of being masked: an MFMA output row depends only on
+// its own row of x, and those rows are never stored.
 #pragma once
 
 #include "ksq_common.h"
@@ -20,9 +30,9 @@ namespace ksq {
 struct SplitKParams {
   void* y;
   const void* x;
-  const u32x4* w;
-  const uint16_t* scales;
-  const uint8_t* zeros;
+  const void* w;
+  const void* scales;
+  const void* zeros;
   uint32_t M, N, K;
   // grouped (MoE) mode
   const int32_t* sorted_ids;
@@ -30,14 +40,33 @@ struct SplitKParams {
   const int32_t* num_post_pad;
   const float* topk_w;
   uint32_t numel, top_k;
+  uint32_t x_bytes;  // extent of x, below 1 GiB
+  uint32_t nibble_mask, magic2;  // 0x000f000f and T::kMagic2, passed in so that they live in registers
 };
 
-template <typename T, int MT, int NT, int WAVES, int GROUP, bool HAS_ZP, bool GROUPED>
-__global__ void __launch_bounds__(WAVES * 64) w4a16_splitk_kernel(SplitKParams p) {
+// Eight codes of a packed dword -> MFMA operand holding magic+code (nibble i and i+4 are the pair k=2i, 2i+1).
+// mask (0x000f000f) and magic2 arrive as kernel arguments rather than literals: with both in registers the
+// compiler folds each and/or pair into one v_and_or_b32, which a literal operand would forbid on this ISA.
+template <typename T>
+__device__ __forceinline__ typename T::frag dequant_magic_fast(uint32_t w, uint32_t mask, uint32_t magic2) {
+  u32x4 v;
+  v.x = (w & mask) | magic2;
+  v.y = ((w >> 4) & mask) | magic2;
+  v.z = ((w >> 8) & mask) | magic2;
+  v.w = ((w >> 12) & mask) | magic2;
+  return as_frag<T>(v);
+}
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, static_cast<int>(bytes), 0x00020000);
+}
+
+template <typename T, int MT, int NT, int WAVES, int LOOK, int OCC, int GROUP, bool HAS_ZP, bool GROUPED>
+__global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKParams p) {
   constexpr int GPT = 128 / GROUP;  // groups per k-tile
   constexpr int SPG = GROUP / 32;   // MFMA k-steps per group
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lrow = lane & 15;
   const int lq = lane >> 4;
   const uint32_t KT = p.K / 128;
@@ -46,9 +75,8 @@ __global__ void __launch_bounds__(WAVES * 64) w4a16_splitk_kernel(SplitKParams p
 
   __shared__ f32x4 red[WAVES][NT * MT][64];
 
-  // ---- which rows of x this lane feeds, and where they go
+  // ---- rows of x this lane feeds (row operand: lane l supplies row l%16, k = 8*(l/16)..+7 of each k-step)
   uint32_t xrow[MT];
-  bool ok[MT];
   size_t tile_base = 0;  // first weight tile of the expert, in tiles
   size_t sz_base = 0;    // first scale / zero element of the expert
   if (GROUPED) {
@@ -60,116 +88,156 @@ __global__ void __launch_bounds__(WAVES * 64) w4a16_splitk_kernel(SplitKParams p
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       uint32_t sid = static_cast<uint32_t>(p.sorted_ids[pos0 + mt * 16 + lrow]);
-      ok[mt] = sid < p.numel;
+      sid = sid < p.numel ? sid : p.numel - 1;
       xrow[mt] = sid / p.top_k;
     }
   } else {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-      xrow[mt] = blockIdx.y * (16 * MT) + mt * 16 + lrow;
-      ok[mt] = xrow[mt] < p.M;
+      uint32_t r = blockIdx.y * (16 * MT) + mt * 16 + lrow;
+      xrow[mt] = r < p.M ? r : p.M - 1;
     }
   }
 
-  const u32x4* wbase[NT];
-  const uint16_t* sbase[NT];
-  const uint8_t* zbase[NT];
+  // ---- buffer resources: bases are wavefront-uniform, lanes add a fixed offset, k-tiles a scalar offset
+  const uint32_t w_tile_stride = KT * 1024;  // bytes between consecutive column tiles
+  const uint32_t s_tile_stride = G * 32;
+  const uint32_t z_tile_stride = G * 16;
+  const __amdgpu_buffer_rsrc_t wr = make_rsrc(
+      static_cast<const char*>(p.w) + (tile_base + static_cast<size_t>(nt0) * KT) * 1024, NT * w_tile_stride);
+  const __amdgpu_buffer_rsrc_t sr = make_rsrc(
+      static_cast<const char*>(p.scales) + (sz_base + static_cast<size_t>(nt0) * G * 16) * 2, NT * s_tile_stride);
+  const __amdgpu_buffer_rsrc_t zr = make_rsrc(
+      HAS_ZP ? static_cast<const char*>(p.zeros) + sz_base + static_cast<size_t>(nt0) * G * 16 : nullptr,
+      HAS_ZP ? NT * z_tile_stride : 0);
+  // x spans less than 1 GiB (checked on the host), so offset kOutOfRange is past this constant extent
+  const __amdgpu_buffer_rsrc_t xr = make_rsrc(p.x, 0x3fffffffu);
+  const uint32_t w_off = lane * 16;
+  const uint32_t s_off = lrow * 2;
+  const uint32_t z_off = lrow;
+  uint32_t x_off[MT];
 #pragma unroll
-  for (int t = 0; t < NT; ++t) {
-    wbase[t] = p.w + (tile_base + static_cast<size_t>(nt0 + t) * KT) * 64 + lane;
-    sbase[t] = p.scales + sz_base + static_cast<size_t>(nt0 + t) * G * 16 + 4 * lq;
-    zbase[t] = HAS_ZP ? p.zeros + sz_base + static_cast<size_t>(nt0 + t) * G * 16 + 4 * lq : nullptr;
-  }
-  const uint16_t* xbase[MT];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
-    xbase[mt] = static_cast<const uint16_t*>(p.x) + static_cast<size_t>(xrow[mt]) * p.K + lq * 8;
+  for (int mt = 0; mt < MT; ++mt) x_off[mt] = (xrow[mt] * p.K + lq * 8) * 2;
 
+  // acc[t][mt][i]: column (nt0+t)*16 + lrow, row mt*16 + 4*lq + i
   f32x4 acc[NT][MT];
 #pragma unroll
   for (int t = 0; t < NT; ++t)
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[t][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  struct Stage {
-    u32x4 wq[NT];
+  struct Slot {  // one weight tile with its scales / zero points
+    u32x4 wq;
+    uint32_t sc[GPT];  // 16-bit scale and 8-bit zero point, each widened into a register of its own so that no
+    uint32_t zp[GPT];  // packing of ring slots ties loads of different groups together
+  };
+  struct XBuf {
     u32x4 xf[MT][4];
-    u32x2 sc[NT][GPT];
-    uint32_t zp[NT][GPT];
+  };
+  // Scalar byte offsets of one k-tile in the four buffers.  A k-tile past the end of K gets kOutOfRange:
+  // buffer loads beyond the resource's extent return zero, zero x and zero scales contribute nothing, and every
+  // wavefront runs the same instruction sequence, so the waits count exactly the loads allowed to stay in flight.
+  constexpr uint32_t kOutOfRange = 0x40000000u;
+  struct KOff {
+    uint32_t w, s, z, x;
+  };
+  const uint32_t kt_begin = 0;
+  const uint32_t kt_end = KT;
+  auto koff = [&](uint32_t round) {
+    const uint32_t kt = kt_begin + wave + round * WAVES;
+    const bool ok = kt < kt_end;
+    KOff o;
+    // readfirstlane pins the offsets to scalar registers (a vector offset would make every load a waterfall loop)
+    o.w = __builtin_amdgcn_readfirstlane(ok ? kt * 1024u : kOutOfRange);
+    o.s = __builtin_amdgcn_readfirstlane(ok ? kt * (GPT * 32u) : kOutOfRange);
+    o.z = __builtin_amdgcn_readfirstlane(ok ? kt * (GPT * 16u) : kOutOfRange);
+    o.x = __builtin_amdgcn_readfirstlane(ok ? kt * 256u : kOutOfRange);
+    return o;
   };
 
-  auto load_stage = [&](Stage& s, uint32_t kt) {
+  auto load_slot = [&](Slot& s, int t, const KOff& o) {
+    s.wq = __builtin_amdgcn_raw_buffer_load_b128(wr, w_off, t * w_tile_stride + o.w, 2);
 #pragma unroll
-    for (int t = 0; t < NT; ++t) s.wq[t] = __builtin_nontemporal_load(wbase[t] + static_cast<size_t>(kt) * 64);
+    for (int gi = 0; gi < GPT; ++gi) {
+      s.sc[gi] = __builtin_amdgcn_raw_buffer_load_b16(sr, s_off, t * s_tile_stride + o.s + gi * 32, 0);
+      if (HAS_ZP) s.zp[gi] = __builtin_amdgcn_raw_buffer_load_b8(zr, z_off, t * z_tile_stride + o.z + gi * 16, 0);
+    }
+  };
+  auto load_x = [&](XBuf& b, const KOff& o) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-      for (int d = 0; d < 4; ++d)
-        s.xf[mt][d] = ok[mt] ? *reinterpret_cast<const u32x4*>(xbase[mt] + kt * 128 + d * 32) : u32x4{0, 0, 0, 0};
-#pragma unroll
-    for (int t = 0; t < NT; ++t)
-#pragma unroll
-      for (int gi = 0; gi < GPT; ++gi) {
-        s.sc[t][gi] = *reinterpret_cast<const u32x2*>(sbase[t] + (static_cast<size_t>(kt) * GPT + gi) * 16);
-        if (HAS_ZP) s.zp[t][gi] = *reinterpret_cast<const uint32_t*>(zbase[t] + (static_cast<size_t>(kt) * GPT + gi) * 16);
-      }
+      for (int d = 0; d < 4; ++d) b.xf[mt][d] = __builtin_amdgcn_raw_buffer_load_b128(xr, x_off[mt], o.x + d * 64, 0);
   };
 
   const typename T::frag ones = as_frag<T>(u32x4{T::kOne2, T::kOne2, T::kOne2, T::kOne2});
+  uint32_t magic2 = p.magic2;
+  asm volatile("" : "+v"(magic2));  // no instruction: keeps the value in a VGPR so the three-operand form applies
+  const uint32_t nmask = p.nibble_mask;
 
-  auto compute_stage = [&](const Stage& s) {
+  auto sum_x = [&](const XBuf& b, f32x4 (&sx)[GPT][MT]) {
 #pragma unroll
-    for (int gi = 0; gi < GPT; ++gi) {
-      float sx[MT];
+    for (int gi = 0; gi < GPT; ++gi)
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
         f32x4 r{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int d = gi * SPG; d < (gi + 1) * SPG; ++d) r = T::mfma(ones, as_frag<T>(s.xf[mt][d]), r);
-        sx[mt] = r.x;
+        for (int d = gi * SPG; d < (gi + 1) * SPG; ++d) r = T::mfma(as_frag<T>(b.xf[mt][d]), ones, r);
+        sx[gi][mt] = r;
       }
+  };
+  auto compute = [&](const Slot& s, const XBuf& b, const f32x4 (&sx)[GPT][MT], int t) {
 #pragma unroll
-      for (int t = 0; t < NT; ++t) {
-        float sc[4], cz[4];
-        sc[0] = T::to_float(static_cast<uint16_t>(s.sc[t][gi].x & 0xffffu));
-        sc[1] = T::to_float(static_cast<uint16_t>(s.sc[t][gi].x >> 16));
-        sc[2] = T::to_float(static_cast<uint16_t>(s.sc[t][gi].y & 0xffffu));
-        sc[3] = T::to_float(static_cast<uint16_t>(s.sc[t][gi].y >> 16));
+    for (int gi = 0; gi < GPT; ++gi) {
+      const float sc = T::lo_to_float(s.sc[gi]);
+      const float ncz = HAS_ZP ? -(T::kMagic + static_cast<float>(s.zp[gi])) : -(T::kMagic + 8.0f);
+      typename T::frag wf[SPG];
+#pragma unroll
+      for (int d = 0; d < SPG; ++d) wf[d] = dequant_magic_fast<T>(s.wq[gi * SPG + d], nmask, magic2);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        f32x4 r{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int d = 0; d < SPG; ++d) r = T::mfma(as_frag<T>(b.xf[mt][gi * SPG + d]), wf[d], r);
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-          cz[i] = HAS_ZP ? T::kMagic + static_cast<float>((s.zp[t][gi] >> (8 * i)) & 0xffu) : T::kMagic + 8.0f;
-        typename T::frag wf[SPG];
-#pragma unroll
-        for (int d = 0; d < SPG; ++d) wf[d] = dequant_magic<T>(s.wq[t][gi * SPG + d]);
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          f32x4 r{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-          for (int d = 0; d < SPG; ++d) r = T::mfma(wf[d], as_frag<T>(s.xf[mt][gi * SPG + d]), r);
-#pragma unroll
-          for (int i = 0; i < 4; ++i) acc[t][mt][i] += sc[i] * (r[i] - cz[i] * sx[mt]);
-        }
+          acc[t][mt][i] = __builtin_fmaf(sc, __builtin_fmaf(ncz, sx[gi][mt][i], r[i]), acc[t][mt][i]);
       }
     }
   };
 
-  // ---- main loop, one stage of loads in flight ahead of the math
-  uint32_t kt = wave;
-  if (kt < KT) {
-    Stage cur;
-    load_stage(cur, kt);
-    for (;;) {
-      uint32_t nk = kt + WAVES;
-      if (nk < KT) {
-        Stage nxt;
-        load_stage(nxt, nk);
-        compute_stage(cur);
-        cur = nxt;
-        kt = nk;
-      } else {
-        compute_stage(cur);
-        break;
+  // ---- main loop.  The ring holds LOOK k-tiles, each a load group of NT weight tiles (with scales / zero points)
+  // followed by the x fragments; a group is refilled for round cur+LOOK while round cur is consumed, so LOOK-1
+  // whole groups stay in flight behind every wait.  The round count is uniform over the workgroup and a multiple
+  // of LOOK, the surplus rounds load zeros.
+  const uint32_t slice_len = kt_end - kt_begin;
+  const uint32_t rounds = (slice_len + WAVES * LOOK - 1) / (WAVES * LOOK) * LOOK;
+  Slot slot[LOOK][NT];
+  XBuf xb[LOOK];
+#pragma unroll
+  for (int j = 0; j < LOOK; ++j) {
+    const KOff o = koff(j);
+#pragma unroll
+    for (int t = 0; t < NT; ++t) load_slot(slot[j][t], t, o);
+    load_x(xb[j], o);
+    __builtin_amdgcn_sched_barrier(0);  // keep the groups in issue order, the waits below count on it
+  }
+  for (uint32_t it = 0; it < rounds; it += LOOK) {
+#pragma unroll
+    for (int h = 0; h < LOOK; ++h) {
+      const KOff o = koff(it + h + LOOK);  // past the last round this is out of range by construction
+      f32x4 sx[GPT][MT];
+      sum_x(xb[h], sx);
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        compute(slot[h][t], xb[h], sx, t);
+        // the refill must be issued here, not sunk below the remaining math: the barriers pin it in place
+        __builtin_amdgcn_sched_barrier(0);
+        load_slot(slot[h][t], t, o);
+        __builtin_amdgcn_sched_barrier(0);
       }
+      load_x(xb[h], o);
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
 
@@ -187,24 +255,23 @@ __global__ void __launch_bounds__(WAVES * 64) w4a16_splitk_kernel(SplitKParams p
     f32x4 v = red[0][tm][l];
 #pragma unroll
     for (int w = 1; w < WAVES; ++w) v += red[w][tm][l];
-    uint32_t orow;
-    bool valid;
-    float rw = 1.0f;
-    if (GROUPED) {
-      uint32_t sid = static_cast<uint32_t>(p.sorted_ids[blockIdx.y * (16 * MT) + mt * 16 + (l & 15)]);
-      valid = sid < p.numel;
-      orow = sid;
-      if (valid && p.topk_w) rw = p.topk_w[sid];
-    } else {
-      orow = blockIdx.y * (16 * MT) + mt * 16 + (l & 15);
-      valid = orow < p.M;
-    }
-    if (valid) {
-      u32x2 o;
-      o.x = pack2(T::from_float(v[0] * rw), T::from_float(v[1] * rw));
-      o.y = pack2(T::from_float(v[2] * rw), T::from_float(v[3] * rw));
-      uint16_t* yp = static_cast<uint16_t*>(p.y) + static_cast<size_t>(orow) * p.N + (nt0 + t) * 16 + 4 * (l >> 4);
-      *reinterpret_cast<u32x2*>(yp) = o;
+    const uint32_t col = (nt0 + t) * 16 + (l & 15);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t r = mt * 16 + 4 * (l >> 4) + i;
+      uint32_t orow;
+      bool valid;
+      float rw = 1.0f;
+      if (GROUPED) {
+        uint32_t sid = static_cast<uint32_t>(p.sorted_ids[blockIdx.y * (16 * MT) + r]);
+        valid = sid < p.numel;
+        orow = sid;
+        if (valid && p.topk_w) rw = p.topk_w[sid];
+      } else {
+        orow = blockIdx.y * (16 * MT) + r;
+        valid = orow < p.M;
+      }
+      if (valid) static_cast<uint16_t*>(p.y)[static_cast<size_t>(orow) * p.N + col] = T::from_float(v[i] * rw);
     }
   }
 }

@@ -3,7 +3,7 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libksq_hip.so")
+LIB_PATH = os.environ.get("KSQ_LIB_PATH", os.path.join(_HERE, "libksq_hip.so"))
 
 F16, BF16, F32 = 0, 1, 2
 SRC_GPTQ, SRC_AWQ, SRC_MOE_NK, SRC_INT4X2_KN = 0, 1, 2, 3
