@@ -34,6 +34,13 @@ SplitKChoice select_splitk_blocks(int mt, size_t m_blocks, size_t n, size_t k) {
   return c;
 }
 
+// Regime switch.  W4A16 moves 0.5 byte per weight and 2*m flops: on this part the HBM and MFMA bounds cross near
+// m = 80; the split-K kernel handles up to two 16-row tiles per workgroup, the tile kernel takes over above that.
+bool use_mfma_tile(size_t m, size_t n, size_t k, size_t group) {
+  (void)k;
+  return m > 32 && group == 128 && n % 256 == 0;
+}
+
 }  // namespace ksq
 
 using namespace ksq;
@@ -46,6 +53,16 @@ KSQ_EXPORT int ksq_select_tile(int kind, size_t m, size_t n, size_t k, int dtype
   switch (kind) {
     case KSQ_KIND_W4A16:
     case KSQ_KIND_MOE_W4A16: {
+      if (kind == KSQ_KIND_W4A16 && use_mfma_tile(m, n, k, 128)) {
+        d->kernel = KSQ_KERNEL_MFMA_TILE;
+        d->block_m = m <= 128 ? 128 : 256;
+        d->block_n = 256;
+        d->block_k = 64;
+        d->waves = 8;
+        d->split_k = 1;
+        d->grid = static_cast<int32_t>(div_up(m, d->block_m) * (n / 256));
+        return KSQ_OK;
+      }
       SplitKChoice c = select_splitk(m, n, k);
       d->kernel = KSQ_KERNEL_SPLITK_WAVE;
       d->block_m = 16 * c.mt;

@@ -5,6 +5,7 @@
 #include "ksq_common.h"
 #include "tile_select.h"
 #include "w4a16_splitk.h"
+#include "w4a16_tile.h"
 
 namespace ksq {
 namespace {
@@ -74,6 +75,27 @@ int dispatch_tile(SplitKParams& p, SplitKChoice c, uint32_t m_blocks, size_t gro
   return fail(KSQ_ERR_UNSUPPORTED, "no split-K kernel for mt=%d nt=%d waves=%d", c.mt, c.nt, c.waves);
 }
 
+template <typename T, int WAVES_M, int WAVES_N, int WM, int WN>
+int launch_tile(const TileParams& p0, hipStream_t s) {
+  constexpr int BM = WAVES_M * WM * 16, BN = WAVES_N * WN * 16;
+  TileParams p = p0;
+  p.tiles_m = static_cast<uint32_t>(div_up(p.M, BM));
+  p.tiles_n = p.N / BN;
+  const size_t lds = 2 * (BM / 16) * 2 * 1024;
+  const unsigned grid = p.tiles_m * p.tiles_n;
+  if (p.zeros)
+    w4a16_tile_kernel<T, WAVES_M, WAVES_N, WM, WN, true><<<grid, WAVES_M * WAVES_N * 64, lds, s>>>(p);
+  else
+    w4a16_tile_kernel<T, WAVES_M, WAVES_N, WM, WN, false><<<grid, WAVES_M * WAVES_N * 64, lds, s>>>(p);
+  return KSQ_OK;
+}
+
+template <typename T>
+int dispatch_mfma_tile(const TileParams& p, hipStream_t s) {
+  if (p.M <= 128) return launch_tile<T, 1, 8, 8, 2>(p, s);  // 128 x 256
+  return launch_tile<T, 2, 4, 8, 4>(p, s);                  // 256 x 256
+}
+
 int check_common(const char* fn, const void* y, const void* x, const void* w, const void* sc, size_t n, size_t k,
                  size_t group, int dtype) {
   if (!y || !x || !w || !sc) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: null pointer", fn);
@@ -106,7 +128,9 @@ KSQ_EXPORT int ksq_w4a16_gemm(void* y, const void* x, const void* w_packed, cons
   if (int rc = check_common(fn, y, x, w_packed, scales_packed, n, k, group, dtype)) return rc;
   (void)workspace; (void)workspace_bytes;
   if (m == 0) return KSQ_OK;
-  if (m > 0x7fffffffull || m * k * 2 >= 0x40000000ull) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: m too large", fn);
+  if (m > 0x7fffffffull) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: m too large", fn);
+  if (!use_mfma_tile(m, n, k, group) && m * k * 2 >= 0x40000000ull)
+    return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: m too large for this shape", fn);
   SplitKParams p{};
   p.y = y;
   p.x = x;
@@ -117,6 +141,20 @@ KSQ_EXPORT int ksq_w4a16_gemm(void* y, const void* x, const void* w_packed, cons
   p.N = static_cast<uint32_t>(n);
   p.K = static_cast<uint32_t>(k);
   p.x_bytes = static_cast<uint32_t>(m * k * 2);
+  if (use_mfma_tile(m, n, k, group)) {
+    TileParams tp{};
+    tp.y = y;
+    tp.x = x;
+    tp.w = w_packed;
+    tp.scales = scales_packed;
+    tp.zeros = zeros_packed;
+    tp.M = static_cast<uint32_t>(m);
+    tp.N = static_cast<uint32_t>(n);
+    tp.K = static_cast<uint32_t>(k);
+    int rc = dtype == KSQ_F16 ? dispatch_mfma_tile<F16>(tp, as_stream(stream)) : dispatch_mfma_tile<BF16>(tp, as_stream(stream));
+    if (rc) return rc;
+    return check_launch(fn);
+  }
   SplitKChoice c = select_splitk(m, n, k);
   if (const char* f = getenv("KSQ_FORCE_SPLITK")) sscanf(f, "%d,%d,%d", &c.mt, &c.nt, &c.waves);
   const size_t m_blocks = div_up(m, 16 * c.mt);

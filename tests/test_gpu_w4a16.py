@@ -42,7 +42,27 @@ def test_cfg1_gptq_fp16(ops, M):
 def test_cfg2_awq_bf16(ops, M, N, K):
     d = H.make_w4a16(2000 + M + N, M, N, K, 128, H.BF16, awq=True, s_lo=0.003, s_hi=0.015)
     y = run_case(ops, d)
-    H.check_gemm(y, H.w4a16_oracle(d), H.BF16, "cfg2 M=%d N=%d K=%d" % (M, N, K))
+    H.check_gemm(y, H.w4a16_oracle(d), H.BF16, "cfg2 M=%d N=%d K=%d" % (M, N, K), weights_rounded=M > 32)
+
+
+# prefill regime (MFMA tile kernel): ragged M, both dtypes, with and without zero points
+@pytest.mark.parametrize("dtype", [H.F16, H.BF16])
+@pytest.mark.parametrize("awq", [False, True])
+@pytest.mark.parametrize("M,N,K", [(33, 256, 256), (130, 512, 1024), (300, 768, 512), (512, 14336, 4096)])
+def test_prefill_tile_kernel(ops, dtype, awq, M, N, K):
+    from ksanallm_amd import lib as L
+    assert L.select_tile(L.KIND_W4A16, M, N, K, dtype)["kernel"] == 1
+    d = H.make_w4a16(3000 + M + N, M, N, K, 128, dtype, awq=awq, x_std=0.5, s_lo=0.002, s_hi=0.01, z_lo=0, z_hi=15)
+    y = run_case(ops, d)
+    H.check_gemm(y, H.w4a16_oracle(d), dtype, "prefill M=%d N=%d K=%d" % (M, N, K), weights_rounded=True)
+
+
+# config 3 shape (Qwen-32B-like, GPTQ fp16) at a row count the CPU oracle finishes in seconds
+@pytest.mark.parametrize("N,K", [(25600, 5120), (5120, 25600)])
+def test_cfg3_gptq_fp16_prefill(ops, N, K):
+    d = H.make_w4a16(3100 + N, 256, N, K, 128, H.F16, awq=False, x_std=0.5, s_lo=0.002, s_hi=0.01)
+    y = run_case(ops, d)
+    H.check_gemm(y, H.w4a16_oracle(d), H.F16, "cfg3 N=%d K=%d" % (N, K), weights_rounded=True)
 
 
 @pytest.mark.parametrize("dtype", [H.F16, H.BF16])
