@@ -154,6 +154,14 @@ int ksq_moe_w4a16_gemm(void* out, const void* x, const void* w_packed, const voi
                        const void* num_post_pad, size_t numel, size_t top_k, size_t E, size_t n, size_t k,
                        size_t group, size_t block_m, int dtype, void* stream);
 
+/* Router: softmax over the E gating logits of every token in fp32, the top_k largest probabilities in descending
+ * order (ties: lower expert id first), weights = probability * routed_scaling_factor, optionally renormalised to
+ * sum to routed_scaling_factor over the top_k first (norm_topk_prob).  gating [tokens, E] in `dtype` (KSQ_F32
+ * allowed), topk_w fp32 [tokens, top_k], topk_ids int32 [tokens, top_k].  E <= 1024, top_k <= 32.
+ * Replaces InvokeBasicSoftmaxTopk (K/grouped_topk/grouped_topk.cu:678-755), the routing step in front of the path. */
+int ksq_moe_topk_softmax(const void* gating, void* topk_w, void* topk_ids, size_t tokens, size_t E, size_t top_k,
+                         int norm_topk_prob, float routed_scaling_factor, int dtype, void* stream);
+
 /* out[r, i] = T(silu(x[r, i]) * x[r, inter + i]), fp32 math a / (1 + expf(-a)) * b.
  * Replaces InvokeSiluAndMul (K/moe_utils/moe_utils.cu:893-905). */
 int ksq_moe_silu_mul(const void* x, void* out, size_t rows, size_t inter, int dtype, void* stream);

@@ -51,5 +51,28 @@ def build(verbose=False, jobs=None):
     return LIB
 
 
+LAYERS = os.path.join(HERE, "layers")
+LAYERS_LIB = os.path.join(HERE, "libksq_layers.so")
+LAYER_TEST = os.path.join(ROOT, "tests", "cpp", "layer_test")
+
+
+def build_layers():
+    """C++ layer classes (host code only) -> libksq_layers.so, and the driver tests/cpp/layer_test that links them."""
+    srcs = sorted(os.path.join(LAYERS, f) for f in os.listdir(LAYERS) if f.endswith(".cpp"))
+    common = [HIPCC, "-std=c++17", "-O2", "-fPIC", "-I" + os.path.join(ROOT, "include"), "-I" + LAYERS,
+              "-Wno-unused-command-line-argument"]
+    link = ["-L" + HERE, "-lksq_hip", "-Wl,-rpath,$ORIGIN"]
+    r = subprocess.run(common + ["-shared", "-o", LAYERS_LIB] + srcs + link, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("layer build failed:\n" + r.stderr)
+    r = subprocess.run(common + ["-o", LAYER_TEST, os.path.join(ROOT, "tests", "cpp", "layer_test.cpp"),
+                                 "-L" + HERE, "-lksq_layers", "-lksq_hip",
+                                 "-Wl,-rpath,$ORIGIN/../../ksanallm_amd"], capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("layer test build failed:\n" + r.stderr)
+    return LAYERS_LIB, LAYER_TEST
+
+
 if __name__ == "__main__":
     print(build(verbose=True))
+    print(build_layers())

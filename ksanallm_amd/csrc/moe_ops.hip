@@ -129,6 +129,81 @@ __global__ void __launch_bounds__(256) moe_sum_kernel(const uint16_t* __restrict
   *reinterpret_cast<u32x4*>(out + t * d + c) = o;
 }
 
+// one wavefront per token: lane l holds experts l, l+64, ... (at most 16 each)
+template <typename LOAD>
+__global__ void __launch_bounds__(256) topk_softmax_kernel(const void* __restrict__ gating, float* __restrict__ topk_w,
+                                                           int32_t* __restrict__ topk_ids, uint32_t tokens,
+                                                           uint32_t E, uint32_t top_k, int norm, float scaling) {
+  const uint32_t token = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (token >= tokens) return;
+  float v[16];
+  float mx = -INFINITY;
+#pragma unroll
+  for (int j = 0; j < 16; ++j) {
+    const uint32_t e = j * 64 + lane;
+    v[j] = e < E ? LOAD::get(gating, static_cast<size_t>(token) * E + e) : -INFINITY;
+    mx = fmaxf(mx, v[j]);
+  }
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+  float sum = 0.f;
+#pragma unroll
+  for (int j = 0; j < 16; ++j) {
+    const uint32_t e = j * 64 + lane;
+    v[j] = e < E ? expf(v[j] - mx) : -1.0f;  // -1 never wins the arg-max below
+    sum += e < E ? v[j] : 0.f;
+  }
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) sum += __shfl_xor(sum, off, 64);
+  float picked_sum = 0.f;
+  float my_w = 0.f;
+  int my_id = 0;
+  for (uint32_t r = 0; r < top_k; ++r) {
+    float best = -2.0f;
+    uint32_t best_e = 0xffffffffu;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      const uint32_t e = j * 64 + lane;
+      if (v[j] > best) {  // ascending e inside a lane: strict > keeps the lower id on ties
+        best = v[j];
+        best_e = e;
+      }
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+      const float ob = __shfl_xor(best, off, 64);
+      const uint32_t oe = __shfl_xor(best_e, off, 64);
+      if (ob > best || (ob == best && oe < best_e)) {
+        best = ob;
+        best_e = oe;
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 16; ++j)
+      if (static_cast<uint32_t>(j * 64 + lane) == best_e) v[j] = -1.0f;
+    const float prob = best / sum;
+    picked_sum += prob;
+    if (static_cast<uint32_t>(lane) == r) {
+      my_w = prob;
+      my_id = static_cast<int>(best_e);
+    }
+  }
+  if (static_cast<uint32_t>(lane) < top_k) {
+    const float w = norm ? my_w / picked_sum : my_w;
+    topk_w[static_cast<size_t>(token) * top_k + lane] = w * scaling;
+    topk_ids[static_cast<size_t>(token) * top_k + lane] = my_id;
+  }
+}
+
+struct LoadF32 {
+  static __device__ __forceinline__ float get(const void* p, size_t i) { return static_cast<const float*>(p)[i]; }
+};
+template <typename T>
+struct Load16 {
+  static __device__ __forceinline__ float get(const void* p, size_t i) { return T::to_float(static_cast<const uint16_t*>(p)[i]); }
+};
+
 void align_geometry(size_t numel, uint32_t* chunks, uint32_t* per) {
   size_t c = div_up(numel, 8);
   if (c < 1) c = 1;
@@ -170,6 +245,31 @@ KSQ_EXPORT int ksq_moe_align(const void* topk_ids, size_t numel, size_t E, size_
       static_cast<uint32_t>(block_m), static_cast<uint32_t>(cap), static_cast<int32_t*>(sorted_ids),
       static_cast<int32_t*>(expert_ids), static_cast<int32_t*>(num_post_pad), static_cast<int32_t*>(scratch), chunks,
       per);
+  return check_launch(fn);
+}
+
+KSQ_EXPORT int ksq_moe_topk_softmax(const void* gating, void* topk_w, void* topk_ids, size_t tokens, size_t E,
+                                    size_t top_k, int norm_topk_prob, float routed_scaling_factor, int dtype,
+                                    void* stream) {
+  const char* fn = "ksq_moe_topk_softmax";
+  if (!gating || !topk_w || !topk_ids) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: null pointer", fn);
+  if (E == 0 || E > 1024 || top_k == 0 || top_k > 32 || top_k > E)
+    return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: need 1 <= top_k <= min(32, E) and E <= 1024", fn);
+  if (tokens == 0) return KSQ_OK;
+  if (tokens > 0x7fffffffull) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: too many tokens", fn);
+  const unsigned blocks = static_cast<unsigned>(div_up(tokens, 4));
+  float* w = static_cast<float*>(topk_w);
+  int32_t* ids = static_cast<int32_t*>(topk_ids);
+  const uint32_t t = static_cast<uint32_t>(tokens), e = static_cast<uint32_t>(E), k = static_cast<uint32_t>(top_k);
+  hipStream_t st = as_stream(stream);
+  if (dtype == KSQ_F32)
+    topk_softmax_kernel<LoadF32><<<blocks, 256, 0, st>>>(gating, w, ids, t, e, k, norm_topk_prob, routed_scaling_factor);
+  else if (dtype == KSQ_F16)
+    topk_softmax_kernel<Load16<F16>><<<blocks, 256, 0, st>>>(gating, w, ids, t, e, k, norm_topk_prob, routed_scaling_factor);
+  else if (dtype == KSQ_BF16)
+    topk_softmax_kernel<Load16<BF16>><<<blocks, 256, 0, st>>>(gating, w, ids, t, e, k, norm_topk_prob, routed_scaling_factor);
+  else
+    return fail(KSQ_ERR_UNSUPPORTED, "%s: unknown dtype %d", fn, dtype);
   return check_launch(fn);
 }
 

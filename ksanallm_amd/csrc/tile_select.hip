@@ -48,7 +48,9 @@ using namespace ksq;
 KSQ_EXPORT int ksq_select_tile(int kind, size_t m, size_t n, size_t k, int dtype, ksq_tile_desc* d) {
   if (!d) return fail(KSQ_ERR_INVALID_ARGUMENT, "ksq_select_tile: null descriptor");
   if (m == 0 || n == 0 || k == 0) return fail(KSQ_ERR_INVALID_ARGUMENT, "ksq_select_tile: empty problem");
-  (void)dtype;
+  if (dtype != KSQ_F16 && dtype != KSQ_BF16) return fail(KSQ_ERR_UNSUPPORTED, "ksq_select_tile: dtype %d has no kernel", dtype);
+  if (k % 128 != 0 || n % 16 != 0)
+    return fail(KSQ_ERR_UNSUPPORTED, "ksq_select_tile: no kernel for n=%zu k=%zu (k must be a multiple of 128, n of 16)", n, k);
   *d = ksq_tile_desc{};
   switch (kind) {
     case KSQ_KIND_W4A16:

@@ -1,0 +1,43 @@
+#include "quant_weight_repack.h"
+
+namespace ksana_llm {
+
+Tensor PackGroupQuantWeight(const Tensor& qweight, const Tensor& scales, const Tensor* qzeros, QuantMode method,
+                            size_t group_size, int rank, hipStream_t stream) {
+  const char* who = "PackGroupQuantWeight";
+  if (method != QUANT_GPTQ && method != QUANT_AWQ) KLLM_THROW("PackGroupQuantWeight: method must be GPTQ or AWQ");
+  if (qweight.shape.size() != 2 || scales.shape.size() != 2) KLLM_THROW("PackGroupQuantWeight: 2-D tensors expected");
+  const bool awq = method == QUANT_AWQ;
+  const size_t K = awq ? qweight.shape[0] : qweight.shape[0] * 8;
+  const size_t N = awq ? qweight.shape[1] * 8 : qweight.shape[1];
+  if (scales.shape[0] * group_size != K || scales.shape[1] != N) KLLM_THROW("PackGroupQuantWeight: scales shape mismatch");
+  if (awq && !qzeros) KLLM_THROW("PackGroupQuantWeight: AWQ needs qzeros");
+  const int dtype = KsqDtype(scales.dtype, who);
+
+  Tensor packed(MemoryLocation::LOCATION_DEVICE, TYPE_I4_GROUP, {K, N / 2}, rank);
+  KsqCheck(ksq_w4a16_repack(qweight.GetPtr<void>(), awq ? KSQ_SRC_AWQ : KSQ_SRC_GPTQ, packed.GetPtr<void>(), 1, K, N, stream), who);
+  packed.scales = std::make_shared<Tensor>(MemoryLocation::LOCATION_DEVICE, scales.dtype, scales.shape, rank);
+  KsqCheck(ksq_w4a16_repack_scales(scales.GetPtr<void>(), KSQ_SCALE_GN, packed.scales->GetPtr<void>(), 1, K, N, group_size, dtype, stream), who);
+  if (awq) {
+    packed.zeros = std::make_shared<Tensor>(MemoryLocation::LOCATION_DEVICE, TYPE_UINT8, std::vector<size_t>{K / group_size, N}, rank);
+    KsqCheck(ksq_w4a16_repack_zeros(qzeros->GetPtr<void>(), KSQ_ZERO_AWQ_PACKED, packed.zeros->GetPtr<void>(), K, N, group_size, stream), who);
+  }
+  return packed;
+}
+
+Tensor PackMoeExpertWeight(const Tensor& experts, const Tensor& scales, size_t group_size, int rank, hipStream_t stream) {
+  const char* who = "PackMoeExpertWeight";
+  if (experts.shape.size() != 3 || scales.shape.size() != 3) KLLM_THROW("PackMoeExpertWeight: 3-D tensors expected");
+  const size_t E = experts.shape[0], N = experts.shape[1], K = experts.shape[2] * 2;
+  if (scales.shape[0] != E || scales.shape[1] != N || scales.shape[2] * group_size != K) {
+    KLLM_THROW("PackMoeExpertWeight: scales shape mismatch");
+  }
+  const int dtype = KsqDtype(scales.dtype, who);
+  Tensor packed(MemoryLocation::LOCATION_DEVICE, TYPE_UINT4x2, experts.shape, rank);
+  KsqCheck(ksq_w4a16_repack(experts.GetPtr<void>(), KSQ_SRC_MOE_NK, packed.GetPtr<void>(), E, K, N, stream), who);
+  packed.scales = std::make_shared<Tensor>(MemoryLocation::LOCATION_DEVICE, scales.dtype, scales.shape, rank);
+  KsqCheck(ksq_w4a16_repack_scales(scales.GetPtr<void>(), KSQ_SCALE_NG, packed.scales->GetPtr<void>(), E, K, N, group_size, dtype, stream), who);
+  return packed;
+}
+
+}  // namespace ksana_llm

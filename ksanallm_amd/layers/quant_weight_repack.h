@@ -1,0 +1,24 @@
+// Loader-side half of the path: turns the tensors a GPTQ / AWQ checkpoint holds into the single packed weight tensor
+// the layers consume, with its scale / zero-point tensors bound as side tensors.
+// Stands where the reference converts layouts after slicing for tensor parallelism:
+//   dense   QuantWeight::ConvertGroupTensor / PackAndBindGroupTensor  (src/ksana_llm/models/quant/quant_weight.cpp:321-520,
+//           716-753) with CutlassUtils / MarlinUtils / MacheteUtils    (src/ksana_llm/models/quant/*_utils.cpp)
+//   experts the [E, N, K/2] uint4x2 stacks of the moe-int4 loader      (src/ksana_llm/models/quant/quant_weight.cpp:182-319)
+// All device work is enqueued on `stream`; the sources may be released once the stream has drained.
+#pragma once
+
+#include "base_layer.h"
+
+namespace ksana_llm {
+
+// qweight: GPTQ [K/8, N] int32 or AWQ [K, N/8] int32 (device).  scales: [K/group, N] in T.  qzeros: AWQ only,
+// [K/group, N/8] int32 (nullptr for GPTQ, whose symmetric zero point 8 is implicit).
+// Returns a TYPE_I4_GROUP tensor of logical shape {K, N/2} with `scales` (and `zeros`) bound.
+Tensor PackGroupQuantWeight(const Tensor& qweight, const Tensor& scales, const Tensor* qzeros, QuantMode method,
+                            size_t group_size, int rank, hipStream_t stream);
+
+// experts: [E, N, K/2] uint8, low nibble = even k.  scales: [E, N, K/group] in T.
+// Returns a TYPE_UINT4x2 tensor of logical shape {E, N, K/2} with `scales` bound.
+Tensor PackMoeExpertWeight(const Tensor& experts, const Tensor& scales, size_t group_size, int rank, hipStream_t stream);
+
+}  // namespace ksana_llm

@@ -1,0 +1,79 @@
+#include "w4a16_matmul_layer.h"
+
+namespace ksana_llm {
+
+Status W4A16MatMulLayer::Init(const std::vector<std::any>& parameters, const RuntimeConfig& runtime_config,
+                              std::shared_ptr<Context> context, int rank) {
+  STATUS_CHECK_FAILURE(BaseLayer::Init(parameters, runtime_config, context, rank));
+  if (parameters.size() < 9) {
+    return Status(RET_INVALID_ARGUMENT, std::string(Name()) + ": expects 9 init parameters");
+  }
+  int parameter_index = 0;
+  max_m_ = std::any_cast<const size_t>(parameters[parameter_index++]);
+  max_n_ = std::any_cast<const size_t>(parameters[parameter_index++]);
+  max_k_ = std::any_cast<const size_t>(parameters[parameter_index++]);
+  groupsize_ = std::any_cast<const size_t>(parameters[parameter_index++]);
+  is_awq_ = std::any_cast<const bool>(parameters[parameter_index++]);
+  is_gptq_desc_ = std::any_cast<const bool>(parameters[parameter_index++]);
+  is_k_full_ = std::any_cast<const bool>(parameters[parameter_index++]);
+  [[maybe_unused]] bool use_gemv_cuda_core = std::any_cast<const bool>(parameters[parameter_index++]);  // no analogue
+  weight_data_type_ = std::any_cast<const DataType>(parameters[parameter_index++]);
+  is_k_full_ = is_gptq_desc_ ? is_k_full_ : true;
+  if (is_gptq_desc_) {
+    // act-order checkpoints need the activation columns gathered through `perm`; not built yet
+    return Status(RET_INVALID_ARGUMENT, std::string(Name()) + ": desc_act (act-order) weights are not supported");
+  }
+  return Status();
+}
+
+size_t W4A16MatMulLayer::GetWorkspaceSize() {
+  if (weight_data_type_ != TYPE_I4_GROUP) {
+    KLLM_THROW(std::string("Not supported weight data type: ") + std::to_string(weight_data_type_) + ". " + Name() +
+               " only supports TYPE_I4_GROUP.");
+  }
+  workspace_size_ = ksq_w4a16_workspace_size(max_m_, max_n_, max_k_, groupsize_, KsqDtype(inter_data_type_, Name()));
+  return workspace_size_;
+}
+
+Status W4A16MatMulLayer::Preprocess(const ModelConfig& model_config, const RuntimeConfig& runtime_config) {
+  ksq_tile_desc desc;
+  const int dtype = KsqDtype(inter_data_type_, Name());
+  const size_t probe_m[2] = {1, max_m_ ? max_m_ : 1};
+  for (size_t m : probe_m) {
+    if (ksq_select_tile(KSQ_KIND_W4A16, m, max_n_, max_k_, dtype, &desc) != KSQ_OK) {
+      return Status(RET_INVALID_ARGUMENT, std::string(Name()) + ": " + ksq_last_error_string());
+    }
+  }
+  return Status();
+}
+
+Status W4A16MatMulLayer::Forward(const std::vector<Tensor>& input_tensors, std::vector<Tensor>& output_tensors) {
+  if (weight_data_type_ != TYPE_I4_GROUP) {
+    KLLM_THROW(std::string("Not supported weight data type: ") + std::to_string(weight_data_type_) + ". " + Name() +
+               " only supports TYPE_I4_GROUP.");
+  }
+  const Tensor& weight_tensor = input_tensors[1];
+  if (!weight_tensor.scales) KLLM_THROW(std::string(Name()) + ": weight tensor has no scales bound");
+  if (is_awq_ && !weight_tensor.zeros) KLLM_THROW(std::string(Name()) + ": AWQ weight tensor has no zeros bound");
+  void* p_qweight = weight_tensor.GetPtr<void>();
+  void* p_scales = weight_tensor.scales->GetPtr<void>();
+  void* p_zeros = is_awq_ ? weight_tensor.zeros->GetPtr<void>() : nullptr;
+
+  const size_t m = input_tensors[0].shape[0];
+  const size_t n = max_n_;
+  const size_t k = max_k_;
+  if (input_tensors[0].shape.size() < 2 || input_tensors[0].shape[1] != k) {
+    KLLM_THROW(std::string(Name()) + ": activation inner dimension does not match k");
+  }
+  void* ws = workspace_buffer_ ? workspace_buffer_->GetPtr<void>() : nullptr;
+  const size_t ws_bytes = workspace_buffer_ ? workspace_buffer_->GetTotalBytes() : 0;
+  KsqCheck(ksq_w4a16_gemm(output_tensors[0].GetPtr<void>(), input_tensors[0].GetPtr<void>(), p_qweight, p_scales,
+                          p_zeros, ws, ws_bytes, m, n, k, groupsize_, KsqDtype(inter_data_type_, Name()),
+                          context_->GetComputeStreams()[rank_].Get()),
+           Name());
+  output_tensors[0].shape = {m, n};
+  output_tensors[0].dtype = input_tensors[0].dtype;
+  return Status();
+}
+
+}  // namespace ksana_llm

@@ -156,6 +156,17 @@ def moe_w4a16_gemm(x, w_packed, scales_packed, topk_w, sorted_ids, expert_ids, n
     return out
 
 
+def moe_topk_softmax(gating, top_k, norm_topk_prob=False, routed_scaling_factor=1.0):
+    """InvokeBasicSoftmaxTopk: (topk_weights fp32 [T, top_k], topk_ids int32 [T, top_k])."""
+    tokens, E = gating.shape
+    dt = _l.F32 if gating.dtype == torch.float32 else _dt(gating)
+    w = torch.empty((tokens, top_k), dtype=torch.float32, device=gating.device)
+    ids = torch.empty((tokens, top_k), dtype=torch.int32, device=gating.device)
+    _l.check(_lib.ksq_moe_topk_softmax(_ptr(gating), _ptr(w), _ptr(ids), tokens, E, top_k, int(norm_topk_prob),
+                                       float(routed_scaling_factor), dt, _stream()))
+    return w, ids
+
+
 def silu_and_mul(x, out=None):
     """InvokeSiluAndMul: x [rows, 2*inter] -> [rows, inter]."""
     rows, two = x.shape

@@ -600,6 +600,44 @@ KSQO_API void ksqo_moe_w4a16_gemm(const void* x, const uint8_t* w, const void* s
   }
 }
 
+/* Router: fp32 softmax over the experts, top_k by repeated arg-max (lowest id wins ties), weight = prob * scaling,
+ * or prob / sum(top_k probs) * scaling when norm is set.  K/grouped_topk/grouped_topk.cu:678-733
+ * (BasicSoftmaxTopkKernel); the renormalisation is the norm_topk_prob option of the layer above it. */
+KSQO_API void ksqo_moe_topk_softmax(const void* gating, float* topk_w, int32_t* topk_ids, size_t tokens, size_t E,
+                                    size_t top_k, int norm, float scaling, int dtype) {
+#pragma omp parallel for schedule(static)
+  for (size_t t = 0; t < tokens; ++t) {
+    float* sc = (float*)malloc(E * sizeof(float));
+    float mx = load_t(gating, t * E, dtype);
+    for (size_t e = 0; e < E; ++e) {
+      sc[e] = load_t(gating, t * E + e, dtype);
+      mx = fmaxf(mx, sc[e]);
+    }
+    float sum = 0.f;
+    for (size_t e = 0; e < E; ++e) {
+      sc[e] = expf(sc[e] - mx);
+      sum += sc[e];
+    }
+    float picked = 0.f;
+    for (size_t r = 0; r < top_k; ++r) {
+      size_t best = 0;
+      float bv = -2.f;
+      for (size_t e = 0; e < E; ++e)
+        if (sc[e] > bv) {
+          bv = sc[e];
+          best = e;
+        }
+      sc[best] = -1.f;
+      topk_ids[t * top_k + r] = (int32_t)best;
+      topk_w[t * top_k + r] = bv / sum;
+      picked += bv / sum;
+    }
+    for (size_t r = 0; r < top_k; ++r)
+      topk_w[t * top_k + r] = (norm ? topk_w[t * top_k + r] / picked : topk_w[t * top_k + r]) * scaling;
+    free(sc);
+  }
+}
+
 /* out[r, i] = T( silu(a) * b ) with a = x[r, i], b = x[r, inter + i], math in fp32: a / (1 + expf(-a)) * b.
  * K/moe_utils/moe_utils.cu:597-606. */
 KSQO_API void ksqo_silu_mul(const void* x, void* out, size_t rows, size_t inter, int dtype) {

@@ -301,6 +301,16 @@ def moe_w4a16_gemm(x_bits, w, scales_bits, topk_ids, topk_w, top_k_div, group, m
     return out
 
 
+def moe_topk_softmax(gating, top_k, norm, scaling, dtype):
+    g = _c(gating, _store_dt(dtype))
+    T, E = g.shape
+    w = np.empty((T, top_k), np.float32)
+    ids = np.empty((T, top_k), np.int32)
+    lib().ksqo_moe_topk_softmax(_p(g), _p(w), _p(ids), _sz(T), _sz(E), _sz(top_k), ctypes.c_int(int(norm)),
+                                ctypes.c_float(scaling), ctypes.c_int(dtype))
+    return w, ids
+
+
 def silu_mul(x_bits, dtype):
     x = _c(x_bits, _store_dt(dtype))
     rows, two_i = x.shape

@@ -1,0 +1,295 @@
+// Driver for the C++ layer classes: builds a layer through its factory exactly as model code would, feeds it the raw
+// tensors found in a directory and writes the output next to them.  tests/test_gpu_layers.py creates the inputs,
+// runs this program and compares the output with the CPU oracle.
+//
+//   layer_test w4a16     <dir> <gptq|awq> <f16|bf16> <cutlass|marlin|machete> m n k group
+//   layer_test blockwise <dir> <f16|bf16> m n k fuse_silu_mul
+//   layer_test moe       <dir> <f16|bf16> tokens experts hidden inter topk renorm scaling
+//   layer_test errors
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <fstream>
+#include <iostream>
+
+#include "blockwise_matmul_layer.h"
+#include "layer_factory.h"
+#include "moe_layer.h"
+#include "quant_weight_repack.h"
+#include "w4a16_matmul_layer.h"
+
+using namespace ksana_llm;
+
+#define HIP_OK(expr)                                                                      \
+  do {                                                                                    \
+    hipError_t _e = (expr);                                                               \
+    if (_e != hipSuccess) {                                                               \
+      std::fprintf(stderr, "%s failed: %s\n", #expr, hipGetErrorString(_e));              \
+      std::exit(2);                                                                       \
+    }                                                                                     \
+  } while (0)
+
+static std::vector<char> ReadFile(const std::string& path) {
+  std::ifstream f(path, std::ios::binary | std::ios::ate);
+  if (!f) {
+    std::fprintf(stderr, "cannot open %s\n", path.c_str());
+    std::exit(2);
+  }
+  std::vector<char> buf(static_cast<size_t>(f.tellg()));
+  f.seekg(0);
+  f.read(buf.data(), static_cast<std::streamsize>(buf.size()));
+  return buf;
+}
+
+static Tensor Upload(const std::string& path, DataType dtype, const std::vector<size_t>& shape) {
+  std::vector<char> host = ReadFile(path);
+  Tensor t(MemoryLocation::LOCATION_DEVICE, dtype, shape, 0);
+  if (host.size() != t.GetTotalBytes()) {
+    std::fprintf(stderr, "%s: %zu bytes on disk, %zu expected\n", path.c_str(), host.size(), t.GetTotalBytes());
+    std::exit(2);
+  }
+  HIP_OK(hipMemcpy(t.GetPtr<void>(), host.data(), host.size(), hipMemcpyHostToDevice));
+  return t;
+}
+
+static void Download(const Tensor& t, const std::string& path) {
+  std::vector<char> host(t.GetTotalBytes());
+  HIP_OK(hipDeviceSynchronize());
+  HIP_OK(hipMemcpy(host.data(), t.GetPtr<void>(), host.size(), hipMemcpyDeviceToHost));
+  std::ofstream f(path, std::ios::binary);
+  f.write(host.data(), static_cast<std::streamsize>(host.size()));
+}
+
+static DataType ParseT(const char* s) { return std::strcmp(s, "bf16") == 0 ? TYPE_BF16 : TYPE_FP16; }
+
+static void Drive(std::shared_ptr<BaseLayer> layer, const ModelConfig& mc, const RuntimeConfig& rc,
+                  const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) {
+  size_t ws = layer->GetWorkspaceSize();
+  auto buffer = std::make_shared<Tensor>(MemoryLocation::LOCATION_DEVICE, TYPE_INT8, std::vector<size_t>{ws ? ws : 256}, 0);
+  Status s = layer->SetWorkspaceBuffer(buffer);
+  if (!s.OK()) KLLM_THROW(s.GetMessage());
+  s = layer->Preprocess(mc, rc);
+  if (!s.OK()) KLLM_THROW(s.GetMessage());
+  s = layer->Forward(inputs, outputs);
+  if (!s.OK()) KLLM_THROW(s.GetMessage());
+}
+
+static int RunW4A16(int argc, char** argv) {
+  if (argc < 10) return 2;
+  const std::string dir = argv[2];
+  const bool awq = std::strcmp(argv[3], "awq") == 0;
+  const DataType T = ParseT(argv[4]);
+  const std::string be = argv[5];
+  const size_t m = std::atol(argv[6]), n = std::atol(argv[7]), k = std::atol(argv[8]), group = std::atol(argv[9]);
+  LinearComputeBackend backend = be == "marlin" ? MARLIN_LINEAR_BACKEND : be == "machete" ? MACHETE_LINEAR_BACKEND : CUTLASS_LINEAR_BACKEND;
+
+  hipStream_t stream;
+  HIP_OK(hipStreamCreate(&stream));
+  auto context = std::make_shared<Context>(1, stream);
+  ModelConfig mc;
+  mc.is_quant = true;
+  mc.quant_config.method = awq ? QUANT_AWQ : QUANT_GPTQ;
+  mc.quant_config.group_size = group;
+  RuntimeConfig rc;
+  rc.inter_data_type = T;
+  rc.max_step_token_num = m;
+
+  Tensor qweight = awq ? Upload(dir + "/qweight.bin", TYPE_INT32, {k, n / 8}) : Upload(dir + "/qweight.bin", TYPE_INT32, {k / 8, n});
+  Tensor scales = Upload(dir + "/scales.bin", T, {k / group, n});
+  Tensor qzeros;
+  if (awq) qzeros = Upload(dir + "/qzeros.bin", TYPE_INT32, {k / group, n / 8});
+  Tensor weight = PackGroupQuantWeight(qweight, scales, awq ? &qzeros : nullptr, mc.quant_config.method, group, 0, stream);
+
+  MatMulLayerFactory factory(mc, rc, 0, context);
+  auto layer = factory.CreateLayer(TYPE_I4_GROUP, T, T, factory.GroupMatMulParams(n, k, true), mc.quant_config.method, backend);
+  Tensor x = Upload(dir + "/x.bin", T, {m, k});
+  std::vector<Tensor> outputs{Tensor(MemoryLocation::LOCATION_DEVICE, T, {m, n}, 0)};
+  Drive(layer, mc, rc, {x, weight}, outputs);
+  if (outputs[0].shape != std::vector<size_t>{m, n} || outputs[0].dtype != T) return 3;
+  HIP_OK(hipStreamSynchronize(stream));
+  Download(outputs[0], dir + "/y.bin");
+  return 0;
+}
+
+static int RunBlockwise(int argc, char** argv) {
+  if (argc < 8) return 2;
+  const std::string dir = argv[2];
+  const DataType T = ParseT(argv[3]);
+  const size_t m = std::atol(argv[4]), n = std::atol(argv[5]), k = std::atol(argv[6]);
+  const bool fuse = std::atoi(argv[7]) != 0;
+  hipStream_t stream;
+  HIP_OK(hipStreamCreate(&stream));
+  auto context = std::make_shared<Context>(1, stream);
+  ModelConfig mc;
+  mc.is_quant = true;
+  mc.quant_config.method = QUANT_BLOCK_FP8_E4M3;
+  RuntimeConfig rc;
+  rc.inter_data_type = T;
+  rc.max_step_token_num = (m + 3) / 4 * 4;
+
+  Tensor weight = Upload(dir + "/w.bin", TYPE_FP8_E4M3, {n, k});
+  weight.weight_scales = std::make_shared<Tensor>(Upload(dir + "/w_scale.bin", TYPE_FP32, {(n + 127) / 128, k / 128}));
+  std::vector<std::any> params{rc.max_step_token_num, n, k, size_t(128), weight};
+  MatMulLayerFactory factory(mc, rc, 0, context);
+  auto layer = factory.CreateLayer(TYPE_FP8_E4M3, T, T, params, QUANT_BLOCK_FP8_E4M3, DEFAULT_LINEAR_BACKEND);
+  Tensor x = Upload(dir + "/x.bin", T, {m, fuse ? 2 * k : k});
+  std::vector<Tensor> outputs{Tensor(MemoryLocation::LOCATION_DEVICE, T, {m, n}, 0)};
+  Drive(layer, mc, rc, {x, weight}, outputs);
+  HIP_OK(hipStreamSynchronize(stream));
+  Download(outputs[0], dir + "/y.bin");
+  return 0;
+}
+
+static std::vector<std::any> MoeParams(size_t tokens, size_t E, size_t hidden, size_t inter, size_t topk, bool renorm,
+                                       float scaling, DataType int_dtype = TYPE_UINT4x2) {
+  return {renorm ? MoeScaleNormMode::RE_NORM : MoeScaleNormMode::NO_NORM,
+          tokens,
+          int(0),
+          E,
+          hidden,
+          inter,
+          topk,
+          size_t(1),
+          true,
+          uint32_t(1),
+          uint32_t(1),
+          std::string("softmax"),
+          std::string("greedy"),
+          renorm,
+          scaling,
+          false,
+          false,
+          TYPE_INVALID,
+          int_dtype,
+          int(128),
+          false};
+}
+
+static int RunMoe(int argc, char** argv) {
+  if (argc < 11) return 2;
+  const std::string dir = argv[2];
+  const DataType T = ParseT(argv[3]);
+  const size_t tokens = std::atol(argv[4]), E = std::atol(argv[5]), hidden = std::atol(argv[6]), inter = std::atol(argv[7]),
+               topk = std::atol(argv[8]);
+  const bool renorm = std::atoi(argv[9]) != 0;
+  const float scaling = static_cast<float>(std::atof(argv[10]));
+  hipStream_t stream;
+  HIP_OK(hipStreamCreate(&stream));
+  auto context = std::make_shared<Context>(1, stream);
+  ModelConfig mc;
+  RuntimeConfig rc;
+  rc.inter_data_type = T;
+
+  Tensor w13 = PackMoeExpertWeight(Upload(dir + "/w13.bin", TYPE_UINT8, {E, 2 * inter, hidden / 2}),
+                                   Upload(dir + "/s13.bin", T, {E, 2 * inter, hidden / 128}), 128, 0, stream);
+  Tensor w2 = PackMoeExpertWeight(Upload(dir + "/w2.bin", TYPE_UINT8, {E, hidden, inter / 2}),
+                                  Upload(dir + "/s2.bin", T, {E, hidden, inter / 128}), 128, 0, stream);
+  HIP_OK(hipStreamSynchronize(stream));
+  MoeLayerFactory factory(mc, rc, 0, context);
+  auto layer = factory.CreateLayer(TYPE_UINT8, T, T, MoeParams(tokens, E, hidden, inter, topk, renorm, scaling),
+                                   MOE_QUANT_GPTQ, TRITON_MOE_BACKEND);
+  Tensor x = Upload(dir + "/x.bin", T, {tokens, hidden});
+  Tensor gating = Upload(dir + "/gating.bin", TYPE_FP32, {tokens, E});
+  std::vector<Tensor> outputs{Tensor(MemoryLocation::LOCATION_DEVICE, T, {tokens, hidden}, 0)};
+  Drive(layer, mc, rc, {x, gating, w13, w2}, outputs);
+  HIP_OK(hipStreamSynchronize(stream));
+  Download(outputs[0], dir + "/y.bin");
+  return 0;
+}
+
+// error behaviour that needs no kernel launch
+static int RunErrors() {
+  auto context = std::make_shared<Context>(1, nullptr);
+  ModelConfig mc;
+  RuntimeConfig rc;
+  int failures = 0;
+  auto expect = [&](bool ok, const char* what) {
+    if (!ok) {
+      std::fprintf(stderr, "FAILED: %s\n", what);
+      ++failures;
+    }
+  };
+  auto throws = [](auto&& fn) {
+    try {
+      fn();
+    } catch (const std::exception&) {
+      return true;
+    }
+    return false;
+  };
+  MatMulLayerFactory factory(mc, rc, 0, context);
+  // unknown combination
+  expect(throws([&] { factory.CreateLayer(TYPE_I4_GROUP, TYPE_FP32, TYPE_FP32, {}, QUANT_GPTQ, CUTLASS_LINEAR_BACKEND); }),
+         "fp32 activations have no int4 layer");
+  // too few parameters
+  {
+    CutlassMatMulLayer layer;
+    expect(!layer.Init({size_t(1)}, rc, context, 0).OK(), "short parameter list is rejected");
+  }
+  // act-order rejected
+  {
+    MarlinMatMulLayer layer;
+    std::vector<std::any> p{size_t(16), size_t(256), size_t(256), size_t(128), false, true, true, true, TYPE_I4_GROUP};
+    expect(!layer.Init(p, rc, context, 0).OK(), "desc_act is rejected");
+  }
+  // wrong weight data type surfaces in GetWorkspaceSize, as in the reference
+  {
+    CutlassMatMulLayer layer;
+    std::vector<std::any> p{size_t(16), size_t(256), size_t(256), size_t(128), false, false, true, true, TYPE_FP16};
+    expect(layer.Init(p, rc, context, 0).OK(), "init with foreign weight type succeeds");
+    expect(throws([&] { layer.GetWorkspaceSize(); }), "GetWorkspaceSize throws for a non-int4 weight type");
+  }
+  // shape with no kernel: k not a multiple of 128
+  {
+    MacheteMatMulLayer layer;
+    std::vector<std::any> p{size_t(16), size_t(256), size_t(200), size_t(128), false, false, true, true, TYPE_I4_GROUP};
+    expect(layer.Init(p, rc, context, 0).OK(), "init");
+    expect(!layer.Preprocess(mc, rc).OK(), "Preprocess reports a shape without a kernel");
+  }
+  // blockwise: block size other than 128; forward without workspace
+  {
+    BlockwiseMatMulLayer layer;
+    std::vector<std::any> p{size_t(16), size_t(256), size_t(256), size_t(64), Tensor()};
+    expect(!layer.Init(p, rc, context, 0).OK(), "block size 64 is rejected");
+    BlockwiseMatMulLayer layer2;
+    std::vector<std::any> p2{size_t(16), size_t(256), size_t(256), size_t(128), Tensor()};
+    expect(layer2.Init(p2, rc, context, 0).OK(), "blockwise init");
+    expect(layer2.GetWorkspaceSize() >= 16 * 256 + 16 * 2 * 4, "blockwise workspace holds a_q and a_s");
+    std::vector<Tensor> out{Tensor()};
+    Tensor x(MemoryLocation::LOCATION_DEVICE, TYPE_FP16, {16, 256}, 0, reinterpret_cast<void*>(0x1000));
+    expect(throws([&] { layer2.Forward({x, Tensor()}, out); }), "Forward without a workspace buffer throws");
+  }
+  // moe: fp8 experts / grouped routing rejected, int4 accepted
+  {
+    MoeLayer a, b, c;
+    auto p = MoeParams(64, 8, 256, 256, 2, false, 1.0f);
+    expect(a.Init(p, rc, context, 0).OK(), "moe int4 init");
+    expect(a.GetWorkspaceSize() > 0, "moe workspace size");
+    auto q = p;
+    q[17] = TYPE_BLOCK_FP8_E4M3;
+    expect(!b.Init(q, rc, context, 0).OK(), "fp8 experts are rejected");
+    auto r = p;
+    r[9] = uint32_t(8);
+    expect(!c.Init(r, rc, context, 0).OK(), "grouped routing is rejected");
+    expect(MoeLayer::BlockM(20) == 16 && MoeLayer::BlockM(21) == 32, "block_m thresholds");
+  }
+  std::printf(failures ? "layer errors: %d FAILED\n" : "layer errors: OK\n", failures);
+  return failures ? 1 : 0;
+}
+
+int main(int argc, char** argv) {
+  if (argc < 2) return 2;
+  const std::string mode = argv[1];
+  try {
+    if (mode == "w4a16") return RunW4A16(argc, argv);
+    if (mode == "blockwise") return RunBlockwise(argc, argv);
+    if (mode == "moe") return RunMoe(argc, argv);
+    if (mode == "errors") return RunErrors();
+  } catch (const std::exception& e) {
+    std::fprintf(stderr, "exception: %s\n", e.what());
+    return 4;
+  }
+  return 2;
+}

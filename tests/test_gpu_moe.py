@@ -44,6 +44,22 @@ def test_align_out_of_range_ids_dropped(ops, oracle):
     np.testing.assert_array_equal(s.cpu().numpy(), so)
 
 
+@pytest.mark.parametrize("T,E,topk", [(1, 256, 8), (77, 256, 8), (5, 60, 4), (9, 1000, 6)])
+def test_topk_softmax(ops, oracle, T, E, topk):
+    g = H.gen(T + E)
+    logits = torch.randn((T, E), generator=g)
+    logits[0, :4] = logits[0, 7]  # ties
+    for norm in (False, True):
+        w, ids = ops.moe_topk_softmax(logits.cuda(), topk, norm, 2.5)
+        wo, io = oracle.moe_topk_softmax(logits.numpy(), topk, norm, 2.5, 2)
+        np.testing.assert_array_equal(ids.cpu().numpy(), io)
+        np.testing.assert_allclose(w.cpu().numpy(), wo, rtol=2e-6, atol=1e-9)
+    lb = logits.to(torch.bfloat16)
+    w, ids = ops.moe_topk_softmax(lb.cuda(), topk)
+    wo, io = oracle.moe_topk_softmax(H.bits_of(lb), topk, False, 1.0, H.BF16)
+    np.testing.assert_array_equal(ids.cpu().numpy(), io)
+
+
 @pytest.mark.parametrize("dtype", [H.F16, H.BF16])
 def test_silu_mul_and_sum(ops, oracle, dtype):
     g = H.gen(3)

@@ -326,3 +326,19 @@ def test_silu_mul_and_moe_sum(oracle):
         for j in range(8):
             acc = acc + tt[:, j]
         np.testing.assert_array_equal(oracle.from_bits(oracle.moe_sum(yb, dtype), dtype), acc.float().numpy())
+
+
+def test_topk_softmax_vs_torch(oracle):
+    g = torch.Generator().manual_seed(3)
+    logits = torch.randn((37, 256), generator=g)
+    w, ids = oracle.moe_topk_softmax(logits.numpy(), 8, False, 2.5, oracle.F32)
+    p = torch.softmax(logits, -1)
+    tw, ti = torch.topk(p, 8, dim=-1)
+    np.testing.assert_array_equal(ids, ti.numpy())
+    np.testing.assert_allclose(w, tw.numpy() * 2.5, rtol=1e-5)
+    w2, _ = oracle.moe_topk_softmax(logits.numpy(), 8, True, 1.0, oracle.F32)
+    np.testing.assert_allclose(w2.sum(-1), 1.0, rtol=1e-5)
+    # ties go to the lower expert id
+    flat = np.zeros((1, 16), np.float32)
+    _, ids = oracle.moe_topk_softmax(flat, 4, False, 1.0, oracle.F32)
+    np.testing.assert_array_equal(ids[0], [0, 1, 2, 3])
