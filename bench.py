@@ -27,6 +27,13 @@ MFMA_PEAK = {"f16": 2.5e15, "bf16": 2.5e15, "fp8": 5.0e15}   # dense FLOP/s
 CACHE_BYTES = 320 << 20                            # rotate through more than the Infinity Cache
 
 
+# HBM bytes per launch of a kernel variant, averaged over the cases that run it: rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE (KiB per dispatch), each scaled by the factor the same counter shows for a 256 MiB device copy
+# (`--calibrate-copy`): FETCH_SIZE reads half the bytes moved (x2.0), WRITE_SIZE reads them exactly (x1.0).
+# Keyed by (config, kernel variant); None where no counter run has been made for the current kernel.
+MEASURED_TRAFFIC = {}
+
+
 def seeded(cfg, idx):
     g = torch.Generator(device="cpu")
     g.manual_seed(1000 * cfg + idx)
@@ -45,8 +52,9 @@ def awq_pack_cols(codes):
 
 
 class Case:
-    def __init__(self, name, launch, flops, nbytes, peak_key, kernel):
+    def __init__(self, name, launch, flops, nbytes, peak_key, kernel, copies=1):
         self.name, self.launch, self.flops, self.bytes, self.peak_key, self.kernel = name, launch, flops, nbytes, peak_key, kernel
+        self.copies = copies
         t_hbm = nbytes / HBM_PEAK
         t_mfma = flops / MFMA_PEAK[peak_key]
         self.bound = "hbm" if t_hbm >= t_mfma else "mfma"
@@ -54,7 +62,7 @@ class Case:
 
 
 def copies_needed(weight_bytes):
-    return max(2, min(24, -(-CACHE_BYTES // weight_bytes) + 1))
+    return max(2, min(64, -(-CACHE_BYTES // weight_bytes) + 1))
 
 
 # ------------------------------------------------------------------------------------------------ workloads
@@ -94,8 +102,9 @@ def w4a16_cases(ops, L, cfg, shapes, Ms, dtype, awq, x_std, s_lo, s_hi):
             nbytes = K * N // 2 + G * N * 2 + (G * N // 2 if awq else 0) + 2 * M * K + 2 * M * N
             flops = 2 * M * N * K
             desc = L.select_tile(L.KIND_W4A16, M, N, K, L.F16 if dtype == "f16" else L.BF16)
-            kern = "w4a16_splitk" if desc["kernel"] == 0 else "w4a16_mfma"
-            cases.append(Case("%s:M=%d" % (tag, M), launch, flops, nbytes, dtype, kern))
+            kern = "%s<%dx%d,w%d>" % ("w4a16_splitk_kernel" if desc["kernel"] == 0 else "w4a16_tile_kernel",
+                                      desc["block_m"], desc["block_n"], desc["waves"])
+            cases.append(Case("%s:M=%d" % (tag, M), launch, flops, nbytes, dtype, kern, R))
     return cases, keep
 
 
@@ -134,7 +143,7 @@ def fp8_cases(ops, L, cfg, shapes, Ms):
             cases.append(Case("%s:quant:M=%d" % (tag, M), quant, 0, 2 * M * K + M * K + 4 * M * K // 128, "fp8",
                               "fp8_group_quant"))
             nbytes = N * K + b_s.numel() * 4 + M * K + 4 * M * K // 128 + 2 * M * N
-            cases.append(Case("%s:gemm:M=%d" % (tag, M), gemm, 2 * M * N * K, nbytes, "fp8", "fp8_blockwise_gemm"))
+            cases.append(Case("%s:gemm:M=%d" % (tag, M), gemm, 2 * M * N * K, nbytes, "fp8", "fp8_blockwise_gemm", R))
     return cases, keep
 
 
@@ -193,41 +202,76 @@ def build(cfg, ops, L):
 
 
 # ------------------------------------------------------------------------------------------------ timing
-def time_launches(fn, reps):
-    """Average duration of `reps` back-to-back launches of fn, HIP events on the launch stream (ms)."""
+def capture(fns):
+    """One HIP graph holding the launches of `fns` in order (captured on a side stream, replayed on the current one)."""
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for f in fns:
+            f()
+    return g
+
+
+def time_case(c, use_graph):
+    """Average duration of one launch of case c in ms: HIP events around `reps` back-to-back launches on the launch
+    stream.  With graphs the launches are replayed from one captured graph, which takes the host's per-launch cost
+    (several microseconds from Python) out of the measurement of kernels that run for less than that."""
+    reps = 200 if c.t_bound < 2e-5 else (48 if c.t_bound < 2e-4 else 8)
+    reps = -(-reps // c.copies) * c.copies          # whole turns of the weight-copy rotation
     start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    fn()
-    torch.cuda.synchronize()
-    start.record()
-    for _ in range(reps):
-        fn()
-    end.record()
+    if use_graph:
+        g = capture([c.launch] * reps)
+        g.replay()
+        torch.cuda.synchronize()
+        start.record()
+        g.replay()
+        end.record()
+    else:
+        c.launch()
+        torch.cuda.synchronize()
+        start.record()
+        for _ in range(reps):
+            c.launch()
+        end.record()
     torch.cuda.synchronize()
     return start.elapsed_time(end) / reps
 
 
 def cpu_baseline(cfg, keep, ops):
-    """The oracle's dequantize-then-fp32-GEMM on the host cores, on a bounded sample of the default workload."""
-    if cfg != 2 or not keep:
+    """The oracle's dequantize-to-fp32 + fp32 GEMM on the host cores: one pass over a bounded sample of the workload."""
+    if cfg not in (1, 2) or not keep:
         return None
     import numpy as np
     from oracle import ksq_oracle as orc
     orc.build()
     threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
-    k = keep[0]
-    codes = orc.awq_unpack(k["q"].numpy().view(np.uint32))
-    sb = k["scales"].view(torch.int16).numpy().view(np.uint16)
-    zeros = k["zeros"].numpy()
-    Ms = [1, 8, 32]
-    flops, t = 0, 0.0
-    for M in Ms:
-        xb = k["x"][M].cpu().view(torch.int16).numpy().view(np.uint16)
-        t0 = time.perf_counter()
-        orc.w4a16_gemm(xb, codes, sb, zeros, 128, orc.BF16)
-        t += time.perf_counter() - t0
-        flops += 2 * M * k["N"] * k["K"]
+    prepared = []
+    for k in keep:
+        tag = orc.BF16 if k["x"][min(k["x"])].dtype == torch.bfloat16 else orc.F16
+        if k["awq"]:
+            codes = orc.awq_unpack(k["q"].numpy().view(np.uint32))
+            zeros = k["zeros"].numpy()
+        else:
+            codes = orc.gptq_unpack(k["q"].numpy().view(np.uint32))
+            zeros = None
+        sb = k["scales"].view(torch.int16).numpy().view(np.uint16)
+        xs = {M: k["x"][M].cpu().view(torch.int16).numpy().view(np.uint16) for M in sorted(k["x"])}
+        prepared.append((k, tag, codes, zeros, sb, xs))
+    # whole passes over the workload until at least 10 s of wall time have been spent (30 s cap inside a pass)
+    flops, t, passes = 0, 0.0, 0
+    while t < 10.0:
+        for k, tag, codes, zeros, sb, xs in prepared:
+            for M, xb in xs.items():
+                t0 = time.perf_counter()
+                orc.w4a16_gemm(xb, codes, sb, zeros, 128, tag)
+                t += time.perf_counter() - t0
+                flops += 2 * M * k["N"] * k["K"]
+                if t > 30.0:
+                    break
+        passes += 1
+    names = ", ".join("%s(%dx%d) M in {%s}" % (k["tag"], k["N"], k["K"], ",".join(map(str, xs)))
+                      for k, _, _, _, _, xs in prepared)
     return {"value": round(flops / t / 1e12, 6), "unit": "TFLOP/s", "cores": threads, "kind": "port",
-            "sample": "gate_up 14336x4096 AWQ bf16, M in {1,8,32}, dequant-to-fp32 + fp32 GEMM, one pass each",
+            "sample": "%d pass(es) of the oracle (dequantize to fp32, fp32 GEMM, OpenMP) over %s" % (passes, names),
             "seconds": round(t, 3)}
 
 
@@ -239,6 +283,10 @@ def main():
     ap.add_argument("--config", type=int, default=2, help="BASELINE.json config number 1..5 (default 2)")
     ap.add_argument("--only", default="", help="substring filter on case names (for profiling one case)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-graph", action="store_true", help="launch every kernel from Python instead of replaying "
+                    "captured HIP graphs (adds the host's per-launch cost to short kernels)")
+    ap.add_argument("--calibrate-copy", action="store_true", help="run only a 256 MiB device-to-device copy a few "
+                    "times (the known-size kernel hardware traffic counters are scaled by) and exit")
     ap.add_argument("--details", action="store_true", help="also print a per-case table to stderr")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -246,6 +294,16 @@ def main():
                          "multi-GPU leg, every case is already a per-GPU shape)" % args.gpus)
     if not torch.cuda.is_available():
         raise SystemExit("bench.py needs a GPU")
+
+    if args.calibrate_copy:
+        n = 256 << 20
+        src = torch.randint(0, 255, (n,), dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_bytes_read": n, "copy_bytes_written": n, "launches": 5}))
+        return
 
     from ksanallm_amd import lib as L
     from ksanallm_amd import ops
@@ -256,18 +314,32 @@ def main():
         if not cases:
             raise SystemExit("--only matched no case")
 
-    def step():
+    use_graph = not args.no_graph
+    n_graphs = max(c.copies for c in cases)
+
+    def eager_step(_i=0):
         for c in cases:
             c.launch()
 
-    for _ in range(args.warmup):
-        step()
+    if use_graph:
+        # one captured graph per turn of the weight-copy rotation; step i replays graph i % n_graphs
+        eager_step()
+        torch.cuda.synchronize()
+        graphs = [capture([c.launch for c in cases]) for _ in range(n_graphs)]
+
+        def step(i):
+            graphs[i % n_graphs].replay()
+    else:
+        step = eager_step
+
+    for i in range(args.warmup):
+        step(i)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     start.record()
-    for _ in range(args.steps):
-        step()
+    for i in range(args.steps):
+        step(args.warmup + i)
     end.record()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
@@ -276,8 +348,7 @@ def main():
     # per-case kernel timing, same stream, after the timed region
     per_case = []
     for c in cases:
-        reps = 200 if c.t_bound < 2e-5 else (50 if c.t_bound < 2e-4 else 10)
-        ms = time_launches(c.launch, reps)
+        ms = time_case(c, use_graph)
         sec = ms * 1e-3
         per_case.append({
             "case": c.name, "kernel": c.kernel, "us": round(ms * 1e3, 2), "tflops": round(c.flops / sec / 1e12, 3),
@@ -289,17 +360,37 @@ def main():
     total_bytes = sum(c.bytes for c in cases)
     step_s = ms_per_step * 1e-3
 
-    dom_i = max(range(len(cases)), key=lambda i: per_case[i]["us"])
-    dc, dp = cases[dom_i], per_case[dom_i]
-    if dc.bound == "hbm":
-        roof = {"bound": "hbm", "achieved": dp["gbps"], "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                "frac": round(dp["gbps"] * 1e9 / HBM_PEAK, 4), "traffic": None}
+    # dominant kernel = the kernel variant with the largest share of the step; its launches average over the cases
+    # that run it, which is also what a profiler's per-kernel average shows
+    groups = {}
+    for c, p in zip(cases, per_case):
+        g = groups.setdefault(c.kernel, {"us": 0.0, "flops": 0, "bytes": 0, "t_hbm": 0.0, "t_mfma": 0.0, "n": 0,
+                                         "peak_key": c.peak_key, "cases": []})
+        g["us"] += p["us"]
+        g["flops"] += c.flops
+        g["bytes"] += c.bytes
+        g["t_hbm"] += c.bytes / HBM_PEAK
+        g["t_mfma"] += c.flops / MFMA_PEAK[c.peak_key]
+        g["n"] += 1
+        g["cases"].append(c.name)
+    dk = max(groups, key=lambda k: groups[k]["us"])
+    g = groups[dk]
+    sec = g["us"] * 1e-6
+    if g["t_hbm"] >= g["t_mfma"]:
+        ach = g["bytes"] / sec / 1e9
+        roof = {"bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                "frac": round(ach * 1e9 / HBM_PEAK, 4)}
     else:
-        roof = {"bound": "mfma", "achieved": dp["tflops"], "peak": MFMA_PEAK[dc.peak_key] / 1e12, "unit": "TFLOP/s",
-                "frac": round(dp["tflops"] * 1e12 / MFMA_PEAK[dc.peak_key], 4), "traffic": None}
-    roof["kernel"] = dp["kernel"]
-    roof["case"] = dp["case"]
-    roof["launch_us"] = dp["us"]
+        ach = g["flops"] / sec / 1e12
+        roof = {"bound": "mfma", "achieved": round(ach, 3), "peak": MFMA_PEAK[g["peak_key"]] / 1e12, "unit": "TFLOP/s",
+                "frac": round(ach * 1e12 / MFMA_PEAK[g["peak_key"]], 4)}
+    traffic = MEASURED_TRAFFIC.get((args.config, dk))
+    roof["traffic"] = traffic
+    roof["kernel"] = dk
+    roof["cases"] = g["cases"]
+    roof["avg_launch_us"] = round(g["us"] / g["n"], 2)
+    roof["algorithmic_bytes_per_launch"] = g["bytes"] // g["n"]
+    roof["algorithmic_flops_per_launch"] = g["flops"] // g["n"]
 
     out = {
         "metric": METRIC, "value": round(100.0 * total_bound / step_s, 3), "unit": "% of roofline",
@@ -307,7 +398,7 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic",
         "config": {"workload": workload, "cases": len(cases), "config_index": args.config - 1},
         "tflops": round(total_flops / step_s / 1e12, 3), "hbm_gbps": round(total_bytes / step_s / 1e9, 1),
-        "wall_ms_per_step": round(wall_ms, 5),
+        "wall_ms_per_step": round(wall_ms, 5), "launch": "hip graph replay" if use_graph else "python launches",
         "peaks": {"hbm_gbps": HBM_PEAK / 1e9, "mfma_tflops": {k: v / 1e12 for k, v in MFMA_PEAK.items()}},
         "roofline": roof, "per_case": per_case,
     }
