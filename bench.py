@@ -94,10 +94,12 @@ def w4a16_cases(ops, L, cfg, shapes, Ms, dtype, awq, x_std, s_lo, s_hi):
             x = (torch.randn((M, K), generator=seeded(cfg, 100 * si + mi + 10)) * x_std).to(tdt).to(dev)
             y = torch.empty((M, N), dtype=tdt, device=dev)
             keep[-1].setdefault("x", {})[M] = x
+            need = L.load().ksq_w4a16_workspace_size(M, N, K, 128, L.F16 if dtype == "f16" else L.BF16)
+            ws = torch.empty(need, dtype=torch.uint8, device=dev) if need else None
 
-            def launch(x=x, y=y, N=N, K=K, wps=wps, sps=sps, zps=zps, state=state, R=R):
+            def launch(x=x, y=y, N=N, K=K, wps=wps, sps=sps, zps=zps, state=state, R=R, ws=ws):
                 i = state["i"] = (state["i"] + 1) % R
-                ops.w4a16_gemm(x, wps[i], sps[i], zps[i], N, K, 128, out=y)
+                ops.w4a16_gemm(x, wps[i], sps[i], zps[i], N, K, 128, out=y, workspace=ws)
 
             nbytes = K * N // 2 + G * N * 2 + (G * N // 2 if awq else 0) + 2 * M * K + 2 * M * N
             flops = 2 * M * N * K

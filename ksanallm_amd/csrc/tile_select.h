@@ -15,8 +15,16 @@ SplitKChoice select_splitk(size_t m, size_t n, size_t k);
 // same rule for a grid of m_blocks row blocks of 16*mt rows each (MoE: one block per aligned expert segment)
 SplitKChoice select_splitk_blocks(int mt, size_t m_blocks, size_t n, size_t k);
 
-// true when the MFMA tile kernel (prefill regime) serves the shape: m above the decode range, group 128 and n a
-// multiple of its 256-column workgroup tile
+// true when the MFMA tile kernel (prefill regime) serves the shape: m above the decode range and group 128
 bool use_mfma_tile(size_t m, size_t n, size_t k, size_t group);
+
+// Grid of the MFMA tile kernel: block_m x 256 output tiles, and a split of K over workgroups when the output tiles
+// alone would leave most of the 256 CUs idle.  splits > 1 needs splits*m*n fp32 of workspace.
+struct TilePlan {
+  int block_m;  // 128 or 256
+  unsigned tiles_m, tiles_n, splits, kt_per_split;
+  size_t workspace_bytes;
+};
+TilePlan plan_mfma_tile(size_t m, size_t n, size_t k);
 
 }  // namespace ksq

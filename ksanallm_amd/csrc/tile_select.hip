@@ -38,7 +38,32 @@ SplitKChoice select_splitk_blocks(int mt, size_t m_blocks, size_t n, size_t k) {
 // m = 80; the split-K kernel handles up to two 16-row tiles per workgroup, the tile kernel takes over above that.
 bool use_mfma_tile(size_t m, size_t n, size_t k, size_t group) {
   (void)k;
-  return m > 32 && group == 128 && n % 256 == 0;
+  (void)n;
+  return m > 32 && group == 128;
+}
+
+// 256-row tiles halve the weight traffic per output row, 128-row tiles waste less when m sits just above a multiple
+// of 256.  With fewer than 192 output tiles the k range is cut into up to 256/tiles pieces of at least 4 k-tiles (512 k)
+// each; the fp32 partial tiles are summed by a second, bandwidth-bound kernel.
+TilePlan plan_mfma_tile(size_t m, size_t n, size_t k) {
+  TilePlan t{};
+  const size_t rem = (m - 1) % 256;
+  t.block_m = (m <= 128 || (m < 1024 && rem < 128)) ? 128 : 256;
+  t.tiles_m = static_cast<unsigned>(div_up(m, t.block_m));
+  t.tiles_n = static_cast<unsigned>(div_up(n, 256));
+  const unsigned kt = static_cast<unsigned>(k / 128);
+  const unsigned tiles = t.tiles_m * t.tiles_n;
+  unsigned want = 1;
+  if (tiles < static_cast<unsigned>(kNumCU) * 3 / 4) {
+    want = kNumCU / tiles;
+    const unsigned cap = kt / 4 ? kt / 4 : 1;
+    want = want < cap ? want : cap;
+    if (want < 1) want = 1;
+  }
+  t.kt_per_split = static_cast<unsigned>(div_up(kt, want));
+  t.splits = static_cast<unsigned>(div_up(kt, t.kt_per_split));
+  t.workspace_bytes = t.splits > 1 ? static_cast<size_t>(t.splits) * m * n * 4 : 0;
+  return t;
 }
 
 }  // namespace ksq
@@ -56,13 +81,14 @@ KSQ_EXPORT int ksq_select_tile(int kind, size_t m, size_t n, size_t k, int dtype
     case KSQ_KIND_W4A16:
     case KSQ_KIND_MOE_W4A16: {
       if (kind == KSQ_KIND_W4A16 && use_mfma_tile(m, n, k, 128)) {
+        const TilePlan t = plan_mfma_tile(m, n, k);
         d->kernel = KSQ_KERNEL_MFMA_TILE;
-        d->block_m = m <= 128 ? 128 : 256;
+        d->block_m = t.block_m;
         d->block_n = 256;
         d->block_k = 64;
         d->waves = 8;
-        d->split_k = 1;
-        d->grid = static_cast<int32_t>(div_up(m, d->block_m) * (n / 256));
+        d->split_k = static_cast<int32_t>(t.splits);
+        d->grid = static_cast<int32_t>(t.tiles_m * t.tiles_n * t.splits);
         return KSQ_OK;
       }
       SplitKChoice c = select_splitk(m, n, k);

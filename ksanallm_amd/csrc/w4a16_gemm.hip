@@ -3,6 +3,8 @@
 #include <cstdlib>
 
 #include "ksq_common.h"
+#include <atomic>
+
 #include "tile_select.h"
 #include "w4a16_splitk.h"
 #include "w4a16_tile.h"
@@ -75,25 +77,40 @@ int dispatch_tile(SplitKParams& p, SplitKChoice c, uint32_t m_blocks, size_t gro
   return fail(KSQ_ERR_UNSUPPORTED, "no split-K kernel for mt=%d nt=%d waves=%d", c.mt, c.nt, c.waves);
 }
 
-template <typename T, int WAVES_M, int WAVES_N, int WM, int WN>
-int launch_tile(const TileParams& p0, hipStream_t s) {
-  constexpr int BM = WAVES_M * WM * 16, BN = WAVES_N * WN * 16;
-  TileParams p = p0;
-  p.tiles_m = static_cast<uint32_t>(div_up(p.M, BM));
-  p.tiles_n = p.N / BN;
-  const size_t lds = 2 * (BM / 16) * 2 * 1024;
-  const unsigned grid = p.tiles_m * p.tiles_n;
-  if (p.zeros)
-    w4a16_tile_kernel<T, WAVES_M, WAVES_N, WM, WN, true><<<grid, WAVES_M * WAVES_N * 64, lds, s>>>(p);
-  else
-    w4a16_tile_kernel<T, WAVES_M, WAVES_N, WM, WN, false><<<grid, WAVES_M * WAVES_N * 64, lds, s>>>(p);
+template <typename T, int WM, bool HAS_ZP>
+int launch_tile_zp(const TileParams& p, hipStream_t s) {
+  constexpr int kLds = 4 * WM * 2 * 1024;  // NS stages of WM*2 fragments
+  static std::atomic<bool> configured{false};
+  if (!configured.load(std::memory_order_acquire)) {
+    // more dynamic LDS than the 64 KiB a kernel may use without asking
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&w4a16_tile_kernel<T, WM, HAS_ZP>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
+    if (e != hipSuccess) return fail(KSQ_ERR_LAUNCH, "hipFuncSetAttribute(LDS %d): %s", kLds, hipGetErrorString(e));
+    configured.store(true, std::memory_order_release);
+  }
+  const unsigned grid = p.tiles_m * p.tiles_n * p.splits;
+  w4a16_tile_kernel<T, WM, HAS_ZP><<<grid, 512, kLds, s>>>(p);
   return KSQ_OK;
 }
 
 template <typename T>
-int dispatch_mfma_tile(const TileParams& p, hipStream_t s) {
-  if (p.M <= 128) return launch_tile<T, 1, 8, 8, 2>(p, s);  // 128 x 256
-  return launch_tile<T, 2, 4, 8, 4>(p, s);                  // 256 x 256
+int dispatch_mfma_tile(TileParams p, const TilePlan& plan, hipStream_t s) {
+  p.tiles_m = plan.tiles_m;
+  p.tiles_n = plan.tiles_n;
+  p.splits = plan.splits;
+  p.kt_per_split = plan.kt_per_split;
+  int rc;
+  if (plan.block_m == 128)
+    rc = p.zeros ? launch_tile_zp<T, 8, true>(p, s) : launch_tile_zp<T, 8, false>(p, s);
+  else
+    rc = p.zeros ? launch_tile_zp<T, 16, true>(p, s) : launch_tile_zp<T, 16, false>(p, s);
+  if (rc) return rc;
+  if (plan.splits > 1) {
+    const size_t mn = static_cast<size_t>(p.M) * p.N;
+    const unsigned blocks = static_cast<unsigned>(div_up(mn, 256 * 8));
+    splitk_reduce_kernel<T><<<blocks, 256, 0, s>>>(p.partial, static_cast<uint16_t*>(p.y), mn, plan.splits);
+  }
+  return KSQ_OK;
 }
 
 int check_common(const char* fn, const void* y, const void* x, const void* w, const void* sc, size_t n, size_t k,
@@ -117,8 +134,17 @@ int check_common(const char* fn, const void* y, const void* x, const void* w, co
 using namespace ksq;
 
 KSQ_EXPORT size_t ksq_w4a16_workspace_size(size_t max_m, size_t n, size_t k, size_t group, int dtype) {
-  (void)max_m; (void)n; (void)k; (void)group; (void)dtype;
-  return 0;  // every reduction happens inside a workgroup
+  (void)dtype;
+  // the decode kernel reduces inside a workgroup; only the split-K form of the tile kernel needs fp32 partials
+  if (n == 0 || k == 0 || k % 128 != 0) return 0;
+  size_t need = 0;
+  for (size_t m = 33; m <= max_m; ++m) {
+    if (!use_mfma_tile(m, n, k, group)) break;
+    const TilePlan t = plan_mfma_tile(m, n, k);
+    if (t.splits == 1 && t.block_m == 256 && m % 256 == 0) break;  // the grid only grows from here on
+    need = t.workspace_bytes > need ? t.workspace_bytes : need;
+  }
+  return need;
 }
 
 KSQ_EXPORT int ksq_w4a16_gemm(void* y, const void* x, const void* w_packed, const void* scales_packed,
@@ -126,7 +152,6 @@ KSQ_EXPORT int ksq_w4a16_gemm(void* y, const void* x, const void* w_packed, cons
                               size_t k, size_t group, int dtype, void* stream) {
   const char* fn = "ksq_w4a16_gemm";
   if (int rc = check_common(fn, y, x, w_packed, scales_packed, n, k, group, dtype)) return rc;
-  (void)workspace; (void)workspace_bytes;
   if (m == 0) return KSQ_OK;
   if (m > 0x7fffffffull) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: m too large", fn);
   if (!use_mfma_tile(m, n, k, group) && m * k * 2 >= 0x40000000ull)
@@ -151,7 +176,16 @@ KSQ_EXPORT int ksq_w4a16_gemm(void* y, const void* x, const void* w_packed, cons
     tp.M = static_cast<uint32_t>(m);
     tp.N = static_cast<uint32_t>(n);
     tp.K = static_cast<uint32_t>(k);
-    int rc = dtype == KSQ_F16 ? dispatch_mfma_tile<F16>(tp, as_stream(stream)) : dispatch_mfma_tile<BF16>(tp, as_stream(stream));
+    const TilePlan plan = plan_mfma_tile(m, n, k);
+    if (plan.splits > 1) {
+      if (!workspace || workspace_bytes < plan.workspace_bytes || !aligned16(workspace))
+        return fail(KSQ_ERR_WORKSPACE, "%s: m=%zu n=%zu k=%zu needs %zu bytes of 16-byte aligned workspace, got %zu", fn,
+                    m, n, k, plan.workspace_bytes, workspace ? workspace_bytes : size_t(0));
+      tp.partial = static_cast<float*>(workspace);
+    }
+    if (256 * k * 2 > 0xffffffffull) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: k too large", fn);
+    int rc = dtype == KSQ_F16 ? dispatch_mfma_tile<F16>(tp, plan, as_stream(stream))
+                              : dispatch_mfma_tile<BF16>(tp, plan, as_stream(stream));
     if (rc) return rc;
     return check_launch(fn);
   }

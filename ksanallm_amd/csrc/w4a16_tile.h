@@ -1,17 +1,23 @@
-// Prefill-regime W4A16 kernel (MFMA-bound): a workgroup of 8 wavefronts computes a BM x 256 output tile.
+// Prefill-regime W4A16 kernel (MFMA-bound): a workgroup of 8 wavefronts computes a BM x 256 output tile
+// (BM = 256 or 128) over a contiguous range of k-tiles (split-K across workgroups when the grid would not fill the chip).
 //
-//   - x (activations) is staged through LDS in MFMA fragment order, double buffered, 64 k per stage: each 1 KiB
-//     fragment (16 rows x 32 k) is read back with one conflict-free ds_read_b128 per lane;
-//   - packed int4 weights never touch LDS: the wavefronts split the 256 columns between them (WN column tiles of
-//     16 each), so every weight fragment belongs to exactly one wavefront, which loads its 1 KiB tiles straight
-//     from global memory (16 bytes per lane, one k-tile of 128 every other stage) and dequantizes them in
-//     registers to T with scale and zero point applied, (code - zp) * s;
+//   - x (activations) goes global -> LDS without touching registers: every wavefront issues global_load_lds_dwordx4
+//     for whole 1 KiB MFMA fragments (16 rows x 32 k; lane l supplies row l%16, k 8*(l/16)..+7 and lands at
+//     base + 16*l), into a ring of NS stages of 64 k each.  The fragment is read back with one conflict-free
+//     ds_read_b128 per lane.  Three stages are in flight while one is consumed.
+//   - packed int4 weights never touch LDS: the 8 wavefronts split the 256 columns (2 column tiles of 16 each), so
+//     every weight fragment belongs to exactly one wavefront and no weight is dequantized twice.  A wavefront loads
+//     its 1 KiB tiles straight from global memory (16 bytes per lane) three stages ahead and dequantizes them in
+//     registers to T with (code - zp) * s applied.
+//   - all vector memory loads of the main loop are issued from inline assembly in a fixed order, the same number
+//     every stage (addresses are clamped past the end), so that one `s_waitcnt vmcnt(N)` per stage with a constant N
+//     releases exactly the stage that is needed: vmcnt retires in issue order.  The registers a wait makes valid are
+//     tied to that wait as in/out operands, which keeps the compiler from scheduling their uses above it.
 //   - the weights are the row operand of v_mfma_f32_16x16x32 and x the column operand, so a lane ends up with four
-//     consecutive output columns of one row and stores them as one 8-byte word; accumulation runs over the whole K
-//     inside the MFMA, there is no per-group epilogue.
+//     consecutive output columns of one row and stores them as one 8-byte word (or 16 bytes of fp32 partials).
 //
-// Workgroup ids are remapped so that the eight XCDs each work on a contiguous band of column tiles and sweep the
-// row tiles fastest: the weight band of a workgroup is shared by its neighbours on the same L2.
+// Workgroup ids are remapped so that the eight XCDs each work on a contiguous band of (column tile, k-split) pairs and
+// sweep the row tiles fastest: the weight band of a workgroup is shared by its neighbours on the same L2.
 #pragma once
 
 #include "ksq_common.h"
@@ -24,8 +30,10 @@ struct TileParams {
   const void* w;
   const void* scales;
   const void* zeros;
+  float* partial;  // [splits][M][N] fp32 when splits > 1
   uint32_t M, N, K;
   uint32_t tiles_m, tiles_n;
+  uint32_t splits, kt_per_split;
 };
 
 // dequantize one packed dword (8 codes) to 8 T values with (code - zp) * s applied
@@ -80,9 +88,9 @@ struct Dequant<BF16, HAS_ZP> {
     return __builtin_bit_cast(uint32_t, r);
   }
   __device__ __forceinline__ BF16::frag operator()(uint32_t w) const {
-    const uint32_t e = w & 0x0f0f0f0fu;         // nibbles 0,2,4,6 -> k = 0, 4, 1, 5   (nibble i <-> k pair order)
-    const uint32_t o = (w >> 4) & 0x0f0f0f0fu;  // nibbles 1,3,5,7 -> k = 2, 6, 3, 7
     // nibble p holds k = {0,2,4,6,1,3,5,7}[p]: even nibbles p=0,2,4,6 -> k=0,4,1,5 ; odd p=1,3,5,7 -> k=2,6,3,7
+    const uint32_t e = w & 0x0f0f0f0fu;
+    const uint32_t o = (w >> 4) & 0x0f0f0f0fu;
     const float k0 = static_cast<float>(e & 0xffu), k4 = static_cast<float>((e >> 8) & 0xffu);
     const float k1 = static_cast<float>((e >> 16) & 0xffu), k5 = static_cast<float>(e >> 24);
     const float k2 = static_cast<float>(o & 0xffu), k6 = static_cast<float>((o >> 8) & 0xffu);
@@ -96,57 +104,81 @@ struct Dequant<BF16, HAS_ZP> {
   }
 };
 
-// WAVES_M x WAVES_N wavefronts, each WM x WN tiles of 16x16.  BM = WAVES_M*WM*16, BN = WAVES_N*WN*16.
-template <typename T, int WAVES_M, int WAVES_N, int WM, int WN, bool HAS_ZP>
-__global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, 1) w4a16_tile_kernel(TileParams p) {
-  constexpr int THREADS = WAVES_M * WAVES_N * 64;
-  constexpr int BM = WAVES_M * WM * 16;
-  constexpr int BN = WAVES_N * WN * 16;
-  constexpr int BK = 64;                       // k per LDS stage
-  constexpr int FRAGS = (BM / 16) * (BK / 32);  // 1 KiB fragments per stage
-  constexpr int STAGE_BYTES = FRAGS * 1024;
-  constexpr int A_LOADS = BM * BK * 2 / 16 / THREADS;  // 16-byte chunks per thread per stage
-  static_assert(BM * BK * 2 / 16 % THREADS == 0, "A tile must split evenly over the threads");
+// One column tile's packed weights, scale and zero point for one k-tile of 128.
+struct WSlot {
+  u32x4 wq;
+  uint32_t sc;
+  uint32_t zp;
+};
 
-  extern __shared__ __attribute__((aligned(16))) char lds[];  // 2 * STAGE_BYTES
+// 8 wavefronts side by side along N; each computes WM x 2 tiles of 16x16.  BM = 16*WM, BN = 256.
+template <typename T, int WM, bool HAS_ZP>
+__global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
+  constexpr int WAVES = 8;
+  constexpr int WN = 2;
+  constexpr int BM = WM * 16;
+  constexpr int BN = WAVES * WN * 16;
+  constexpr int BK = 64;                 // k per LDS stage
+  constexpr int NS = 4;                  // LDS stages
+  constexpr int FRAGS = WM * (BK / 32);  // 1 KiB fragments per stage
+  constexpr int STAGE_BYTES = FRAGS * 1024;
+  constexpr int AP = FRAGS / WAVES;      // fragments this wavefront fetches per stage
+  constexpr int WL = HAS_ZP ? 3 : 2;     // loads per weight slot
+  constexpr int L = WL + AP;             // vector memory loads per wavefront per stage
+  constexpr int WAIT_N = (NS - 2) * L;   // loads issued after the stage that is about to be consumed
+  static_assert(FRAGS % WAVES == 0 && AP % 2 == 0, "fragments must split evenly, in k pairs, over the wavefronts");
+  static_assert(WAIT_N < 64, "vmcnt is a 6-bit counter");
+
+  extern __shared__ __attribute__((aligned(16))) char lds[];  // NS * STAGE_BYTES
 
   const int lane = threadIdx.x & 63;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const uint32_t wm = wave / WAVES_N, wn = wave % WAVES_N;
   const int lrow = lane & 15, lq = lane >> 4;
   const uint32_t KT = p.K / 128;
 
-  // ---- XCD-aware tile id: workgroup b runs on XCD b%8; give every XCD a contiguous range of tiles, row tile fastest
-  const uint32_t total = p.tiles_m * p.tiles_n;
+  // ---- XCD-aware work id: workgroup b runs on XCD b%8; every XCD gets a contiguous range, row tile fastest
+  const uint32_t total = p.tiles_m * p.tiles_n * p.splits;
   uint32_t bid = blockIdx.x;
   {
     const uint32_t per = total / 8, rem = total % 8;
     const uint32_t xcd = bid % 8, local = bid / 8;
-    // XCDs 0..rem-1 own per+1 tiles, the rest own per
-    bid = xcd * per + (xcd < rem ? xcd : rem) + local;
+    bid = xcd * per + (xcd < rem ? xcd : rem) + local;  // XCDs 0..rem-1 own per+1 items
   }
-  const uint32_t tile_n = bid / p.tiles_m, tile_m = bid % p.tiles_m;
+  const uint32_t tile_m = bid % p.tiles_m;
+  const uint32_t rest = bid / p.tiles_m;
+  const uint32_t split = rest % p.splits, tile_n = rest / p.splits;
   const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
+  const uint32_t kt_begin = split * p.kt_per_split;
+  const uint32_t kt_count = (KT - kt_begin) < p.kt_per_split ? (KT - kt_begin) : p.kt_per_split;
+  const uint32_t stages = kt_count * 2;
 
-  // ---- A (x) staging: thread t copies chunks q = j*THREADS + t ; row = q / 8, 16-byte chunk c = q % 8 of the row
-  const char* a_src[A_LOADS];
-  uint32_t a_dst[A_LOADS];
+  // ---- x staging: this wavefront fetches fragments f = wave*AP + 2j + {0,1}: row block f/2, k half f%2
+  const char* x_tile = static_cast<const char*>(p.x) + (static_cast<size_t>(m0) * p.K + kt_begin * 128) * 2;
+  uint32_t a_voff[AP / 2];
 #pragma unroll
-  for (int j = 0; j < A_LOADS; ++j) {
-    const uint32_t q = j * THREADS + threadIdx.x;
-    uint32_t row = q / 8;
-    const uint32_t c = q % 8;
-    uint32_t grow = m0 + row;
-    grow = grow < p.M ? grow : p.M - 1;
-    a_src[j] = static_cast<const char*>(p.x) + (static_cast<size_t>(grow) * p.K) * 2 + c * 16;
-    a_dst[j] = (((row / 16) * (BK / 32) + c / 4) * 64 + (c % 4) * 16 + row % 16) * 16;
+  for (int j = 0; j < AP / 2; ++j) {
+    const uint32_t rb = wave * (AP / 2) + j;
+    uint32_t row = rb * 16 + lrow;
+    row = (m0 + row < p.M) ? row : (p.M - 1 - m0);  // rows past M repeat the last row; their results are dropped
+    a_voff[j] = (row * p.K + lq * 8) * 2;
   }
+  const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<size_t>((__attribute__((address_space(3))) char*)lds));
+  const uint32_t a_lds_wave = lds_base + wave * AP * 1024;
 
-  // ---- weights: this wavefront's WN column tiles
-  const uint32_t nt0 = n0 / 16 + wn * WN;
-  const u32x4* wsrc = static_cast<const u32x4*>(p.w) + static_cast<size_t>(nt0) * KT * 64 + lane;
-  const uint16_t* ssrc = static_cast<const uint16_t*>(p.scales) + static_cast<size_t>(nt0) * KT * 16 + lrow;
-  const uint8_t* zsrc = HAS_ZP ? static_cast<const uint8_t*>(p.zeros) + static_cast<size_t>(nt0) * KT * 16 + lrow : nullptr;
+  // ---- weights: this wavefront's two column tiles (clamped inside N; results of clamped tiles are not stored)
+  const uint32_t n_tiles = p.N / 16;
+  const uint32_t nt0 = n0 / 16 + wave * WN;
+  const char* w_base[WN];
+  const char* s_base[WN];
+  const char* z_base[WN];
+#pragma unroll
+  for (int t = 0; t < WN; ++t) {
+    const uint32_t nt = (nt0 + t < n_tiles) ? nt0 + t : n_tiles - 1;
+    w_base[t] = static_cast<const char*>(p.w) + (static_cast<size_t>(nt) * KT + kt_begin) * 1024;
+    s_base[t] = static_cast<const char*>(p.scales) + (static_cast<size_t>(nt) * KT + kt_begin) * 32;
+    z_base[t] = HAS_ZP ? static_cast<const char*>(p.zeros) + (static_cast<size_t>(nt) * KT + kt_begin) * 16 : nullptr;
+  }
+  const uint32_t w_voff = lane * 16, s_voff = lrow * 2, z_voff = lrow;
 
   f32x4 acc[WN][WM];
 #pragma unroll
@@ -154,40 +186,54 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, 1) w4a16_tile_kernel(Ti
 #pragma unroll
     for (int i = 0; i < WM; ++i) acc[t][i] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  u32x4 areg[A_LOADS];
-  u32x4 wq[WN];       // current k-tile's packed weights
-  u32x4 wq_next[WN];
-  uint32_t sc[WN], sc_next[WN], zp[WN], zp_next[WN];
+  WSlot ring[3][WN];  // k-tiles kt, kt+1, kt+2 (indexed kt % 3)
 
-  auto load_a = [&](uint32_t k0) {
-#pragma unroll
-    for (int j = 0; j < A_LOADS; ++j) areg[j] = *reinterpret_cast<const u32x4*>(a_src[j] + static_cast<size_t>(k0) * 2);
-  };
-  auto store_a = [&](int buf) {
-#pragma unroll
-    for (int j = 0; j < A_LOADS; ++j) *reinterpret_cast<u32x4*>(lds + buf * STAGE_BYTES + a_dst[j]) = areg[j];
-  };
-  auto load_w = [&](u32x4 (&dst)[WN], uint32_t (&s)[WN], uint32_t (&z)[WN], uint32_t kt) {
-#pragma unroll
-    for (int t = 0; t < WN; ++t) {
-      dst[t] = wsrc[(static_cast<size_t>(t) * KT + kt) * 64];
-      s[t] = ssrc[(static_cast<size_t>(t) * KT + kt) * 16];
-      z[t] = HAS_ZP ? zsrc[(static_cast<size_t>(t) * KT + kt) * 16] : 8u;
+  // ---- issue helpers (inline assembly: the compiler neither reorders nor counts these loads)
+  auto load_w = [&](WSlot& dst, int t, uint32_t kt) {
+    kt = kt < kt_count ? kt : kt_count - 1;
+    const char* wp = w_base[t] + static_cast<size_t>(kt) * 1024;
+    const char* sp = s_base[t] + static_cast<size_t>(kt) * 32;
+    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(dst.wq) : "v"(w_voff), "s"(wp) : "memory");
+    asm volatile("global_load_ushort %0, %1, %2" : "=v"(dst.sc) : "v"(s_voff), "s"(sp) : "memory");
+    if (HAS_ZP) {
+      const char* zp = z_base[t] + static_cast<size_t>(kt) * 16;
+      asm volatile("global_load_ubyte %0, %1, %2" : "=v"(dst.zp) : "v"(z_voff), "s"(zp) : "memory");
+    } else {
+      dst.zp = 8u;
     }
   };
+  auto load_a = [&](uint32_t stage) {
+    const uint32_t st = stage < stages ? stage : stages - 1;
+    const char* src = x_tile + static_cast<size_t>(st) * (BK * 2);
+    const uint32_t dst = __builtin_amdgcn_readfirstlane(a_lds_wave + (stage % NS) * STAGE_BYTES);
+#pragma unroll
+    for (int j = 0; j < AP / 2; ++j) {
+      // the instruction offset of an LDS-targeted load is added to the LDS address as well as to the global one:
+      // the second fragment's 64-byte global offset is taken back out of its LDS base
+      const uint32_t d0 = dst + (2 * j) * 1024, d1 = d0 + 1024 - 64;
+      asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %2" ::"v"(a_voff[j]), "s"(d0), "s"(src)
+                   : "memory");
+      asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %2 offset:64" ::"v"(a_voff[j]), "s"(d1),
+                   "s"(src)
+                   : "memory");
+    }
+  };
+  // wait until at most WAIT_N loads are outstanding; `fresh` is the weight slot that becomes valid with this wait
+  auto wait_stage = [&](WSlot& fresh) {
+    asm volatile("s_waitcnt vmcnt(%3)" : "+v"(fresh.wq), "+v"(fresh.sc), "+v"(fresh.zp) : "n"(WAIT_N) : "memory");
+  };
+  auto tie = [&](WSlot& slot) { asm volatile("" : "+v"(slot.wq), "+v"(slot.sc), "+v"(slot.zp)::"memory"); };
 
-  // half = 0/1: which 64-wide half of the current k-tile this stage covers
-  auto compute = [&](int buf, int half) {
-    const char* abase = lds + buf * STAGE_BYTES + (wm * WM * (BK / 32)) * 1024 + lane * 16;
+  auto compute = [&](uint32_t slot, WSlot (&w)[WN], int half) {
+    const char* abase = lds + slot * STAGE_BYTES + lane * 16;
+    Dequant<T, HAS_ZP> dq[WN];
+#pragma unroll
+    for (int t = 0; t < WN; ++t) dq[t].set(w[t].sc, w[t].zp);
 #pragma unroll
     for (int ks = 0; ks < BK / 32; ++ks) {
       typename T::frag bfrag[WN];
 #pragma unroll
-      for (int t = 0; t < WN; ++t) {
-        Dequant<T, HAS_ZP> dq;
-        dq.set(sc[t], zp[t]);
-        bfrag[t] = dq(wq[t][half * 2 + ks]);
-      }
+      for (int t = 0; t < WN; ++t) bfrag[t] = dq[t](w[t].wq[half * 2 + ks]);
 #pragma unroll
       for (int i = 0; i < WM; ++i) {
         const u32x4 a = *reinterpret_cast<const u32x4*>(abase + (i * (BK / 32) + ks) * 1024);
@@ -197,45 +243,83 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, 1) w4a16_tile_kernel(Ti
     }
   };
 
-  // ---- pipeline: stage s covers k in [64 s, 64 s + 64); k-tile = s / 2
-  const uint32_t stages = p.K / BK;
+  // ---- schedule.  Stage j issues [weight slot W_j][x stage j+3]; W_j is column tile j%2 of k-tile j/2 + 2 (j even)
+  // or (j+3)/2 (j odd), i.e. the two slots of a k-tile are issued 4 and 3 stages before its first stage.  Stage s is
+  // consumed after a wait that leaves exactly the loads of stages s-2 and s-1 outstanding.
+  load_w(ring[0][0], 0, 0);  // virtual stage -4
+  load_w(ring[0][1], 1, 0);  // virtual stage -3
   load_a(0);
-  load_w(wq, sc, zp, 0);
-  store_a(0);
-  __syncthreads();
-  for (uint32_t s = 0; s < stages; ++s) {
-    const int buf = s & 1;
-    const int half = s & 1;
-    if (s + 1 < stages) load_a((s + 1) * BK);
-    if (half == 0 && (s >> 1) + 1 < KT) load_w(wq_next, sc_next, zp_next, (s >> 1) + 1);
-    compute(buf, half);
-    if (s + 1 < stages) store_a(buf ^ 1);
-    if (half == 1) {
+  load_w(ring[1][0], 0, 1);  // virtual stage -2
+  load_a(1);
+  load_w(ring[1][1], 1, 1);  // virtual stage -1
+  load_a(2);
+
+  for (uint32_t base = 0; base < stages; base += 6) {
 #pragma unroll
-      for (int t = 0; t < WN; ++t) {
-        wq[t] = wq_next[t];
-        sc[t] = sc_next[t];
-        zp[t] = zp_next[t];
+    for (int u = 0; u < 6; ++u) {
+      const uint32_t s = base + u;
+      // the slot issued three stages ago becomes valid now (ring indices are static because base % 6 == 0)
+      constexpr int kPrevOf[6] = {3, 4, 5, 0, 1, 2};  // (u - 3) mod 6
+      const int j = kPrevOf[u];
+      WSlot& fresh = (j % 2 == 0) ? ring[(j / 2 + 2) % 3][0] : ring[((j + 3) / 2) % 3][1];
+      wait_stage(fresh);
+      if (u == 0) tie(ring[0][0]);  // issued before x stage 0 in the prologue: complete, but tied to no wait of its own
+      __syncthreads();
+      // issue stage s: weight slot W_s, then x stage s+3 (its LDS slot was consumed in stage s-1 and every wavefront
+      // is past that: the barrier above follows their compute of s-1)
+      if (u % 2 == 0) {
+        load_w(ring[(u / 2 + 2) % 3][0], 0, s / 2 + 2);
+      } else {
+        load_w(ring[((u + 3) / 2) % 3][1], 1, (s + 3) / 2);
       }
+      load_a(s + 3);
+      if (s < stages) compute(s % NS, ring[(u / 2) % 3], u % 2);
     }
-    __syncthreads();
   }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // drain the clamped prefetches before the LDS is released
 
   // ---- store: lane holds row m = l%16 of the 16x16 tile and columns 4*(l/16) .. +3
 #pragma unroll
   for (int i = 0; i < WM; ++i) {
-    const uint32_t row = m0 + (wm * WM + i) * 16 + lrow;
+    const uint32_t row = m0 + i * 16 + lrow;
     if (row < p.M) {
 #pragma unroll
       for (int t = 0; t < WN; ++t) {
-        u32x2 o;
-        o.x = pack2(T::from_float(acc[t][i][0]), T::from_float(acc[t][i][1]));
-        o.y = pack2(T::from_float(acc[t][i][2]), T::from_float(acc[t][i][3]));
-        uint16_t* yp = static_cast<uint16_t*>(p.y) + static_cast<size_t>(row) * p.N + (nt0 + t) * 16 + 4 * lq;
-        *reinterpret_cast<u32x2*>(yp) = o;
+        if (nt0 + t < n_tiles) {
+          const size_t col = static_cast<size_t>(nt0 + t) * 16 + 4 * lq;
+          if (p.splits == 1) {
+            u32x2 o;
+            o.x = pack2(T::from_float(acc[t][i][0]), T::from_float(acc[t][i][1]));
+            o.y = pack2(T::from_float(acc[t][i][2]), T::from_float(acc[t][i][3]));
+            *reinterpret_cast<u32x2*>(static_cast<uint16_t*>(p.y) + static_cast<size_t>(row) * p.N + col) = o;
+          } else {
+            float* dst = p.partial + (static_cast<size_t>(split) * p.M + row) * p.N + col;
+            *reinterpret_cast<f32x4*>(dst) = acc[t][i];
+          }
+        }
       }
     }
   }
+}
+
+// y[m, n] = T(sum over splits of partial[s, m, n]), 8 outputs per thread, summed in split order
+template <typename T>
+__global__ void __launch_bounds__(256) splitk_reduce_kernel(const float* __restrict__ partial, uint16_t* __restrict__ y,
+                                                            size_t mn, uint32_t splits) {
+  const size_t i = (static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x) * 8;
+  if (i >= mn) return;
+  f32x4 a = *reinterpret_cast<const f32x4*>(partial + i);
+  f32x4 b = *reinterpret_cast<const f32x4*>(partial + i + 4);
+  for (uint32_t s = 1; s < splits; ++s) {
+    a += *reinterpret_cast<const f32x4*>(partial + s * mn + i);
+    b += *reinterpret_cast<const f32x4*>(partial + s * mn + i + 4);
+  }
+  u32x4 o;
+  o.x = pack2(T::from_float(a[0]), T::from_float(a[1]));
+  o.y = pack2(T::from_float(a[2]), T::from_float(a[3]));
+  o.z = pack2(T::from_float(b[0]), T::from_float(b[1]));
+  o.w = pack2(T::from_float(b[2]), T::from_float(b[3]));
+  *reinterpret_cast<u32x4*>(y + i) = o;
 }
 
 }  // namespace ksq

@@ -93,11 +93,28 @@ def w4a16_workspace_size(max_m, n, k, group, dtype):
     return _lib.ksq_w4a16_workspace_size(max_m, n, k, group, dtype)
 
 
+_WORKSPACES = {}
+
+
+def _w4a16_workspace(device, m, n, k, group, dt):
+    """A per-device scratch tensor large enough for this call (grown on demand, like the engine's shared workspace)."""
+    need = _lib.ksq_w4a16_workspace_size(m, n, k, group, dt)
+    if need == 0:
+        return None
+    cur = _WORKSPACES.get(device)
+    if cur is None or cur.numel() < need:
+        cur = torch.empty(need, dtype=torch.uint8, device=device)
+        _WORKSPACES[device] = cur
+    return cur
+
+
 def w4a16_gemm(x, w_packed, scales_packed, zeros_packed, n, k, group, out=None, workspace=None):
     """InvokeFpAIntBGroupCudaGemm / InvokeFpAIntBGroupCutlassGemm / InvokeMarlinGemm / InvokeMacheteGemm."""
     m = x.shape[0]
     if out is None:
         out = torch.empty((m, n), dtype=x.dtype, device=x.device)
+    if workspace is None:
+        workspace = _w4a16_workspace(x.device, m, n, k, group, _dt(x))
     ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
     _l.check(_lib.ksq_w4a16_gemm(_ptr(out), _ptr(x), _ptr(w_packed), _ptr(scales_packed), _ptr(zeros_packed),
                                  _ptr(workspace), ws_bytes, m, n, k, group, _dt(x), _stream()))
