@@ -141,7 +141,7 @@ KSQ_EXPORT size_t ksq_w4a16_workspace_size(size_t max_m, size_t n, size_t k, siz
   for (size_t m = 33; m <= max_m; ++m) {
     if (!use_mfma_tile(m, n, k, group)) break;
     const TilePlan t = plan_mfma_tile(m, n, k);
-    if (t.splits == 1 && t.block_m == 256 && m % 256 == 0) break;  // the grid only grows from here on
+    if (t.splits == 1 && m % 256 == 0 && m >= 1024) break;  // the grid only grows from here on
     need = t.workspace_bytes > need ? t.workspace_bytes : need;
   }
   return need;

@@ -4,7 +4,9 @@
 //   - x (activations) goes global -> LDS without touching registers: every wavefront issues global_load_lds_dwordx4
 //     for whole 1 KiB MFMA fragments (16 rows x 32 k; lane l supplies row l%16, k 8*(l/16)..+7 and lands at
 //     base + 16*l), into a ring of NS stages of 64 k each.  The fragment is read back with one conflict-free
-//     ds_read_b128 per lane.  Three stages are in flight while one is consumed.
+//     ds_read_b128 per lane, DEPTH fragments ahead of the MFMAs that use it.  Two to three stages are in flight
+//     while one is consumed; the one barrier per stage sits in the middle of the stage, so the fragment reads never
+//     drain at a stage boundary.
 //   - packed int4 weights never touch LDS: the 8 wavefronts split the 256 columns (2 column tiles of 16 each), so
 //     every weight fragment belongs to exactly one wavefront and no weight is dequantized twice.  A wavefront loads
 //     its 1 KiB tiles straight from global memory (16 bytes per lane) three stages ahead and dequantizes them in
@@ -16,9 +18,11 @@
 //   - the weights are the row operand of v_mfma_f32_16x16x32 and x the column operand, so a lane ends up with four
 //     consecutive output columns of one row and stores them as one 8-byte word (or 16 bytes of fp32 partials).
 //
-// Workgroup ids are remapped so that the eight XCDs each work on a contiguous band of (column tile, k-split) pairs and
-// sweep the row tiles fastest: the weight band of a workgroup is shared by its neighbours on the same L2.
+// Workgroup ids are remapped so that the workgroups running on one XCD at the same time form a compact block of
+// row tiles x column tiles: both operands are then shared through that XCD's L2.
 #pragma once
+
+#include <type_traits>
 
 #include "ksq_common.h"
 
@@ -136,17 +140,27 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
   const int lrow = lane & 15, lq = lane >> 4;
   const uint32_t KT = p.K / 128;
 
-  // ---- XCD-aware work id: workgroup b runs on XCD b%8; every XCD gets a contiguous range, row tile fastest
-  const uint32_t total = p.tiles_m * p.tiles_n * p.splits;
-  uint32_t bid = blockIdx.x;
+  // ---- work id.  Workgroup b runs on XCD b%8 and the b/8-th of that XCD's workgroups start in order, 32 at a time
+  // (one per CU).  Every XCD gets a contiguous range of a linear tile order in which 32 consecutive items form a block
+  // of 4 row tiles x 8 (column tile, k-split) pairs: the workgroups that share an L2 at any moment read 4 activation
+  // tiles and 8 weight strips between them instead of 16 and 2, which cuts the traffic into the L2 by more than half.
+  constexpr uint32_t GN = 8;
+  const uint32_t cols = p.tiles_n * p.splits;
+  const uint32_t total = p.tiles_m * cols;
+  uint32_t lin = blockIdx.x;
   {
     const uint32_t per = total / 8, rem = total % 8;
-    const uint32_t xcd = bid % 8, local = bid / 8;
-    bid = xcd * per + (xcd < rem ? xcd : rem) + local;  // XCDs 0..rem-1 own per+1 items
+    const uint32_t xcd = lin % 8, local = lin / 8;
+    lin = xcd * per + (xcd < rem ? xcd : rem) + local;  // XCDs 0..rem-1 own per+1 items
   }
-  const uint32_t tile_m = bid % p.tiles_m;
-  const uint32_t rest = bid / p.tiles_m;
-  const uint32_t split = rest % p.splits, tile_n = rest / p.splits;
+  const uint32_t band_items = p.tiles_m * GN;
+  const uint32_t band = lin / band_items;
+  const uint32_t c0 = band * GN;
+  const uint32_t width = (cols - c0) < GN ? (cols - c0) : GN;
+  const uint32_t within = lin - band * band_items;
+  const uint32_t tile_m = within / width;
+  const uint32_t col = c0 + within % width;
+  const uint32_t split = col % p.splits, tile_n = col / p.splits;
   const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
   const uint32_t kt_begin = split * p.kt_per_split;
   const uint32_t kt_count = (KT - kt_begin) < p.kt_per_split ? (KT - kt_begin) : p.kt_per_split;
@@ -189,91 +203,165 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
   WSlot ring[3][WN];  // k-tiles kt, kt+1, kt+2 (indexed kt % 3)
 
   // ---- issue helpers (inline assembly: the compiler neither reorders nor counts these loads)
-  auto load_w = [&](WSlot& dst, int t, uint32_t kt) {
+  // Every group of loads is ONE assembly statement that opens with `s_nop 4`: all its scalar operands are in place
+  // before the statement starts, and should the compiler have produced one of them with a VALU instruction
+  // (v_readfirstlane), the five wait states a vector memory instruction needs after that have passed.  The compiler
+  // inserts such wait states for its own instructions, not inside assembly.
+  auto load_w = [&](WSlot (&dst)[WN], uint32_t kt) {
+    static_assert(WN == 2, "the load group below names two column tiles");
     kt = kt < kt_count ? kt : kt_count - 1;
-    const char* wp = w_base[t] + static_cast<size_t>(kt) * 1024;
-    const char* sp = s_base[t] + static_cast<size_t>(kt) * 32;
-    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(dst.wq) : "v"(w_voff), "s"(wp) : "memory");
-    asm volatile("global_load_ushort %0, %1, %2" : "=v"(dst.sc) : "v"(s_voff), "s"(sp) : "memory");
+    const char* w0 = w_base[0] + static_cast<size_t>(kt) * 1024;
+    const char* w1 = w_base[1] + static_cast<size_t>(kt) * 1024;
+    const char* s0 = s_base[0] + static_cast<size_t>(kt) * 32;
+    const char* s1 = s_base[1] + static_cast<size_t>(kt) * 32;
     if (HAS_ZP) {
-      const char* zp = z_base[t] + static_cast<size_t>(kt) * 16;
-      asm volatile("global_load_ubyte %0, %1, %2" : "=v"(dst.zp) : "v"(z_voff), "s"(zp) : "memory");
+      const char* z0 = z_base[0] + static_cast<size_t>(kt) * 16;
+      const char* z1 = z_base[1] + static_cast<size_t>(kt) * 16;
+      asm volatile(
+          "s_nop 4\n\t"
+          "global_load_dwordx4 %0, %6, %9\n\t"
+          "global_load_ushort %1, %7, %10\n\t"
+          "global_load_ubyte %2, %8, %11\n\t"
+          "global_load_dwordx4 %3, %6, %12\n\t"
+          "global_load_ushort %4, %7, %13\n\t"
+          "global_load_ubyte %5, %8, %14"
+          : "=&v"(dst[0].wq), "=&v"(dst[0].sc), "=&v"(dst[0].zp), "=&v"(dst[1].wq), "=&v"(dst[1].sc), "=&v"(dst[1].zp)
+          : "v"(w_voff), "v"(s_voff), "v"(z_voff), "s"(w0), "s"(s0), "s"(z0), "s"(w1), "s"(s1), "s"(z1)
+          : "memory");
     } else {
-      dst.zp = 8u;
+      asm volatile(
+          "s_nop 4\n\t"
+          "global_load_dwordx4 %0, %4, %6\n\t"
+          "global_load_ushort %1, %5, %7\n\t"
+          "global_load_dwordx4 %2, %4, %8\n\t"
+          "global_load_ushort %3, %5, %9"
+          : "=&v"(dst[0].wq), "=&v"(dst[0].sc), "=&v"(dst[1].wq), "=&v"(dst[1].sc)
+          : "v"(w_voff), "v"(s_voff), "s"(w0), "s"(s0), "s"(w1), "s"(s1)
+          : "memory");
+      dst[0].zp = 8u;
+      dst[1].zp = 8u;
     }
   };
+  // x stage `stage` -> LDS slot stage % NS.  The instruction offset of an LDS-targeted load is added to the LDS address
+  // as well as to the global one: the second fragment's 64-byte global offset is taken back out of its LDS base.
   auto load_a = [&](uint32_t stage) {
     const uint32_t st = stage < stages ? stage : stages - 1;
     const char* src = x_tile + static_cast<size_t>(st) * (BK * 2);
-    const uint32_t dst = __builtin_amdgcn_readfirstlane(a_lds_wave + (stage % NS) * STAGE_BYTES);
-#pragma unroll
-    for (int j = 0; j < AP / 2; ++j) {
-      // the instruction offset of an LDS-targeted load is added to the LDS address as well as to the global one:
-      // the second fragment's 64-byte global offset is taken back out of its LDS base
-      const uint32_t d0 = dst + (2 * j) * 1024, d1 = d0 + 1024 - 64;
-      asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %2" ::"v"(a_voff[j]), "s"(d0), "s"(src)
-                   : "memory");
-      asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %2 offset:64" ::"v"(a_voff[j]), "s"(d1),
-                   "s"(src)
-                   : "memory");
+    const uint32_t d0 = __builtin_amdgcn_readfirstlane(a_lds_wave + (stage % NS) * STAGE_BYTES);
+    const uint32_t d1 = d0 + 1024 - 64;
+    if (AP == 2) {
+      asm volatile(
+          "s_nop 4\n\t"
+          "s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %3\n\t"
+          "s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %3 offset:64"
+          :
+          : "v"(a_voff[0]), "s"(d0), "s"(d1), "s"(src)
+          : "memory");
+    } else {
+      static_assert(AP == 2 || AP == 4, "two or four fragments per wavefront and stage");
+      const uint32_t d2 = d0 + 2048, d3 = d1 + 2048;
+      asm volatile(
+          "s_nop 4\n\t"
+          "s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %6\n\t"
+          "s_mov_b32 m0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %6 offset:64\n\t"
+          "s_mov_b32 m0, %4\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %6\n\t"
+          "s_mov_b32 m0, %5\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %6 offset:64"
+          :
+          : "v"(a_voff[0]), "v"(a_voff[AP / 2 - 1]), "s"(d0), "s"(d1), "s"(d2), "s"(d3), "s"(src)
+          : "memory");
     }
   };
-  // wait until at most WAIT_N loads are outstanding; `fresh` is the weight slot that becomes valid with this wait
-  auto wait_stage = [&](WSlot& fresh) {
-    asm volatile("s_waitcnt vmcnt(%3)" : "+v"(fresh.wq), "+v"(fresh.sc), "+v"(fresh.zp) : "n"(WAIT_N) : "memory");
+  // wait until at most `n` loads are outstanding; the weight slots named become valid with this wait and are tied to it
+  auto wait_tie = [&](auto n, WSlot (&fresh)[WN]) {
+    asm volatile("s_waitcnt vmcnt(%6)"
+                 : "+v"(fresh[0].wq), "+v"(fresh[0].sc), "+v"(fresh[0].zp), "+v"(fresh[1].wq), "+v"(fresh[1].sc),
+                   "+v"(fresh[1].zp)
+                 : "n"(decltype(n)::value)
+                 : "memory");
   };
-  auto tie = [&](WSlot& slot) { asm volatile("" : "+v"(slot.wq), "+v"(slot.sc), "+v"(slot.zp)::"memory"); };
+  auto wait_only = [&](auto n) { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(decltype(n)::value) : "memory"); };
 
-  auto compute = [&](uint32_t slot, WSlot (&w)[WN], int half) {
-    const char* abase = lds + slot * STAGE_BYTES + lane * 16;
-    Dequant<T, HAS_ZP> dq[WN];
+  // ---- compute pipeline, in steps of 32 k (two per stage).  A fragments are read DEPTH ahead of the MFMAs that use
+  // them, across step and stage boundaries; the weight fragments of step g+1 are dequantized while step g multiplies.
+  constexpr int DEPTH = 4;
+  static_assert(WM % DEPTH == 0, "the A prefetch ring must divide the row tiles");
+  u32x4 abuf[DEPTH];
+  typename T::frag bcur[WN], bnext[WN];
+  Dequant<T, HAS_ZP> dq[WN];
+
+  auto frag_ptr = [&](uint32_t slot, int ks) { return lds + slot * STAGE_BYTES + ks * 1024 + lane * 16; };
+  // `wn`/`dn`: weight slot and dword (32-k block of its k-tile) the NEXT step uses
+  auto step = [&](uint32_t slot, int ks, WSlot (&wn)[WN], int dn) {
+    const char* cur = frag_ptr(slot, ks);
+    const char* nxt = ks == 0 ? frag_ptr(slot, 1) : frag_ptr((slot + 1) % NS, 0);
+    if (dn == 0) {
 #pragma unroll
-    for (int t = 0; t < WN; ++t) dq[t].set(w[t].sc, w[t].zp);
-#pragma unroll
-    for (int ks = 0; ks < BK / 32; ++ks) {
-      typename T::frag bfrag[WN];
-#pragma unroll
-      for (int t = 0; t < WN; ++t) bfrag[t] = dq[t](w[t].wq[half * 2 + ks]);
-#pragma unroll
-      for (int i = 0; i < WM; ++i) {
-        const u32x4 a = *reinterpret_cast<const u32x4*>(abase + (i * (BK / 32) + ks) * 1024);
-#pragma unroll
-        for (int t = 0; t < WN; ++t) acc[t][i] = T::mfma(bfrag[t], as_frag<T>(a), acc[t][i]);
-      }
+      for (int t = 0; t < WN; ++t) dq[t].set(wn[t].sc, wn[t].zp);
     }
+#pragma unroll
+    for (int i = 0; i < WM; ++i) {
+      const u32x4 a = abuf[i % DEPTH];
+      const int ni = i + DEPTH;
+      abuf[i % DEPTH] = ni < WM ? *reinterpret_cast<const u32x4*>(cur + ni * 2048)
+                                : *reinterpret_cast<const u32x4*>(nxt + (ni - WM) * 2048);
+#pragma unroll
+      for (int t = 0; t < WN; ++t) acc[t][i] = T::mfma(bcur[t], as_frag<T>(a), acc[t][i]);
+      if (i == 1) bnext[0] = dq[0](wn[0].wq[dn]);
+      if (i == WM / 2 + 1) bnext[1] = dq[1](wn[1].wq[dn]);
+      __builtin_amdgcn_sched_barrier(0x6);  // VALU / SALU may move; LDS reads and MFMAs keep this order
+    }
+#pragma unroll
+    for (int t = 0; t < WN; ++t) bcur[t] = bnext[t];
   };
 
-  // ---- schedule.  Stage j issues [weight slot W_j][x stage j+3]; W_j is column tile j%2 of k-tile j/2 + 2 (j even)
-  // or (j+3)/2 (j odd), i.e. the two slots of a k-tile are issued 4 and 3 stages before its first stage.  Stage s is
-  // consumed after a wait that leaves exactly the loads of stages s-2 and s-1 outstanding.
-  load_w(ring[0][0], 0, 0);  // virtual stage -4
-  load_w(ring[0][1], 1, 0);  // virtual stage -3
-  load_a(0);
-  load_w(ring[1][0], 0, 1);  // virtual stage -2
+  // ---- schedule.  One synchronisation point per stage, in its middle ("sync c" sits between the two steps of
+  // stage c): wait for x stage c+1, barrier, then issue [weights of k-tile c/2+2 when c is even][x stage c+3] - the LDS
+  // slot of stage c+3 is the one stage c-1 used, and every wavefront is past that.  Weights of k-tile kt are issued at
+  // sync 2kt-4, complete at sync 2kt-2 and are first dequantized during the last step of k-tile kt-1.
+  // Loads outstanding after x stage c+1 at sync c: those of sync c-1, i.e. AP, plus 2*WL when c-1 is even.
+  using WaitEven = std::integral_constant<int, AP>;
+  using WaitOdd = std::integral_constant<int, AP + WN * WL>;
+  using WaitFirst = std::integral_constant<int, 2 * AP + WN * WL>;
+  load_w(ring[0], 0);  // sync -4
+  load_a(0);           // sync -3
+  load_w(ring[1], 1);  // sync -2
   load_a(1);
-  load_w(ring[1][1], 1, 1);  // virtual stage -1
-  load_a(2);
+  load_a(2);           // sync -1
+  wait_tie(WaitFirst{}, ring[0]);  // x stage 0 and k-tile 0 are in
+  __builtin_amdgcn_s_barrier();
+#pragma unroll
+  for (int t = 0; t < WN; ++t) {
+    dq[t].set(ring[0][t].sc, ring[0][t].zp);
+    bcur[t] = dq[t](ring[0][t].wq[0]);
+  }
+#pragma unroll
+  for (int j = 0; j < DEPTH; ++j) abuf[j] = *reinterpret_cast<const u32x4*>(frag_ptr(0, 0) + j * 2048);
 
   for (uint32_t base = 0; base < stages; base += 6) {
 #pragma unroll
     for (int u = 0; u < 6; ++u) {
       const uint32_t s = base + u;
-      // the slot issued three stages ago becomes valid now (ring indices are static because base % 6 == 0)
-      constexpr int kPrevOf[6] = {3, 4, 5, 0, 1, 2};  // (u - 3) mod 6
-      const int j = kPrevOf[u];
-      WSlot& fresh = (j % 2 == 0) ? ring[(j / 2 + 2) % 3][0] : ring[((j + 3) / 2) % 3][1];
-      wait_stage(fresh);
-      if (u == 0) tie(ring[0][0]);  // issued before x stage 0 in the prologue: complete, but tied to no wait of its own
-      __syncthreads();
-      // issue stage s: weight slot W_s, then x stage s+3 (its LDS slot was consumed in stage s-1 and every wavefront
-      // is past that: the barrier above follows their compute of s-1)
+      const uint32_t slot = s % NS;
+      constexpr int kDummy = 0;
+      (void)kDummy;
+      // first step of the stage: k block 2*(u%2) of k-tile u/2; the next step uses block 2*(u%2)+1 of the same tile
+      if (s < stages) step(slot, 0, ring[(u / 2) % 3], 2 * (u % 2) + 1);
+      // sync s
       if (u % 2 == 0) {
-        load_w(ring[(u / 2 + 2) % 3][0], 0, s / 2 + 2);
+        wait_tie(WaitEven{}, ring[(u / 2 + 1) % 3]);  // k-tile s/2+1, issued at sync s-2
       } else {
-        load_w(ring[((u + 3) / 2) % 3][1], 1, (s + 3) / 2);
+        wait_only(WaitOdd{});
       }
+      __builtin_amdgcn_s_barrier();
+      if (u % 2 == 0) load_w(ring[(u / 2 + 2) % 3], s / 2 + 2);
       load_a(s + 3);
-      if (s < stages) compute(s % NS, ring[(u / 2) % 3], u % 2);
+      // second step: the next step is block 2 of this k-tile (u even) or block 0 of the next k-tile (u odd)
+      if (s < stages) {
+        if (u % 2 == 0)
+          step(slot, 1, ring[(u / 2) % 3], 2);
+        else
+          step(slot, 1, ring[(u / 2 + 1) % 3], 0);
+      }
     }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // drain the clamped prefetches before the LDS is released
