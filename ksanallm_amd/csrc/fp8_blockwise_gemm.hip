@@ -3,7 +3,12 @@
 // Both operands are K-contiguous bytes, which is what v_mfma_f32_16x16x128_f8f6f4 wants: lane l supplies the 32
 // bytes k = 32*(l/16) .. +31 of row l%16.  Weights are the row operand, activations the column operand, so a lane's
 // four results are four consecutive output columns of one token.
+#include <atomic>
+
+#include "fp8_tile.h"
 #include "ksq_common.h"
+#include "splitk_reduce.h"
+#include "tile_select.h"
 
 namespace ksq {
 namespace {
@@ -143,21 +148,60 @@ int dispatch(const Fp8Params& p, hipStream_t s) {
   return KSQ_OK;
 }
 
+template <typename TO>
+int launch_fp8_tile(const Fp8Params& q, const TilePlan& plan, float* partial, hipStream_t s) {
+  constexpr int kLds = 2 * 32 * 2048;
+  static std::atomic<bool> configured{false};
+  if (!configured.load(std::memory_order_acquire)) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&fp8_tile_kernel<TO>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
+    if (e != hipSuccess) return fail(KSQ_ERR_LAUNCH, "hipFuncSetAttribute(LDS %d): %s", kLds, hipGetErrorString(e));
+    configured.store(true, std::memory_order_release);
+  }
+  Fp8TileParams p{};
+  p.a = q.a;
+  p.a_s = q.a_s;
+  p.b = q.b;
+  p.b_s = q.b_s;
+  p.out = q.out;
+  p.partial = partial;
+  p.M = q.M;
+  p.N = q.N;
+  p.K = q.K;
+  p.tiles_m = plan.tiles_m;
+  p.tiles_n = plan.tiles_n;
+  p.splits = plan.splits;
+  p.kb_per_split = plan.kt_per_split;
+  fp8_tile_kernel<TO><<<plan.tiles_m * plan.tiles_n * plan.splits, 512, kLds, s>>>(p);
+  if (plan.splits > 1) {
+    const size_t mn = static_cast<size_t>(p.M) * p.N;
+    splitk_reduce_kernel<TO><<<static_cast<unsigned>(div_up(mn, 256 * 8)), 256, 0, s>>>(partial, static_cast<uint16_t*>(p.out), mn,
+                                                                                   plan.splits);
+  }
+  return KSQ_OK;
+}
+
 }  // namespace
 }  // namespace ksq
 
 using namespace ksq;
 
 KSQ_EXPORT size_t ksq_fp8_blockwise_workspace_size(size_t max_m, size_t n, size_t k) {
-  (void)max_m; (void)n; (void)k;
-  return 0;
+  // only the split-K form of the tile kernel needs scratch: fp32 partial tiles
+  if (n == 0 || k == 0 || k % 128 != 0) return 0;
+  size_t need = 0;
+  for (size_t m = 65; m <= max_m; ++m) {
+    const TilePlan t = plan_fp8_tile(m, n, k);
+    if (t.splits == 1 && m % 256 == 0) break;  // the grid only grows from here on
+    need = t.workspace_bytes > need ? t.workspace_bytes : need;
+  }
+  return need;
 }
 
 KSQ_EXPORT int ksq_fp8_blockwise_gemm(const void* a_q, const void* a_s, const void* b, const void* b_s, void* out,
                                       size_t m, size_t n, size_t k, int out_dtype, void* workspace,
                                       size_t workspace_bytes, void* stream) {
   const char* fn = "ksq_fp8_blockwise_gemm";
-  (void)workspace; (void)workspace_bytes;
   if (!a_q || !a_s || !b || !b_s || !out) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: null pointer", fn);
   if (!aligned16(a_q) || !aligned16(b) || !aligned16(out) || (reinterpret_cast<uintptr_t>(a_s) & 3u) ||
       (reinterpret_cast<uintptr_t>(b_s) & 3u))
@@ -173,7 +217,19 @@ KSQ_EXPORT int ksq_fp8_blockwise_gemm(const void* a_q, const void* a_s, const vo
   Fp8Params p{static_cast<const uint8_t*>(a_q), static_cast<const float*>(a_s), static_cast<const uint8_t*>(b),
               static_cast<const float*>(b_s), out, static_cast<uint32_t>(m), static_cast<uint32_t>(n),
               static_cast<uint32_t>(k)};
-  int rc = out_dtype == KSQ_F16 ? dispatch<F16>(p, as_stream(stream)) : dispatch<BF16>(p, as_stream(stream));
+  int rc;
+  if (use_fp8_tile(m, n, k)) {
+    const TilePlan plan = plan_fp8_tile(m, n, k);
+    if (plan.splits > 1 && (!workspace || workspace_bytes < plan.workspace_bytes || !aligned16(workspace)))
+      return fail(KSQ_ERR_WORKSPACE, "%s: m=%zu n=%zu k=%zu needs %zu bytes of 16-byte aligned workspace, got %zu", fn, m,
+                  n, k, plan.workspace_bytes, workspace ? workspace_bytes : size_t(0));
+    if (256 * k > 0xffffffffull) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: k too large", fn);
+    float* partial = plan.splits > 1 ? static_cast<float*>(workspace) : nullptr;
+    rc = out_dtype == KSQ_F16 ? launch_fp8_tile<F16>(p, plan, partial, as_stream(stream))
+                              : launch_fp8_tile<BF16>(p, plan, partial, as_stream(stream));
+  } else {
+    rc = out_dtype == KSQ_F16 ? dispatch<F16>(p, as_stream(stream)) : dispatch<BF16>(p, as_stream(stream));
+  }
   if (rc) return rc;
   return check_launch(fn);
 }

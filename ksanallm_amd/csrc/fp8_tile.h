@@ -1,0 +1,258 @@
+// Prefill-regime blockwise-FP8 kernel (MFMA-bound): a workgroup of 8 wavefronts (2 along M x 4 along N) computes a
+// 256 x 256 output tile over a contiguous range of 128-deep k-blocks.
+//
+//   - both operands are e4m3 bytes, K-contiguous, and need no conversion, so both go global -> LDS without touching
+//     registers (global_load_lds_dwordx4), one 128-deep k-block (32 KiB of activations + 32 KiB of weights) per stage,
+//     two stages.  A 16-row x 128-byte MFMA operand is kept as a 2 KiB fragment in which lane L's 32 bytes sit at
+//     32*L: two loads of 64 contiguous bytes per row fill it, and a lane reads its operand back with two ds_read_b128.
+//   - one v_mfma_f32_16x16x128_f8f6f4 covers exactly one scale block: its result goes to a scratch tile and is folded
+//     into the accumulator with a_s[kb, m] * b_s[n/128, kb] by four fp32 FMAs, issued under the following MFMA.
+//   - weights are the MFMA row operand, activations the column operand: a lane holds four consecutive output columns
+//     of one token (8-byte stores) and needs one activation scale per row tile.
+//   - loads are issued from inline assembly one stage ahead; a single `s_waitcnt vmcnt(0)` + barrier per stage makes
+//     the next stage visible and releases the LDS slot that was just consumed.
+#pragma once
+
+#include "ksq_common.h"
+
+namespace ksq {
+
+struct Fp8TileParams {
+  const uint8_t* a;   // [m, k]
+  const float* a_s;   // [k/128, m]
+  const uint8_t* b;   // [n, k]
+  const float* b_s;   // [ceil(n/128), k/128]
+  void* out;          // [m, n]
+  float* partial;     // [splits][m][n] fp32 when splits > 1
+  uint32_t M, N, K;
+  uint32_t tiles_m, tiles_n;
+  uint32_t splits, kb_per_split;
+};
+
+__device__ __forceinline__ f32x4 mfma_fp8_k128(i32x8 a, i32x8 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
+}
+
+template <typename TO>
+__global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
+  constexpr int WAVES_N = 4;
+  constexpr int WM = 8, WN = 4;  // 16x16 tiles per wavefront: 128 tokens x 64 weight rows
+  constexpr int BM = 256, BN = 256;
+  constexpr int FRAG = 2048;                  // bytes of one 16 x 128 operand fragment
+  constexpr int STAGE_BYTES = 32 * FRAG;      // 16 activation + 16 weight fragments
+  constexpr int W_FRAG0 = 16;                 // first weight fragment of a stage
+
+  extern __shared__ __attribute__((aligned(16))) char lds[];  // 2 * STAGE_BYTES
+
+  const int lane = threadIdx.x & 63;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t wm = wave / WAVES_N, wn = wave % WAVES_N;
+  const int lrow = lane & 15, lq = lane >> 4;
+  const uint32_t KB = p.K / 128;
+
+  // ---- work id: 32 consecutive items of one XCD form a block of 4 row tiles x 8 (column tile, k-split) pairs
+  constexpr uint32_t GN = 8;
+  const uint32_t cols = p.tiles_n * p.splits;
+  const uint32_t total = p.tiles_m * cols;
+  uint32_t lin = blockIdx.x;
+  {
+    const uint32_t per = total / 8, rem = total % 8;
+    const uint32_t xcd = lin % 8, local = lin / 8;
+    lin = xcd * per + (xcd < rem ? xcd : rem) + local;
+  }
+  const uint32_t band_items = p.tiles_m * GN;
+  const uint32_t band = lin / band_items;
+  const uint32_t c0 = band * GN;
+  const uint32_t width = (cols - c0) < GN ? (cols - c0) : GN;
+  const uint32_t within = lin - band * band_items;
+  const uint32_t tile_m = within / width;
+  const uint32_t col = c0 + within % width;
+  const uint32_t split = col % p.splits, tile_n = col / p.splits;
+  const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
+  const uint32_t kb_begin = split * p.kb_per_split;
+  const uint32_t kb_count = (KB - kb_begin) < p.kb_per_split ? (KB - kb_begin) : p.kb_per_split;
+
+  // ---- operand staging.  Wavefronts 0..3 fetch the activation fragments 4w..4w+3, wavefronts 4..7 the weight
+  // fragments 4(w-4)..+3.  Load lane j supplies 16 bytes: row (j/2)%16, byte 64h + 32*((j/2)/16) + 16*(j%2) of the
+  // k-block, h = 0/1 being the instruction; it lands at fragment + 1024h + 16j, i.e. MFMA lane L = 32h + j/2 finds
+  // its 32 bytes at 32L.
+  const bool stage_act = wave < 4;
+  const uint32_t frag0 = (wave & 3) * 4;
+  const uint8_t* g_tile = stage_act ? p.a + static_cast<size_t>(m0) * p.K : p.b + static_cast<size_t>(n0) * p.K;
+  g_tile += static_cast<size_t>(kb_begin) * 128;
+  const uint32_t row_limit = stage_act ? p.M - m0 : p.N - n0;  // rows of this tile inside the matrix
+  uint32_t d_voff[4];
+#pragma unroll
+  for (int f = 0; f < 4; ++f) {
+    uint32_t row = (frag0 + f) * 16 + ((lane >> 1) & 15);
+    row = row < row_limit ? row : row_limit - 1;  // rows past the edge repeat the last row; their results are dropped
+    d_voff[f] = row * p.K + 32 * ((lane >> 5) & 1) + 16 * (lane & 1);
+  }
+  const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<size_t>((__attribute__((address_space(3))) char*)lds));
+  const uint32_t d_lds = lds_base + ((stage_act ? 0 : W_FRAG0) + frag0) * FRAG;
+
+  // ---- scales: one activation scale per row tile and lane (token = column l%16 of the MFMA result), one weight
+  // scale per wavefront and k-block (its 64 weight rows lie inside one 128-row scale block)
+  uint32_t s_voff[WM];
+#pragma unroll
+  for (int i = 0; i < WM; ++i) {
+    uint32_t row = m0 + wm * 128 + i * 16 + lrow;
+    row = row < p.M ? row : p.M - 1;
+    s_voff[i] = row * 4;
+  }
+  const char* as_base = reinterpret_cast<const char*>(p.a_s) + static_cast<size_t>(kb_begin) * p.M * 4;
+  const uint32_t n_wave = n0 + wn * 64;
+  const uint32_t nblk = (n_wave < p.N ? n_wave : p.N - 1) / 128;
+  const char* bs_base = reinterpret_cast<const char*>(p.b_s + static_cast<size_t>(nblk) * KB + kb_begin);
+  const uint32_t zero_voff = 0;
+
+  float as[WM];
+  float bs;
+
+  // Every group of loads is one assembly statement opening with `s_nop 4`: its scalar operands are in place before
+  // it starts, and the wait states a vector memory instruction needs after a VALU write of a scalar register have
+  // passed whatever produced them.
+  auto load_scales = [&](uint32_t kb) {
+    kb = kb < kb_count ? kb : kb_count - 1;
+    const char* ap = as_base + static_cast<size_t>(kb) * p.M * 4;
+    const char* bp = bs_base + static_cast<size_t>(kb) * 4;
+    asm volatile(
+        "s_nop 4\n\t"
+        "global_load_dword %0, %9, %18\n\t"
+        "global_load_dword %1, %10, %18\n\t"
+        "global_load_dword %2, %11, %18\n\t"
+        "global_load_dword %3, %12, %18\n\t"
+        "global_load_dword %4, %13, %18\n\t"
+        "global_load_dword %5, %14, %18\n\t"
+        "global_load_dword %6, %15, %18\n\t"
+        "global_load_dword %7, %16, %18\n\t"
+        "global_load_dword %8, %17, %19"
+        : "=&v"(as[0]), "=&v"(as[1]), "=&v"(as[2]), "=&v"(as[3]), "=&v"(as[4]), "=&v"(as[5]), "=&v"(as[6]), "=&v"(as[7]),
+          "=&v"(bs)
+        : "v"(s_voff[0]), "v"(s_voff[1]), "v"(s_voff[2]), "v"(s_voff[3]), "v"(s_voff[4]), "v"(s_voff[5]), "v"(s_voff[6]),
+          "v"(s_voff[7]), "v"(zero_voff), "s"(ap), "s"(bp)
+        : "memory");
+  };
+  // operands of k-block `kb` -> LDS slot kb % 2.  The instruction offset of an LDS-targeted load is added to the LDS
+  // address as well as to the global one: the second half's 64-byte global offset is taken out of its LDS base.
+  auto load_operands = [&](uint32_t kb) {
+    const uint32_t k = kb < kb_count ? kb : kb_count - 1;
+    const uint8_t* src = g_tile + static_cast<size_t>(k) * 128;
+    const uint32_t f0 = __builtin_amdgcn_readfirstlane(d_lds + (kb & 1) * STAGE_BYTES);
+    const uint32_t f0h = f0 + 1024 - 64;
+    const uint32_t f1 = f0 + FRAG, f1h = f0h + FRAG;
+    const uint32_t f2 = f1 + FRAG, f2h = f1h + FRAG;
+    const uint32_t f3 = f2 + FRAG, f3h = f2h + FRAG;
+    asm volatile(
+        "s_nop 4\n\t"
+        "s_mov_b32 m0, %4\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %12\n\t"
+        "s_mov_b32 m0, %5\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %12 offset:64\n\t"
+        "s_mov_b32 m0, %6\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %12\n\t"
+        "s_mov_b32 m0, %7\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %12 offset:64\n\t"
+        "s_mov_b32 m0, %8\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %12\n\t"
+        "s_mov_b32 m0, %9\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %12 offset:64\n\t"
+        "s_mov_b32 m0, %10\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %3, %12\n\t"
+        "s_mov_b32 m0, %11\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %3, %12 offset:64"
+        :
+        : "v"(d_voff[0]), "v"(d_voff[1]), "v"(d_voff[2]), "v"(d_voff[3]), "s"(f0), "s"(f0h), "s"(f1), "s"(f1h),
+          "s"(f2), "s"(f2h), "s"(f3), "s"(f3h), "s"(src)
+        : "memory");
+  };
+  // everything issued so far has landed; the scale registers become valid with this wait and are tied to it
+  auto wait_all = [&]() {
+    asm volatile("s_waitcnt vmcnt(0)"
+                 : "+v"(as[0]), "+v"(as[1]), "+v"(as[2]), "+v"(as[3]), "+v"(as[4]), "+v"(as[5]), "+v"(as[6]), "+v"(as[7]),
+                   "+v"(bs)
+                 :
+                 : "memory");
+  };
+
+  f32x4 acc[WN][WM];
+#pragma unroll
+  for (int t = 0; t < WN; ++t)
+#pragma unroll
+    for (int i = 0; i < WM; ++i) acc[t][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  auto read_frag = [&](const char* base) {
+    const i32x4 lo = *reinterpret_cast<const i32x4*>(base);
+    const i32x4 hi = *reinterpret_cast<const i32x4*>(base + 16);
+    return i32x8{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+  };
+
+  // one k-block: 32 MFMAs; the scale FMAs of MFMA j are placed after MFMA j+2 so that they run in its shadow
+  auto compute = [&](uint32_t slot, const float (&sc)[WM]) {
+    const char* act = lds + slot * STAGE_BYTES + (wm * WM) * FRAG + lane * 32;
+    const char* wgt = lds + slot * STAGE_BYTES + (W_FRAG0 + wn * WN) * FRAG + lane * 32;
+    i32x8 wf[WN];
+#pragma unroll
+    for (int t = 0; t < WN; ++t) wf[t] = read_frag(wgt + t * FRAG);
+    i32x8 af[2];
+    af[0] = read_frag(act);
+    f32x4 tmp[3];
+    const f32x4 zero{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < WM * WN + 2; ++j) {
+      const int i = j / WN, t = j % WN;
+      if (j < WM * WN) {
+        if (t == 0 && i + 1 < WM) af[(i + 1) & 1] = read_frag(act + (i + 1) * FRAG);
+        tmp[j % 3] = mfma_fp8_k128(wf[t], af[i & 1], zero);
+      }
+      if (j >= 2) {  // the MFMA issued two places earlier has left the pipeline by now
+        const int pi = (j - 2) / WN, pt = (j - 2) % WN;
+        const f32x4 r = tmp[(j - 2) % 3];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[pt][pi][e] = __builtin_fmaf(r[e], sc[pi], acc[pt][pi][e]);
+      }
+      __builtin_amdgcn_sched_barrier(0x4);  // keep MFMAs, FMAs and LDS reads in this order (scalar ALU may move)
+    }
+  };
+
+  // ---- schedule: stage c computes k-block c out of LDS slot c%2 while the operands of c+1 and its scales are in
+  // flight; at the end of the stage everything has to have landed (vmcnt(0)), the barrier makes it visible and tells
+  // every wavefront that slot c%2 is free, and the operands of c+2 are issued into it.
+  load_scales(0);
+  load_operands(0);
+  wait_all();
+  __builtin_amdgcn_s_barrier();
+  float sc[WM];
+#pragma unroll
+  for (int i = 0; i < WM; ++i) sc[i] = as[i] * bs;
+  load_scales(1);
+  load_operands(1);
+
+  for (uint32_t c = 0; c < kb_count; ++c) {
+    compute(c & 1, sc);
+    wait_all();  // operands and scales of c+1
+    __builtin_amdgcn_s_barrier();
+#pragma unroll
+    for (int i = 0; i < WM; ++i) sc[i] = as[i] * bs;
+    load_scales(c + 2);
+    load_operands(c + 2);
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // drain the clamped prefetches before the LDS is released
+
+  // ---- store: lane holds token m = l%16 of the tile and weight rows (output columns) 4*(l/16) .. +3
+#pragma unroll
+  for (int i = 0; i < WM; ++i) {
+    const uint32_t row = m0 + wm * 128 + i * 16 + lrow;
+    if (row < p.M) {
+#pragma unroll
+      for (int t = 0; t < WN; ++t) {
+        const uint32_t ncol = n_wave + t * 16 + 4 * lq;
+        if (ncol < p.N) {
+          if (p.splits == 1) {
+            u32x2 o;
+            o.x = pack2(TO::from_float(acc[t][i][0]), TO::from_float(acc[t][i][1]));
+            o.y = pack2(TO::from_float(acc[t][i][2]), TO::from_float(acc[t][i][3]));
+            *reinterpret_cast<u32x2*>(static_cast<uint16_t*>(p.out) + static_cast<size_t>(row) * p.N + ncol) = o;
+          } else {
+            float* dst = p.partial + (static_cast<size_t>(split) * p.M + row) * p.N + ncol;
+            *reinterpret_cast<f32x4*>(dst) = acc[t][i];
+          }
+        }
+      }
+    }
+  }
+}
+
+}  // namespace ksq

@@ -27,4 +27,9 @@ struct TilePlan {
 };
 TilePlan plan_mfma_tile(size_t m, size_t n, size_t k);
 
+// Blockwise FP8: rows of activations above which the 256 x 256 MFMA tile kernel replaces the split-K wavefront kernel,
+// and its grid (block_m is always 256; kt_per_split counts 128-deep k-blocks).
+bool use_fp8_tile(size_t m, size_t n, size_t k);
+TilePlan plan_fp8_tile(size_t m, size_t n, size_t k);
+
 }  // namespace ksq

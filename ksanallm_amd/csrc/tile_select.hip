@@ -71,6 +71,32 @@ TilePlan plan_mfma_tile(size_t m, size_t n, size_t k) {
   return t;
 }
 
+bool use_fp8_tile(size_t m, size_t n, size_t k) {
+  (void)n;
+  (void)k;
+  return m > 64;
+}
+
+TilePlan plan_fp8_tile(size_t m, size_t n, size_t k) {
+  TilePlan t{};
+  t.block_m = 256;
+  t.tiles_m = static_cast<unsigned>(div_up(m, 256));
+  t.tiles_n = static_cast<unsigned>(div_up(n, 256));
+  const unsigned kb = static_cast<unsigned>(k / 128);
+  const unsigned tiles = t.tiles_m * t.tiles_n;
+  unsigned want = 1;
+  if (tiles < static_cast<unsigned>(kNumCU) * 3 / 4) {
+    want = kNumCU / tiles;
+    const unsigned cap = kb / 4 ? kb / 4 : 1;
+    want = want < cap ? want : cap;
+    if (want < 1) want = 1;
+  }
+  t.kt_per_split = static_cast<unsigned>(div_up(kb, want));
+  t.splits = static_cast<unsigned>(div_up(kb, t.kt_per_split));
+  t.workspace_bytes = t.splits > 1 ? static_cast<size_t>(t.splits) * m * n * 4 : 0;
+  return t;
+}
+
 }  // namespace ksq
 
 using namespace ksq;
@@ -106,15 +132,30 @@ KSQ_EXPORT int ksq_select_tile(int kind, size_t m, size_t n, size_t k, int dtype
       d->grid = static_cast<int32_t>((n / 16 / c.nt) * div_up(m, 16 * c.mt));
       return KSQ_OK;
     }
-    case KSQ_KIND_FP8_BLOCKWISE:
-      d->kernel = KSQ_KERNEL_MFMA_TILE;
-      d->block_m = 16;
+    case KSQ_KIND_FP8_BLOCKWISE: {
+      if (use_fp8_tile(m, n, k)) {
+        const TilePlan t = plan_fp8_tile(m, n, k);
+        d->kernel = KSQ_KERNEL_MFMA_TILE;
+        d->block_m = 256;
+        d->block_n = 256;
+        d->block_k = 128;
+        d->waves = 8;
+        d->split_k = static_cast<int32_t>(t.splits);
+        d->grid = static_cast<int32_t>(t.tiles_m * t.tiles_n * t.splits);
+        return KSQ_OK;
+      }
+      // decode: 16 weight rows x (16|32|64) tokens per workgroup, the wavefronts split K between them
+      const int mt = m <= 16 ? 1 : (m <= 32 ? 2 : 4);
+      const int waves = (k / 128 >= 64 && mt < 4) ? 16 : 8;
+      d->kernel = KSQ_KERNEL_SPLITK_WAVE;
+      d->block_m = 16 * mt;
       d->block_n = 16;
       d->block_k = 128;
-      d->waves = 4;
-      d->split_k = 1;
-      d->grid = static_cast<int32_t>(div_up(m, 16) * div_up(n, 16));
+      d->waves = waves;
+      d->split_k = waves;
+      d->grid = static_cast<int32_t>(div_up(m, 16 * mt) * (n / 16));
       return KSQ_OK;
+    }
     default:
       return fail(KSQ_ERR_INVALID_ARGUMENT, "ksq_select_tile: unknown kind %d", kind);
   }

@@ -140,6 +140,12 @@ def fp8_blockwise_gemm(a_q, a_s, b, b_s, out_dtype=torch.bfloat16, out=None, wor
     n = b.shape[0]
     if out is None:
         out = torch.empty((m, n), dtype=out_dtype, device=a_q.device)
+    if workspace is None:
+        need = _lib.ksq_fp8_blockwise_workspace_size(m, n, k)
+        if need:
+            workspace = _WORKSPACES.get(a_q.device)
+            if workspace is None or workspace.numel() < need:
+                workspace = _WORKSPACES[a_q.device] = torch.empty(need, dtype=torch.uint8, device=a_q.device)
     ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
     _l.check(_lib.ksq_fp8_blockwise_gemm(_ptr(a_q), _ptr(a_s), _ptr(b), _ptr(b_s), _ptr(out), m, n, k, _dt(out),
                                          _ptr(workspace), ws_bytes, _stream()))

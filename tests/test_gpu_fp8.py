@@ -128,6 +128,26 @@ def test_blockwise_gemm(ops, oracle, m, n, k):
     H.check_gemm(out, ref, H.BF16, "fp8 m=%d n=%d k=%d" % (m, n, k))
 
 
+# prefill regime (256 x 256 MFMA tile kernel): ragged M and N, odd k-block counts, split-K through the workspace
+@pytest.mark.parametrize("m,n,k", [(65, 256, 128), (300, 2320, 1152), (256, 7168, 2048), (1024, 512, 4096),
+                                   (130, 4096, 7168)])
+def test_blockwise_gemm_tile_kernel(ops, oracle, m, n, k):
+    from ksanallm_amd import lib as L
+    desc = L.select_tile(L.KIND_FP8_BLOCKWISE, m, n, k, H.BF16)
+    assert desc["kernel"] == 1
+    x, bq, bs = make_fp8_problem(oracle, 4400 + m + n, m, n, k)
+    q, s = ops.per_token_group_quant_fp8(x.cuda(), k, 128, True)
+    out = ops.fp8_blockwise_gemm(q, s, torch.from_numpy(bq).cuda(), torch.from_numpy(bs).cuda(), torch.bfloat16)
+    ref = oracle.fp8_blockwise_gemm(q.cpu().numpy(), s.cpu().numpy(), bq, bs, True)
+    H.check_gemm(out, ref, H.BF16, "fp8 tile m=%d n=%d k=%d split=%d" % (m, n, k, desc["split_k"]))
+    if desc["split_k"] > 1:
+        small = torch.empty(64, dtype=torch.uint8, device="cuda")
+        with pytest.raises(L.KsqError) as e:
+            ops.fp8_blockwise_gemm(q, s, torch.from_numpy(bq).cuda(), torch.from_numpy(bs).cuda(), torch.bfloat16,
+                                   workspace=small)
+        assert e.value.code == 3
+
+
 def test_blockwise_gemm_partial_scale_row_and_fp16_out(ops, oracle):
     m, n, k = 7, 208, 384  # n not a multiple of 128: the last scale row covers 80 weight rows
     x, bq, bs = make_fp8_problem(oracle, 4321, m, n, k, H.F16)
