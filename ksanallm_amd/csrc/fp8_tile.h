@@ -3,14 +3,15 @@
 //
 //   - both operands are e4m3 bytes, K-contiguous, and need no conversion, so both go global -> LDS without touching
 //     registers (global_load_lds_dwordx4), one 128-deep k-block (32 KiB of activations + 32 KiB of weights) per stage,
-//     two stages.  A 16-row x 128-byte MFMA operand is kept as a 2 KiB fragment in which lane L's 32 bytes sit at
-//     32*L: two loads of 64 contiguous bytes per row fill it, and a lane reads its operand back with two ds_read_b128.
+//     two stages.  A 16-row x 128-byte MFMA operand is kept as a 2 KiB fragment filled by two loads of 64 contiguous
+//     bytes per row, its 16-byte pieces swizzled so that a lane reads its operand back with two ds_read_b128 free of
+//     bank conflicts.
 //   - one v_mfma_f32_16x16x128_f8f6f4 covers exactly one scale block: its result goes to a scratch tile and is folded
 //     into the accumulator with a_s[kb, m] * b_s[n/128, kb] by four fp32 FMAs, issued under the following MFMA.
 //   - weights are the MFMA row operand, activations the column operand: a lane holds four consecutive output columns
 //     of one token (8-byte stores) and needs one activation scale per row tile.
-//   - loads are issued from inline assembly one stage ahead; a single `s_waitcnt vmcnt(0)` + barrier per stage makes
-//     the next stage visible and releases the LDS slot that was just consumed.
+//   - the loads of the next k-block are issued from inline assembly under the first MFMAs of a stage; a single
+//     `s_waitcnt vmcnt(0)` + barrier per stage makes them visible and releases the LDS slot that was just consumed.
 #pragma once
 
 #include "ksq_common.h"
@@ -73,9 +74,11 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
   const uint32_t kb_count = (KB - kb_begin) < p.kb_per_split ? (KB - kb_begin) : p.kb_per_split;
 
   // ---- operand staging.  Wavefronts 0..3 fetch the activation fragments 4w..4w+3, wavefronts 4..7 the weight
-  // fragments 4(w-4)..+3.  Load lane j supplies 16 bytes: row (j/2)%16, byte 64h + 32*((j/2)/16) + 16*(j%2) of the
-  // k-block, h = 0/1 being the instruction; it lands at fragment + 1024h + 16j, i.e. MFMA lane L = 32h + j/2 finds
-  // its 32 bytes at 32L.
+  // fragments 4(w-4)..+3.  A fragment (16 rows x 128 bytes) is two loads, one per 64-byte half h of the rows; in a
+  // load four consecutive lanes take the four 16-byte pieces of one row (64 contiguous bytes: the granularity at which
+  // the memory pipeline runs at full rate).  Load lane j lands at 1024h + 16j = 1024h + 64*(j/4) + 16*(j%4) and
+  // fetches piece (j%4) ^ (j/16) of row j/4, so that MFMA lane (row r, k slot q) finds its two pieces 2(q%2)+p at
+  // 1024*(q/2) + 64r + 16*((2(q%2)+p) ^ (r/4)): the sixteen lanes that read together hit different bank groups.
   const bool stage_act = wave < 4;
   const uint32_t frag0 = (wave & 3) * 4;
   const uint8_t* g_tile = stage_act ? p.a + static_cast<size_t>(m0) * p.K : p.b + static_cast<size_t>(n0) * p.K;
@@ -84,9 +87,9 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
   uint32_t d_voff[4];
 #pragma unroll
   for (int f = 0; f < 4; ++f) {
-    uint32_t row = (frag0 + f) * 16 + ((lane >> 1) & 15);
+    uint32_t row = (frag0 + f) * 16 + (lane >> 2);
     row = row < row_limit ? row : row_limit - 1;  // rows past the edge repeat the last row; their results are dropped
-    d_voff[f] = row * p.K + 32 * ((lane >> 5) & 1) + 16 * (lane & 1);
+    d_voff[f] = row * p.K + 16 * ((lane & 3) ^ (lane >> 4));
   }
   const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<size_t>((__attribute__((address_space(3))) char*)lds));
   const uint32_t d_lds = lds_base + ((stage_act ? 0 : W_FRAG0) + frag0) * FRAG;
@@ -173,21 +176,27 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
 #pragma unroll
     for (int i = 0; i < WM; ++i) acc[t][i] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+  const uint32_t rd_lo = 1024 * (lq >> 1) + 64 * lrow + 16 * ((2 * (lq & 1)) ^ (lrow >> 2));
+  const uint32_t rd_hi = rd_lo ^ 16;
   auto read_frag = [&](const char* base) {
-    const i32x4 lo = *reinterpret_cast<const i32x4*>(base);
-    const i32x4 hi = *reinterpret_cast<const i32x4*>(base + 16);
+    const i32x4 lo = *reinterpret_cast<const i32x4*>(base + rd_lo);
+    const i32x4 hi = *reinterpret_cast<const i32x4*>(base + rd_hi);
     return i32x8{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
   };
 
-  // one k-block: 32 MFMAs; the scale FMAs of MFMA j are placed after MFMA j+2 so that they run in its shadow
-  auto compute = [&](uint32_t slot, const float (&sc)[WM]) {
-    const char* act = lds + slot * STAGE_BYTES + (wm * WM) * FRAG + lane * 32;
-    const char* wgt = lds + slot * STAGE_BYTES + (W_FRAG0 + wn * WN) * FRAG + lane * 32;
+  // one k-block: 32 MFMAs; the scale FMAs of MFMA j are placed after MFMA j+2 so that they run in its shadow, and the
+  // loads of k-block `next` (scales, then operands into the LDS slot the previous stage used) are issued after the
+  // first and second row tile: a vector memory instruction takes several issue cycles, which are free there.
+  auto compute = [&](uint32_t slot, const float (&sc)[WM], uint32_t next) {
+    const char* act = lds + slot * STAGE_BYTES + (wm * WM) * FRAG;
+    const char* wgt = lds + slot * STAGE_BYTES + (W_FRAG0 + wn * WN) * FRAG;
     i32x8 wf[WN];
-#pragma unroll
-    for (int t = 0; t < WN; ++t) wf[t] = read_frag(wgt + t * FRAG);
     i32x8 af[2];
+    wf[0] = read_frag(wgt);
     af[0] = read_frag(act);
+#pragma unroll
+    for (int t = 1; t < WN; ++t) wf[t] = read_frag(wgt + t * FRAG);
+    __builtin_amdgcn_sched_barrier(0x4);
     f32x4 tmp[3];
     const f32x4 zero{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -197,6 +206,7 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
         if (t == 0 && i + 1 < WM) af[(i + 1) & 1] = read_frag(act + (i + 1) * FRAG);
         tmp[j % 3] = mfma_fp8_k128(wf[t], af[i & 1], zero);
       }
+      __builtin_amdgcn_sched_barrier(0x4);
       if (j >= 2) {  // the MFMA issued two places earlier has left the pipeline by now
         const int pi = (j - 2) / WN, pt = (j - 2) % WN;
         const f32x4 r = tmp[(j - 2) % 3];
@@ -204,12 +214,14 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
         for (int e = 0; e < 4; ++e) acc[pt][pi][e] = __builtin_fmaf(r[e], sc[pi], acc[pt][pi][e]);
       }
       __builtin_amdgcn_sched_barrier(0x4);  // keep MFMAs, FMAs and LDS reads in this order (scalar ALU may move)
+      if (j == WN - 1) load_scales(next);
+      if (j == 2 * WN - 1) load_operands(next);
     }
   };
 
-  // ---- schedule: stage c computes k-block c out of LDS slot c%2 while the operands of c+1 and its scales are in
-  // flight; at the end of the stage everything has to have landed (vmcnt(0)), the barrier makes it visible and tells
-  // every wavefront that slot c%2 is free, and the operands of c+2 are issued into it.
+  // ---- schedule: stage c computes k-block c out of LDS slot c%2 and, a quarter of the way in, issues the loads of
+  // k-block c+1 into the other slot (every wavefront left it at the previous barrier).  At the end of the stage they
+  // have to have landed (vmcnt(0)); the barrier makes them visible to all wavefronts.
   load_scales(0);
   load_operands(0);
   wait_all();
@@ -217,17 +229,13 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
   float sc[WM];
 #pragma unroll
   for (int i = 0; i < WM; ++i) sc[i] = as[i] * bs;
-  load_scales(1);
-  load_operands(1);
 
   for (uint32_t c = 0; c < kb_count; ++c) {
-    compute(c & 1, sc);
+    compute(c & 1, sc, c + 1);
     wait_all();  // operands and scales of c+1
     __builtin_amdgcn_s_barrier();
 #pragma unroll
     for (int i = 0; i < WM; ++i) sc[i] = as[i] * bs;
-    load_scales(c + 2);
-    load_operands(c + 2);
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // drain the clamped prefetches before the LDS is released
 

@@ -50,11 +50,12 @@ TilePlan plan_mfma_tile(size_t m, size_t n, size_t k) {
   const size_t rem = (m - 1) % 256;
   t.block_m = (m <= 128 || (m < 1024 && rem < 128)) ? 128 : 256;
   t.tiles_n = static_cast<unsigned>(div_up(n, 256));
-  // where 256-row tiles leave the grid under-filled but 128-row tiles fill it, take those (the weights are then fetched
+  // where 256-row tiles leave more than half of the CUs idle but 128-row tiles fill the grid, take those (the weights are then fetched
   // twice as often, out of the L2 / Infinity Cache) rather than split K: fp32 partial tiles cost 8 bytes of HBM
   // traffic per output element and split.  Where neither fills it, 256-row tiles with a deeper split measured faster.
   const unsigned fill = static_cast<unsigned>(kNumCU) * 3 / 4;
-  if (t.block_m == 256 && div_up(m, 256) * t.tiles_n < fill && div_up(m, 128) * t.tiles_n >= fill) t.block_m = 128;
+  if (t.block_m == 256 && div_up(m, 256) * t.tiles_n < static_cast<unsigned>(kNumCU) / 2 && div_up(m, 128) * t.tiles_n >= fill)
+    t.block_m = 128;
   t.tiles_m = static_cast<unsigned>(div_up(m, t.block_m));
   const unsigned kt = static_cast<unsigned>(k / 128);
   const unsigned tiles = t.tiles_m * t.tiles_n;

@@ -2,9 +2,9 @@
 // (BM = 256 or 128) over a contiguous range of k-tiles (split-K across workgroups when the grid would not fill the chip).
 //
 //   - x (activations) goes global -> LDS without touching registers: every wavefront issues global_load_lds_dwordx4
-//     for whole 1 KiB MFMA fragments (16 rows x 32 k; lane l supplies row l%16, k 8*(l/16)..+7 and lands at
-//     base + 16*l), into a ring of NS stages of 64 k each.  The fragment is read back with one conflict-free
-//     ds_read_b128 per lane, DEPTH fragments ahead of the MFMAs that use it.  Two to three stages are in flight
+//     for whole 1 KiB MFMA fragments (16 rows x 32 k, four lanes per row so that every load touches 64 contiguous
+//     bytes per row, pieces swizzled so that the read-back is free of bank conflicts), into a ring of NS stages of
+//     64 k each.  The fragment is read back with one ds_read_b128 per lane, DEPTH fragments ahead of the MFMAs that use it.  Two to three stages are in flight
 //     while one is consumed; the one barrier per stage sits in the middle of the stage, so the fragment reads never
 //     drain at a stage boundary.
 //   - packed int4 weights never touch LDS: the 8 wavefronts split the 256 columns (2 column tiles of 16 each), so
@@ -167,16 +167,22 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
   const uint32_t kt_count = (KT - kt_begin) < p.kt_per_split ? (KT - kt_begin) : p.kt_per_split;
   const uint32_t stages = kt_count * 2;
 
-  // ---- x staging: this wavefront fetches fragments f = wave*AP + 2j + {0,1}: row block f/2, k half f%2
+  // ---- x staging: this wavefront fetches fragments f = wave*AP + 2j + {0,1}: row block f/2, k half f%2.
+  // A fragment (16 rows x 32 k = 64 bytes per row) is fetched by ONE load in which four consecutive lanes take the
+  // four 16-byte pieces of one row - 64 contiguous bytes, the granularity at which the memory pipeline runs at full
+  // rate (16-byte pieces of four different rows run at a quarter of it).  Load lane j lands at 16*j = 64*(j/4) +
+  // 16*(j%4); it fetches piece (j%4) ^ (j/16) of row j/4, so that MFMA lane (row r, k piece q) finds its operand at
+  // 64*r + 16*(q ^ (r/4)): the sixteen lanes that read together (same q) then hit sixteen different bank groups.
   const char* x_tile = static_cast<const char*>(p.x) + (static_cast<size_t>(m0) * p.K + kt_begin * 128) * 2;
   uint32_t a_voff[AP / 2];
 #pragma unroll
   for (int j = 0; j < AP / 2; ++j) {
     const uint32_t rb = wave * (AP / 2) + j;
-    uint32_t row = rb * 16 + lrow;
+    uint32_t row = rb * 16 + (lane >> 2);
     row = (m0 + row < p.M) ? row : (p.M - 1 - m0);  // rows past M repeat the last row; their results are dropped
-    a_voff[j] = (row * p.K + lq * 8) * 2;
+    a_voff[j] = (row * p.K + 8 * ((lane & 3) ^ (lane >> 4))) * 2;
   }
+  const uint32_t a_rd = 64 * lrow + 16 * (lq ^ (lrow >> 2));  // this lane's operand inside a fragment
   const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<size_t>((__attribute__((address_space(3))) char*)lds));
   const uint32_t a_lds_wave = lds_base + wave * AP * 1024;
 
@@ -290,7 +296,7 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
   typename T::frag bcur[WN], bnext[WN];
   Dequant<T, HAS_ZP> dq[WN];
 
-  auto frag_ptr = [&](uint32_t slot, int ks) { return lds + slot * STAGE_BYTES + ks * 1024 + lane * 16; };
+  auto frag_ptr = [&](uint32_t slot, int ks) { return lds + slot * STAGE_BYTES + ks * 1024 + a_rd; };
   // `wn`/`dn`: weight slot and dword (32-k block of its k-tile) the NEXT step uses
   auto step = [&](uint32_t slot, int ks, WSlot (&wn)[WN], int dn) {
     const char* cur = frag_ptr(slot, ks);
