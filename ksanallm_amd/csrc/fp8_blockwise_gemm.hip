@@ -150,12 +150,15 @@ int dispatch(const Fp8Params& p, hipStream_t s) {
 
 template <typename TO>
 int launch_fp8_tile(const Fp8Params& q, const TilePlan& plan, float* partial, hipStream_t s) {
-  constexpr int kLds = 2 * 32 * 2048;
+  // two operand stages, two stages of activation scales, the weight scales of the k range
+  constexpr int kLdsMax = 160 * 1024;
+  const size_t lds = 2 * 32 * 2048 + 2 * 1024 + 2 * static_cast<size_t>(plan.kt_per_split) * 4;
+  if (lds > kLdsMax) return fail(KSQ_ERR_UNSUPPORTED, "k range of %u blocks per workgroup does not fit the LDS", plan.kt_per_split);
   static std::atomic<bool> configured{false};
   if (!configured.load(std::memory_order_acquire)) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&fp8_tile_kernel<TO>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
-    if (e != hipSuccess) return fail(KSQ_ERR_LAUNCH, "hipFuncSetAttribute(LDS %d): %s", kLds, hipGetErrorString(e));
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLdsMax);
+    if (e != hipSuccess) return fail(KSQ_ERR_LAUNCH, "hipFuncSetAttribute(LDS %d): %s", kLdsMax, hipGetErrorString(e));
     configured.store(true, std::memory_order_release);
   }
   Fp8TileParams p{};
@@ -172,7 +175,7 @@ int launch_fp8_tile(const Fp8Params& q, const TilePlan& plan, float* partial, hi
   p.tiles_n = plan.tiles_n;
   p.splits = plan.splits;
   p.kb_per_split = plan.kt_per_split;
-  fp8_tile_kernel<TO><<<plan.tiles_m * plan.tiles_n * plan.splits, 512, kLds, s>>>(p);
+  fp8_tile_kernel<TO><<<plan.tiles_m * plan.tiles_n * plan.splits, 512, lds, s>>>(p);
   if (plan.splits > 1) {
     const size_t mn = static_cast<size_t>(p.M) * p.N;
     splitk_reduce_kernel<TO><<<static_cast<unsigned>(div_up(mn, 256 * 8)), 256, 0, s>>>(partial, static_cast<uint16_t*>(p.out), mn,

@@ -8,6 +8,8 @@
 //     bank conflicts.
 //   - one v_mfma_f32_16x16x128_f8f6f4 covers exactly one scale block: its result goes to a scratch tile and is folded
 //     into the accumulator with a_s[kb, m] * b_s[n/128, kb] by four fp32 FMAs, issued under the following MFMA.
+//   - activation scales reach the lanes through LDS as well (one small LDS-targeted load per stage), the weight
+//     scales of the workgroup's k range are staged there once: no per-lane scale loads in the loop.
 //   - weights are the MFMA row operand, activations the column operand: a lane holds four consecutive output columns
 //     of one token (8-byte stores) and needs one activation scale per row tile.
 //   - the loads of the next k-block are issued from inline assembly under the first MFMAs of a stage; a single
@@ -94,47 +96,41 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
   const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<size_t>((__attribute__((address_space(3))) char*)lds));
   const uint32_t d_lds = lds_base + ((stage_act ? 0 : W_FRAG0) + frag0) * FRAG;
 
-  // ---- scales: one activation scale per row tile and lane (token = column l%16 of the MFMA result), one weight
-  // scale per wavefront and k-block (its 64 weight rows lie inside one 128-row scale block)
-  uint32_t s_voff[WM];
-#pragma unroll
-  for (int i = 0; i < WM; ++i) {
-    uint32_t row = m0 + wm * 128 + i * 16 + lrow;
-    row = row < p.M ? row : p.M - 1;
-    s_voff[i] = row * 4;
-  }
+  // ---- scales.  Activation scales of a k-block are 256 consecutive floats (a_s is token-contiguous): wavefronts 0..3
+  // copy 64 of them each into LDS with one 4-byte-per-lane LDS-targeted load per stage.  The weight scales of the
+  // workgroup's two 128-row scale blocks, for its whole k range, are copied into LDS once.  A lane needs one activation
+  // scale per row tile (token = column l%16 of the MFMA result) and one weight scale per k-block.
+  constexpr int SCALE_BASE = 2 * STAGE_BYTES;    // [2 slots][256] activation scales, then [2][kb_count] weight scales
+  constexpr int BS_BASE = SCALE_BASE + 2 * 1024;
+  uint32_t s_row = m0 + (wave & 3) * 64 + lane;
+  s_row = s_row < p.M ? s_row : p.M - 1;
+  const uint32_t s_voff = s_row * 4;
   const char* as_base = reinterpret_cast<const char*>(p.a_s) + static_cast<size_t>(kb_begin) * p.M * 4;
+  const uint32_t s_lds = lds_base + SCALE_BASE + (wave & 3) * 256;
   const uint32_t n_wave = n0 + wn * 64;
-  const uint32_t nblk = (n_wave < p.N ? n_wave : p.N - 1) / 128;
-  const char* bs_base = reinterpret_cast<const char*>(p.b_s + static_cast<size_t>(nblk) * KB + kb_begin);
-  const uint32_t zero_voff = 0;
-
-  float as[WM];
-  float bs;
+  {
+    const uint32_t nb_last = (p.N - 1) / 128;
+    for (uint32_t t = threadIdx.x; t < 2 * kb_count; t += 512) {
+      const uint32_t blk = t / kb_count, kb = t - blk * kb_count;
+      uint32_t nb = n0 / 128 + blk;
+      nb = nb < nb_last ? nb : nb_last;
+      reinterpret_cast<float*>(lds + BS_BASE)[t] = p.b_s[static_cast<size_t>(nb) * KB + kb_begin + kb];
+    }
+  }
+  const float* bs_lds = reinterpret_cast<const float*>(lds + BS_BASE) + (wn >> 1) * kb_count;
+  const float* as_lds = reinterpret_cast<const float*>(lds + SCALE_BASE) + wm * 128 + lrow;
 
   // Every group of loads is one assembly statement opening with `s_nop 4`: its scalar operands are in place before
   // it starts, and the wait states a vector memory instruction needs after a VALU write of a scalar register have
   // passed whatever produced them.
   auto load_scales = [&](uint32_t kb) {
-    kb = kb < kb_count ? kb : kb_count - 1;
-    const char* ap = as_base + static_cast<size_t>(kb) * p.M * 4;
-    const char* bp = bs_base + static_cast<size_t>(kb) * 4;
-    asm volatile(
-        "s_nop 4\n\t"
-        "global_load_dword %0, %9, %18\n\t"
-        "global_load_dword %1, %10, %18\n\t"
-        "global_load_dword %2, %11, %18\n\t"
-        "global_load_dword %3, %12, %18\n\t"
-        "global_load_dword %4, %13, %18\n\t"
-        "global_load_dword %5, %14, %18\n\t"
-        "global_load_dword %6, %15, %18\n\t"
-        "global_load_dword %7, %16, %18\n\t"
-        "global_load_dword %8, %17, %19"
-        : "=&v"(as[0]), "=&v"(as[1]), "=&v"(as[2]), "=&v"(as[3]), "=&v"(as[4]), "=&v"(as[5]), "=&v"(as[6]), "=&v"(as[7]),
-          "=&v"(bs)
-        : "v"(s_voff[0]), "v"(s_voff[1]), "v"(s_voff[2]), "v"(s_voff[3]), "v"(s_voff[4]), "v"(s_voff[5]), "v"(s_voff[6]),
-          "v"(s_voff[7]), "v"(zero_voff), "s"(ap), "s"(bp)
-        : "memory");
+    if (wave < 4) {
+      const uint32_t k = kb < kb_count ? kb : kb_count - 1;
+      const char* ap = as_base + static_cast<size_t>(k) * p.M * 4;
+      const uint32_t d = __builtin_amdgcn_readfirstlane(s_lds + (kb & 1) * 1024);
+      asm volatile("s_nop 4\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, %2" ::"v"(s_voff), "s"(d), "s"(ap)
+                   : "memory");
+    }
   };
   // operands of k-block `kb` -> LDS slot kb % 2.  The instruction offset of an LDS-targeted load is added to the LDS
   // address as well as to the global one: the second half's 64-byte global offset is taken out of its LDS base.
@@ -161,14 +157,8 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
           "s"(f2), "s"(f2h), "s"(f3), "s"(f3h), "s"(src)
         : "memory");
   };
-  // everything issued so far has landed; the scale registers become valid with this wait and are tied to it
-  auto wait_all = [&]() {
-    asm volatile("s_waitcnt vmcnt(0)"
-                 : "+v"(as[0]), "+v"(as[1]), "+v"(as[2]), "+v"(as[3]), "+v"(as[4]), "+v"(as[5]), "+v"(as[6]), "+v"(as[7]),
-                   "+v"(bs)
-                 :
-                 : "memory");
-  };
+  // everything this wavefront issued so far has landed
+  auto wait_all = [&]() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
 
   f32x4 acc[WN][WM];
 #pragma unroll
@@ -187,7 +177,13 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
   // one k-block: 32 MFMAs; the scale FMAs of MFMA j are placed after MFMA j+2 so that they run in its shadow, and the
   // loads of k-block `next` (scales, then operands into the LDS slot the previous stage used) are issued after the
   // first and second row tile: a vector memory instruction takes several issue cycles, which are free there.
-  auto compute = [&](uint32_t slot, const float (&sc)[WM], uint32_t next) {
+  auto compute = [&](uint32_t slot, uint32_t kb, uint32_t next) {
+    float sc[WM];
+    {
+      const float bs = bs_lds[kb];
+#pragma unroll
+      for (int i = 0; i < WM; ++i) sc[i] = as_lds[slot * 256 + i * 16] * bs;
+    }
     const char* act = lds + slot * STAGE_BYTES + (wm * WM) * FRAG;
     const char* wgt = lds + slot * STAGE_BYTES + (W_FRAG0 + wn * WN) * FRAG;
     i32x8 wf[WN];
@@ -225,17 +221,12 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
   load_scales(0);
   load_operands(0);
   wait_all();
-  __builtin_amdgcn_s_barrier();
-  float sc[WM];
-#pragma unroll
-  for (int i = 0; i < WM; ++i) sc[i] = as[i] * bs;
+  __syncthreads();  // also publishes the weight-scale table written with ordinary stores above
 
   for (uint32_t c = 0; c < kb_count; ++c) {
-    compute(c & 1, sc, c + 1);
+    compute(c & 1, c, c + 1);
     wait_all();  // operands and scales of c+1
     __builtin_amdgcn_s_barrier();
-#pragma unroll
-    for (int i = 0; i < WM; ++i) sc[i] = as[i] * bs;
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // drain the clamped prefetches before the LDS is released
 
