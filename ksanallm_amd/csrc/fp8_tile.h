@@ -102,11 +102,15 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
   // scale per row tile (token = column l%16 of the MFMA result) and one weight scale per k-block.
   constexpr int SCALE_BASE = 2 * STAGE_BYTES;    // [2 slots][256] activation scales, then [2][kb_count] weight scales
   constexpr int BS_BASE = SCALE_BASE + 2 * 1024;
-  uint32_t s_row = m0 + (wave & 3) * 64 + lane;
-  s_row = s_row < p.M ? s_row : p.M - 1;
+  // M % 4 == 0: wavefront 0 copies all 256 with one 16-byte-per-lane load (lanes whose four tokens lie past M repeat
+  // the last four).  Otherwise wavefronts 0..3 copy 64 each, 4 bytes per lane, every lane clamped on its own.
+  const bool s_vec = (p.M & 3) == 0;
+  uint32_t s_row = s_vec ? m0 + 4 * lane : m0 + (wave & 3) * 64 + lane;
+  const uint32_t s_last = s_vec ? p.M - 4 : p.M - 1;
+  s_row = s_row < s_last ? s_row : s_last;
   const uint32_t s_voff = s_row * 4;
   const char* as_base = reinterpret_cast<const char*>(p.a_s) + static_cast<size_t>(kb_begin) * p.M * 4;
-  const uint32_t s_lds = lds_base + SCALE_BASE + (wave & 3) * 256;
+  const uint32_t s_lds = lds_base + SCALE_BASE + (s_vec ? 0 : (wave & 3) * 256);
   const uint32_t n_wave = n0 + wn * 64;
   {
     const uint32_t nb_last = (p.N - 1) / 128;
@@ -124,10 +128,14 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
   // it starts, and the wait states a vector memory instruction needs after a VALU write of a scalar register have
   // passed whatever produced them.
   auto load_scales = [&](uint32_t kb) {
-    if (wave < 4) {
-      const uint32_t k = kb < kb_count ? kb : kb_count - 1;
-      const char* ap = as_base + static_cast<size_t>(k) * p.M * 4;
-      const uint32_t d = __builtin_amdgcn_readfirstlane(s_lds + (kb & 1) * 1024);
+    const uint32_t k = kb < kb_count ? kb : kb_count - 1;
+    const char* ap = as_base + static_cast<size_t>(k) * p.M * 4;
+    const uint32_t d = __builtin_amdgcn_readfirstlane(s_lds + (kb & 1) * 1024);
+    if (s_vec) {
+      if (wave == 0)
+        asm volatile("s_nop 4\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %2" ::"v"(s_voff), "s"(d), "s"(ap)
+                     : "memory");
+    } else if (wave < 4) {
       asm volatile("s_nop 4\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, %2" ::"v"(s_voff), "s"(d), "s"(ap)
                    : "memory");
     }
@@ -176,7 +184,7 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
 
   // one k-block: 32 MFMAs; the scale FMAs of MFMA j are placed after MFMA j+2 so that they run in its shadow, and the
   // loads of k-block `next` (scales, then operands into the LDS slot the previous stage used) are issued after the
-  // first and second row tile: a vector memory instruction takes several issue cycles, which are free there.
+  // first MFMA.
   auto compute = [&](uint32_t slot, uint32_t kb, uint32_t next) {
     float sc[WM];
     {
@@ -210,8 +218,10 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
         for (int e = 0; e < 4; ++e) acc[pt][pi][e] = __builtin_fmaf(r[e], sc[pi], acc[pt][pi][e]);
       }
       __builtin_amdgcn_sched_barrier(0x4);  // keep MFMAs, FMAs and LDS reads in this order (scalar ALU may move)
-      if (j == WN - 1) load_scales(next);
-      if (j == 2 * WN - 1) load_operands(next);
+      if (j == 0) {  // right behind the first MFMA: the longest flight time the two LDS stages allow
+        load_scales(next);
+        load_operands(next);
+      }
     }
   };
 
@@ -220,7 +230,7 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
   // have to have landed (vmcnt(0)); the barrier makes them visible to all wavefronts.
   load_scales(0);
   load_operands(0);
-  wait_all();
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();  // also publishes the weight-scale table written with ordinary stores above
 
   for (uint32_t c = 0; c < kb_count; ++c) {
