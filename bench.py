@@ -31,7 +31,19 @@ CACHE_BYTES = 320 << 20                            # rotate through more than th
 # WRITE_SIZE (KiB per dispatch), each scaled by the factor the same counter shows for a 256 MiB device copy
 # (`--calibrate-copy`): FETCH_SIZE reads half the bytes moved (x2.0), WRITE_SIZE reads them exactly (x1.0).
 # Keyed by (config, kernel variant); None where no counter run has been made for the current kernel.
-MEASURED_TRAFFIC = {}
+MEASURED_TRAFFIC = {
+    (2, "w4a16_splitk_kernel<16x16,w4>"): 31874075,
+    (2, "w4a16_splitk_kernel<16x64,w4>"): 31246449,
+    (2, "w4a16_splitk_kernel<32x16,w4>"): 38395318,
+    (2, "w4a16_splitk_kernel<32x64,w4>"): 33821620,
+    (2, "w4a16_tile_kernel<128x256,w8>"): 84562638,
+    (2, "w4a16_tile_kernel<256x256,w8>"): 221588892,
+    (3, "w4a16_tile_kernel<256x256,w8>"): 1246797628,
+    (4, "fp8_group_quant"): 27623708,
+    (4, "fp8_splitk_kernel<16x16,w16>"): 134519524,
+    (4, "fp8_splitk_kernel<16x16,w8>"): 134076218,
+    (4, "fp8_tile_kernel<256x256,w8>"): 261946688,
+}
 
 
 def seeded(cfg, idx):
@@ -137,15 +149,21 @@ def fp8_cases(ops, L, cfg, shapes, Ms):
             def quant(x=x, a_q=a_q, a_s=a_s, K=K):
                 ops.per_token_group_quant_fp8(x, K, 128, True, False, q=a_q, s=a_s)
 
-            def gemm(a_q=a_q, a_s=a_s, y=y, bs_=bs_, b_sd=b_sd, state=state, R=R):
+            need = L.load().ksq_fp8_blockwise_workspace_size(M, N, K)
+            ws = torch.empty(need, dtype=torch.uint8, device=dev) if need else None
+
+            def gemm(a_q=a_q, a_s=a_s, y=y, bs_=bs_, b_sd=b_sd, state=state, R=R, ws=ws):
                 i = state["i"] = (state["i"] + 1) % R
-                ops.fp8_blockwise_gemm(a_q, a_s, bs_[i], b_sd, out=y)
+                ops.fp8_blockwise_gemm(a_q, a_s, bs_[i], b_sd, out=y, workspace=ws)
 
             quant()
             cases.append(Case("%s:quant:M=%d" % (tag, M), quant, 0, 2 * M * K + M * K + 4 * M * K // 128, "fp8",
                               "fp8_group_quant"))
             nbytes = N * K + b_s.numel() * 4 + M * K + 4 * M * K // 128 + 2 * M * N
-            cases.append(Case("%s:gemm:M=%d" % (tag, M), gemm, 2 * M * N * K, nbytes, "fp8", "fp8_blockwise_gemm", R))
+            desc = L.select_tile(L.KIND_FP8_BLOCKWISE, M, N, K, L.BF16)
+            kern = "%s<%dx%d,w%d>" % ("fp8_splitk_kernel" if desc["kernel"] == 0 else "fp8_tile_kernel",
+                                      desc["block_m"], desc["block_n"], desc["waves"])
+            cases.append(Case("%s:gemm:M=%d" % (tag, M), gemm, 2 * M * N * K, nbytes, "fp8", kern, R))
     return cases, keep
 
 
