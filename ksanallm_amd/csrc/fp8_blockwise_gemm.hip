@@ -4,6 +4,8 @@
 // bytes k = 32*(l/16) .. +31 of row l%16.  Weights are the row operand, activations the column operand, so a lane's
 // four results are four consecutive output columns of one token.
 #include <atomic>
+#include <cstdio>
+#include <cstdlib>
 
 #include "fp8_tile.h"
 #include "ksq_common.h"
@@ -32,121 +34,144 @@ __device__ __forceinline__ i32x8 load32(const uint8_t* p) {
   return i32x8{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
 }
 
-// Decode regime: a workgroup owns 16 weight rows and MT*16 tokens; wavefront w takes the 128-wide k-blocks
-// w, w+WAVES, ...; partials are summed through LDS in wavefront order.
-template <typename TO, int MT, int WAVES>
+// Decode regime (HBM-bound): a workgroup owns 16 weight rows and MT*16 tokens; wavefront w takes the 128-wide
+// k-blocks w, w+WAVES, ... and keeps LOOK of them in flight (a ring of register stages, refilled in place right after
+// use; blocks past the end are clamped to the last one and given a zero scale, so that control flow stays uniform and
+// the compiler's wait counts stay exact).  Partials are summed through LDS in wavefront order.
+template <typename TO, int MT, int NT, int WAVES, int LOOK>
 __global__ void __launch_bounds__(WAVES * 64) fp8_splitk_kernel(Fp8Params p) {
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lrow = lane & 15;
   const int lq = lane >> 4;
   const uint32_t KB = p.K / 128;
-  const uint32_t n0 = blockIdx.x * 16;
+  const uint32_t n0 = blockIdx.x * (16 * NT);  // NT strips of 16 weight rows share every activation fragment
   const uint32_t m0 = blockIdx.y * (16 * MT);
 
-  __shared__ f32x4 red[WAVES][MT][64];
+  __shared__ f32x4 red[WAVES][NT][MT][64];
 
   const uint8_t* bptr = p.b + static_cast<size_t>(n0 + lrow) * p.K + lq * 32;
-  const float* bs = p.b_s + static_cast<size_t>(n0 / 128) * KB;
+  const float* bs = p.b_s + static_cast<size_t>(n0 / 128) * KB;  // 16*NT <= 128 rows: one scale block
   const uint8_t* aptr[MT];
-  uint32_t arow[MT];
-  bool ok[MT];
+  const float* asptr[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
-    arow[mt] = m0 + mt * 16 + lrow;
-    ok[mt] = arow[mt] < p.M;
-    aptr[mt] = p.a + static_cast<size_t>(ok[mt] ? arow[mt] : 0) * p.K + lq * 32;
+    uint32_t row = m0 + mt * 16 + lrow;
+    row = row < p.M ? row : p.M - 1;  // rows past M repeat the last token; their results are not stored
+    aptr[mt] = p.a + static_cast<size_t>(row) * p.K + lq * 32;
+    asptr[mt] = p.a_s + row;
   }
 
-  f32x4 acc[MT];
+  f32x4 acc[NT][MT];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   struct Stage {
-    i32x8 w;
-    i32x8 a[MT];
-    float sc[MT];
+    i32x4 w0[NT], w1[NT];
+    i32x4 a0[MT], a1[MT];
+    float as[MT];
+    float ws;
   };
+  Stage ring[LOOK];
   auto load_stage = [&](Stage& s, uint32_t kb) {
-    const i32x4* wp = reinterpret_cast<const i32x4*>(bptr + static_cast<size_t>(kb) * 128);
-    i32x4 lo = __builtin_nontemporal_load(wp), hi = __builtin_nontemporal_load(wp + 1);
-    s.w = i32x8{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-    const float wsc = bs[kb];
+    const bool live = kb < KB;
+    kb = live ? kb : KB - 1;
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const i32x4* wp = reinterpret_cast<const i32x4*>(bptr + static_cast<size_t>(nt) * 16 * p.K + static_cast<size_t>(kb) * 128);
+      s.w0[nt] = __builtin_nontemporal_load(wp);
+      s.w1[nt] = __builtin_nontemporal_load(wp + 1);
+    }
+    s.ws = live ? bs[kb] : 0.f;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-      if (ok[mt]) {
-        s.a[mt] = load32(aptr[mt] + static_cast<size_t>(kb) * 128);
-        s.sc[mt] = p.a_s[static_cast<size_t>(kb) * p.M + arow[mt]] * wsc;
-      } else {
-        s.a[mt] = i32x8{0, 0, 0, 0, 0, 0, 0, 0};
-        s.sc[mt] = 0.f;
-      }
+      const i32x4* ap = reinterpret_cast<const i32x4*>(aptr[mt] + static_cast<size_t>(kb) * 128);
+      s.a0[mt] = ap[0];
+      s.a1[mt] = ap[1];
+      s.as[mt] = asptr[mt][static_cast<size_t>(kb) * p.M];
     }
   };
   auto compute_stage = [&](const Stage& s) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-      f32x4 r = mfma_fp8_128(s.w, s.a[mt], f32x4{0.f, 0.f, 0.f, 0.f});
+      const i32x8 a{s.a0[mt].x, s.a0[mt].y, s.a0[mt].z, s.a0[mt].w, s.a1[mt].x, s.a1[mt].y, s.a1[mt].z, s.a1[mt].w};
+      const float sc = s.as[mt] * s.ws;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) acc[mt][i] += r[i] * s.sc[mt];
+      for (int nt = 0; nt < NT; ++nt) {
+        const i32x8 w{s.w0[nt].x, s.w0[nt].y, s.w0[nt].z, s.w0[nt].w, s.w1[nt].x, s.w1[nt].y, s.w1[nt].z, s.w1[nt].w};
+        const f32x4 r = mfma_fp8_128(w, a, f32x4{0.f, 0.f, 0.f, 0.f});
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[nt][mt][i] = __builtin_fmaf(r[i], sc, acc[nt][mt][i]);
+      }
     }
   };
 
-  uint32_t kb = wave;
-  if (kb < KB) {
-    Stage cur;
-    load_stage(cur, kb);
-    for (;;) {
-      uint32_t nk = kb + WAVES;
-      if (nk < KB) {
-        Stage nxt;
-        load_stage(nxt, nk);
-        compute_stage(cur);
-        cur = nxt;
-        kb = nk;
-      } else {
-        compute_stage(cur);
-        break;
-      }
+  const uint32_t rounds = (KB + WAVES - 1) / WAVES;  // k-blocks this wavefront may own
+#pragma unroll
+  for (int h = 0; h < LOOK; ++h) {
+    load_stage(ring[h], wave + h * WAVES);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  for (uint32_t it = 0; it < rounds; it += LOOK) {
+#pragma unroll
+    for (int h = 0; h < LOOK; ++h) {
+      compute_stage(ring[h]);
+      __builtin_amdgcn_sched_barrier(0);
+      load_stage(ring[h], wave + (it + h + LOOK) * WAVES);
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
 
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) red[wave][mt][lane] = acc[mt];
-  __syncthreads();
-  for (int idx = threadIdx.x; idx < MT * 64; idx += WAVES * 64) {
-    const int l = idx & 63, mt = idx >> 6;
-    f32x4 v = red[0][mt][l];
+  for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-    for (int w = 1; w < WAVES; ++w) v += red[w][mt][l];
+    for (int mt = 0; mt < MT; ++mt) red[wave][nt][mt][lane] = acc[nt][mt];
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < NT * MT * 64; idx += WAVES * 64) {
+    const int l = idx & 63, mt = (idx >> 6) % MT, nt = (idx >> 6) / MT;
+    f32x4 v = red[0][nt][mt][l];
+#pragma unroll
+    for (int w = 1; w < WAVES; ++w) v += red[w][nt][mt][l];
     const uint32_t row = m0 + mt * 16 + (l & 15);
     if (row < p.M) {
       u32x2 o;
       o.x = pack2(TO::from_float(v[0]), TO::from_float(v[1]));
       o.y = pack2(TO::from_float(v[2]), TO::from_float(v[3]));
-      uint16_t* yp = static_cast<uint16_t*>(p.out) + static_cast<size_t>(row) * p.N + n0 + 4 * (l >> 4);
+      uint16_t* yp = static_cast<uint16_t*>(p.out) + static_cast<size_t>(row) * p.N + n0 + nt * 16 + 4 * (l >> 4);
       *reinterpret_cast<u32x2*>(yp) = o;
     }
   }
 }
 
+template <typename TO, int MT, int NT, int WAVES, int LOOK>
+void launch_splitk(const Fp8Params& p, hipStream_t s) {
+  dim3 grid(p.N / (16 * NT), static_cast<unsigned>(div_up(p.M, 16 * MT)), 1);
+  fp8_splitk_kernel<TO, MT, NT, WAVES, LOOK><<<grid, WAVES * 64, 0, s>>>(p);
+}
+
 template <typename TO>
 int dispatch(const Fp8Params& p, hipStream_t s) {
-  const uint32_t KB = p.K / 128;
-  const int mt = p.M <= 16 ? 1 : (p.M <= 32 ? 2 : 4);
-  const bool w16 = KB >= 64 && mt < 4;
-  dim3 grid(p.N / 16, static_cast<unsigned>(div_up(p.M, 16 * mt)), 1);
-  if (mt == 1) {
-    if (w16) fp8_splitk_kernel<TO, 1, 16><<<grid, 1024, 0, s>>>(p);
-    else fp8_splitk_kernel<TO, 1, 8><<<grid, 512, 0, s>>>(p);
-  } else if (mt == 2) {
-    if (w16) fp8_splitk_kernel<TO, 2, 16><<<grid, 1024, 0, s>>>(p);
-    else fp8_splitk_kernel<TO, 2, 8><<<grid, 512, 0, s>>>(p);
-  } else {
-    fp8_splitk_kernel<TO, 4, 8><<<grid, 512, 0, s>>>(p);
-  }
-  return KSQ_OK;
+  const int mt = p.M <= 16 ? 1 : 2;
+  // Measured on MI355X: four wavefronts per workgroup with a shallow ring stream fastest (the grid already holds
+  // thousands of wavefronts; deeper rings only cost registers, i.e. resident wavefronts).
+  // the activation fragments are as large as the weight fragments: two strips share them once there are several
+  // tokens, or when K is the long dimension (few strips, long streams)
+  int nt = (p.M > 8 || p.K > p.N) ? 2 : 1;
+  if (p.N % (16 * nt) != 0) nt = 1;
+#define KSQ_CASE(MT_, NT_) \
+  if (mt == MT_ && nt == NT_) { launch_splitk<TO, MT_, NT_, 4, 2>(p, s); return KSQ_OK; }
+  KSQ_CASE(1, 1) KSQ_CASE(1, 2) KSQ_CASE(2, 1) KSQ_CASE(2, 2)
+#undef KSQ_CASE
+  return fail(KSQ_ERR_UNSUPPORTED, "no fp8 decode kernel for mt=%d nt=%d", mt, nt);
 }
+
+}  // namespace
+}  // namespace ksq
+
+namespace ksq {
+namespace {
 
 template <typename TO>
 int launch_fp8_tile(const Fp8Params& q, const TilePlan& plan, float* partial, hipStream_t s) {
@@ -193,7 +218,7 @@ KSQ_EXPORT size_t ksq_fp8_blockwise_workspace_size(size_t max_m, size_t n, size_
   // only the split-K form of the tile kernel needs scratch: fp32 partial tiles
   if (n == 0 || k == 0 || k % 128 != 0) return 0;
   size_t need = 0;
-  for (size_t m = 65; m <= max_m; ++m) {
+  for (size_t m = 33; m <= max_m; ++m) {
     const TilePlan t = plan_fp8_tile(m, n, k);
     if (t.splits == 1 && m % 256 == 0) break;  // the grid only grows from here on
     need = t.workspace_bytes > need ? t.workspace_bytes : need;

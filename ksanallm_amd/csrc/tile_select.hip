@@ -75,7 +75,7 @@ TilePlan plan_mfma_tile(size_t m, size_t n, size_t k) {
 bool use_fp8_tile(size_t m, size_t n, size_t k) {
   (void)n;
   (void)k;
-  return m > 64;
+  return m > 32;  // above two 16-token tiles the MFMA tile kernel (with split-K) measured faster than the streaming one
 }
 
 TilePlan plan_fp8_tile(size_t m, size_t n, size_t k) {
@@ -146,15 +146,16 @@ KSQ_EXPORT int ksq_select_tile(int kind, size_t m, size_t n, size_t k, int dtype
         return KSQ_OK;
       }
       // decode: 16 weight rows x (16|32|64) tokens per workgroup, the wavefronts split K between them
-      const int mt = m <= 16 ? 1 : (m <= 32 ? 2 : 4);
-      const int waves = (k / 128 >= 64 && mt < 4) ? 16 : 8;
+      const int mt = m <= 16 ? 1 : 2;
+      const int waves = 4;
       d->kernel = KSQ_KERNEL_SPLITK_WAVE;
+      const int nt = ((m > 8 || k > n) && n % 32 == 0) ? 2 : 1;
       d->block_m = 16 * mt;
-      d->block_n = 16;
+      d->block_n = 16 * nt;
       d->block_k = 128;
       d->waves = waves;
       d->split_k = waves;
-      d->grid = static_cast<int32_t>(div_up(m, 16 * mt) * (n / 16));
+      d->grid = static_cast<int32_t>(div_up(m, 16 * mt) * (n / (16 * nt)));
       return KSQ_OK;
     }
     default:
