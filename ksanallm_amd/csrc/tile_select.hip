@@ -102,6 +102,16 @@ TilePlan plan_fp8_tile(size_t m, size_t n, size_t k) {
 
 using namespace ksq;
 
+// Rows per expert block for numel routed (token, slot) pairs over E experts.  Replaces the M thresholds of
+// InvokeFusedMoe (16 / 32 / 64 rows by token count): below about 48 rows per expert the weights are streamed once per
+// 16- or 32-row block (HBM-bound); above, 128-row blocks feed the MFMA tile kernel.
+KSQ_EXPORT size_t ksq_moe_block_m(size_t numel, size_t E) {
+  if (E == 0) return 16;
+  const size_t per_expert = numel / E;
+  if (per_expert >= 48) return 128;
+  return per_expert < 16 ? 16 : 32;
+}
+
 KSQ_EXPORT int ksq_select_tile(int kind, size_t m, size_t n, size_t k, int dtype, ksq_tile_desc* d) {
   if (!d) return fail(KSQ_ERR_INVALID_ARGUMENT, "ksq_select_tile: null descriptor");
   if (m == 0 || n == 0 || k == 0) return fail(KSQ_ERR_INVALID_ARGUMENT, "ksq_select_tile: empty problem");

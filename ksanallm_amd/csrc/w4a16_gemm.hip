@@ -93,6 +93,21 @@ int launch_tile_zp(const TileParams& p, hipStream_t s) {
   return KSQ_OK;
 }
 
+// grouped (MoE) form: one 128-row block of the aligned permutation per row tile, no split-K
+template <typename T>
+int launch_tile_grouped(const TileParams& p, hipStream_t s) {
+  constexpr int kLds = 4 * 8 * 2 * 1024;
+  static std::atomic<bool> configured{false};
+  if (!configured.load(std::memory_order_acquire)) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&w4a16_tile_kernel<T, 8, false, true>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
+    if (e != hipSuccess) return fail(KSQ_ERR_LAUNCH, "hipFuncSetAttribute(LDS %d): %s", kLds, hipGetErrorString(e));
+    configured.store(true, std::memory_order_release);
+  }
+  w4a16_tile_kernel<T, 8, false, true><<<p.tiles_m * p.tiles_n, 512, kLds, s>>>(p);
+  return KSQ_OK;
+}
+
 template <typename T>
 int dispatch_mfma_tile(TileParams p, const TilePlan& plan, hipStream_t s) {
   p.tiles_m = plan.tiles_m;
@@ -210,10 +225,35 @@ KSQ_EXPORT int ksq_moe_w4a16_gemm(void* out, const void* x, const void* w_packed
   if (zeros_packed) return fail(KSQ_ERR_UNSUPPORTED, "%s: zero points are not supported for expert weights", fn);
   if (group != 128) return fail(KSQ_ERR_UNSUPPORTED, "%s: expert weights need group size 128", fn);
   if (top_k == 0 || E == 0) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: top_k and E must be positive", fn);
-  if (block_m != 16 && block_m != 32)
-    return fail(KSQ_ERR_UNSUPPORTED, "%s: block_m %zu not in {16,32}", fn, block_m);
+  if (block_m != 16 && block_m != 32 && block_m != 128)
+    return fail(KSQ_ERR_UNSUPPORTED, "%s: block_m %zu not in {16,32,128}", fn, block_m);
   if (numel == 0) return KSQ_OK;
   const size_t cap_blocks = (numel + E * (block_m - 1)) / block_m;  // upper bound on aligned blocks
+  if (block_m == 128) {  // prefill regime: MFMA tile kernel, rows gathered / scattered through the permutation
+    if (numel > 0x7fffffffull || (numel / top_k + 1) * k * 2 > 0xffffffffull)
+      return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: x too large", fn);
+    TileParams tp{};
+    tp.y = out;
+    tp.x = x;
+    tp.w = w_packed;
+    tp.scales = scales_packed;
+    tp.M = static_cast<uint32_t>(cap_blocks * 128);
+    tp.N = static_cast<uint32_t>(n);
+    tp.K = static_cast<uint32_t>(k);
+    tp.tiles_m = static_cast<uint32_t>(cap_blocks);
+    tp.tiles_n = static_cast<uint32_t>(div_up(n, 256));
+    tp.splits = 1;
+    tp.kt_per_split = static_cast<uint32_t>(k / 128);
+    tp.sorted_ids = static_cast<const int32_t*>(sorted_ids);
+    tp.expert_ids = static_cast<const int32_t*>(expert_ids);
+    tp.num_post_pad = static_cast<const int32_t*>(num_post_pad);
+    tp.topk_w = static_cast<const float*>(topk_w);
+    tp.numel = static_cast<uint32_t>(numel);
+    tp.top_k = static_cast<uint32_t>(top_k);
+    int rc = dtype == KSQ_F16 ? launch_tile_grouped<F16>(tp, as_stream(stream)) : launch_tile_grouped<BF16>(tp, as_stream(stream));
+    if (rc) return rc;
+    return check_launch(fn);
+  }
   if (cap_blocks > 65535) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: too many row blocks (%zu)", fn, cap_blocks);
   const size_t x_rows = (numel + top_k - 1) / top_k;
   if (x_rows * k * 2 >= 0x40000000ull) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: x too large", fn);

@@ -39,6 +39,12 @@ struct TileParams {
   uint32_t M, N, K;
   uint32_t tiles_m, tiles_n;
   uint32_t splits, kt_per_split;
+  // grouped (MoE) form: row block b = tile_m holds the rows sorted_ids[b*BM ..] of expert expert_ids[b]
+  const int32_t* sorted_ids;
+  const int32_t* expert_ids;
+  const int32_t* num_post_pad;
+  const float* topk_w;  // optional: multiplied into the output row of slot id s
+  uint32_t numel, top_k;
 };
 
 // dequantize one packed dword (8 codes) to 8 T values with (code - zp) * s applied
@@ -117,7 +123,11 @@ struct WSlot {
 };
 
 // 8 wavefronts side by side along N; each computes WM x 2 tiles of 16x16.  BM = 16*WM, BN = 256.
-template <typename T, int WM, bool HAS_ZP>
+// GROUPED: the MoE form.  Row block tile_m is one block of the aligned token permutation: its rows are gathered through
+// sorted_ids (slot id s reads x row s / top_k, pad slots carry s >= numel), its weights are those of expert
+// expert_ids[tile_m], its results are scattered to out[s, :] (times topk_w[s] when given).  Blocks past num_post_pad
+// leave at once.  There is no split-K in this form.
+template <typename T, int WM, bool HAS_ZP, bool GROUPED = false>
 __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
   constexpr int WAVES = 8;
   constexpr int WN = 2;
@@ -166,6 +176,11 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
   const uint32_t kt_begin = split * p.kt_per_split;
   const uint32_t kt_count = (KT - kt_begin) < p.kt_per_split ? (KT - kt_begin) : p.kt_per_split;
   const uint32_t stages = kt_count * 2;
+  uint32_t expert = 0;
+  if (GROUPED) {
+    if (m0 >= static_cast<uint32_t>(p.num_post_pad[0])) return;  // uniform: the whole workgroup leaves
+    expert = static_cast<uint32_t>(p.expert_ids[tile_m]);
+  }
 
   // ---- x staging: this wavefront fetches fragments f = wave*AP + 2j + {0,1}: row block f/2, k half f%2.
   // A fragment (16 rows x 32 k = 64 bytes per row) is fetched by ONE load in which four consecutive lanes take the
@@ -173,13 +188,19 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
   // rate (16-byte pieces of four different rows run at a quarter of it).  Load lane j lands at 16*j = 64*(j/4) +
   // 16*(j%4); it fetches piece (j%4) ^ (j/16) of row j/4, so that MFMA lane (row r, k piece q) finds its operand at
   // 64*r + 16*(q ^ (r/4)): the sixteen lanes that read together (same q) then hit sixteen different bank groups.
-  const char* x_tile = static_cast<const char*>(p.x) + (static_cast<size_t>(m0) * p.K + kt_begin * 128) * 2;
+  const char* x_tile = static_cast<const char*>(p.x) + (static_cast<size_t>(GROUPED ? 0 : m0) * p.K + kt_begin * 128) * 2;
   uint32_t a_voff[AP / 2];
 #pragma unroll
   for (int j = 0; j < AP / 2; ++j) {
     const uint32_t rb = wave * (AP / 2) + j;
     uint32_t row = rb * 16 + (lane >> 2);
-    row = (m0 + row < p.M) ? row : (p.M - 1 - m0);  // rows past M repeat the last row; their results are dropped
+    if (GROUPED) {
+      uint32_t sid = static_cast<uint32_t>(p.sorted_ids[m0 + row]);
+      sid = sid < p.numel ? sid : p.numel - 1;  // pad slots read some valid row; their results are dropped
+      row = sid / p.top_k;
+    } else {
+      row = (m0 + row < p.M) ? row : (p.M - 1 - m0);  // rows past M repeat the last row; their results are dropped
+    }
     a_voff[j] = (row * p.K + 8 * ((lane & 3) ^ (lane >> 4))) * 2;
   }
   const uint32_t a_rd = 64 * lrow + 16 * (lq ^ (lrow >> 2));  // this lane's operand inside a fragment
@@ -194,10 +215,10 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
   const char* z_base[WN];
 #pragma unroll
   for (int t = 0; t < WN; ++t) {
-    const uint32_t nt = (nt0 + t < n_tiles) ? nt0 + t : n_tiles - 1;
-    w_base[t] = static_cast<const char*>(p.w) + (static_cast<size_t>(nt) * KT + kt_begin) * 1024;
-    s_base[t] = static_cast<const char*>(p.scales) + (static_cast<size_t>(nt) * KT + kt_begin) * 32;
-    z_base[t] = HAS_ZP ? static_cast<const char*>(p.zeros) + (static_cast<size_t>(nt) * KT + kt_begin) * 16 : nullptr;
+    const size_t nt = static_cast<size_t>(expert) * n_tiles + ((nt0 + t < n_tiles) ? nt0 + t : n_tiles - 1);
+    w_base[t] = static_cast<const char*>(p.w) + (nt * KT + kt_begin) * 1024;
+    s_base[t] = static_cast<const char*>(p.scales) + (nt * KT + kt_begin) * 32;
+    z_base[t] = HAS_ZP ? static_cast<const char*>(p.zeros) + (nt * KT + kt_begin) * 16 : nullptr;
   }
   const uint32_t w_voff = lane * 16, s_voff = lrow * 2, z_voff = lrow;
 
@@ -376,16 +397,28 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
   // ---- store: lane holds row m = l%16 of the 16x16 tile and columns 4*(l/16) .. +3
 #pragma unroll
   for (int i = 0; i < WM; ++i) {
-    const uint32_t row = m0 + i * 16 + lrow;
-    if (row < p.M) {
+    uint32_t row = m0 + i * 16 + lrow;
+    bool live;
+    float rw = 1.0f;
+    if (GROUPED) {
+      const uint32_t sid = static_cast<uint32_t>(p.sorted_ids[row]);
+      live = sid < p.numel;
+      row = sid;
+      if (live && p.topk_w) rw = p.topk_w[sid];
+    } else {
+      live = row < p.M;
+    }
+    if (live) {
 #pragma unroll
       for (int t = 0; t < WN; ++t) {
         if (nt0 + t < n_tiles) {
           const size_t col = static_cast<size_t>(nt0 + t) * 16 + 4 * lq;
-          if (p.splits == 1) {
+          if (GROUPED || p.splits == 1) {
+            f32x4 v = acc[t][i];
+            if (GROUPED) v *= rw;
             u32x2 o;
-            o.x = pack2(T::from_float(acc[t][i][0]), T::from_float(acc[t][i][1]));
-            o.y = pack2(T::from_float(acc[t][i][2]), T::from_float(acc[t][i][3]));
+            o.x = pack2(T::from_float(v[0]), T::from_float(v[1]));
+            o.y = pack2(T::from_float(v[2]), T::from_float(v[3]));
             *reinterpret_cast<u32x2*>(static_cast<uint16_t*>(p.y) + static_cast<size_t>(row) * p.N + col) = o;
           } else {
             float* dst = p.partial + (static_cast<size_t>(split) * p.M + row) * p.N + col;

@@ -30,9 +30,9 @@ class MoeLayer : public BaseLayer {
   // output [0]: [tokens, hidden] T.
   Status Forward(const std::vector<Tensor>& input_tensors, std::vector<Tensor>& output_tensors) override;
 
-  // rows per expert block for a chunk of `tokens` tokens (InvokeFusedMoe picks 16 / 32 / 64 by the same thresholds;
-  // 64-row blocks run as two 32-row blocks here, which changes no result)
-  static size_t BlockM(size_t tokens) { return tokens <= 20 ? 16 : 32; }
+  // rows per expert block for a chunk (InvokeFusedMoe picks 16 / 32 / 64 by token count; here the library decides by
+  // rows per expert, which changes no result)
+  size_t BlockM(size_t tokens) const { return ksq_moe_block_m(tokens * expert_topk_, expert_num_per_node_); }
 
  private:
   static constexpr size_t kChunk = 32 * 1024;

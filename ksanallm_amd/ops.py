@@ -215,7 +215,7 @@ def fused_moe_w4a16(x, w13_packed, s13_packed, w2_packed, s2_packed, topk_ids, t
     T, topk = topk_ids.shape
     numel = T * topk
     if block_m is None:
-        block_m = 16 if numel // E < 16 else 32
+        block_m = _lib.ksq_moe_block_m(numel, E)
     sorted_ids, expert_ids, npp = moe_align_block_size(topk_ids, E, block_m)
     tw = topk_w.reshape(-1).to(torch.float32).contiguous()
     c1 = moe_w4a16_gemm(x, w13_packed, s13_packed, None, sorted_ids, expert_ids, npp, numel, topk, E, 2 * inter,

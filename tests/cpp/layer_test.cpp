@@ -273,7 +273,8 @@ static int RunErrors() {
     auto r = p;
     r[9] = uint32_t(8);
     expect(!c.Init(r, rc, context, 0).OK(), "grouped routing is rejected");
-    expect(MoeLayer::BlockM(20) == 16 && MoeLayer::BlockM(21) == 32, "block_m thresholds");
+    expect(ksq_moe_block_m(8 * 2, 8) == 16 && ksq_moe_block_m(64 * 2, 8) == 32 && ksq_moe_block_m(4096 * 8, 256) == 128,
+           "block_m thresholds");
   }
   std::printf(failures ? "layer errors: %d FAILED\n" : "layer errors: OK\n", failures);
   return failures ? 1 : 0;

@@ -52,7 +52,7 @@ def ulp(ref, dtype):
     return 2.0 ** (np.floor(np.log2(a)) - mant)
 
 
-def check_gemm(y_gpu, ref_f32, dtype, what="", weights_rounded=False):
+def check_gemm(y_gpu, ref_f32, dtype, what="", weights_rounded=False, rel_l2_max=5e-3):
     """rel-L2 <= 5e-3 and max-abs <= 2e-2 against the fp32-accumulated dequant reference.
 
     Two forms of the absolute bound are used and the raw maximum is returned for reporting:
@@ -71,7 +71,7 @@ def check_gemm(y_gpu, ref_f32, dtype, what="", weights_rounded=False):
     assert np.all(np.isfinite(y)), what
     rel_l2 = np.linalg.norm(y - ref) / max(np.linalg.norm(ref), 1e-30)
     err = np.abs(y - ref)
-    assert rel_l2 <= 5e-3, "%s rel-L2 %.3e" % (what, rel_l2)
+    assert rel_l2 <= rel_l2_max, "%s rel-L2 %.3e" % (what, rel_l2)
     norm = err.max() / max(1.0, np.abs(ref).max())
     assert norm <= 2e-2, "%s normalised max-abs %.3e (raw %.3e)" % (what, norm, err.max())
     if not weights_rounded:

@@ -74,7 +74,7 @@ def test_blockwise_layer(tmp_path, oracle, dtype, m, n, k, fuse):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("dtype,tokens,renorm,scaling", [(H.BF16, 1, 0, 2.5), (H.F16, 24, 1, 1.0), (H.BF16, 70, 0, 1.0)])
+@pytest.mark.parametrize("dtype,tokens,renorm,scaling", [(H.BF16, 1, 0, 2.5), (H.F16, 24, 1, 1.0), (H.BF16, 70, 0, 1.0), (H.BF16, 400, 0, 1.0)])
 def test_moe_layer(tmp_path, oracle, dtype, tokens, renorm, scaling):
     E, hidden, inter, topk = 16, 256, 128, 4
     g = H.gen(9200 + tokens)
@@ -92,4 +92,7 @@ def test_moe_layer(tmp_path, oracle, dtype, tokens, renorm, scaling):
     tw, ids = oracle.moe_topk_softmax(gating.numpy(), topk, bool(renorm), scaling, 2)
     ref = oracle.moe_forward(H.bits_of(x), w13.numpy(), H.bits_of(s13), w2.numpy(), H.bits_of(s2), ids, tw, 128, dtype)
     ref = oracle.from_bits(ref, dtype)
-    H.check_gemm(y, ref, dtype, "moe layer")
+    # from 48 rows per expert on both GEMMs run through the MFMA tile kernel, which rounds the dequantized weights to T:
+    # each GEMM on its own is held to 5e-3 (tests/test_gpu_moe.py), two in a row compound to sqrt(2) of that
+    rounded = tokens * topk // E >= 48
+    H.check_gemm(y, ref, dtype, "moe layer", weights_rounded=rounded, rel_l2_max=5e-3 * (2 ** 0.5 if rounded else 1.0))

@@ -100,7 +100,7 @@ def pack_moe(ops, d):
 
 
 @pytest.mark.parametrize("dtype", [H.F16, H.BF16])
-@pytest.mark.parametrize("T,bm", [(1, 16), (5, 16), (64, 16), (64, 32)])
+@pytest.mark.parametrize("T,bm", [(1, 16), (5, 16), (64, 16), (64, 32), (64, 128), (300, 128), (512, 128)])
 def test_grouped_gemm_stages(ops, oracle, dtype, T, bm):
     d = make_moe(oracle, 5000 + T, 16, 256, 128, T, 4, 128, dtype)
     w13p, s13p, w2p, s2p = pack_moe(ops, d)
@@ -110,16 +110,16 @@ def test_grouped_gemm_stages(ops, oracle, dtype, T, bm):
                             d["hidden"], 128, bm)
     ref1 = oracle.moe_w4a16_gemm(H.bits_of(d["x"]), d["w13"].numpy(), H.bits_of(d["s13"]), d["ids"].numpy(),
                                  d["tw"].numpy(), d["topk"], 128, False, dtype)
-    H.check_gemm(c1, ref1, dtype, "moe gemm1")
+    H.check_gemm(c1, ref1, dtype, "moe gemm1", weights_rounded=bm == 128)
     c2 = ops.silu_and_mul(c1)
     c3 = ops.moe_w4a16_gemm(c2, w2p, s2p, d["tw"].cuda().reshape(-1), s, e, npp, numel, 1, d["E"], d["hidden"],
                             d["inter"], 128, bm)
     ref3 = oracle.moe_w4a16_gemm(H.bits_of(c2.cpu()), d["w2"].numpy(), H.bits_of(d["s2"]), d["ids"].numpy(),
                                  d["tw"].numpy(), 1, 128, True, dtype)
-    H.check_gemm(c3, ref3, dtype, "moe gemm2")
+    H.check_gemm(c3, ref3, dtype, "moe gemm2", weights_rounded=bm == 128)
 
 
-@pytest.mark.parametrize("T", [1, 64])
+@pytest.mark.parametrize("T", [1, 64, 2048])
 def test_moe_block_deepseek_shape(ops, oracle, T):
     """256 experts, hidden 7168, inter 2048, top-8; weights for all experts are generated but only touched ones
     matter.  Scaled to 32 experts' worth of memory on the host by reusing expert slabs."""
@@ -142,4 +142,8 @@ def test_moe_block_deepseek_shape(ops, oracle, T):
     ref = oracle.from_bits(ref, H.BF16)
     # intermediate tensors are rounded to bf16 at three places in both implementations, so the end-to-end
     # comparison carries those roundings: rel-L2 stays the gate, the absolute bound is the GEMM one
-    H.check_gemm(out, ref, H.BF16, "moe block T=%d" % T)
+    # T = 2048 runs both GEMMs through the MFMA tile kernel, which rounds every dequantized weight to bf16 (each GEMM
+    # on its own is held to 5e-3 in test_grouped_gemm_stages); two such GEMMs in a row compound to sqrt(2) of that
+    rounded = T * topk // E >= 48
+    H.check_gemm(out, ref, H.BF16, "moe block T=%d" % T, weights_rounded=rounded,
+                 rel_l2_max=5e-3 * (2 ** 0.5 if rounded else 1.0))
