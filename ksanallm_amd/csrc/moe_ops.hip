@@ -79,6 +79,121 @@ __global__ void __launch_bounds__(kAlignThreads) moe_align_kernel(const int32_t*
   }
 }
 
+// ---- the same sort for many ids: two launches over `chunks` workgroups ---------------------------------------------
+constexpr int kChunkThreads = 256;
+constexpr uint32_t kMaxChunks = 128;
+
+// Launch 1: workgroup c counts its chunk's ids per expert into cnt[c][e]; all workgroups together fill `sorted` with
+// the padding value.
+__global__ void __launch_bounds__(kChunkThreads) moe_align_count_kernel(const int32_t* __restrict__ ids, uint32_t numel,
+                                                                        uint32_t E, uint32_t capacity,
+                                                                        int32_t* __restrict__ sorted,
+                                                                        int32_t* __restrict__ cnt, uint32_t per) {
+  extern __shared__ int32_t lds[];  // [E]
+  const uint32_t tid = threadIdx.x;
+  for (uint32_t e = tid; e < E; e += kChunkThreads) lds[e] = 0;
+  for (uint32_t i = blockIdx.x * kChunkThreads + tid; i < capacity; i += gridDim.x * kChunkThreads)
+    sorted[i] = static_cast<int32_t>(numel);
+  __syncthreads();
+  const uint32_t begin = blockIdx.x * per;
+  const uint32_t end = (begin + per < numel) ? begin + per : numel;
+  for (uint32_t i = begin + tid; i < end; i += kChunkThreads) {
+    uint32_t e = static_cast<uint32_t>(ids[i]);
+    if (e < E) atomicAdd(&lds[e], 1);
+  }
+  __syncthreads();
+  for (uint32_t e = tid; e < E; e += kChunkThreads) cnt[blockIdx.x * E + e] = lds[e];
+}
+
+// Launch 2: every workgroup sums the count table (ids of each expert before its chunk, and in total), scans the padded
+// totals over experts, and places its chunk's ids in rounds of 256: inside a round an id's rank is the number of equal
+// ids at lower positions, so the order inside an expert ascends with the flat index.  Workgroup 0 also writes
+// expert_ids and num_post_pad.
+__global__ void __launch_bounds__(kChunkThreads) moe_align_place_kernel(const int32_t* __restrict__ ids, uint32_t numel,
+                                                                        uint32_t E, uint32_t block_m,
+                                                                        int32_t* __restrict__ sorted,
+                                                                        int32_t* __restrict__ expert_ids,
+                                                                        int32_t* __restrict__ num_post_pad,
+                                                                        const int32_t* __restrict__ cnt, uint32_t chunks,
+                                                                        uint32_t per) {
+  extern __shared__ int32_t lds[];  // scan_a[E+1] scan_b[E+1] next[E] round[256]
+  const uint32_t tid = threadIdx.x;
+  const uint32_t EP = E + 1;
+  int32_t* scan_a = lds;
+  int32_t* scan_b = lds + EP;
+  int32_t* next = lds + 2 * EP;
+  int32_t* round = next + E;
+  const uint32_t c = blockIdx.x;
+  const int32_t bm = static_cast<int32_t>(block_m);
+
+  for (uint32_t e = tid; e < E; e += kChunkThreads) {
+    int32_t before = 0, total = 0;
+#pragma unroll 8
+    for (uint32_t c2 = 0; c2 < chunks; ++c2) {
+      int32_t v = cnt[c2 * E + e];
+      total += v;
+      before += (c2 < c) ? v : 0;
+    }
+    next[e] = before;
+    scan_a[e + 1] = (total + bm - 1) / bm * bm;
+  }
+  if (tid == 0) scan_a[0] = 0;
+  __syncthreads();
+  int32_t* src = scan_a;
+  int32_t* dst = scan_b;
+  for (uint32_t off = 1; off < EP; off <<= 1) {
+    for (uint32_t i = tid; i < EP; i += kChunkThreads) dst[i] = src[i] + (i >= off ? src[i - off] : 0);
+    __syncthreads();
+    int32_t* t = src;
+    src = dst;
+    dst = t;
+  }
+  const int32_t* first = src;
+  if (c == 0) {
+    if (tid == 0) num_post_pad[0] = first[E];
+    for (uint32_t e = tid; e < E; e += kChunkThreads)
+      for (int32_t s = first[e]; s < first[e + 1]; s += bm) expert_ids[s / bm] = static_cast<int32_t>(e);
+  }
+  for (uint32_t e = tid; e < E; e += kChunkThreads) next[e] += first[e];
+  __syncthreads();
+
+  const uint32_t begin = c * per;
+  const uint32_t end = (begin + per < numel) ? begin + per : numel;
+  for (uint32_t r0 = begin; r0 < end; r0 += kChunkThreads) {
+    const uint32_t i = r0 + tid;
+    uint32_t e = (i < end) ? static_cast<uint32_t>(ids[i]) : 0xffffffffu;
+    if (e >= E) e = 0xffffffffu;
+    round[tid] = static_cast<int32_t>(e);
+    __syncthreads();
+    int32_t pos = 0;
+    bool last = true;
+    if (e != 0xffffffffu) {
+      int32_t rank = 0;
+      for (uint32_t j = 0; j < kChunkThreads; ++j) {
+        const bool same = static_cast<uint32_t>(round[j]) == e;
+        rank += (same && j < tid) ? 1 : 0;
+        last = last && !(same && j > tid);
+      }
+      pos = next[e] + rank;
+      sorted[pos] = static_cast<int32_t>(i);
+    }
+    __syncthreads();
+    if (e != 0xffffffffu && last) next[e] = pos + 1;
+    __syncthreads();
+  }
+}
+
+void chunk_geometry(size_t numel, uint32_t* chunks, uint32_t* per) {
+  size_t c = div_up(numel, kChunkThreads);
+  if (c > kMaxChunks) c = kMaxChunks;
+  const size_t p = div_up(div_up(numel, c), kChunkThreads) * kChunkThreads;
+  *per = static_cast<uint32_t>(p);
+  *chunks = static_cast<uint32_t>(div_up(numel, p));
+}
+
+// ids from which the two-launch sort is used
+constexpr size_t kParallelAlignFrom = 2048;
+
 template <typename T>
 __global__ void __launch_bounds__(256) silu_mul_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ out,
                                                        size_t rows, uint32_t inter) {
@@ -225,7 +340,10 @@ KSQ_EXPORT size_t ksq_moe_align_capacity(size_t numel, size_t E, size_t block_m)
 KSQ_EXPORT size_t ksq_moe_align_scratch_bytes(size_t numel, size_t E) {
   uint32_t chunks, per;
   align_geometry(numel, &chunks, &per);
-  return (static_cast<size_t>(chunks) + 1) * E * sizeof(int32_t);
+  size_t bytes = (static_cast<size_t>(chunks) + 1) * E * sizeof(int32_t);
+  chunk_geometry(numel, &chunks, &per);
+  const size_t parallel = static_cast<size_t>(chunks) * E * sizeof(int32_t);
+  return bytes > parallel ? bytes : parallel;
 }
 
 KSQ_EXPORT int ksq_moe_align(const void* topk_ids, size_t numel, size_t E, size_t block_m, void* sorted_ids,
@@ -238,6 +356,17 @@ KSQ_EXPORT int ksq_moe_align(const void* topk_ids, size_t numel, size_t E, size_
   const size_t cap = ksq_moe_align_capacity(numel, E, block_m);
   if (cap > 0x7fffffffull) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: too many ids", fn);
   uint32_t chunks, per;
+  if (numel >= kParallelAlignFrom) {
+    chunk_geometry(numel, &chunks, &per);
+    moe_align_count_kernel<<<chunks, kChunkThreads, E * sizeof(int32_t), as_stream(stream)>>>(
+        static_cast<const int32_t*>(topk_ids), static_cast<uint32_t>(numel), static_cast<uint32_t>(E),
+        static_cast<uint32_t>(cap), static_cast<int32_t*>(sorted_ids), static_cast<int32_t*>(scratch), per);
+    moe_align_place_kernel<<<chunks, kChunkThreads, (3 * E + 2 + kChunkThreads) * sizeof(int32_t), as_stream(stream)>>>(
+        static_cast<const int32_t*>(topk_ids), static_cast<uint32_t>(numel), static_cast<uint32_t>(E),
+        static_cast<uint32_t>(block_m), static_cast<int32_t*>(sorted_ids), static_cast<int32_t*>(expert_ids),
+        static_cast<int32_t*>(num_post_pad), static_cast<const int32_t*>(scratch), chunks, per);
+    return check_launch(fn);
+  }
   align_geometry(numel, &chunks, &per);
   const size_t lds = 2 * (E + 1) * sizeof(int32_t);
   moe_align_kernel<<<1, kAlignThreads, lds, as_stream(stream)>>>(

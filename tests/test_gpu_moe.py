@@ -44,6 +44,19 @@ def test_align_out_of_range_ids_dropped(ops, oracle):
     np.testing.assert_array_equal(s.cpu().numpy(), so)
 
 
+@pytest.mark.parametrize("numel,E,bm", [(2048, 7, 128), (2049, 4096, 16), (33333, 300, 32), (70001, 1, 128)])
+def test_align_many_ids_ragged(ops, oracle, numel, E, bm):
+    # the sort over several workgroups: ragged chunk ends, ids outside [0, E), one expert, the largest expert count
+    g = H.gen(numel + E)
+    ids = torch.randint(-3, E + 3, (numel,), generator=g, dtype=torch.int32)
+    s, e, npp = ops.moe_align_block_size(ids.cuda(), E, bm)
+    so, eo, nppo = oracle.moe_align(ids.numpy(), E, bm)
+    assert npp.item() == nppo
+    np.testing.assert_array_equal(s.cpu().numpy(), so)
+    nb = nppo // bm
+    np.testing.assert_array_equal(e.cpu().numpy()[:nb], eo[:nb])
+
+
 @pytest.mark.parametrize("T,E,topk", [(1, 256, 8), (77, 256, 8), (5, 60, 4), (9, 1000, 6)])
 def test_topk_softmax(ops, oracle, T, E, topk):
     g = H.gen(T + E)
