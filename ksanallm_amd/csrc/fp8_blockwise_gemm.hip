@@ -177,8 +177,9 @@ template <typename TO>
 int launch_fp8_tile(const Fp8Params& q, const TilePlan& plan, float* partial, hipStream_t s) {
   // two operand stages, two stages of activation scales, the weight scales of the k range
   constexpr int kLdsMax = 160 * 1024;
-  const size_t lds = 2 * 32 * 2048 + 2 * 1024 + 2 * static_cast<size_t>(plan.kt_per_split) * 4;
-  if (lds > kLdsMax) return fail(KSQ_ERR_UNSUPPORTED, "k range of %u blocks per workgroup does not fit the LDS", plan.kt_per_split);
+  const size_t kb_max = (plan.main_items || plan.splits == 1) ? q.K / 128 : plan.kt_per_split;  // whole tiles span all of K
+  const size_t lds = 2 * 32 * 2048 + 2 * 1024 + 2 * kb_max * 4;
+  if (lds > kLdsMax) return fail(KSQ_ERR_UNSUPPORTED, "k range of %zu blocks per workgroup does not fit the LDS", kb_max);
   static std::atomic<bool> configured{false};
   if (!configured.load(std::memory_order_acquire)) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&fp8_tile_kernel<TO>),
@@ -198,13 +199,14 @@ int launch_fp8_tile(const Fp8Params& q, const TilePlan& plan, float* partial, hi
   p.K = q.K;
   p.tiles_m = plan.tiles_m;
   p.tiles_n = plan.tiles_n;
+  p.main_items = plan.main_items;
   p.splits = plan.splits;
   p.kb_per_split = plan.kt_per_split;
-  fp8_tile_kernel<TO><<<plan.tiles_m * plan.tiles_n * plan.splits, 512, lds, s>>>(p);
+  fp8_tile_kernel<TO><<<plan.grid, 512, lds, s>>>(p);
   if (plan.splits > 1) {
-    const size_t mn = static_cast<size_t>(p.M) * p.N;
-    splitk_reduce_kernel<TO><<<static_cast<unsigned>(div_up(mn, 256 * 8)), 256, 0, s>>>(partial, static_cast<uint16_t*>(p.out), mn,
-                                                                                   plan.splits);
+    const unsigned cut = plan.tiles_m * plan.tiles_n - plan.main_items;
+    splitk_reduce_kernel<TO, 256><<<cut * 32, 256, 0, s>>>(partial, static_cast<uint16_t*>(p.out), p.M, p.N, p.tiles_m, p.tiles_n,
+                                                          p.main_items, p.splits);
   }
   return KSQ_OK;
 }
@@ -218,10 +220,12 @@ KSQ_EXPORT size_t ksq_fp8_blockwise_workspace_size(size_t max_m, size_t n, size_
   // only the split-K form of the tile kernel needs scratch: fp32 partial tiles
   if (n == 0 || k == 0 || k % 128 != 0) return 0;
   size_t need = 0;
-  for (size_t m = 33; m <= max_m; ++m) {
+  // the plan is the same for all m of a band of 256 rows
+  for (size_t band_end = 256; max_m > 32; band_end += 256) {
+    const size_t m = band_end < max_m ? band_end : max_m;
     const TilePlan t = plan_fp8_tile(m, n, k);
-    if (t.splits == 1 && m % 256 == 0) break;  // the grid only grows from here on
     need = t.workspace_bytes > need ? t.workspace_bytes : need;
+    if (m == max_m) break;
   }
   return need;
 }

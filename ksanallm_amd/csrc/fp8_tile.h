@@ -17,6 +17,7 @@
 #pragma once
 
 #include "ksq_common.h"
+#include "tile_work.h"
 
 namespace ksq {
 
@@ -26,10 +27,10 @@ struct Fp8TileParams {
   const uint8_t* b;   // [n, k]
   const float* b_s;   // [ceil(n/128), k/128]
   void* out;          // [m, n]
-  float* partial;     // [splits][m][n] fp32 when splits > 1
+  float* partial;     // [slot][part][256][256] fp32 tiles of the workgroups that compute a part of K
   uint32_t M, N, K;
   uint32_t tiles_m, tiles_n;
-  uint32_t splits, kb_per_split;
+  uint32_t main_items, splits, kb_per_split;  // tile_work.h
 };
 
 __device__ __forceinline__ f32x4 mfma_fp8_k128(i32x8 a, i32x8 b, f32x4 c) {
@@ -53,27 +54,15 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
   const int lrow = lane & 15, lq = lane >> 4;
   const uint32_t KB = p.K / 128;
 
-  // ---- work id: 32 consecutive items of one XCD form a block of 4 row tiles x 8 (column tile, k-split) pairs
-  constexpr uint32_t GN = 8;
-  const uint32_t cols = p.tiles_n * p.splits;
-  const uint32_t total = p.tiles_m * cols;
-  uint32_t lin = blockIdx.x;
-  {
-    const uint32_t per = total / 8, rem = total % 8;
-    const uint32_t xcd = lin % 8, local = lin / 8;
-    lin = xcd * per + (xcd < rem ? xcd : rem) + local;
-  }
-  const uint32_t band_items = p.tiles_m * GN;
-  const uint32_t band = lin / band_items;
-  const uint32_t c0 = band * GN;
-  const uint32_t width = (cols - c0) < GN ? (cols - c0) : GN;
-  const uint32_t within = lin - band * band_items;
-  const uint32_t tile_m = within / width;
-  const uint32_t col = c0 + within % width;
-  const uint32_t split = col % p.splits, tile_n = col / p.splits;
+  // ---- work id (tile_work.h): output tile and the part of K this workgroup computes
+  // (the divisions inside run on the vector unit: readfirstlane brings the wave-uniform results back to scalars)
+  const TileWork work = tile_work(blockIdx.x, p.tiles_m, p.tiles_n, p.main_items, p.splits);
+  const uint32_t tile_m = __builtin_amdgcn_readfirstlane(work.tile_m), tile_n = __builtin_amdgcn_readfirstlane(work.tile_n);
+  const uint32_t part = __builtin_amdgcn_readfirstlane(work.part), slot = __builtin_amdgcn_readfirstlane(work.slot);
+  const bool direct = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(work.direct)) != 0;
   const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
-  const uint32_t kb_begin = split * p.kb_per_split;
-  const uint32_t kb_count = (KB - kb_begin) < p.kb_per_split ? (KB - kb_begin) : p.kb_per_split;
+  const uint32_t kb_begin = direct ? 0 : part * p.kb_per_split;
+  const uint32_t kb_count = direct ? KB : ((KB - kb_begin) < p.kb_per_split ? (KB - kb_begin) : p.kb_per_split);
 
   // ---- operand staging.  Wavefronts 0..3 fetch the activation fragments 4w..4w+3, wavefronts 4..7 the weight
   // fragments 4(w-4)..+3.  A fragment (16 rows x 128 bytes) is two loads, one per 64-byte half h of the rows; in a
@@ -249,13 +238,13 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
       for (int t = 0; t < WN; ++t) {
         const uint32_t ncol = n_wave + t * 16 + 4 * lq;
         if (ncol < p.N) {
-          if (p.splits == 1) {
+          if (direct) {
             u32x2 o;
             o.x = pack2(TO::from_float(acc[t][i][0]), TO::from_float(acc[t][i][1]));
             o.y = pack2(TO::from_float(acc[t][i][2]), TO::from_float(acc[t][i][3]));
             *reinterpret_cast<u32x2*>(static_cast<uint16_t*>(p.out) + static_cast<size_t>(row) * p.N + ncol) = o;
           } else {
-            float* dst = p.partial + (static_cast<size_t>(split) * p.M + row) * p.N + ncol;
+            float* dst = p.partial + ((static_cast<size_t>(slot) * p.splits + part) * BM + (row - m0)) * BN + (ncol - n0);
             *reinterpret_cast<f32x4*>(dst) = acc[t][i];
           }
         }

@@ -2,27 +2,37 @@
 #pragma once
 
 #include "ksq_common.h"
+#include "tile_work.h"
 
 namespace ksq {
 
-// y[m, n] = T(sum over splits of partial[s, m, n]), 8 outputs per thread, summed in split order
-template <typename T>
+// Partial tiles lie as [slot][part][BM][256] fp32.  One workgroup sums 2048 consecutive elements (8 rows) of one slot,
+// 8 per thread, in part order, and writes the rows and columns that are inside the matrix.
+template <typename T, int BM>
 __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float* __restrict__ partial, uint16_t* __restrict__ y,
-                                                            size_t mn, uint32_t splits) {
-  const size_t i = (static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x) * 8;
-  if (i >= mn) return;
-  f32x4 a = *reinterpret_cast<const f32x4*>(partial + i);
-  f32x4 b = *reinterpret_cast<const f32x4*>(partial + i + 4);
+                                                            uint32_t M, uint32_t N, uint32_t tiles_m, uint32_t tiles_n,
+                                                            uint32_t main_items, uint32_t splits) {
+  constexpr uint32_t BN = 256;
+  constexpr uint32_t kBlocksPerTile = BM * BN / 2048;
+  const uint32_t slot = blockIdx.x / kBlocksPerTile;
+  const uint32_t e = (blockIdx.x % kBlocksPerTile) * 2048 + threadIdx.x * 8;
+  uint32_t tile_m, tile_n;
+  tile_of_slot(slot, tiles_m, tiles_n, main_items, &tile_m, &tile_n);
+  const uint32_t row = tile_m * BM + e / BN, col = tile_n * BN + e % BN;
+  if (row >= M || col >= N) return;
+  const float* src = partial + static_cast<size_t>(slot) * splits * (BM * BN) + e;
+  f32x4 a = *reinterpret_cast<const f32x4*>(src);
+  f32x4 b = *reinterpret_cast<const f32x4*>(src + 4);
   for (uint32_t s = 1; s < splits; ++s) {
-    a += *reinterpret_cast<const f32x4*>(partial + s * mn + i);
-    b += *reinterpret_cast<const f32x4*>(partial + s * mn + i + 4);
+    a += *reinterpret_cast<const f32x4*>(src + static_cast<size_t>(s) * (BM * BN));
+    b += *reinterpret_cast<const f32x4*>(src + static_cast<size_t>(s) * (BM * BN) + 4);
   }
   u32x4 o;
   o.x = pack2(T::from_float(a[0]), T::from_float(a[1]));
   o.y = pack2(T::from_float(a[2]), T::from_float(a[3]));
   o.z = pack2(T::from_float(b[0]), T::from_float(b[1]));
   o.w = pack2(T::from_float(b[2]), T::from_float(b[3]));
-  *reinterpret_cast<u32x4*>(y + i) = o;
+  *reinterpret_cast<u32x4*>(y + static_cast<size_t>(row) * N + col) = o;
 }
 
 }  // namespace ksq

@@ -18,11 +18,12 @@ SplitKChoice select_splitk_blocks(int mt, size_t m_blocks, size_t n, size_t k);
 // true when the MFMA tile kernel (prefill regime) serves the shape: m above the decode range and group 128
 bool use_mfma_tile(size_t m, size_t n, size_t k, size_t group);
 
-// Grid of the MFMA tile kernel: block_m x 256 output tiles, and a split of K over workgroups when the output tiles
-// alone would leave most of the 256 CUs idle.  splits > 1 needs splits*m*n fp32 of workspace.
+// Grid of the MFMA tile kernel: block_m x 256 output tiles; the first main_items tiles (in the order of tile_work.h)
+// are computed whole, the others in `splits` parts of kt_per_split k-steps whose fp32 partial tiles go through the
+// workspace.  main_items == 0 and splits > 1: every tile is cut (grids far smaller than the chip).
 struct TilePlan {
   int block_m;  // 128 or 256
-  unsigned tiles_m, tiles_n, splits, kt_per_split;
+  unsigned tiles_m, tiles_n, main_items, splits, kt_per_split, grid;
   size_t workspace_bytes;
 };
 TilePlan plan_mfma_tile(size_t m, size_t n, size_t k);

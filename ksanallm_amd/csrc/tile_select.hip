@@ -45,6 +45,47 @@ bool use_mfma_tile(size_t m, size_t n, size_t k, size_t group) {
 // 256-row tiles halve the weight traffic per output row, 128-row tiles waste less when m sits just above a multiple
 // of 256.  With fewer than 192 output tiles the k range is cut into up to 256/tiles pieces of at least 4 k-tiles (512 k)
 // each; the fp32 partial tiles are summed by a second, bandwidth-bound kernel.
+// How to spread `tiles` output tiles of `kt` k-steps over the CUs.  Costs are in k-steps of one workgroup:
+//   fixed    prologue + epilogue of a workgroup
+//   partial  storing an fp32 partial tile instead of the output tile (and reading it back in the reduction)
+//   reduce   launch of the reduction pass, plus per_unit for every partial tile it reads
+// Candidates: every tile whole (ceil(tiles/CUs) rounds), or the full rounds whole and the tiles of the last, partly
+// filled round cut into s parts of K.  A part is at least 4 k-steps and at most 512 partial tiles are written.
+struct SpreadCost {
+  double fixed, partial, reduce, per_unit;
+};
+
+void spread_tiles(unsigned tiles, unsigned kt, const SpreadCost& c, TilePlan* t) {
+  const unsigned cus = static_cast<unsigned>(kNumCU);
+  const unsigned full = tiles / cus * cus, rem = tiles - full;
+  double best = div_up(tiles, cus) * (kt + c.fixed);
+  t->main_items = 0;
+  t->splits = 1;
+  t->kt_per_split = kt;
+  if (rem == 0) return;
+  for (unsigned s = 2; s <= 16; ++s) {
+    const unsigned per = static_cast<unsigned>(div_up(kt, s));
+    if (per < 4) break;
+    if (div_up(kt, per) != s) continue;  // the same parts as a smaller s
+    const unsigned units = rem * s;
+    if (units > 512) break;
+    const double cost = (full / cus) * (kt + c.fixed) + div_up(units, cus) * (per + c.fixed + c.partial) + c.reduce + units * c.per_unit;
+    if (cost < best) {
+      best = cost;
+      t->main_items = full;
+      t->splits = s;
+      t->kt_per_split = per;
+    }
+  }
+}
+
+void finish_plan(TilePlan* t) {
+  const unsigned tiles = t->tiles_m * t->tiles_n;
+  const unsigned cut = t->splits > 1 ? tiles - t->main_items : 0;
+  t->grid = t->main_items + (tiles - t->main_items) * t->splits;
+  t->workspace_bytes = static_cast<size_t>(cut) * t->splits * t->block_m * 256 * sizeof(float);
+}
+
 TilePlan plan_mfma_tile(size_t m, size_t n, size_t k) {
   TilePlan t{};
   const size_t rem = (m - 1) % 256;
@@ -57,18 +98,9 @@ TilePlan plan_mfma_tile(size_t m, size_t n, size_t k) {
   if (t.block_m == 256 && div_up(m, 256) * t.tiles_n < static_cast<unsigned>(kNumCU) / 2 && div_up(m, 128) * t.tiles_n >= fill)
     t.block_m = 128;
   t.tiles_m = static_cast<unsigned>(div_up(m, t.block_m));
-  const unsigned kt = static_cast<unsigned>(k / 128);
-  const unsigned tiles = t.tiles_m * t.tiles_n;
-  unsigned want = 1;
-  if (tiles < fill) {
-    want = kNumCU / tiles;
-    const unsigned cap = kt / 4 ? kt / 4 : 1;
-    want = want < cap ? want : cap;
-    if (want < 1) want = 1;
-  }
-  t.kt_per_split = static_cast<unsigned>(div_up(kt, want));
-  t.splits = static_cast<unsigned>(div_up(kt, t.kt_per_split));
-  t.workspace_bytes = t.splits > 1 ? static_cast<size_t>(t.splits) * m * n * 4 : 0;
+  static const SpreadCost cost{3.0, 3.0, 2.0, 0.02};
+  spread_tiles(t.tiles_m * t.tiles_n, static_cast<unsigned>(k / 128), cost, &t);
+  finish_plan(&t);
   return t;
 }
 
@@ -83,18 +115,9 @@ TilePlan plan_fp8_tile(size_t m, size_t n, size_t k) {
   t.block_m = 256;
   t.tiles_m = static_cast<unsigned>(div_up(m, 256));
   t.tiles_n = static_cast<unsigned>(div_up(n, 256));
-  const unsigned kb = static_cast<unsigned>(k / 128);
-  const unsigned tiles = t.tiles_m * t.tiles_n;
-  unsigned want = 1;
-  if (tiles < static_cast<unsigned>(kNumCU) * 3 / 4) {
-    want = kNumCU / tiles;
-    const unsigned cap = kb / 4 ? kb / 4 : 1;
-    want = want < cap ? want : cap;
-    if (want < 1) want = 1;
-  }
-  t.kt_per_split = static_cast<unsigned>(div_up(kb, want));
-  t.splits = static_cast<unsigned>(div_up(kb, t.kt_per_split));
-  t.workspace_bytes = t.splits > 1 ? static_cast<size_t>(t.splits) * m * n * 4 : 0;
+  static const SpreadCost cost{8.0, 6.0, 4.0, 0.05};
+  spread_tiles(t.tiles_m * t.tiles_n, static_cast<unsigned>(k / 128), cost, &t);
+  finish_plan(&t);
   return t;
 }
 
@@ -130,7 +153,7 @@ KSQ_EXPORT int ksq_select_tile(int kind, size_t m, size_t n, size_t k, int dtype
         d->block_k = 64;
         d->waves = 8;
         d->split_k = static_cast<int32_t>(t.splits);
-        d->grid = static_cast<int32_t>(t.tiles_m * t.tiles_n * t.splits);
+        d->grid = static_cast<int32_t>(t.grid);
         return KSQ_OK;
       }
       SplitKChoice c = select_splitk(m, n, k);
@@ -152,7 +175,7 @@ KSQ_EXPORT int ksq_select_tile(int kind, size_t m, size_t n, size_t k, int dtype
         d->block_k = 128;
         d->waves = 8;
         d->split_k = static_cast<int32_t>(t.splits);
-        d->grid = static_cast<int32_t>(t.tiles_m * t.tiles_n * t.splits);
+        d->grid = static_cast<int32_t>(t.grid);
         return KSQ_OK;
       }
       // decode: 16 weight rows x (16|32|64) tokens per workgroup, the wavefronts split K between them

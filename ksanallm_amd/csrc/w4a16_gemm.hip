@@ -78,7 +78,7 @@ int dispatch_tile(SplitKParams& p, SplitKChoice c, uint32_t m_blocks, size_t gro
 }
 
 template <typename T, int WM, bool HAS_ZP>
-int launch_tile_zp(const TileParams& p, hipStream_t s) {
+int launch_tile_zp(const TileParams& p, unsigned grid, hipStream_t s) {
   constexpr int kLds = 4 * WM * 2 * 1024;  // NS stages of WM*2 fragments
   static std::atomic<bool> configured{false};
   if (!configured.load(std::memory_order_acquire)) {
@@ -88,7 +88,6 @@ int launch_tile_zp(const TileParams& p, hipStream_t s) {
     if (e != hipSuccess) return fail(KSQ_ERR_LAUNCH, "hipFuncSetAttribute(LDS %d): %s", kLds, hipGetErrorString(e));
     configured.store(true, std::memory_order_release);
   }
-  const unsigned grid = p.tiles_m * p.tiles_n * p.splits;
   w4a16_tile_kernel<T, WM, HAS_ZP><<<grid, 512, kLds, s>>>(p);
   return KSQ_OK;
 }
@@ -112,18 +111,22 @@ template <typename T>
 int dispatch_mfma_tile(TileParams p, const TilePlan& plan, hipStream_t s) {
   p.tiles_m = plan.tiles_m;
   p.tiles_n = plan.tiles_n;
+  p.main_items = plan.main_items;
   p.splits = plan.splits;
   p.kt_per_split = plan.kt_per_split;
   int rc;
   if (plan.block_m == 128)
-    rc = p.zeros ? launch_tile_zp<T, 8, true>(p, s) : launch_tile_zp<T, 8, false>(p, s);
+    rc = p.zeros ? launch_tile_zp<T, 8, true>(p, plan.grid, s) : launch_tile_zp<T, 8, false>(p, plan.grid, s);
   else
-    rc = p.zeros ? launch_tile_zp<T, 16, true>(p, s) : launch_tile_zp<T, 16, false>(p, s);
+    rc = p.zeros ? launch_tile_zp<T, 16, true>(p, plan.grid, s) : launch_tile_zp<T, 16, false>(p, plan.grid, s);
   if (rc) return rc;
   if (plan.splits > 1) {
-    const size_t mn = static_cast<size_t>(p.M) * p.N;
-    const unsigned blocks = static_cast<unsigned>(div_up(mn, 256 * 8));
-    splitk_reduce_kernel<T><<<blocks, 256, 0, s>>>(p.partial, static_cast<uint16_t*>(p.y), mn, plan.splits);
+    const unsigned cut = plan.tiles_m * plan.tiles_n - plan.main_items;
+    uint16_t* y = static_cast<uint16_t*>(p.y);
+    if (plan.block_m == 128)
+      splitk_reduce_kernel<T, 128><<<cut * 16, 256, 0, s>>>(p.partial, y, p.M, p.N, p.tiles_m, p.tiles_n, p.main_items, p.splits);
+    else
+      splitk_reduce_kernel<T, 256><<<cut * 32, 256, 0, s>>>(p.partial, y, p.M, p.N, p.tiles_m, p.tiles_n, p.main_items, p.splits);
   }
   return KSQ_OK;
 }
@@ -153,11 +156,14 @@ KSQ_EXPORT size_t ksq_w4a16_workspace_size(size_t max_m, size_t n, size_t k, siz
   // the decode kernel reduces inside a workgroup; only the split-K form of the tile kernel needs fp32 partials
   if (n == 0 || k == 0 || k % 128 != 0) return 0;
   size_t need = 0;
-  for (size_t m = 33; m <= max_m; ++m) {
-    if (!use_mfma_tile(m, n, k, group)) break;
-    const TilePlan t = plan_mfma_tile(m, n, k);
-    if (t.splits == 1 && m % 256 == 0 && m >= 1024) break;  // the grid only grows from here on
-    need = t.workspace_bytes > need ? t.workspace_bytes : need;
+  // the plan is the same for all m of a band of 128 rows
+  for (size_t band_end = 128; max_m > 32; band_end += 128) {
+    const size_t m = band_end < max_m ? band_end : max_m;
+    if (use_mfma_tile(m, n, k, group)) {
+      const TilePlan t = plan_mfma_tile(m, n, k);
+      need = t.workspace_bytes > need ? t.workspace_bytes : need;
+    }
+    if (m == max_m) break;
   }
   return need;
 }
@@ -242,6 +248,7 @@ KSQ_EXPORT int ksq_moe_w4a16_gemm(void* out, const void* x, const void* w_packed
     tp.K = static_cast<uint32_t>(k);
     tp.tiles_m = static_cast<uint32_t>(cap_blocks);
     tp.tiles_n = static_cast<uint32_t>(div_up(n, 256));
+    tp.main_items = 0;
     tp.splits = 1;
     tp.kt_per_split = static_cast<uint32_t>(k / 128);
     tp.sorted_ids = static_cast<const int32_t*>(sorted_ids);

@@ -25,6 +25,7 @@
 #include <type_traits>
 
 #include "ksq_common.h"
+#include "tile_work.h"
 #include "splitk_reduce.h"
 
 namespace ksq {
@@ -35,10 +36,10 @@ struct TileParams {
   const void* w;
   const void* scales;
   const void* zeros;
-  float* partial;  // [splits][M][N] fp32 when splits > 1
+  float* partial;  // [slot][part][BM][256] fp32 tiles of the workgroups that compute a part of K
   uint32_t M, N, K;
   uint32_t tiles_m, tiles_n;
-  uint32_t splits, kt_per_split;
+  uint32_t main_items, splits, kt_per_split;  // tile_work.h
   // grouped (MoE) form: row block b = tile_m holds the rows sorted_ids[b*BM ..] of expert expert_ids[b]
   const int32_t* sorted_ids;
   const int32_t* expert_ids;
@@ -151,30 +152,15 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
   const int lrow = lane & 15, lq = lane >> 4;
   const uint32_t KT = p.K / 128;
 
-  // ---- work id.  Workgroup b runs on XCD b%8 and the b/8-th of that XCD's workgroups start in order, 32 at a time
-  // (one per CU).  Every XCD gets a contiguous range of a linear tile order in which 32 consecutive items form a block
-  // of 4 row tiles x 8 (column tile, k-split) pairs: the workgroups that share an L2 at any moment read 4 activation
-  // tiles and 8 weight strips between them instead of 16 and 2, which cuts the traffic into the L2 by more than half.
-  constexpr uint32_t GN = 8;
-  const uint32_t cols = p.tiles_n * p.splits;
-  const uint32_t total = p.tiles_m * cols;
-  uint32_t lin = blockIdx.x;
-  {
-    const uint32_t per = total / 8, rem = total % 8;
-    const uint32_t xcd = lin % 8, local = lin / 8;
-    lin = xcd * per + (xcd < rem ? xcd : rem) + local;  // XCDs 0..rem-1 own per+1 items
-  }
-  const uint32_t band_items = p.tiles_m * GN;
-  const uint32_t band = lin / band_items;
-  const uint32_t c0 = band * GN;
-  const uint32_t width = (cols - c0) < GN ? (cols - c0) : GN;
-  const uint32_t within = lin - band * band_items;
-  const uint32_t tile_m = within / width;
-  const uint32_t col = c0 + within % width;
-  const uint32_t split = col % p.splits, tile_n = col / p.splits;
+  // ---- work id (tile_work.h): output tile and the part of K this workgroup computes
+  // (the divisions inside run on the vector unit: readfirstlane brings the wave-uniform results back to scalars)
+  const TileWork work = tile_work(blockIdx.x, p.tiles_m, p.tiles_n, p.main_items, p.splits);
+  const uint32_t tile_m = __builtin_amdgcn_readfirstlane(work.tile_m), tile_n = __builtin_amdgcn_readfirstlane(work.tile_n);
+  const uint32_t part = __builtin_amdgcn_readfirstlane(work.part), slot = __builtin_amdgcn_readfirstlane(work.slot);
+  const bool direct = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(work.direct)) != 0;
   const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
-  const uint32_t kt_begin = split * p.kt_per_split;
-  const uint32_t kt_count = (KT - kt_begin) < p.kt_per_split ? (KT - kt_begin) : p.kt_per_split;
+  const uint32_t kt_begin = direct ? 0 : part * p.kt_per_split;
+  const uint32_t kt_count = direct ? KT : ((KT - kt_begin) < p.kt_per_split ? (KT - kt_begin) : p.kt_per_split);
   const uint32_t stages = kt_count * 2;
   uint32_t expert = 0;
   if (GROUPED) {
@@ -413,7 +399,7 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
       for (int t = 0; t < WN; ++t) {
         if (nt0 + t < n_tiles) {
           const size_t col = static_cast<size_t>(nt0 + t) * 16 + 4 * lq;
-          if (GROUPED || p.splits == 1) {
+          if (GROUPED || direct) {
             f32x4 v = acc[t][i];
             if (GROUPED) v *= rw;
             u32x2 o;
@@ -421,7 +407,7 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
             o.y = pack2(T::from_float(v[2]), T::from_float(v[3]));
             *reinterpret_cast<u32x2*>(static_cast<uint16_t*>(p.y) + static_cast<size_t>(row) * p.N + col) = o;
           } else {
-            float* dst = p.partial + (static_cast<size_t>(split) * p.M + row) * p.N + col;
+            float* dst = p.partial + ((static_cast<size_t>(slot) * p.splits + part) * BM + (row - m0)) * BN + (col - n0);
             *reinterpret_cast<f32x4*>(dst) = acc[t][i];
           }
         }

@@ -148,6 +148,20 @@ def test_blockwise_gemm_tile_kernel(ops, oracle, m, n, k):
         assert e.value.code == 3
 
 
+# a little more than one round of tiles: the first 256 tiles are computed whole, the rest cut along K
+def test_blockwise_gemm_whole_and_cut_tiles(ops, oracle):
+    from ksanallm_amd import lib as L
+    m, n, k = 1030, 13328, 4096
+    desc = L.select_tile(L.KIND_FP8_BLOCKWISE, m, n, k, H.BF16)
+    tiles = 5 * 53
+    assert desc["kernel"] == 1 and desc["split_k"] > 1 and desc["grid"] == 256 + (tiles - 256) * desc["split_k"]
+    x, bq, bs = make_fp8_problem(oracle, 4500, m, n, k)
+    q, s = ops.per_token_group_quant_fp8(x.cuda(), k, 128, True)
+    out = ops.fp8_blockwise_gemm(q, s, torch.from_numpy(bq).cuda(), torch.from_numpy(bs).cuda(), torch.bfloat16)
+    ref = oracle.fp8_blockwise_gemm(q.cpu().numpy(), s.cpu().numpy(), bq, bs, True)
+    H.check_gemm(out, ref, H.BF16, "fp8 whole + cut tiles")
+
+
 def test_blockwise_gemm_partial_scale_row_and_fp16_out(ops, oracle):
     m, n, k = 7, 208, 384  # n not a multiple of 128: the last scale row covers 80 weight rows
     x, bq, bs = make_fp8_problem(oracle, 4321, m, n, k, H.F16)

@@ -80,6 +80,19 @@ def test_prefill_split_k(ops, dtype, M, N, K):
     assert e.value.code == 3
 
 
+# a little more than one round of tiles: the first 256 tiles are computed whole, the rest cut along K (ragged M and N)
+@pytest.mark.parametrize("dtype,awq", [(H.F16, False), (H.BF16, True)])
+def test_prefill_whole_and_cut_tiles(ops, dtype, awq):
+    from ksanallm_amd import lib as L
+    M, N, K = 1030, 13328, 2048
+    desc = L.select_tile(L.KIND_W4A16, M, N, K, dtype)
+    tiles = 5 * 53
+    assert desc["kernel"] == 1 and desc["split_k"] > 1 and desc["grid"] == 256 + (tiles - 256) * desc["split_k"]
+    d = H.make_w4a16(3300, M, N, K, 128, dtype, awq=awq, x_std=0.5, s_lo=0.002, s_hi=0.01, z_lo=0, z_hi=15)
+    y = run_case(ops, d)
+    H.check_gemm(y, H.w4a16_oracle(d), dtype, "whole + cut tiles", weights_rounded=True)
+
+
 # config 3 shape (Qwen-32B-like, GPTQ fp16) at a row count the CPU oracle finishes in seconds
 @pytest.mark.parametrize("N,K", [(25600, 5120), (5120, 25600)])
 def test_cfg3_gptq_fp16_prefill(ops, N, K):
