@@ -165,6 +165,24 @@ int ksq_moe_w4a16_gemm(void* out, const void* x, const void* w_packed, const voi
 int ksq_moe_topk_softmax(const void* gating, void* topk_w, void* topk_ids, size_t tokens, size_t E, size_t top_k,
                          int norm_topk_prob, float routed_scaling_factor, int dtype, void* stream);
 
+/* Grouped router (DeepSeek-V2/V3 style).  Per token, in fp32:
+ *   score  = softmax(gating) (KSQ_SCORE_SOFTMAX) or 1 / (1 + expf(-gating)) (KSQ_SCORE_SIGMOID)
+ *   choose = score + e_bias[expert] when e_bias (fp32 [E]) is given, else score
+ *   the E experts form num_expert_group equal groups; a group ranks by the sum of its two largest choose values
+ *   (e_bias given) or by its largest (e_bias NULL); the topk_group best groups are kept (ties: lower group first)
+ *   the top_k largest choose values among the kept groups select the experts (descending; ties: lower id first)
+ *   weight = score of the selected expert (never the biased value), / sum over the top_k when renormalize,
+ *   * routed_scaling_factor.
+ * num_expert_group = topk_group = 1 with e_bias NULL is plain top-k routing with either scoring function.
+ * E <= 1024 and a multiple of num_expert_group <= 64, top_k <= min(32, topk_group * E / num_expert_group).
+ * Replaces InvokeGroupedTopk (S/kernels/nvidia/moe_kernel_wrapper.cpp:264-347: the fused sigmoid + bias form and
+ * the general tensor-op form) and InvokeDeepSeekV3GroupedTopk (K/grouped_topk/grouped_topk.cu:507-665). */
+#define KSQ_SCORE_SOFTMAX 0
+#define KSQ_SCORE_SIGMOID 1
+int ksq_moe_grouped_topk(const void* gating, const void* e_bias, void* topk_w, void* topk_ids, size_t tokens, size_t E,
+                         size_t top_k, size_t num_expert_group, size_t topk_group, int scoring, int renormalize,
+                         float routed_scaling_factor, int dtype, void* stream);
+
 /* out[r, i] = T(silu(x[r, i]) * x[r, inter + i]), fp32 math a / (1 + expf(-a)) * b.
  * Replaces InvokeSiluAndMul (K/moe_utils/moe_utils.cu:893-905). */
 int ksq_moe_silu_mul(const void* x, void* out, size_t rows, size_t inter, int dtype, void* stream);

@@ -319,6 +319,143 @@ struct Load16 {
   static __device__ __forceinline__ float get(const void* p, size_t i) { return T::to_float(static_cast<const uint16_t*>(p)[i]); }
 };
 
+// Grouped routing (DeepSeek-V2/V3): one wavefront per token, lane l holds experts l, l+64, ... (at most 16 each).
+//   score   = softmax(gating) or sigmoid(gating), fp32
+//   choose  = score + bias (bias given) or score
+//   group g = experts [g*per_group, (g+1)*per_group): its rank value is the sum of its two largest choose values
+//             (bias given) or its largest one; the topk_group best groups stay, all other experts are out
+//   top_k rounds of wave arg-max over choose pick the experts (descending, the lower id wins ties); the routing
+//   weight of a pick is its score (without bias), divided by the sum of the picks when renormalize, times scaling.
+// Group rank values are built from the choose values staged in LDS (one row of E floats per wavefront).
+template <typename LOAD>
+__global__ void __launch_bounds__(256) grouped_topk_kernel(const void* __restrict__ gating, const float* __restrict__ bias,
+                                                           float* __restrict__ topk_w, int32_t* __restrict__ topk_ids,
+                                                           uint32_t tokens, uint32_t E, uint32_t top_k, uint32_t groups,
+                                                           uint32_t topk_group, int sigmoid, int renorm, float scaling) {
+  extern __shared__ float lds_choose[];  // [4][E]
+  const uint32_t wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const uint32_t token_raw = blockIdx.x * 4 + wave;
+  const bool active = token_raw < tokens;
+  const uint32_t token = active ? token_raw : tokens - 1;  // idle wavefronts repeat the last token and store nothing
+  const uint32_t per_group = E / groups;
+  float* choose_row = lds_choose + wave * E;
+
+  float score[16], choose[16];
+  float mx = -INFINITY;
+#pragma unroll
+  for (int j = 0; j < 16; ++j) {
+    const uint32_t e = j * 64 + lane;
+    score[j] = e < E ? LOAD::get(gating, static_cast<size_t>(token) * E + e) : -INFINITY;
+    mx = fmaxf(mx, score[j]);
+  }
+  if (sigmoid) {
+#pragma unroll
+    for (int j = 0; j < 16; ++j) score[j] = 1.0f / (1.0f + expf(-score[j]));
+  } else {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+    float sum = 0.f;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      const uint32_t e = j * 64 + lane;
+      score[j] = e < E ? expf(score[j] - mx) : 0.f;
+      sum += score[j];
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) sum += __shfl_xor(sum, off, 64);
+#pragma unroll
+    for (int j = 0; j < 16; ++j) score[j] = score[j] / sum;
+  }
+#pragma unroll
+  for (int j = 0; j < 16; ++j) {
+    const uint32_t e = j * 64 + lane;
+    choose[j] = e < E ? score[j] + (bias ? bias[e] : 0.f) : -INFINITY;
+    if (e < E) choose_row[e] = choose[j];
+  }
+  __syncthreads();
+
+  // rank value of group g = lane (groups <= 64)
+  float rank = -INFINITY;
+  if (static_cast<uint32_t>(lane) < groups) {
+    float m1 = -INFINITY, m2 = -INFINITY;
+    const float* g = choose_row + lane * per_group;
+    for (uint32_t i = 0; i < per_group; ++i) {
+      const float c = g[i];
+      if (c > m1) {
+        m2 = m1;
+        m1 = c;
+      } else if (c > m2) {
+        m2 = c;
+      }
+    }
+    rank = bias ? m1 + m2 : m1;
+  }
+  uint64_t kept = 0;
+  for (uint32_t r = 0; r < topk_group; ++r) {
+    float best = rank;
+    uint32_t best_g = static_cast<uint32_t>(lane) < groups ? lane : 0xffffffffu;
+    if ((kept >> lane) & 1) best_g = 0xffffffffu;  // taken: never wins
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+      const float ob = __shfl_xor(best, off, 64);
+      const uint32_t og = __shfl_xor(best_g, off, 64);
+      const bool mine = best_g != 0xffffffffu, theirs = og != 0xffffffffu;
+      if (theirs && (!mine || ob > best || (ob == best && og < best_g))) {
+        best = ob;
+        best_g = og;
+      }
+    }
+    if (best_g != 0xffffffffu) kept |= 1ull << best_g;
+  }
+  uint32_t taken = 0;  // bit j: expert j*64+lane is out (group not kept, past E, or already picked)
+#pragma unroll
+  for (int j = 0; j < 16; ++j) {
+    const uint32_t e = j * 64 + lane;
+    if (e >= E || !((kept >> (e / per_group)) & 1)) taken |= 1u << j;
+  }
+
+  float picked_sum = 0.f, my_w = 0.f;
+  int my_id = 0;
+  for (uint32_t r = 0; r < top_k; ++r) {
+    float best = 0.f, best_s = 0.f;
+    uint32_t best_e = 0xffffffffu;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      if (!((taken >> j) & 1) && (best_e == 0xffffffffu || choose[j] > best)) {  // ascending e: > keeps the lower id
+        best = choose[j];
+        best_s = score[j];
+        best_e = j * 64 + lane;
+      }
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+      const float ob = __shfl_xor(best, off, 64);
+      const float os = __shfl_xor(best_s, off, 64);
+      const uint32_t oe = __shfl_xor(best_e, off, 64);
+      const bool mine = best_e != 0xffffffffu, theirs = oe != 0xffffffffu;
+      if (theirs && (!mine || ob > best || (ob == best && oe < best_e))) {
+        best = ob;
+        best_s = os;
+        best_e = oe;
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 16; ++j)
+      if (static_cast<uint32_t>(j * 64 + lane) == best_e) taken |= 1u << j;
+    picked_sum += best_s;
+    if (static_cast<uint32_t>(lane) == r) {
+      my_w = best_s;
+      my_id = static_cast<int>(best_e);
+    }
+  }
+  if (active && static_cast<uint32_t>(lane) < top_k) {
+    const float w = renorm ? my_w / picked_sum : my_w;
+    topk_w[static_cast<size_t>(token) * top_k + lane] = w * scaling;
+    topk_ids[static_cast<size_t>(token) * top_k + lane] = my_id;
+  }
+}
+
 void align_geometry(size_t numel, uint32_t* chunks, uint32_t* per) {
   size_t c = div_up(numel, 8);
   if (c < 1) c = 1;
@@ -397,6 +534,46 @@ KSQ_EXPORT int ksq_moe_topk_softmax(const void* gating, void* topk_w, void* topk
     topk_softmax_kernel<Load16<F16>><<<blocks, 256, 0, st>>>(gating, w, ids, t, e, k, norm_topk_prob, routed_scaling_factor);
   else if (dtype == KSQ_BF16)
     topk_softmax_kernel<Load16<BF16>><<<blocks, 256, 0, st>>>(gating, w, ids, t, e, k, norm_topk_prob, routed_scaling_factor);
+  else
+    return fail(KSQ_ERR_UNSUPPORTED, "%s: unknown dtype %d", fn, dtype);
+  return check_launch(fn);
+}
+
+KSQ_EXPORT int ksq_moe_grouped_topk(const void* gating, const void* e_bias, void* topk_w, void* topk_ids, size_t tokens,
+                                    size_t E, size_t top_k, size_t num_expert_group, size_t topk_group, int scoring,
+                                    int renormalize, float routed_scaling_factor, int dtype, void* stream) {
+  const char* fn = "ksq_moe_grouped_topk";
+  if (!gating || !topk_w || !topk_ids) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: null pointer", fn);
+  if (E == 0 || E > 1024 || top_k == 0 || top_k > 32 || top_k > E)
+    return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: need 1 <= top_k <= min(32, E) and E <= 1024", fn);
+  if (num_expert_group == 0 || num_expert_group > 64 || E % num_expert_group != 0)
+    return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: need 1 <= num_expert_group <= 64 dividing E", fn);
+  if (topk_group == 0 || topk_group > num_expert_group)
+    return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: need 1 <= topk_group <= num_expert_group", fn);
+  const size_t per_group = E / num_expert_group;
+  if (e_bias && per_group < 2)
+    return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: with a bias a group is ranked by its two best experts and needs two", fn);
+  if (top_k > topk_group * per_group)
+    return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: top_k %zu exceeds the %zu experts of the kept groups", fn, top_k, topk_group * per_group);
+  if (scoring != KSQ_SCORE_SOFTMAX && scoring != KSQ_SCORE_SIGMOID)
+    return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: unknown scoring function %d", fn, scoring);
+  if (tokens == 0) return KSQ_OK;
+  if (tokens > 0x7fffffffull) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: too many tokens", fn);
+  const unsigned blocks = static_cast<unsigned>(div_up(tokens, 4));
+  const size_t lds = 4 * E * sizeof(float);
+  float* w = static_cast<float*>(topk_w);
+  int32_t* ids = static_cast<int32_t*>(topk_ids);
+  const float* b = static_cast<const float*>(e_bias);
+  const uint32_t t = static_cast<uint32_t>(tokens), e = static_cast<uint32_t>(E), k = static_cast<uint32_t>(top_k);
+  const uint32_t g = static_cast<uint32_t>(num_expert_group), kg = static_cast<uint32_t>(topk_group);
+  const int sig = scoring == KSQ_SCORE_SIGMOID;
+  hipStream_t st = as_stream(stream);
+  if (dtype == KSQ_F32)
+    grouped_topk_kernel<LoadF32><<<blocks, 256, lds, st>>>(gating, b, w, ids, t, e, k, g, kg, sig, renormalize, routed_scaling_factor);
+  else if (dtype == KSQ_F16)
+    grouped_topk_kernel<Load16<F16>><<<blocks, 256, lds, st>>>(gating, b, w, ids, t, e, k, g, kg, sig, renormalize, routed_scaling_factor);
+  else if (dtype == KSQ_BF16)
+    grouped_topk_kernel<Load16<BF16>><<<blocks, 256, lds, st>>>(gating, b, w, ids, t, e, k, g, kg, sig, renormalize, routed_scaling_factor);
   else
     return fail(KSQ_ERR_UNSUPPORTED, "%s: unknown dtype %d", fn, dtype);
   return check_launch(fn);

@@ -45,8 +45,14 @@ Status MoeLayer::Init(const std::vector<std::any>& parameters, const RuntimeConf
     return Status(RET_INVALID_ARGUMENT, "MoeLayer: only int4 (TYPE_UINT4x2 / TYPE_INT4x2) expert weights are built");
   }
   if (!use_vllm_moe_) return Status(RET_INVALID_ARGUMENT, "MoeLayer: only the use_vllm_moe flow is built");
-  if (scoring_func_ != "softmax" || num_expert_group_ != 1 || use_e_score_correction_bias_) {
-    return Status(RET_INVALID_ARGUMENT, "MoeLayer: only ungrouped softmax routing is built");
+  if (scoring_func_ != "softmax" && scoring_func_ != "sigmoid") {
+    return Status(RET_INVALID_ARGUMENT, "MoeLayer: unsupported scoring function: " + scoring_func_);
+  }
+  if (num_expert_group_ == 0 || num_expert_group_ > 64 || expert_num_per_node_ % num_expert_group_ != 0 ||
+      expert_groups_topk_ == 0 || expert_groups_topk_ > num_expert_group_ ||
+      expert_topk_ > expert_groups_topk_ * (expert_num_per_node_ / num_expert_group_)) {
+    return Status(RET_INVALID_ARGUMENT, "MoeLayer: expert groups must divide the experts (at most 64 groups) and the "
+                                        "kept groups must hold at least topk experts");
   }
   if (runtime_config.parallel_basic_config.expert_parallel_size * runtime_config.parallel_basic_config.expert_world_size != 1) {
     return Status(RET_INVALID_ARGUMENT, "MoeLayer: expert parallelism is not built");
@@ -123,10 +129,25 @@ Status MoeLayer::Forward(const std::vector<Tensor>& input_tensors, std::vector<T
 
   const int gating_dtype = input_tensors[1].dtype == TYPE_FP32 ? KSQ_F32 : KsqDtype(input_tensors[1].dtype, "MoeLayer");
   const bool renormalize = norm_topk_prob_ || moe_scale_norm_mode_ == MoeScaleNormMode::RE_NORM;
-  KsqCheck(ksq_moe_topk_softmax(input_tensors[1].GetPtr<void>(), topk_weights, topk_ids, num_tokens,
-                                expert_num_per_node_, expert_topk_, renormalize ? 1 : 0, routed_scaling_factor_,
-                                gating_dtype, stream),
-           "MoeLayer");
+  // routing (MoeLayer::ExecuteGroupedTopk of the reference, moe_layer.cpp:380-420): the correction bias is input 5
+  const void* e_bias = nullptr;
+  if (use_e_score_correction_bias_) {
+    if (input_tensors.size() <= 5) KLLM_THROW("MoeLayer: use_e_score_correction_bias needs the bias as input tensor 5");
+    if (input_tensors[5].dtype != TYPE_FP32) KLLM_THROW("MoeLayer: e_score_correction_bias must be fp32");
+    e_bias = input_tensors[5].GetPtr<void>();
+  }
+  if (scoring_func_ == "softmax" && num_expert_group_ == 1 && !e_bias) {
+    KsqCheck(ksq_moe_topk_softmax(input_tensors[1].GetPtr<void>(), topk_weights, topk_ids, num_tokens,
+                                  expert_num_per_node_, expert_topk_, renormalize ? 1 : 0, routed_scaling_factor_,
+                                  gating_dtype, stream),
+             "MoeLayer");
+  } else {
+    KsqCheck(ksq_moe_grouped_topk(input_tensors[1].GetPtr<void>(), e_bias, topk_weights, topk_ids, num_tokens,
+                                  expert_num_per_node_, expert_topk_, num_expert_group_, expert_groups_topk_,
+                                  scoring_func_ == "sigmoid" ? KSQ_SCORE_SIGMOID : KSQ_SCORE_SOFTMAX,
+                                  renormalize ? 1 : 0, routed_scaling_factor_, gating_dtype, stream),
+             "MoeLayer");
+  }
 
   const char* hidden = input_tensors[0].GetPtr<char>();
   char* out = output_tensors[0].GetPtr<char>();

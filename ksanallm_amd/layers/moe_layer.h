@@ -1,10 +1,10 @@
 // Fused MoE layer for int4 group-quantized experts (the "moe-int4" path: weights [E, N, K/2] uint4x2 with per-group
 // scales, activations in T).  Mirrors src/ksana_llm/layers/moe_layer.h:42 and nvidia/moe_layer.cpp:38-380 together with
 // InvokeFusedMoe (src/ksana_llm/kernels/nvidia/moe_kernel_wrapper.cpp:466-657):
-//   router (softmax + top-k) -> align/permute -> grouped GEMM gate_up -> silu*mul -> grouped GEMM down (x routing
+//   router (softmax top-k, or grouped / sigmoid / bias-corrected top-k with the bias as input tensor 5) -> align/permute -> grouped GEMM gate_up -> silu*mul -> grouped GEMM down (x routing
 //   weight) -> sum over top-k, processed in chunks of 32768 tokens, all scratch carved out of one workspace buffer.
-// Expert parallelism, DeepEP, EPLB, grouped (DeepSeek-V3 sigmoid) routing and the fp8 / w4afp8 weight types of the
-// reference class are not part of this path and make Init fail with a message.
+// Expert parallelism, DeepEP, EPLB and the fp8 / w4afp8 weight types of the reference class are not part of this path
+// and make Init fail with a message.
 #pragma once
 
 #include "base_layer.h"

@@ -46,6 +46,7 @@ SIGNATURES = {
                                  c_sz, c_i, c_p]),
     "ksq_moe_block_m": (c_sz, [c_sz, c_sz]),
     "ksq_moe_topk_softmax": (c_i, [c_p, c_p, c_p, c_sz, c_sz, c_sz, c_i, ctypes.c_float, c_i, c_p]),
+    "ksq_moe_grouped_topk": (c_i, [c_p, c_p, c_p, c_p, c_sz, c_sz, c_sz, c_sz, c_sz, c_i, c_i, ctypes.c_float, c_i, c_p]),
     "ksq_moe_silu_mul": (c_i, [c_p, c_p, c_sz, c_sz, c_i, c_p]),
     "ksq_moe_sum": (c_i, [c_p, c_p, c_sz, c_sz, c_sz, c_i, c_p]),
     "ksq_select_tile": (c_i, [c_i, c_sz, c_sz, c_sz, c_i, ctypes.POINTER(TileDesc)]),

@@ -190,6 +190,24 @@ def moe_topk_softmax(gating, top_k, norm_topk_prob=False, routed_scaling_factor=
     return w, ids
 
 
+def moe_grouped_topk(gating, top_k, num_expert_group=1, topk_group=1, scoring_func="softmax", e_bias=None,
+                     renormalize=False, routed_scaling_factor=1.0):
+    """InvokeGroupedTopk: (topk_weights fp32 [T, top_k], topk_ids int32 [T, top_k]); e_bias fp32 [E] or None."""
+    tokens, E = gating.shape
+    if scoring_func not in ("softmax", "sigmoid"):
+        raise ValueError("Unsupported scoring function: %s" % scoring_func)
+    dt = _l.F32 if gating.dtype == torch.float32 else _dt(gating)
+    w = torch.empty((tokens, top_k), dtype=torch.float32, device=gating.device)
+    ids = torch.empty((tokens, top_k), dtype=torch.int32, device=gating.device)
+    if e_bias is not None and e_bias.dtype != torch.float32:
+        raise ValueError("e_bias must be fp32")
+    _l.check(_lib.ksq_moe_grouped_topk(_ptr(gating), _ptr(e_bias) if e_bias is not None else None, _ptr(w), _ptr(ids),
+                                       tokens, E, top_k, num_expert_group, topk_group,
+                                       1 if scoring_func == "sigmoid" else 0, int(renormalize),
+                                       float(routed_scaling_factor), dt, _stream()))
+    return w, ids
+
+
 def silu_and_mul(x, out=None):
     """InvokeSiluAndMul: x [rows, 2*inter] -> [rows, inter]."""
     rows, two = x.shape

@@ -638,6 +638,75 @@ KSQO_API void ksqo_moe_topk_softmax(const void* gating, float* topk_w, int32_t* 
   }
 }
 
+/* Grouped router.  Follows the reference's CPU restatement of DeepSeek-V3 routing
+ * (3rdparty/LLM_kernels/tests/references/deepseek_v3_grouped_topk.h:139-236: sigmoid, + bias, group rank = sum of the
+ * two largest, top groups, top_k over the kept groups, weights from the unbiased scores, / sum * scaling) and the
+ * tensor-op form of S/kernels/nvidia/moe_kernel_wrapper.cpp:286-347 for the other options (softmax scoring, no
+ * bias -> group rank = largest, renormalize off, experts outside the kept groups excluded outright).
+ * Picks are by repeated arg-max, the lower index winning ties.
+ * Pinned by tests/test_oracle_golden.py against the published DeepSeek-V3 formula written with torch tensor ops. */
+KSQO_API void ksqo_moe_grouped_topk(const void* gating, const float* bias, float* topk_w, int32_t* topk_ids,
+                                    size_t tokens, size_t E, size_t top_k, size_t groups, size_t topk_group,
+                                    int sigmoid, int renorm, float scaling, int dtype) {
+  const size_t per = E / groups;
+#pragma omp parallel for schedule(static)
+  for (size_t t = 0; t < tokens; ++t) {
+    float* score = (float*)malloc(E * sizeof(float));
+    float* choose = (float*)malloc(E * sizeof(float));
+    float* rank = (float*)malloc(groups * sizeof(float));
+    char* kept = (char*)calloc(groups, 1);
+    char* taken = (char*)calloc(E, 1);
+    if (sigmoid) {
+      for (size_t e = 0; e < E; ++e) score[e] = 1.0f / (1.0f + expf(-load_t(gating, t * E + e, dtype)));
+    } else {
+      float mx = load_t(gating, t * E, dtype), sum = 0.f;
+      for (size_t e = 0; e < E; ++e) mx = fmaxf(mx, load_t(gating, t * E + e, dtype));
+      for (size_t e = 0; e < E; ++e) {
+        score[e] = expf(load_t(gating, t * E + e, dtype) - mx);
+        sum += score[e];
+      }
+      for (size_t e = 0; e < E; ++e) score[e] = score[e] / sum;
+    }
+    for (size_t e = 0; e < E; ++e) choose[e] = score[e] + (bias ? bias[e] : 0.f);
+    for (size_t g = 0; g < groups; ++g) {
+      float m1 = -INFINITY, m2 = -INFINITY;
+      for (size_t i = 0; i < per; ++i) {
+        const float c = choose[g * per + i];
+        if (c > m1) {
+          m2 = m1;
+          m1 = c;
+        } else if (c > m2) {
+          m2 = c;
+        }
+      }
+      rank[g] = bias ? m1 + m2 : m1;
+    }
+    for (size_t r = 0; r < topk_group; ++r) {
+      size_t best = groups;
+      for (size_t g = 0; g < groups; ++g)
+        if (!kept[g] && (best == groups || rank[g] > rank[best])) best = g;
+      kept[best] = 1;
+    }
+    float picked = 0.f;
+    for (size_t r = 0; r < top_k; ++r) {
+      size_t best = E;
+      for (size_t e = 0; e < E; ++e)
+        if (kept[e / per] && !taken[e] && (best == E || choose[e] > choose[best])) best = e;
+      topk_ids[t * top_k + r] = (int32_t)best;
+      topk_w[t * top_k + r] = score[best];
+      picked += score[best];
+      taken[best] = 1;
+    }
+    for (size_t r = 0; r < top_k; ++r)
+      topk_w[t * top_k + r] = (renorm ? topk_w[t * top_k + r] / picked : topk_w[t * top_k + r]) * scaling;
+    free(score);
+    free(choose);
+    free(rank);
+    free(kept);
+    free(taken);
+  }
+}
+
 /* out[r, i] = T( silu(a) * b ) with a = x[r, i], b = x[r, inter + i], math in fp32: a / (1 + expf(-a)) * b.
  * K/moe_utils/moe_utils.cu:597-606. */
 KSQO_API void ksqo_silu_mul(const void* x, void* out, size_t rows, size_t inter, int dtype) {

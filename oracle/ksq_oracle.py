@@ -311,6 +311,18 @@ def moe_topk_softmax(gating, top_k, norm, scaling, dtype):
     return w, ids
 
 
+def moe_grouped_topk(gating, bias, top_k, groups, topk_group, sigmoid, renorm, scaling, dtype):
+    g = _c(gating, _store_dt(dtype))
+    T, E = g.shape
+    w = np.empty((T, top_k), np.float32)
+    ids = np.empty((T, top_k), np.int32)
+    b = None if bias is None else _c(bias, np.float32)
+    lib().ksqo_moe_grouped_topk(_p(g), None if b is None else _p(b), _p(w), _p(ids), _sz(T), _sz(E), _sz(top_k),
+                                _sz(groups), _sz(topk_group), ctypes.c_int(int(sigmoid)), ctypes.c_int(int(renorm)),
+                                ctypes.c_float(scaling), ctypes.c_int(dtype))
+    return w, ids
+
+
 def silu_mul(x_bits, dtype):
     x = _c(x_bits, _store_dt(dtype))
     rows, two_i = x.shape

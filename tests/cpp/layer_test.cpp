@@ -143,7 +143,9 @@ static int RunBlockwise(int argc, char** argv) {
 }
 
 static std::vector<std::any> MoeParams(size_t tokens, size_t E, size_t hidden, size_t inter, size_t topk, bool renorm,
-                                       float scaling, DataType int_dtype = TYPE_UINT4x2) {
+                                       float scaling, DataType int_dtype = TYPE_UINT4x2, uint32_t groups = 1,
+                                       uint32_t topk_group = 1, const std::string& scoring = "softmax",
+                                       bool use_bias = false) {
   return {renorm ? MoeScaleNormMode::RE_NORM : MoeScaleNormMode::NO_NORM,
           tokens,
           int(0),
@@ -153,13 +155,13 @@ static std::vector<std::any> MoeParams(size_t tokens, size_t E, size_t hidden, s
           topk,
           size_t(1),
           true,
-          uint32_t(1),
-          uint32_t(1),
-          std::string("softmax"),
+          groups,
+          topk_group,
+          scoring,
           std::string("greedy"),
           renorm,
           scaling,
-          false,
+          use_bias,
           false,
           TYPE_INVALID,
           int_dtype,
@@ -175,6 +177,10 @@ static int RunMoe(int argc, char** argv) {
                topk = std::atol(argv[8]);
   const bool renorm = std::atoi(argv[9]) != 0;
   const float scaling = static_cast<float>(std::atof(argv[10]));
+  // optional grouped routing: groups topk_group scoring use_bias (bias.bin: fp32 [E])
+  const uint32_t groups = argc > 11 ? std::atoi(argv[11]) : 1, topk_group = argc > 12 ? std::atoi(argv[12]) : 1;
+  const std::string scoring = argc > 13 ? argv[13] : "softmax";
+  const bool use_bias = argc > 14 && std::atoi(argv[14]) != 0;
   hipStream_t stream;
   HIP_OK(hipStreamCreate(&stream));
   auto context = std::make_shared<Context>(1, stream);
@@ -188,12 +194,19 @@ static int RunMoe(int argc, char** argv) {
                                   Upload(dir + "/s2.bin", T, {E, hidden, inter / 128}), 128, 0, stream);
   HIP_OK(hipStreamSynchronize(stream));
   MoeLayerFactory factory(mc, rc, 0, context);
-  auto layer = factory.CreateLayer(TYPE_UINT8, T, T, MoeParams(tokens, E, hidden, inter, topk, renorm, scaling),
+  auto layer = factory.CreateLayer(TYPE_UINT8, T, T,
+                                   MoeParams(tokens, E, hidden, inter, topk, renorm, scaling, TYPE_UINT4x2, groups,
+                                             topk_group, scoring, use_bias),
                                    MOE_QUANT_GPTQ, TRITON_MOE_BACKEND);
   Tensor x = Upload(dir + "/x.bin", T, {tokens, hidden});
   Tensor gating = Upload(dir + "/gating.bin", TYPE_FP32, {tokens, E});
   std::vector<Tensor> outputs{Tensor(MemoryLocation::LOCATION_DEVICE, T, {tokens, hidden}, 0)};
-  Drive(layer, mc, rc, {x, gating, w13, w2}, outputs);
+  std::vector<Tensor> inputs{x, gating, w13, w2};
+  if (use_bias) {
+    inputs.push_back(Tensor());  // input 4 (expert map) is not used on this path
+    inputs.push_back(Upload(dir + "/bias.bin", TYPE_FP32, {E}));
+  }
+  Drive(layer, mc, rc, inputs, outputs);
   HIP_OK(hipStreamSynchronize(stream));
   Download(outputs[0], dir + "/y.bin");
   return 0;
@@ -261,7 +274,7 @@ static int RunErrors() {
     Tensor x(MemoryLocation::LOCATION_DEVICE, TYPE_FP16, {16, 256}, 0, reinterpret_cast<void*>(0x1000));
     expect(throws([&] { layer2.Forward({x, Tensor()}, out); }), "Forward without a workspace buffer throws");
   }
-  // moe: fp8 experts / grouped routing rejected, int4 accepted
+  // moe: fp8 experts / impossible expert groups rejected, int4 and grouped routing accepted
   {
     MoeLayer a, b, c;
     auto p = MoeParams(64, 8, 256, 256, 2, false, 1.0f);
@@ -271,8 +284,19 @@ static int RunErrors() {
     q[17] = TYPE_BLOCK_FP8_E4M3;
     expect(!b.Init(q, rc, context, 0).OK(), "fp8 experts are rejected");
     auto r = p;
-    r[9] = uint32_t(8);
-    expect(!c.Init(r, rc, context, 0).OK(), "grouped routing is rejected");
+    r[9] = uint32_t(4);   // 4 groups of 2 experts, 2 kept: top-2 fits
+    r[10] = uint32_t(2);
+    r[11] = std::string("sigmoid");
+    expect(c.Init(r, rc, context, 0).OK(), "grouped sigmoid routing init");
+    MoeLayer d, e, f;
+    r[9] = uint32_t(3);
+    expect(!d.Init(r, rc, context, 0).OK(), "groups that do not divide the experts are rejected");
+    r[9] = uint32_t(8);   // groups of one expert, 1 kept: top-2 does not fit
+    r[10] = uint32_t(1);
+    expect(!e.Init(r, rc, context, 0).OK(), "kept groups smaller than topk are rejected");
+    r = p;
+    r[11] = std::string("tanh");
+    expect(!f.Init(r, rc, context, 0).OK(), "unknown scoring function is rejected");
     expect(ksq_moe_block_m(8 * 2, 8) == 16 && ksq_moe_block_m(64 * 2, 8) == 32 && ksq_moe_block_m(4096 * 8, 256) == 128,
            "block_m thresholds");
   }

@@ -74,8 +74,11 @@ def test_blockwise_layer(tmp_path, oracle, dtype, m, n, k, fuse):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("dtype,tokens,renorm,scaling", [(H.BF16, 1, 0, 2.5), (H.F16, 24, 1, 1.0), (H.BF16, 70, 0, 1.0), (H.BF16, 400, 0, 1.0)])
-def test_moe_layer(tmp_path, oracle, dtype, tokens, renorm, scaling):
+@pytest.mark.parametrize("dtype,tokens,renorm,scaling,routing", [
+    (H.BF16, 1, 0, 2.5, None), (H.F16, 24, 1, 1.0, None), (H.BF16, 70, 0, 1.0, None), (H.BF16, 400, 0, 1.0, None),
+    # DeepSeek-V3 style routing: 4 groups of 4 experts, 2 kept, sigmoid scores with a correction bias (layer input 5)
+    (H.BF16, 33, 1, 2.5, (4, 2, "sigmoid", True)), (H.F16, 5, 0, 1.0, (2, 1, "softmax", False))])
+def test_moe_layer(tmp_path, oracle, dtype, tokens, renorm, scaling, routing):
     E, hidden, inter, topk = 16, 256, 128, 4
     g = H.gen(9200 + tokens)
     w13 = torch.randint(0, 256, (E, 2 * inter, hidden // 2), generator=g, dtype=torch.uint8)
@@ -87,9 +90,19 @@ def test_moe_layer(tmp_path, oracle, dtype, tokens, renorm, scaling):
     for name, arr in (("w13", w13.numpy()), ("w2", w2.numpy()), ("s13", H.bits_of(s13)), ("s2", H.bits_of(s2)),
                       ("x", H.bits_of(x)), ("gating", gating.numpy())):
         arr.tofile(tmp_path / (name + ".bin"))
-    run_driver("moe", tmp_path, TNAME[dtype], tokens, E, hidden, inter, topk, renorm, scaling)
+    if routing is None:
+        run_driver("moe", tmp_path, TNAME[dtype], tokens, E, hidden, inter, topk, renorm, scaling)
+        tw, ids = oracle.moe_topk_softmax(gating.numpy(), topk, bool(renorm), scaling, 2)
+    else:
+        groups, topk_group, scoring, use_bias = routing
+        bias = (torch.rand(E, generator=g) * 0.2 - 0.1) if use_bias else None
+        if use_bias:
+            bias.numpy().tofile(tmp_path / "bias.bin")
+        run_driver("moe", tmp_path, TNAME[dtype], tokens, E, hidden, inter, topk, renorm, scaling, groups, topk_group,
+                   scoring, int(use_bias))
+        tw, ids = oracle.moe_grouped_topk(gating.numpy(), None if bias is None else bias.numpy(), topk, groups,
+                                          topk_group, scoring == "sigmoid", bool(renorm), scaling, 2)
     y = read_out(tmp_path / "y.bin", dtype, (tokens, hidden))
-    tw, ids = oracle.moe_topk_softmax(gating.numpy(), topk, bool(renorm), scaling, 2)
     ref = oracle.moe_forward(H.bits_of(x), w13.numpy(), H.bits_of(s13), w2.numpy(), H.bits_of(s2), ids, tw, 128, dtype)
     ref = oracle.from_bits(ref, dtype)
     # from 48 rows per expert on both GEMMs run through the MFMA tile kernel, which rounds the dequantized weights to T:

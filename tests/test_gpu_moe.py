@@ -73,6 +73,66 @@ def test_topk_softmax(ops, oracle, T, E, topk):
     np.testing.assert_array_equal(ids.cpu().numpy(), io)
 
 
+def _check_routing(w, ids, wo, io, choose_gap_ok):
+    """ids equal as sets per token; where they differ (expf on the GPU and on the host may round differently and swap
+    two near-equal scores) the two experts' weights must agree to 3e-4, the reference test's own allowance."""
+    w, ids = w.cpu().numpy(), ids.cpu().numpy()
+    order, order_o = np.argsort(ids, -1), np.argsort(io, -1)
+    ids_s, io_s = np.take_along_axis(ids, order, -1), np.take_along_axis(io, order_o, -1)
+    w_s, wo_s = np.take_along_axis(w, order, -1), np.take_along_axis(wo, order_o, -1)
+    diff = ids_s != io_s
+    assert diff.mean() <= choose_gap_ok
+    np.testing.assert_allclose(w_s[~diff], wo_s[~diff], rtol=2e-5, atol=1e-8)
+    np.testing.assert_allclose(np.sort(w, -1), np.sort(wo, -1), atol=3e-4)
+
+
+@pytest.mark.parametrize("T,E,topk,groups,topk_group,scoring,use_bias,renorm", [
+    (2048, 256, 8, 8, 4, "sigmoid", True, True),     # DeepSeek-V3, the reference test's first config
+    (2048, 128, 4, 4, 2, "sigmoid", True, True),     # its second config
+    (77, 160, 6, 8, 3, "softmax", False, False),     # DeepSeek-V2
+    (5, 64, 6, 1, 1, "sigmoid", False, True),
+    (9, 1000, 6, 1, 1, "softmax", False, True),
+    (1, 256, 8, 8, 4, "sigmoid", True, True),
+])
+def test_grouped_topk(ops, oracle, T, E, topk, groups, topk_group, scoring, use_bias, renorm):
+    g = H.gen(T + E)
+    logits = torch.rand((T, E), generator=g) * 1.98 - 0.99
+    bias = (torch.rand(E, generator=g) * 0.009 - 0.01) if use_bias else None
+    for dtype, lt in ((oracle.F32, logits), (H.BF16, logits.to(torch.bfloat16)), (H.F16, logits.to(torch.float16))):
+        w, ids = ops.moe_grouped_topk(lt.cuda(), topk, groups, topk_group, scoring, None if bias is None else bias.cuda(),
+                                      renorm, 2.5)
+        src = lt.numpy() if dtype == oracle.F32 else H.bits_of(lt)
+        wo, io = oracle.moe_grouped_topk(src, None if bias is None else bias.numpy(), topk, groups, topk_group,
+                                         scoring == "sigmoid", renorm, 2.5, dtype)
+        # 16-bit logits tie often (few distinct values): ties resolve identically (lower id), so ids still match
+        _check_routing(w, ids, wo, io, 1e-3)
+        if renorm:
+            np.testing.assert_allclose(w.cpu().numpy().sum(-1), 2.5, rtol=1e-5)
+
+
+def test_grouped_topk_matches_plain_softmax_router(ops):
+    g = H.gen(5)
+    logits = torch.randn((33, 256), generator=g).cuda()
+    w0, i0 = ops.moe_topk_softmax(logits, 8, True, 2.5)
+    w1, i1 = ops.moe_grouped_topk(logits, 8, 1, 1, "softmax", None, True, 2.5)
+    assert torch.equal(i0, i1)
+    torch.testing.assert_close(w0, w1, rtol=1e-6, atol=0)
+
+
+def test_grouped_topk_rejects_bad_arguments(ops):
+    from ksanallm_amd import lib as L
+    x = torch.zeros((2, 256), device="cuda")
+    for kw in (dict(num_expert_group=7), dict(num_expert_group=8, topk_group=9), dict(num_expert_group=128, topk_group=1),
+               dict(top_k=40), dict(num_expert_group=64, topk_group=1, top_k=8)):
+        args = dict(top_k=8, num_expert_group=8, topk_group=4)
+        args.update(kw)
+        with pytest.raises(L.KsqError) as e:
+            ops.moe_grouped_topk(x, args["top_k"], args["num_expert_group"], args["topk_group"], "sigmoid")
+        assert e.value.code == 1
+    with pytest.raises(ValueError):
+        ops.moe_grouped_topk(x, 8, 8, 4, "tanh")
+
+
 @pytest.mark.parametrize("dtype", [H.F16, H.BF16])
 def test_silu_mul_and_sum(ops, oracle, dtype):
     g = H.gen(3)

@@ -342,3 +342,65 @@ def test_topk_softmax_vs_torch(oracle):
     flat = np.zeros((1, 16), np.float32)
     _, ids = oracle.moe_topk_softmax(flat, 4, False, 1.0, oracle.F32)
     np.testing.assert_array_equal(ids[0], [0, 1, 2, 3])
+
+
+def _grouped_topk_torch(logits, bias, top_k, groups, topk_group, sigmoid, renorm, scaling):
+    """The published DeepSeek-V2/V3 routing formula with tensor ops (the form S/kernels/nvidia/moe_kernel_wrapper.cpp:286-347
+    spells out): an independent statement of what the oracle's loops compute."""
+    T, E = logits.shape
+    scores = torch.sigmoid(logits) if sigmoid else torch.softmax(logits, -1)
+    original = scores
+    if bias is not None:
+        scores = scores + bias
+        group_scores = scores.view(T, groups, -1).topk(2, -1)[0].sum(-1)
+    else:
+        group_scores = scores.view(T, groups, -1).max(-1)[0]
+    group_idx = torch.topk(group_scores, topk_group, -1)[1]
+    mask = torch.zeros_like(group_scores).scatter_(1, group_idx, 1)
+    score_mask = mask.unsqueeze(-1).expand(T, groups, E // groups).reshape(T, -1)
+    tmp = scores.masked_fill(~score_mask.bool(), float("-inf"))
+    ids = torch.topk(tmp, top_k, -1)[1]
+    w = original.gather(1, ids)
+    if renorm:
+        w = w / w.sum(-1, keepdim=True)
+    return w * scaling, ids
+
+
+@pytest.mark.parametrize("E,top_k,groups,topk_group,sigmoid,use_bias,renorm", [
+    (256, 8, 8, 4, True, True, True),      # DeepSeek-V3 (the reference test's first config)
+    (128, 4, 4, 2, True, True, True),      # the reference test's second config
+    (160, 6, 8, 3, False, False, False),   # DeepSeek-V2: softmax, group rank = max, no renormalisation
+    (64, 6, 1, 1, True, False, True),      # ungrouped sigmoid
+    (60, 4, 1, 1, False, False, True),     # ungrouped softmax, E not a multiple of 64
+])
+def test_grouped_topk_vs_torch(oracle, E, top_k, groups, topk_group, sigmoid, use_bias, renorm):
+    g = torch.Generator().manual_seed(E + top_k)
+    logits = torch.rand((301, E), generator=g) * 1.98 - 0.99      # U(-0.99, 0.99) as in the reference's test
+    bias = (torch.rand(E, generator=g) * 0.009 - 0.01) if use_bias else None   # U(-0.01, -0.001)
+    w, ids = oracle.moe_grouped_topk(logits.numpy(), None if bias is None else bias.numpy(), top_k, groups, topk_group,
+                                     sigmoid, renorm, 2.5, oracle.F32)
+    tw, ti = _grouped_topk_torch(logits, bias, top_k, groups, topk_group, sigmoid, renorm, 2.5)
+    np.testing.assert_array_equal(ids, ti.numpy())
+    np.testing.assert_allclose(w, tw.numpy(), rtol=2e-5)
+    if renorm:
+        np.testing.assert_allclose(w.sum(-1), 2.5, rtol=1e-5)   # the reference test's EXPECT_NEAR(sum, routed_scaling_factor)
+    # every pick lies in a kept group: at most topk_group distinct groups per token
+    per = E // groups
+    assert max(len(set((row // per).tolist())) for row in ids) <= topk_group
+
+
+def test_grouped_topk_ties_and_group_rank(oracle):
+    # 2 groups of 4; group 1 holds the single largest value but group 0 the larger top-2 sum: with a bias the rank is
+    # the top-2 sum (group 0 kept), without it the maximum (group 1 kept)
+    logits = np.array([[2.0, 2.0, -5, -5, 3.0, -5, -5, -5]], np.float32)
+    zero = np.zeros(8, np.float32)
+    _, ids = oracle.moe_grouped_topk(logits, zero, 2, 2, 1, True, True, 1.0, oracle.F32)
+    np.testing.assert_array_equal(ids[0], [0, 1])      # equal scores: lower id first
+    w, ids = oracle.moe_grouped_topk(logits, None, 2, 2, 1, True, False, 1.0, oracle.F32)
+    np.testing.assert_array_equal(ids[0], [4, 5])
+    np.testing.assert_allclose(w[0], [1 / (1 + np.exp(-3.0)), 1 / (1 + np.exp(5.0))], rtol=1e-6)
+    # weights come from the unbiased score: a large bias changes the pick, not the weight
+    bias = np.array([0, 0, 0, 10, 0, 0, 0, 0], np.float32)
+    w, ids = oracle.moe_grouped_topk(logits, bias, 1, 1, 1, True, False, 1.0, oracle.F32)
+    assert ids[0, 0] == 3
+    np.testing.assert_allclose(w[0, 0], 1 / (1 + np.exp(5.0)), rtol=1e-6)
