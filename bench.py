@@ -200,6 +200,41 @@ def moe_cases(ops, L, cfg, Ts, E=256, hidden=7168, inter=2048, topk=8, distinct=
     return cases, []
 
 
+def moe_fp8_cases(ops, L, cfg, Ts, E=256, hidden=7168, inter=2048, topk=8, distinct=32):
+    """Block-fp8 experts (DeepSeek-V3's own expert format): weights e4m3 [E, N, K] + fp32 scales per 128 x 128 block."""
+    dev = "cuda"
+    g = seeded(cfg, 0)
+    tdt = torch.bfloat16
+    rep = E // distinct
+
+    def experts(n, k):
+        # random e4m3 codes without NaN (exponent-mantissa 0x7f) and scales of the size amax/448 gives for N(0, 0.02)
+        q = torch.randint(0, 256, (distinct, n, k), generator=g, dtype=torch.uint8)
+        q = torch.where((q & 0x7f) == 0x7f, q & 0xfe, q)
+        s = torch.rand((distinct, n // 128, k // 128), generator=g) * 1e-4 + 1e-4
+        return q.to(dev).repeat(rep, 1, 1), s.to(dev).repeat(rep, 1, 1)
+
+    w13, s13 = experts(2 * inter, hidden)
+    w2, s2 = experts(hidden, inter)
+    per_expert = (2 * inter * hidden + hidden * inter) + (2 * inter * hidden + hidden * inter) // (128 * 128) * 4
+    cases = []
+    for ti, T in enumerate(Ts):
+        gx = seeded(cfg, 10 + ti)
+        x = torch.randn((T, hidden), generator=gx).to(tdt).to(dev)
+        logits = torch.randn((T, E), generator=gx)
+        tw, ids = torch.topk(torch.softmax(logits, -1), topk, dim=-1)
+        touched = int(torch.unique(ids).numel())
+        ids_d, tw_d = ids.to(torch.int32).to(dev), tw.float().contiguous().to(dev)
+
+        def launch(x=x, ids_d=ids_d, tw_d=tw_d):
+            ops.fused_moe_fp8_blockwise(x, w13, s13, w2, s2, ids_d, tw_d)
+
+        nbytes = per_expert * touched + 2 * T * hidden * 2 + 64 * T
+        flops = 2 * T * topk * (2 * inter * hidden + hidden * inter)
+        cases.append(Case("moe_fp8:T=%d" % T, launch, flops, nbytes, "fp8", "moe_fp8_blockwise"))
+    return cases, []
+
+
 def build(cfg, ops, L):
     if cfg == 1:
         return ("GPTQ W4A16 fp16 N=K=4096 M in {1,16}",) + w4a16_cases(
@@ -218,6 +253,9 @@ def build(cfg, ops, L):
     if cfg == 5:
         return ("DeepSeek-V3 MoE int4 bf16 E=256 top-8 T in {1,64,512,4096}",) + moe_cases(
             ops, L, 5, [1, 64, 512, 4096]) + ("bf16",)
+    if cfg == 6:  # not one of the reference's five benchmark configurations: the block-fp8 expert path, same shapes as 5
+        return ("DeepSeek-V3 MoE block-fp8 bf16 E=256 top-8 T in {1,64,512,4096}",) + moe_fp8_cases(
+            ops, L, 6, [1, 64, 512, 4096]) + ("fp8",)
     raise SystemExit("unknown --config %d" % cfg)
 
 
@@ -300,7 +338,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--config", type=int, default=2, help="BASELINE.json config number 1..5 (default 2)")
+    ap.add_argument("--config", type=int, default=2, help="BASELINE.json config number 1..5 (default 2); 6 = block-fp8 MoE, same shapes as 5")
     ap.add_argument("--only", default="", help="substring filter on case names (for profiling one case)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-graph", action="store_true", help="launch every kernel from Python instead of replaying "

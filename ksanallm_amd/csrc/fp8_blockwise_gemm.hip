@@ -22,6 +22,13 @@ struct Fp8Params {
   const float* b_s;   // [ceil(n/128), k/128]
   void* out;          // [m, n]
   uint32_t M, N, K;
+  uint32_t as_row_stride, as_kb_stride;  // a_s[row * as_row_stride + kb * as_kb_stride]: (1, M) in the dense form
+  // grouped (MoE) form: row block b holds the slots sorted_ids[b*16*MT ..] of expert expert_ids[b]
+  const int32_t* sorted_ids;
+  const int32_t* expert_ids;
+  const int32_t* num_post_pad;
+  const float* topk_w;
+  uint32_t numel, top_k, scale_rows;  // scale_rows = ceil(N/128): rows of one expert's b_s
 };
 
 __device__ __forceinline__ f32x4 mfma_fp8_128(i32x8 a, i32x8 b, f32x4 c) {
@@ -38,7 +45,10 @@ __device__ __forceinline__ i32x8 load32(const uint8_t* p) {
 // k-blocks w, w+WAVES, ... and keeps LOOK of them in flight (a ring of register stages, refilled in place right after
 // use; blocks past the end are clamped to the last one and given a zero scale, so that control flow stays uniform and
 // the compiler's wait counts stay exact).  Partials are summed through LDS in wavefront order.
-template <typename TO, int MT, int NT, int WAVES, int LOOK>
+// GROUPED: the MoE form.  Row block blockIdx.y is one block of the aligned slot permutation: slot s reads activation
+// row s / top_k (pad slots carry s >= numel), the weights and weight scales are those of expert expert_ids[block], the
+// result goes to out[s, :] (times topk_w[s] when given).  Blocks past num_post_pad leave at once.
+template <typename TO, int MT, int NT, int WAVES, int LOOK, bool GROUPED = false>
 __global__ void __launch_bounds__(WAVES * 64) fp8_splitk_kernel(Fp8Params p) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -50,16 +60,27 @@ __global__ void __launch_bounds__(WAVES * 64) fp8_splitk_kernel(Fp8Params p) {
 
   __shared__ f32x4 red[WAVES][NT][MT][64];
 
-  const uint8_t* bptr = p.b + static_cast<size_t>(n0 + lrow) * p.K + lq * 32;
-  const float* bs = p.b_s + static_cast<size_t>(n0 / 128) * KB;  // 16*NT <= 128 rows: one scale block
+  size_t expert = 0;
+  if (GROUPED) {
+    if (m0 >= static_cast<uint32_t>(p.num_post_pad[0])) return;  // uniform: the whole workgroup leaves
+    expert = static_cast<size_t>(p.expert_ids[blockIdx.y]);
+  }
+  const uint8_t* bptr = p.b + (expert * p.N + n0 + lrow) * p.K + lq * 32;
+  const float* bs = p.b_s + (expert * p.scale_rows + n0 / 128) * KB;  // 16*NT <= 128 rows: one scale block
   const uint8_t* aptr[MT];
   const float* asptr[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     uint32_t row = m0 + mt * 16 + lrow;
-    row = row < p.M ? row : p.M - 1;  // rows past M repeat the last token; their results are not stored
+    if (GROUPED) {
+      uint32_t sid = static_cast<uint32_t>(p.sorted_ids[row]);
+      sid = sid < p.numel ? sid : p.numel - 1;  // pad slots read some valid row; their results are not stored
+      row = sid / p.top_k;
+    } else {
+      row = row < p.M ? row : p.M - 1;  // rows past M repeat the last token; their results are not stored
+    }
     aptr[mt] = p.a + static_cast<size_t>(row) * p.K + lq * 32;
-    asptr[mt] = p.a_s + row;
+    asptr[mt] = p.a_s + static_cast<size_t>(row) * p.as_row_stride;
   }
 
   f32x4 acc[NT][MT];
@@ -90,7 +111,7 @@ __global__ void __launch_bounds__(WAVES * 64) fp8_splitk_kernel(Fp8Params p) {
       const i32x4* ap = reinterpret_cast<const i32x4*>(aptr[mt] + static_cast<size_t>(kb) * 128);
       s.a0[mt] = ap[0];
       s.a1[mt] = ap[1];
-      s.as[mt] = asptr[mt][static_cast<size_t>(kb) * p.M];
+      s.as[mt] = asptr[mt][static_cast<size_t>(kb) * p.as_kb_stride];
     }
   };
   auto compute_stage = [&](const Stage& s) {
@@ -134,8 +155,15 @@ __global__ void __launch_bounds__(WAVES * 64) fp8_splitk_kernel(Fp8Params p) {
     f32x4 v = red[0][nt][mt][l];
 #pragma unroll
     for (int w = 1; w < WAVES; ++w) v += red[w][nt][mt][l];
-    const uint32_t row = m0 + mt * 16 + (l & 15);
-    if (row < p.M) {
+    uint32_t row = m0 + mt * 16 + (l & 15);
+    bool live = row < p.M;
+    if (GROUPED) {
+      const uint32_t sid = static_cast<uint32_t>(p.sorted_ids[row]);
+      live = sid < p.numel;
+      row = sid;
+      if (live && p.topk_w) v *= p.topk_w[sid];
+    }
+    if (live) {
       u32x2 o;
       o.x = pack2(TO::from_float(v[0]), TO::from_float(v[1]));
       o.y = pack2(TO::from_float(v[2]), TO::from_float(v[3]));
@@ -149,6 +177,21 @@ template <typename TO, int MT, int NT, int WAVES, int LOOK>
 void launch_splitk(const Fp8Params& p, hipStream_t s) {
   dim3 grid(p.N / (16 * NT), static_cast<unsigned>(div_up(p.M, 16 * MT)), 1);
   fp8_splitk_kernel<TO, MT, NT, WAVES, LOOK><<<grid, WAVES * 64, 0, s>>>(p);
+}
+
+// grouped (MoE) form: one row block of the aligned permutation per blockIdx.y
+template <typename TO>
+int dispatch_grouped(const Fp8Params& p, int mt, unsigned blocks, hipStream_t s) {
+  const int nt = p.N % 32 == 0 ? 2 : 1;
+#define KSQ_CASE(MT_, NT_)                                                             \
+  if (mt == MT_ && nt == NT_) {                                                        \
+    dim3 grid(p.N / (16 * NT_), blocks, 1);                                            \
+    fp8_splitk_kernel<TO, MT_, NT_, 4, 2, true><<<grid, 4 * 64, 0, s>>>(p);            \
+    return KSQ_OK;                                                                     \
+  }
+  KSQ_CASE(1, 1) KSQ_CASE(1, 2) KSQ_CASE(2, 1) KSQ_CASE(2, 2)
+#undef KSQ_CASE
+  return fail(KSQ_ERR_UNSUPPORTED, "no grouped fp8 kernel for mt=%d nt=%d", mt, nt);
 }
 
 template <typename TO>
@@ -249,6 +292,8 @@ KSQ_EXPORT int ksq_fp8_blockwise_gemm(const void* a_q, const void* a_s, const vo
   Fp8Params p{static_cast<const uint8_t*>(a_q), static_cast<const float*>(a_s), static_cast<const uint8_t*>(b),
               static_cast<const float*>(b_s), out, static_cast<uint32_t>(m), static_cast<uint32_t>(n),
               static_cast<uint32_t>(k)};
+  p.as_row_stride = 1;
+  p.as_kb_stride = static_cast<uint32_t>(m);
   int rc;
   if (use_fp8_tile(m, n, k)) {
     const TilePlan plan = plan_fp8_tile(m, n, k);
@@ -262,6 +307,49 @@ KSQ_EXPORT int ksq_fp8_blockwise_gemm(const void* a_q, const void* a_s, const vo
   } else {
     rc = out_dtype == KSQ_F16 ? dispatch<F16>(p, as_stream(stream)) : dispatch<BF16>(p, as_stream(stream));
   }
+  if (rc) return rc;
+  return check_launch(fn);
+}
+
+KSQ_EXPORT int ksq_moe_fp8_blockwise_gemm(void* out, const void* a_q, const void* a_s, int a_s_column_major, size_t a_rows, const void* b,
+                                          const void* b_s, const void* topk_w, const void* sorted_ids,
+                                          const void* expert_ids, const void* num_post_pad, size_t numel, size_t top_k,
+                                          size_t E, size_t n, size_t k, size_t block_m, int out_dtype, void* stream) {
+  const char* fn = "ksq_moe_fp8_blockwise_gemm";
+  if (!a_q || !a_s || !b || !b_s || !out) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: null pointer", fn);
+  if (!sorted_ids || !expert_ids || !num_post_pad) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: null index buffer", fn);
+  if (!aligned16(a_q) || !aligned16(b) || !aligned16(out) || (reinterpret_cast<uintptr_t>(a_s) & 3u) ||
+      (reinterpret_cast<uintptr_t>(b_s) & 3u))
+    return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: a_q, b, out must be 16-byte aligned, scales 4-byte aligned", fn);
+  if (n == 0 || k == 0 || k % 128 != 0 || n % 16 != 0)
+    return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: need k %% 128 == 0 and n %% 16 == 0 (n=%zu k=%zu)", fn, n, k);
+  if (out_dtype != KSQ_F16 && out_dtype != KSQ_BF16)
+    return fail(KSQ_ERR_UNSUPPORTED, "%s: output dtype must be f16 or bf16", fn);
+  if (top_k == 0 || E == 0) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: top_k and E must be positive", fn);
+  if (block_m != 16 && block_m != 32) return fail(KSQ_ERR_UNSUPPORTED, "%s: block_m %zu not in {16,32}", fn, block_m);
+  if (numel == 0) return KSQ_OK;
+  if (a_rows < (numel + top_k - 1) / top_k)
+    return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: %zu activation rows cannot serve %zu slots of top_k %zu", fn, a_rows, numel, top_k);
+  if (numel > 0x7fffffffull || a_rows > 0x7fffffffull || n > 0x7fffffffull || k > 0x7fffffffull)
+    return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: dimension too large", fn);
+  const size_t cap_blocks = (numel + E * (block_m - 1)) / block_m;  // upper bound on aligned blocks
+  if (cap_blocks > 65535) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: too many row blocks (%zu)", fn, cap_blocks);
+  Fp8Params p{static_cast<const uint8_t*>(a_q), static_cast<const float*>(a_s), static_cast<const uint8_t*>(b),
+              static_cast<const float*>(b_s), out, static_cast<uint32_t>(cap_blocks * block_m), static_cast<uint32_t>(n),
+              static_cast<uint32_t>(k)};
+  p.as_row_stride = a_s_column_major ? 1u : static_cast<uint32_t>(k / 128);
+  p.as_kb_stride = a_s_column_major ? static_cast<uint32_t>(a_rows) : 1u;
+  p.sorted_ids = static_cast<const int32_t*>(sorted_ids);
+  p.expert_ids = static_cast<const int32_t*>(expert_ids);
+  p.num_post_pad = static_cast<const int32_t*>(num_post_pad);
+  p.topk_w = static_cast<const float*>(topk_w);
+  p.numel = static_cast<uint32_t>(numel);
+  p.top_k = static_cast<uint32_t>(top_k);
+  p.scale_rows = static_cast<uint32_t>(div_up(n, 128));
+  const int mt = block_m == 16 ? 1 : 2;
+  const unsigned blocks = static_cast<unsigned>(cap_blocks);
+  int rc = out_dtype == KSQ_F16 ? dispatch_grouped<F16>(p, mt, blocks, as_stream(stream))
+                                : dispatch_grouped<BF16>(p, mt, blocks, as_stream(stream));
   if (rc) return rc;
   return check_launch(fn);
 }

@@ -57,6 +57,9 @@ MoeLayerFactory::MoeLayerFactory(const ModelConfig& model_config, const RuntimeC
   // "deepseek moe-int4" rows of the reference
   builder_map_[{TYPE_UINT8, TYPE_FP16, TYPE_FP16, MOE_QUANT_GPTQ, TRITON_MOE_BACKEND}] = &MoeLayerFactory::BuildLayer<MoeLayer>;
   builder_map_[{TYPE_UINT8, TYPE_BF16, TYPE_BF16, MOE_QUANT_GPTQ, TRITON_MOE_BACKEND}] = &MoeLayerFactory::BuildLayer<MoeLayer>;
+  // "deepseek fp8 blockwise" rows
+  builder_map_[{TYPE_FP8_E4M3, TYPE_FP16, TYPE_FP16, MOE_QUANT_BLOCK_FP8_E4M3, TRITON_MOE_BACKEND}] = &MoeLayerFactory::BuildLayer<MoeLayer>;
+  builder_map_[{TYPE_FP8_E4M3, TYPE_BF16, TYPE_BF16, MOE_QUANT_BLOCK_FP8_E4M3, TRITON_MOE_BACKEND}] = &MoeLayerFactory::BuildLayer<MoeLayer>;
 }
 
 std::shared_ptr<BaseLayer> MoeLayerFactory::CreateLayer(DataType weight_type, DataType input_type, DataType output_type,

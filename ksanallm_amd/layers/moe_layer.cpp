@@ -33,16 +33,22 @@ Status MoeLayer::Init(const std::vector<std::any>& parameters, const RuntimeConf
   group_size_ = std::any_cast<int>(parameters[parameter_index++]);
   apply_weight_ = std::any_cast<bool>(parameters[parameter_index++]);
 
-  // weight / compute type resolution of the reference (moe_layer.cpp:66-86), restricted to the int4 row
+  // weight / compute type resolution of the reference (moe_layer.cpp:66-86): the block-fp8 and the int4 rows
   weight_dtype_ = inter_data_type_;
   compute_dtype_ = inter_data_type_;
-  if (fp8_weight_dtype == TYPE_BLOCK_FP8_E4M3 || fp8_weight_dtype == TYPE_FP8_E4M3) {
-    return Status(RET_INVALID_ARGUMENT, "MoeLayer: fp8 expert weights are not built on this path");
-  }
-  if (int_weight_dtype == TYPE_UINT4x2 || int_weight_dtype == TYPE_INT4x2) {
+  if (fp8_weight_dtype == TYPE_BLOCK_FP8_E4M3) {
+    weight_dtype_ = TYPE_FP8_E4M3;
+    compute_dtype_ = TYPE_BLOCK_FP8_E4M3;
+    if (int_weight_dtype == TYPE_UINT4x2 || int_weight_dtype == TYPE_INT4x2)
+      return Status(RET_INVALID_ARGUMENT, "MoeLayer: int4 weights with fp8 activations (w4afp8) are not built");
+    if (expert_hidden_size_ % 128 != 0 || expert_inter_size_ % 128 != 0)
+      return Status(RET_INVALID_ARGUMENT, "MoeLayer: block-fp8 experts need hidden and inter sizes that are multiples of 128");
+  } else if (fp8_weight_dtype == TYPE_FP8_E4M3) {
+    return Status(RET_INVALID_ARGUMENT, "MoeLayer: per-tensor fp8 expert weights are not built on this path");
+  } else if (int_weight_dtype == TYPE_UINT4x2 || int_weight_dtype == TYPE_INT4x2) {
     weight_dtype_ = int_weight_dtype;
   } else {
-    return Status(RET_INVALID_ARGUMENT, "MoeLayer: only int4 (TYPE_UINT4x2 / TYPE_INT4x2) expert weights are built");
+    return Status(RET_INVALID_ARGUMENT, "MoeLayer: only int4 (TYPE_UINT4x2 / TYPE_INT4x2) or block-fp8 expert weights are built");
   }
   if (!use_vllm_moe_) return Status(RET_INVALID_ARGUMENT, "MoeLayer: only the use_vllm_moe flow is built");
   if (scoring_func_ != "softmax" && scoring_func_ != "sigmoid") {
@@ -57,7 +63,7 @@ Status MoeLayer::Init(const std::vector<std::any>& parameters, const RuntimeConf
   if (runtime_config.parallel_basic_config.expert_parallel_size * runtime_config.parallel_basic_config.expert_world_size != 1) {
     return Status(RET_INVALID_ARGUMENT, "MoeLayer: expert parallelism is not built");
   }
-  if (group_size_ != 128) return Status(RET_INVALID_ARGUMENT, "MoeLayer: expert group size must be 128");
+  if (!IsFp8() && group_size_ != 128) return Status(RET_INVALID_ARGUMENT, "MoeLayer: expert group size must be 128");
   if (expert_topk_ == 0 || expert_topk_ > 32 || expert_num_per_node_ > 1024 || expert_topk_ > expert_num_per_node_) {
     return Status(RET_INVALID_ARGUMENT, "MoeLayer: need 1 <= topk <= min(32, experts), experts <= 1024");
   }
@@ -77,9 +83,17 @@ size_t MoeLayer::GetWorkspaceSize() {
   align_scratch_size_ = AlignAddress(ksq_moe_align_scratch_bytes(numel, expert_num_per_node_));
   cache1_size_ = AlignAddress(numel * expert_inter_size_ * 2 * elem);
   cache2_size_ = AlignAddress(numel * expert_inter_size_ * elem);
+  if (IsFp8()) {
+    // cache2 holds the quantized silu*mul output (codes, then scales); a1 the quantized hidden states of a chunk
+    a2_q_size_ = AlignAddress(numel * expert_inter_size_);
+    cache2_size_ = a2_q_size_ + AlignAddress(numel * (expert_inter_size_ / 128) * sizeof(float));
+    a1_q_size_ = AlignAddress(m * expert_hidden_size_);
+    a1_size_ = a1_q_size_ + AlignAddress(m * (expert_hidden_size_ / 128) * sizeof(float));
+  }
   cache3_size_ = AlignAddress(numel * expert_hidden_size_ * elem);
   cache13_size_ = std::max(cache1_size_, cache3_size_);  // cache1 is dead once silu*mul has run: cache3 reuses it
-  max_ws_bytes_ = topk_weights_size_ + topk_ids_size_ + fused_id_buffer_size_ + align_scratch_size_ + cache13_size_ + cache2_size_;
+  max_ws_bytes_ = topk_weights_size_ + topk_ids_size_ + fused_id_buffer_size_ + align_scratch_size_ + cache13_size_ +
+                  cache2_size_ + a1_size_;
   return max_ws_bytes_;
 }
 
@@ -91,6 +105,13 @@ Status MoeLayer::SetWorkspaceBuffer(const std::shared_ptr<Tensor>& workspace_buf
 Status MoeLayer::Preprocess(const ModelConfig& model_config, const RuntimeConfig& runtime_config) {
   ksq_tile_desc desc;
   const int dtype = KsqDtype(inter_data_type_, "MoeLayer");
+  if (IsFp8()) {
+    if (ksq_select_tile(KSQ_KIND_FP8_BLOCKWISE, 1, expert_inter_size_ * 2, expert_hidden_size_, dtype, &desc) != KSQ_OK ||
+        ksq_select_tile(KSQ_KIND_FP8_BLOCKWISE, 1, expert_hidden_size_, expert_inter_size_, dtype, &desc) != KSQ_OK) {
+      return Status(RET_INVALID_ARGUMENT, std::string("MoeLayer: ") + ksq_last_error_string());
+    }
+    return Status();
+  }
   if (ksq_select_tile(KSQ_KIND_MOE_W4A16, 1, expert_inter_size_ * 2, expert_hidden_size_, dtype, &desc) != KSQ_OK ||
       ksq_select_tile(KSQ_KIND_MOE_W4A16, 1, expert_hidden_size_, expert_inter_size_, dtype, &desc) != KSQ_OK) {
     return Status(RET_INVALID_ARGUMENT, std::string("MoeLayer: ") + ksq_last_error_string());
@@ -107,7 +128,12 @@ Status MoeLayer::Forward(const std::vector<Tensor>& input_tensors, std::vector<T
   const size_t hidden_size = input_tensors[0].shape[1];
   if (hidden_size != expert_hidden_size_) KLLM_THROW("MoeLayer: hidden size mismatch");
   if (num_tokens > max_token_num_) KLLM_THROW("MoeLayer: more tokens than max_token_num");
-  if (!input_tensors[2].scales || !input_tensors[3].scales) KLLM_THROW("MoeLayer: expert weights have no scales bound");
+  if (IsFp8()) {
+    if (!input_tensors[2].weight_scales || !input_tensors[3].weight_scales)
+      KLLM_THROW("MoeLayer: block-fp8 expert weights have no weight_scales bound");
+  } else if (!input_tensors[2].scales || !input_tensors[3].scales) {
+    KLLM_THROW("MoeLayer: expert weights have no scales bound");
+  }
 
   const int dtype = KsqDtype(inter_data_type_, "MoeLayer");
   const size_t elem = GetTypeSize(inter_data_type_);
@@ -126,6 +152,8 @@ Status MoeLayer::Forward(const std::vector<Tensor>& input_tensors, std::vector<T
   char* cache3 = p;
   p += cache13_size_;
   char* cache2 = p;
+  p += cache2_size_;
+  char* a1 = p;  // block-fp8 only
 
   const int gating_dtype = input_tensors[1].dtype == TYPE_FP32 ? KSQ_F32 : KsqDtype(input_tensors[1].dtype, "MoeLayer");
   const bool renormalize = norm_topk_prob_ || moe_scale_norm_mode_ == MoeScaleNormMode::RE_NORM;
@@ -153,8 +181,8 @@ Status MoeLayer::Forward(const std::vector<Tensor>& input_tensors, std::vector<T
   char* out = output_tensors[0].GetPtr<char>();
   const void* w1 = input_tensors[2].GetPtr<void>();
   const void* w2 = input_tensors[3].GetPtr<void>();
-  const void* w1_scale = input_tensors[2].scales->GetPtr<void>();
-  const void* w2_scale = input_tensors[3].scales->GetPtr<void>();
+  const void* w1_scale = IsFp8() ? input_tensors[2].weight_scales->GetPtr<void>() : input_tensors[2].scales->GetPtr<void>();
+  const void* w2_scale = IsFp8() ? input_tensors[3].weight_scales->GetPtr<void>() : input_tensors[3].scales->GetPtr<void>();
   const size_t E = expert_num_per_node_, topk = expert_topk_, inter = expert_inter_size_;
 
   for (size_t begin = 0; begin < num_tokens; begin += kChunk) {
@@ -169,6 +197,24 @@ Status MoeLayer::Forward(const std::vector<Tensor>& input_tensors, std::vector<T
     const float* weights = topk_weights + begin * topk;
 
     KsqCheck(ksq_moe_align(ids, numel, E, block_m, sorted_ids, expert_ids, num_post_pad, align_scratch, stream), "MoeLayer");
+    if (IsFp8()) {
+      // InvokeFusedMoeKernelFunc with compute_dtype TYPE_BLOCK_FP8_E4M3 (moe_kernel_wrapper.cpp:435-456): activations
+      // are quantized per token and 128 channels (scales [rows, k/128]) in front of each GEMM, silu*mul fused into
+      // the second quantization
+      void* a1_s = a1 + a1_q_size_;
+      void* a2_s = cache2 + a2_q_size_;
+      KsqCheck(ksq_fp8_group_quant(hidden + begin * hidden_size * elem, a1, a1_s, tokens, hidden_size, 128, 0, 0, dtype, stream),
+               "MoeLayer");
+      KsqCheck(ksq_moe_fp8_blockwise_gemm(cache1, a1, a1_s, 0, tokens, w1, w1_scale, nullptr, sorted_ids, expert_ids,
+                                          num_post_pad, numel, topk, E, 2 * inter, hidden_size, block_m, dtype, stream),
+               "MoeLayer");
+      KsqCheck(ksq_fp8_group_quant(cache1, cache2, a2_s, numel, inter, 128, 0, 1, dtype, stream), "MoeLayer");
+      KsqCheck(ksq_moe_fp8_blockwise_gemm(cache3, cache2, a2_s, 0, numel, w2, w2_scale, weights, sorted_ids, expert_ids,
+                                          num_post_pad, numel, 1, E, hidden_size, inter, block_m, dtype, stream),
+               "MoeLayer");
+      KsqCheck(ksq_moe_sum(cache3, out + begin * hidden_size * elem, tokens, topk, hidden_size, dtype, stream), "MoeLayer");
+      continue;
+    }
     // gate_up: every (token, slot) row reads hidden[token]
     KsqCheck(ksq_moe_w4a16_gemm(cache1, hidden + begin * hidden_size * elem, w1, w1_scale, nullptr, nullptr, sorted_ids,
                                 expert_ids, num_post_pad, numel, topk, E, 2 * inter, hidden_size, group_size_, block_m,

@@ -1,9 +1,10 @@
 // Fused MoE layer for int4 group-quantized experts (the "moe-int4" path: weights [E, N, K/2] uint4x2 with per-group
-// scales, activations in T).  Mirrors src/ksana_llm/layers/moe_layer.h:42 and nvidia/moe_layer.cpp:38-380 together with
+// scales, activations in T) and for block-quantized fp8 experts (weights [E, N, K] e4m3 with fp32 scales per 128 x 128
+// block bound as weight_scales, activations quantized per token and 128 channels in front of each GEMM).  Mirrors src/ksana_llm/layers/moe_layer.h:42 and nvidia/moe_layer.cpp:38-380 together with
 // InvokeFusedMoe (src/ksana_llm/kernels/nvidia/moe_kernel_wrapper.cpp:466-657):
 //   router (softmax top-k, or grouped / sigmoid / bias-corrected top-k with the bias as input tensor 5) -> align/permute -> grouped GEMM gate_up -> silu*mul -> grouped GEMM down (x routing
 //   weight) -> sum over top-k, processed in chunks of 32768 tokens, all scratch carved out of one workspace buffer.
-// Expert parallelism, DeepEP, EPLB and the fp8 / w4afp8 weight types of the reference class are not part of this path
+// Expert parallelism, DeepEP, EPLB and the per-tensor fp8 / w4afp8 weight types of the reference class are not part of this path
 // and make Init fail with a message.
 #pragma once
 
@@ -32,7 +33,11 @@ class MoeLayer : public BaseLayer {
 
   // rows per expert block for a chunk (InvokeFusedMoe picks 16 / 32 / 64 by token count; here the library decides by
   // rows per expert, which changes no result)
-  size_t BlockM(size_t tokens) const { return ksq_moe_block_m(tokens * expert_topk_, expert_num_per_node_); }
+  size_t BlockM(size_t tokens) const {
+    const size_t bm = ksq_moe_block_m(tokens * expert_topk_, expert_num_per_node_);
+    return IsFp8() && bm > 32 ? 32 : bm;  // the grouped fp8 GEMM has 16- and 32-row blocks
+  }
+  bool IsFp8() const { return compute_dtype_ == TYPE_BLOCK_FP8_E4M3; }
 
  private:
   static constexpr size_t kChunk = 32 * 1024;
@@ -60,6 +65,7 @@ class MoeLayer : public BaseLayer {
   // workspace carve-up (byte sizes, 256-aligned like the reference's AlignAddress)
   size_t topk_weights_size_ = 0, topk_ids_size_ = 0, fused_id_buffer_size_ = 0, align_scratch_size_ = 0;
   size_t cache1_size_ = 0, cache2_size_ = 0, cache3_size_ = 0, cache13_size_ = 0;
+  size_t a1_q_size_ = 0, a1_size_ = 0, a2_q_size_ = 0;  // block-fp8: quantized activations
   size_t max_ws_bytes_ = 0;
 };
 

@@ -45,6 +45,8 @@ SIGNATURES = {
     "ksq_moe_w4a16_gemm": (c_i, [c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_sz, c_sz, c_sz, c_sz, c_sz, c_sz,
                                  c_sz, c_i, c_p]),
     "ksq_moe_block_m": (c_sz, [c_sz, c_sz]),
+    "ksq_moe_fp8_blockwise_gemm": (c_i, [c_p, c_p, c_p, c_i, c_sz, c_p, c_p, c_p, c_p, c_p, c_p, c_sz, c_sz, c_sz, c_sz,
+                                         c_sz, c_sz, c_i, c_p]),
     "ksq_moe_topk_softmax": (c_i, [c_p, c_p, c_p, c_sz, c_sz, c_sz, c_i, ctypes.c_float, c_i, c_p]),
     "ksq_moe_grouped_topk": (c_i, [c_p, c_p, c_p, c_p, c_sz, c_sz, c_sz, c_sz, c_sz, c_i, c_i, ctypes.c_float, c_i, c_p]),
     "ksq_moe_silu_mul": (c_i, [c_p, c_p, c_sz, c_sz, c_i, c_p]),

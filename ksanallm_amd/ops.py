@@ -242,3 +242,40 @@ def fused_moe_w4a16(x, w13_packed, s13_packed, w2_packed, s2_packed, topk_ids, t
     c3 = moe_w4a16_gemm(c2, w2_packed, s2_packed, tw, sorted_ids, expert_ids, npp, numel, 1, E, hidden, inter, group,
                         block_m)
     return moe_sum(c3.view(T, topk, hidden))
+
+
+def moe_fp8_blockwise_gemm(a_q, a_s, a_s_column_major, b, b_s, topk_w, sorted_ids, expert_ids, num_post_pad, numel,
+                           top_k, block_m, out_dtype=torch.bfloat16, out=None):
+    """fp8_w8a8 block-quantized fused_moe_kernel launch: a_q [rows,k] e4m3 bytes, b [E,n,k], b_s [E,n/128,k/128];
+    out [numel, n]."""
+    rows, k = a_q.shape
+    E, n = b.shape[0], b.shape[1]
+    if out is None:
+        out = torch.empty((numel, n), dtype=out_dtype, device=a_q.device)
+    _l.check(_lib.ksq_moe_fp8_blockwise_gemm(_ptr(out), _ptr(a_q), _ptr(a_s), int(a_s_column_major), rows, _ptr(b),
+                                             _ptr(b_s), _ptr(topk_w) if topk_w is not None else None,
+                                             _ptr(sorted_ids), _ptr(expert_ids), _ptr(num_post_pad), numel, top_k, E, n,
+                                             k, block_m, _dt(out), _stream()))
+    return out
+
+
+def fused_moe_fp8_blockwise(x, w13, w13_scale, w2, w2_scale, topk_ids, topk_w, block_m=None):
+    """InvokeFusedMoe<T,false> for block-quantized fp8 experts (S/kernels/nvidia/moe_kernel_wrapper.cpp:463-654 with
+    compute_dtype TYPE_BLOCK_FP8_E4M3): quantize x per token and 128 channels -> align -> GEMM1 -> silu*mul fused into
+    the second quantization -> GEMM2 (* routed weight) -> sum over top-k.  w13 [E, 2*inter, hidden], w2 [E, hidden, inter]
+    e4m3 bytes, scales fp32 per 128 x 128 block."""
+    T, topk = topk_ids.shape
+    E, two_inter, hidden = w13.shape
+    inter = two_inter // 2
+    numel = T * topk
+    if block_m is None:
+        block_m = min(_lib.ksq_moe_block_m(numel, E), 32)
+    sorted_ids, expert_ids, npp = moe_align_block_size(topk_ids, E, block_m)
+    tw = topk_w.reshape(-1).to(torch.float32).contiguous()
+    a1_q, a1_s = per_token_group_quant_fp8(x, hidden, 128, False)
+    c1 = moe_fp8_blockwise_gemm(a1_q, a1_s, False, w13, w13_scale, None, sorted_ids, expert_ids, npp, numel, topk,
+                                block_m, x.dtype)
+    a2_q, a2_s = per_token_group_quant_fp8(c1, inter, 128, False, fuse_silu_mul=True)
+    c3 = moe_fp8_blockwise_gemm(a2_q, a2_s, False, w2, w2_scale, tw, sorted_ids, expert_ids, npp, numel, 1, block_m,
+                                x.dtype)
+    return moe_sum(c3.view(T, topk, hidden))

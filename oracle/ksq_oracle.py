@@ -349,3 +349,31 @@ def moe_forward(x_bits, w13, s13, w2, s2, topk_ids, topk_w, group, dtype):
     c3 = moe_w4a16_gemm(c2b, w2, s2, topk_ids, topk_w, 1, group, True, dtype)
     c3b = to_bits(c3, dtype).reshape(T, topk, -1)
     return moe_sum(c3b, dtype)
+
+
+def moe_fp8_forward(x_bits, w13, w13_scale, w2, w2_scale, topk_ids, topk_w, dtype):
+    """Whole block-fp8 MoE block as S/kernels/nvidia/moe_kernel_wrapper.cpp:435-456 and 616-652 sequence it: quantize the
+    hidden states per token and 128 channels, GEMM1 per expert (no routed weight) -> T, silu*mul fused into the second
+    quantization, GEMM2 (* routed weight) -> T, sum over top-k in T.  Built from the functions above, expert by expert."""
+    ids = np.asarray(topk_ids)
+    T, topk = ids.shape
+    E, two_inter, hidden = w13.shape
+    inter = two_inter // 2
+    a1_q, a1_s = fp8_group_quant(x_bits, hidden, 128, False, False, dtype)
+    c1 = np.zeros((T * topk, two_inter), np.float32)
+    flat = ids.reshape(-1)
+    for e in range(E):
+        slots = np.nonzero(flat == e)[0]
+        if slots.size:
+            rows = slots // topk
+            c1[slots] = fp8_blockwise_gemm(a1_q[rows], a1_s[rows], w13[e], w13_scale[e], False)
+    c1b = to_bits(c1, dtype)
+    a2_q, a2_s = fp8_group_quant(c1b, inter, 128, False, True, dtype)
+    c3 = np.zeros((T * topk, hidden), np.float32)
+    tw = np.asarray(topk_w, np.float32).reshape(-1)
+    for e in range(E):
+        slots = np.nonzero(flat == e)[0]
+        if slots.size:
+            c3[slots] = fp8_blockwise_gemm(a2_q[slots], a2_s[slots], w2[e], w2_scale[e], False) * tw[slots, None]
+    c3b = to_bits(c3, dtype).reshape(T, topk, -1)
+    return moe_sum(c3b, dtype)

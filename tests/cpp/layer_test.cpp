@@ -4,7 +4,8 @@
 //
 //   layer_test w4a16     <dir> <gptq|awq> <f16|bf16> <cutlass|marlin|machete> m n k group
 //   layer_test blockwise <dir> <f16|bf16> m n k fuse_silu_mul
-//   layer_test moe       <dir> <f16|bf16> tokens experts hidden inter topk renorm scaling
+//   layer_test moe       <dir> <f16|bf16> tokens experts hidden inter topk renorm scaling [groups topk_group scoring use_bias]
+//   layer_test moe_fp8   <dir> <f16|bf16> tokens experts hidden inter topk renorm scaling
 //   layer_test errors
 #include <hip/hip_runtime.h>
 
@@ -212,6 +213,38 @@ static int RunMoe(int argc, char** argv) {
   return 0;
 }
 
+// block-fp8 experts: w13.bin [E, 2*inter, hidden] e4m3, s13.bin fp32 [E, 2*inter/128, hidden/128], w2.bin, s2.bin alike
+static int RunMoeFp8(int argc, char** argv) {
+  if (argc < 11) return 2;
+  const std::string dir = argv[2];
+  const DataType T = ParseT(argv[3]);
+  const size_t tokens = std::atol(argv[4]), E = std::atol(argv[5]), hidden = std::atol(argv[6]), inter = std::atol(argv[7]),
+               topk = std::atol(argv[8]);
+  const bool renorm = std::atoi(argv[9]) != 0;
+  const float scaling = static_cast<float>(std::atof(argv[10]));
+  hipStream_t stream;
+  HIP_OK(hipStreamCreate(&stream));
+  auto context = std::make_shared<Context>(1, stream);
+  ModelConfig mc;
+  RuntimeConfig rc;
+  rc.inter_data_type = T;
+  Tensor w13 = Upload(dir + "/w13.bin", TYPE_FP8_E4M3, {E, 2 * inter, hidden});
+  w13.weight_scales = std::make_shared<Tensor>(Upload(dir + "/s13.bin", TYPE_FP32, {E, (2 * inter + 127) / 128, hidden / 128}));
+  Tensor w2 = Upload(dir + "/w2.bin", TYPE_FP8_E4M3, {E, hidden, inter});
+  w2.weight_scales = std::make_shared<Tensor>(Upload(dir + "/s2.bin", TYPE_FP32, {E, (hidden + 127) / 128, inter / 128}));
+  auto params = MoeParams(tokens, E, hidden, inter, topk, renorm, scaling, TYPE_INVALID);
+  params[17] = TYPE_BLOCK_FP8_E4M3;
+  MoeLayerFactory factory(mc, rc, 0, context);
+  auto layer = factory.CreateLayer(TYPE_FP8_E4M3, T, T, params, MOE_QUANT_BLOCK_FP8_E4M3, TRITON_MOE_BACKEND);
+  Tensor x = Upload(dir + "/x.bin", T, {tokens, hidden});
+  Tensor gating = Upload(dir + "/gating.bin", TYPE_FP32, {tokens, E});
+  std::vector<Tensor> outputs{Tensor(MemoryLocation::LOCATION_DEVICE, T, {tokens, hidden}, 0)};
+  Drive(layer, mc, rc, {x, gating, w13, w2}, outputs);
+  HIP_OK(hipStreamSynchronize(stream));
+  Download(outputs[0], dir + "/y.bin");
+  return 0;
+}
+
 // error behaviour that needs no kernel launch
 static int RunErrors() {
   auto context = std::make_shared<Context>(1, nullptr);
@@ -281,8 +314,14 @@ static int RunErrors() {
     expect(a.Init(p, rc, context, 0).OK(), "moe int4 init");
     expect(a.GetWorkspaceSize() > 0, "moe workspace size");
     auto q = p;
+    q[17] = TYPE_FP8_E4M3;
+    expect(!b.Init(q, rc, context, 0).OK(), "per-tensor fp8 experts are rejected");
+    MoeLayer b2, b3;
     q[17] = TYPE_BLOCK_FP8_E4M3;
-    expect(!b.Init(q, rc, context, 0).OK(), "fp8 experts are rejected");
+    expect(!b2.Init(q, rc, context, 0).OK(), "int4 weights with fp8 activations are rejected");
+    q[18] = TYPE_INVALID;
+    expect(b3.Init(q, rc, context, 0).OK(), "block-fp8 experts init");
+    expect(b3.GetWorkspaceSize() > 0 && b3.BlockM(4096) == 32, "block-fp8 workspace and block size");
     auto r = p;
     r[9] = uint32_t(4);   // 4 groups of 2 experts, 2 kept: top-2 fits
     r[10] = uint32_t(2);
@@ -311,6 +350,7 @@ int main(int argc, char** argv) {
     if (mode == "w4a16") return RunW4A16(argc, argv);
     if (mode == "blockwise") return RunBlockwise(argc, argv);
     if (mode == "moe") return RunMoe(argc, argv);
+    if (mode == "moe_fp8") return RunMoeFp8(argc, argv);
     if (mode == "errors") return RunErrors();
   } catch (const std::exception& e) {
     std::fprintf(stderr, "exception: %s\n", e.what());

@@ -109,3 +109,31 @@ def test_moe_layer(tmp_path, oracle, dtype, tokens, renorm, scaling, routing):
     # each GEMM on its own is held to 5e-3 (tests/test_gpu_moe.py), two in a row compound to sqrt(2) of that
     rounded = tokens * topk // E >= 48
     H.check_gemm(y, ref, dtype, "moe layer", weights_rounded=rounded, rel_l2_max=5e-3 * (2 ** 0.5 if rounded else 1.0))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,tokens,renorm,scaling", [(H.BF16, 1, 0, 2.5), (H.F16, 40, 1, 1.0), (H.BF16, 300, 1, 1.0)])
+def test_moe_layer_block_fp8(tmp_path, oracle, dtype, tokens, renorm, scaling):
+    E, hidden, inter, topk = 16, 256, 128, 4
+    g = H.gen(9400 + tokens)
+
+    def experts(n, k):
+        w = (torch.randn((E, n, k), generator=g) * 0.02).to(torch.bfloat16).float().numpy()
+        q = np.empty((E, n, k), np.uint8)
+        s = np.empty((E, (n + 127) // 128, k // 128), np.float32)
+        for e in range(E):
+            q[e], s[e] = oracle.fp8_block_quant_weight(w[e])
+        return q, s
+
+    w13, s13 = experts(2 * inter, hidden)
+    w2, s2 = experts(hidden, inter)
+    x = torch.randn((tokens, hidden), generator=g).to(H.TORCH_DT[dtype])
+    gating = torch.randn((tokens, E), generator=g)
+    for name, arr in (("w13", w13), ("w2", w2), ("s13", s13), ("s2", s2), ("x", H.bits_of(x)), ("gating", gating.numpy())):
+        arr.tofile(tmp_path / (name + ".bin"))
+    run_driver("moe_fp8", tmp_path, TNAME[dtype], tokens, E, hidden, inter, topk, renorm, scaling)
+    y = read_out(tmp_path / "y.bin", dtype, (tokens, hidden))
+    tw, ids = oracle.moe_topk_softmax(gating.numpy(), topk, bool(renorm), scaling, 2)
+    ref = oracle.from_bits(oracle.moe_fp8_forward(H.bits_of(x), w13, s13, w2, s2, ids, tw, dtype), dtype)
+    # GEMM tolerance, as for the block test in tests/test_gpu_moe.py (the fused silu*mul quantizer is not bit-pinned)
+    H.check_gemm(y, ref, dtype, "block-fp8 moe layer")

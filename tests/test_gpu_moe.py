@@ -220,3 +220,62 @@ def test_moe_block_deepseek_shape(ops, oracle, T):
     rounded = T * topk // E >= 48
     H.check_gemm(out, ref, H.BF16, "moe block T=%d" % T, weights_rounded=rounded,
                  rel_l2_max=5e-3 * (2 ** 0.5 if rounded else 1.0))
+
+
+# ---- block-quantized fp8 experts -------------------------------------------------------------------------------------
+
+def _fp8_experts(oracle, seed, E, n, k):
+    g = H.gen(seed)
+    w = (torch.randn((E, n, k), generator=g) * 0.02).to(torch.bfloat16).float().numpy()
+    q = np.empty((E, n, k), np.uint8)
+    s = np.empty((E, (n + 127) // 128, k // 128), np.float32)
+    for e in range(E):
+        q[e], s[e] = oracle.fp8_block_quant_weight(w[e])
+    return q, s
+
+
+@pytest.mark.parametrize("T,E,topk,n,k,bm,colmajor,with_w", [
+    (1, 8, 2, 256, 256, 16, False, False), (70, 8, 2, 208, 384, 16, True, True), (300, 6, 3, 512, 1024, 32, False, True),
+    (33, 16, 4, 4096, 7168, 32, False, False)])
+def test_grouped_fp8_gemm_stage(ops, oracle, T, E, topk, n, k, bm, colmajor, with_w):
+    """One grouped blockwise-fp8 GEMM launch against the per-expert oracle GEMM on the codes the GPU quantizer wrote."""
+    g = H.gen(7000 + T + n)
+    bq, bs = _fp8_experts(oracle, 7100 + n, E, n, k)
+    x = torch.randn((T, k), generator=g).to(torch.bfloat16)
+    ids = torch.stack([torch.randperm(E, generator=g)[:topk] for _ in range(T)]).to(torch.int32)
+    tw = torch.rand((T, topk), generator=g)
+    numel = T * topk
+    q, s = ops.per_token_group_quant_fp8(x.cuda(), k, 128, colmajor)
+    sorted_ids, expert_ids, npp = ops.moe_align_block_size(ids.cuda(), E, bm)
+    out = ops.moe_fp8_blockwise_gemm(q, s, colmajor, torch.from_numpy(bq).cuda(), torch.from_numpy(bs).cuda(),
+                                     tw.reshape(-1).cuda() if with_w else None, sorted_ids, expert_ids, npp, numel, topk,
+                                     bm, torch.bfloat16)
+    qh, sh = q.cpu().numpy(), s.cpu().numpy()
+    ref = np.zeros((numel, n), np.float32)
+    flat = ids.reshape(-1).numpy()
+    for e in range(E):
+        slots = np.nonzero(flat == e)[0]
+        if slots.size:
+            rows = slots // topk
+            a_s = sh[:, rows] if colmajor else sh[rows]
+            ref[slots] = oracle.fp8_blockwise_gemm(qh[rows], np.ascontiguousarray(a_s), bq[e], bs[e], colmajor)
+    if with_w:
+        ref *= tw.reshape(-1, 1).numpy()
+    H.check_gemm(out, ref, H.BF16, "grouped fp8 T=%d n=%d k=%d" % (T, n, k))
+
+
+@pytest.mark.parametrize("dtype", [H.F16, H.BF16])
+@pytest.mark.parametrize("T,E,topk,hidden,inter", [(1, 8, 2, 256, 128), (48, 16, 4, 512, 256), (200, 8, 2, 384, 640)])
+def test_moe_fp8_block(ops, oracle, dtype, T, E, topk, hidden, inter):
+    """Whole block-fp8 MoE block.  The silu*mul front end of the second quantization rounds through T once more than
+    the oracle may (see the quantizer's fused test), so the block is compared at GEMM tolerance, not bit for bit."""
+    g = H.gen(7300 + T + hidden)
+    w13, s13 = _fp8_experts(oracle, 7400 + hidden, E, 2 * inter, hidden)
+    w2, s2 = _fp8_experts(oracle, 7500 + hidden, E, hidden, inter)
+    x = torch.randn((T, hidden), generator=g).to(H.TORCH_DT[dtype])
+    logits = torch.randn((T, E), generator=g)
+    tw, ids = ops.moe_topk_softmax(logits.cuda(), topk, True, 1.0)
+    y = ops.fused_moe_fp8_blockwise(x.cuda(), torch.from_numpy(w13).cuda(), torch.from_numpy(s13).cuda(),
+                                    torch.from_numpy(w2).cuda(), torch.from_numpy(s2).cuda(), ids, tw)
+    ref = oracle.moe_fp8_forward(H.bits_of(x), w13, s13, w2, s2, ids.cpu().numpy(), tw.cpu().numpy(), dtype)
+    H.check_gemm(y, oracle.from_bits(ref, dtype), dtype, "fp8 moe block")
