@@ -128,6 +128,26 @@ int ksq_fp8_blockwise_gemm(const void* a_q, const void* a_s, const void* b, cons
                            size_t n, size_t k, int out_dtype, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------------------------------------------------
+ * Per-tensor / per-channel FP8: x [channels, size] T -> q e4m3 with one fp32 scale per channel (channels = 1: per tensor).
+ *   dynamic (is_static = 0): scale[c] = max(amax|x[c,:]| / 448, 1 / (448 * 512)) is computed and written first
+ *   static  (is_static = 1): scale[c] is read
+ *   q = e4m3(clamp(x / scale, -448, 448)), IEEE division, round to nearest even.
+ * Replaces Fp8E4m3Quantize (S/kernels/nvidia/basic_kernel_wrapper.cpp:1028-1036) = InvokeComputeFP8QuantizeScale +
+ * InvokeQuantizeMatrix (3rdparty/LLM_kernels/csrc/utils/nvidia/cuda_fp8_utils.cu:32-266).
+ * ------------------------------------------------------------------------------------------------------------------ */
+int ksq_fp8_channel_quant(const void* x, void* q, void* scale, size_t channels, size_t size, int is_static, int dtype,
+                          void* stream);
+
+/* Per-tensor-scaled FP8 GEMM: out[m,n] = T((sum_k a_q[m,k] . b[n,k]) * a_scale[0] * b_scale[0]), fp32 accumulation.
+ * a_q [m,k], b [n,k] e4m3 row-major; a_scale, b_scale: one fp32 each in device memory.  k % 128 == 0, n % 16 == 0.
+ * The workspace (256-byte aligned) holds the scales spread into the blockwise layouts and the split-K partials of
+ * the blockwise kernels, which do the work.
+ * Replaces Fp8QuantizedMatMul (S/kernels/nvidia/basic_kernel_wrapper.cpp:1042-1052, cuBLASLt with scale pointers). */
+size_t ksq_fp8_tensor_gemm_workspace_size(size_t max_m, size_t n, size_t k);
+int ksq_fp8_tensor_gemm(const void* a_q, const void* a_scale, const void* b, const void* b_scale, void* out, size_t m,
+                        size_t n, size_t k, int out_dtype, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------------------------------------------------
  * MoE: expert-offset / permutation build, grouped W4A16 GEMM, silu*mul, top-k sum.
  * ------------------------------------------------------------------------------------------------------------------ */
 

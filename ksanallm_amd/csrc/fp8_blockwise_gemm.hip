@@ -254,6 +254,17 @@ int launch_fp8_tile(const Fp8Params& q, const TilePlan& plan, float* partial, hi
   return KSQ_OK;
 }
 
+// per-tensor scales spread into the blockwise layouts
+__global__ void __launch_bounds__(256) fp8_expand_scales_kernel(const float* __restrict__ a_scale, const float* __restrict__ b_scale,
+                                                                float* __restrict__ a_s, size_t na, float* __restrict__ b_s,
+                                                                size_t nb) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (i < na) a_s[i] = a_scale[0];
+  if (i < nb) b_s[i] = b_scale[0];
+}
+
+inline size_t align256(size_t v) { return (v + 255) & ~static_cast<size_t>(255); }
+
 }  // namespace
 }  // namespace ksq
 
@@ -352,4 +363,37 @@ KSQ_EXPORT int ksq_moe_fp8_blockwise_gemm(void* out, const void* a_q, const void
                                 : dispatch_grouped<BF16>(p, mt, blocks, as_stream(stream));
   if (rc) return rc;
   return check_launch(fn);
+}
+
+KSQ_EXPORT size_t ksq_fp8_tensor_gemm_workspace_size(size_t max_m, size_t n, size_t k) {
+  if (n == 0 || k == 0 || k % 128 != 0) return 0;
+  return align256(max_m * (k / 128) * sizeof(float)) + align256(div_up(n, 128) * (k / 128) * sizeof(float)) +
+         ksq_fp8_blockwise_workspace_size(max_m, n, k);
+}
+
+KSQ_EXPORT int ksq_fp8_tensor_gemm(const void* a_q, const void* a_scale, const void* b, const void* b_scale, void* out,
+                                   size_t m, size_t n, size_t k, int out_dtype, void* workspace, size_t workspace_bytes,
+                                   void* stream) {
+  const char* fn = "ksq_fp8_tensor_gemm";
+  if (!a_q || !a_scale || !b || !b_scale || !out) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: null pointer", fn);
+  if ((reinterpret_cast<uintptr_t>(a_scale) & 3u) || (reinterpret_cast<uintptr_t>(b_scale) & 3u))
+    return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: scales must be 4-byte aligned", fn);
+  if (n == 0 || k == 0 || k % 128 != 0 || n % 16 != 0)
+    return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: need k %% 128 == 0 and n %% 16 == 0 (n=%zu k=%zu)", fn, n, k);
+  if (m == 0) return KSQ_OK;
+  const size_t kb = k / 128;
+  const size_t na = m * kb, nb = div_up(n, 128) * kb;
+  const size_t a_bytes = align256(na * sizeof(float)), b_bytes = align256(nb * sizeof(float));
+  const size_t need = a_bytes + b_bytes + ksq_fp8_blockwise_workspace_size(m, n, k);
+  if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u))
+    return fail(KSQ_ERR_WORKSPACE, "%s: m=%zu n=%zu k=%zu needs %zu bytes of 256-byte aligned workspace, got %zu", fn, m, n, k,
+                need, workspace ? workspace_bytes : size_t(0));
+  char* ws = static_cast<char*>(workspace);
+  float* a_s = reinterpret_cast<float*>(ws);
+  float* b_s = reinterpret_cast<float*>(ws + a_bytes);
+  const size_t most = na > nb ? na : nb;
+  fp8_expand_scales_kernel<<<static_cast<unsigned>(div_up(most, 256)), 256, 0, as_stream(stream)>>>(
+      static_cast<const float*>(a_scale), static_cast<const float*>(b_scale), a_s, na, b_s, nb);
+  return ksq_fp8_blockwise_gemm(a_q, a_s, b, b_s, out, m, n, k, out_dtype, ws + a_bytes + b_bytes,
+                                workspace_bytes - a_bytes - b_bytes, stream);
 }

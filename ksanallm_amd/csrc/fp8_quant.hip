@@ -91,6 +91,74 @@ void launch(const void* x, void* q, void* s, uint32_t m, uint32_t k, bool col, b
   }
 }
 
+
+// ---- per-channel / per-tensor quantization (one fp32 scale per row of [channels, size]) ------------------------------
+constexpr float kMinScale = 1.0f / 448.0f / 512.0f;
+
+__global__ void fp8_scale_clear_kernel(float* __restrict__ scale, uint32_t channels) {
+  const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+  if (i < channels) scale[i] = 0.f;
+}
+
+// scale[c] = max(amax(|x[c, :]|) / 448, 1 / (448 * 512)).  Every wavefront folds its maximum in with an integer
+// atomic max on the float's bits (all candidates are positive, so the orders agree); scale[] starts at 0.
+template <typename T>
+__global__ void __launch_bounds__(256) fp8_channel_scale_kernel(const uint16_t* __restrict__ x, float* __restrict__ scale,
+                                                                size_t size, bool vec) {
+  const uint16_t* row = x + static_cast<size_t>(blockIdx.y) * size;
+  const size_t tid = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  const size_t stride = static_cast<size_t>(gridDim.x) * 256;
+  float amax = 0.f;
+  if (vec) {
+    for (size_t i = tid; i < size / 8; i += stride) {
+      const u32x4 raw = *reinterpret_cast<const u32x4*>(row + i * 8);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        amax = fmaxf(amax, fabsf(T::to_float(static_cast<uint16_t>(raw[j] & 0xffffu))));
+        amax = fmaxf(amax, fabsf(T::to_float(static_cast<uint16_t>(raw[j] >> 16))));
+      }
+    }
+  } else {
+    for (size_t i = tid; i < size; i += stride) amax = fmaxf(amax, fabsf(T::to_float(row[i])));
+  }
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+  if ((threadIdx.x & 63) == 0) {
+    const float sc = fmaxf(amax / 448.0f, kMinScale);
+    atomicMax(reinterpret_cast<unsigned int*>(scale + blockIdx.y), __float_as_uint(sc));
+  }
+}
+
+// q[c, i] = e4m3(clamp(x[c, i] / scale[c], -448, 448)), IEEE division, round to nearest even
+template <typename T>
+__global__ void __launch_bounds__(256) fp8_channel_quant_kernel(const uint16_t* __restrict__ x, uint8_t* __restrict__ q,
+                                                                const float* __restrict__ scale, size_t size, bool vec) {
+  const size_t base = static_cast<size_t>(blockIdx.y) * size;
+  const float sc = scale[blockIdx.y];
+  const size_t tid = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  const size_t stride = static_cast<size_t>(gridDim.x) * 256;
+  if (vec) {
+    for (size_t i = tid; i < size / 8; i += stride) {
+      const u32x4 raw = *reinterpret_cast<const u32x4*>(x + base + i * 8);
+      float v[8];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        v[2 * j] = T::to_float(static_cast<uint16_t>(raw[j] & 0xffffu)) / sc;
+        v[2 * j + 1] = T::to_float(static_cast<uint16_t>(raw[j] >> 16)) / sc;
+      }
+      u32x2 out{0u, 0u};
+      out.x = cvt2_e4m3(v[0], v[1], out.x, false);
+      out.x = cvt2_e4m3(v[2], v[3], out.x, true);
+      out.y = cvt2_e4m3(v[4], v[5], out.y, false);
+      out.y = cvt2_e4m3(v[6], v[7], out.y, true);
+      *reinterpret_cast<u32x2*>(q + base + i * 8) = out;
+    }
+  } else {
+    for (size_t i = tid; i < size; i += stride)
+      q[base + i] = static_cast<uint8_t>(cvt2_e4m3(T::to_float(x[base + i]) / sc, 0.f, 0u, false) & 0xffu);
+  }
+}
+
 }  // namespace
 }  // namespace ksq
 
@@ -119,5 +187,33 @@ KSQ_EXPORT int ksq_fp8_group_quant(const void* x, void* q, void* s, size_t m, si
     if (group == 128) KSQ_Q(BF16, 128); else if (group == 64) KSQ_Q(BF16, 64); else KSQ_Q(BF16, 32);
   }
 #undef KSQ_Q
+  return check_launch(fn);
+}
+
+KSQ_EXPORT int ksq_fp8_channel_quant(const void* x, void* q, void* scale, size_t channels, size_t size, int is_static,
+                                     int dtype, void* stream) {
+  const char* fn = "ksq_fp8_channel_quant";
+  if (!x || !q || !scale) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: null pointer", fn);
+  if ((reinterpret_cast<uintptr_t>(x) & 1u) || (reinterpret_cast<uintptr_t>(scale) & 3u))
+    return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: x must be 2-byte, scale 4-byte aligned", fn);
+  if (dtype != KSQ_F16 && dtype != KSQ_BF16) return fail(KSQ_ERR_UNSUPPORTED, "%s: dtype must be f16 or bf16", fn);
+  if (channels == 0 || size == 0) return KSQ_OK;
+  if (channels > 65535) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: at most 65535 channels", fn);
+  // 16-byte loads and 8-byte stores need rows that start on those boundaries
+  const bool vec = size % 8 == 0 && aligned16(x) && (reinterpret_cast<uintptr_t>(q) & 7u) == 0;
+  const size_t work = vec ? size / 8 : size;
+  size_t bx = div_up(work, 256);
+  if (bx > 1024) bx = 1024;
+  const dim3 grid(static_cast<unsigned>(bx), static_cast<unsigned>(channels), 1);
+  hipStream_t st = as_stream(stream);
+  const uint16_t* xp = static_cast<const uint16_t*>(x);
+  float* sp = static_cast<float*>(scale);
+  if (!is_static) {
+    fp8_scale_clear_kernel<<<static_cast<unsigned>(div_up(channels, 256)), 256, 0, st>>>(sp, static_cast<uint32_t>(channels));
+    if (dtype == KSQ_F16) fp8_channel_scale_kernel<F16><<<grid, 256, 0, st>>>(xp, sp, size, vec);
+    else fp8_channel_scale_kernel<BF16><<<grid, 256, 0, st>>>(xp, sp, size, vec);
+  }
+  if (dtype == KSQ_F16) fp8_channel_quant_kernel<F16><<<grid, 256, 0, st>>>(xp, static_cast<uint8_t*>(q), sp, size, vec);
+  else fp8_channel_quant_kernel<BF16><<<grid, 256, 0, st>>>(xp, static_cast<uint8_t*>(q), sp, size, vec);
   return check_launch(fn);
 }

@@ -1,6 +1,7 @@
 #include "layer_factory.h"
 
 #include "blockwise_matmul_layer.h"
+#include "fp8_matmul_layer.h"
 #include "moe_layer.h"
 #include "w4a16_matmul_layer.h"
 
@@ -18,6 +19,7 @@ MatMulLayerFactory::MatMulLayerFactory(const ModelConfig& model_config, const Ru
     }
     builder_map_[{TYPE_FP8_E4M3, t, t, QUANT_BLOCK_FP8_E4M3, DEFAULT_LINEAR_BACKEND}] =
         &MatMulLayerFactory::BuildLayer<BlockwiseMatMulLayer>;
+    builder_map_[{TYPE_FP8_E4M3, t, t, QUANT_FP8_E4M3, DEFAULT_LINEAR_BACKEND}] = &MatMulLayerFactory::BuildLayer<Fp8MatMulLayer>;
   }
 }
 

@@ -279,3 +279,26 @@ def fused_moe_fp8_blockwise(x, w13, w13_scale, w2, w2_scale, topk_ids, topk_w, b
     c3 = moe_fp8_blockwise_gemm(a2_q, a2_s, False, w2, w2_scale, tw, sorted_ids, expert_ids, npp, numel, 1, block_m,
                                 x.dtype)
     return moe_sum(c3.view(T, topk, hidden))
+
+
+def fp8_e4m3_quantize(x, scale=None):
+    """Fp8E4m3Quantize: x [channels, size] -> (codes uint8, scale fp32 [channels]); scale given = static."""
+    channels, size = x.shape
+    q = torch.empty((channels, size), dtype=torch.uint8, device=x.device)
+    static = scale is not None
+    s = scale if static else torch.empty(channels, dtype=torch.float32, device=x.device)
+    _l.check(_lib.ksq_fp8_channel_quant(_ptr(x), _ptr(q), _ptr(s), channels, size, int(static), _dt(x), _stream()))
+    return q, s
+
+
+def fp8_quantized_matmul(a_q, a_scale, b, b_scale, out_dtype=torch.bfloat16, out=None, workspace=None):
+    """Fp8QuantizedMatMul: a_q [m,k], b [n,k] e4m3 bytes, one fp32 device scale each."""
+    m, k = a_q.shape
+    n = b.shape[0]
+    if out is None:
+        out = torch.empty((m, n), dtype=out_dtype, device=a_q.device)
+    if workspace is None:
+        workspace = torch.empty(_lib.ksq_fp8_tensor_gemm_workspace_size(m, n, k), dtype=torch.uint8, device=a_q.device)
+    _l.check(_lib.ksq_fp8_tensor_gemm(_ptr(a_q), _ptr(a_scale), _ptr(b), _ptr(b_scale), _ptr(out), m, n, k, _dt(out),
+                                      _ptr(workspace), workspace.numel(), _stream()))
+    return out

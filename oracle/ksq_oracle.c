@@ -471,6 +471,48 @@ KSQO_API void ksqo_fp8_group_quant(const void* x, uint8_t* q, float* s, size_t m
 }
 
 /* ------------------------------------------------------------------------------------------------
+ * Per-tensor / per-channel FP8
+ * ---------------------------------------------------------------------------------------------- */
+
+/* 3rdparty/LLM_kernels/csrc/utils/nvidia/cuda_fp8_utils.cu:150-256 (scale) and :32-41 (quantize), as called by
+ * Fp8E4m3Quantize (S/kernels/nvidia/basic_kernel_wrapper.cpp:1028-1036):
+ *   dynamic: scale[c] = max(amax|x[c,:]| / 448, 1/(448*512));  q = e4m3(min(max(x / scale, -448), 448)).
+ * Pinned by tests/test_oracle_golden.py against torch's float8_e4m3fn conversion and the reference test's formula
+ * (utils_test.cu:48-56, 136-143). */
+KSQO_API void ksqo_fp8_channel_quant(const void* x, uint8_t* q, float* scale, size_t channels, size_t size,
+                                     int is_static, int dtype) {
+  for (size_t c = 0; c < channels; ++c) {
+    if (!is_static) {
+      float amax = 0.f;
+      for (size_t i = 0; i < size; ++i) amax = fmaxf(amax, fabsf(load_t(x, c * size + i, dtype)));
+      volatile float sc = amax / 448.0f;
+      scale[c] = fmaxf(sc, 1.0f / 448.0f / 512.0f);
+    }
+    volatile float sc = scale[c];
+    for (size_t i = 0; i < size; ++i) {
+      volatile float r = load_t(x, c * size + i, dtype) / sc;
+      q[c * size + i] = ksqo_f32_to_e4m3(fminf(fmaxf(r, -448.0f), 448.0f));
+    }
+  }
+}
+
+/* out[m,n] = (sum_k a[m,k] * b[n,k]) * a_scale * b_scale: what cuBLASLt computes for Fp8QuantizedMatMul
+ * (S/kernels/nvidia/basic_kernel_wrapper.cpp:1042-1052: e4m3 x e4m3, fp32 compute type, scale pointers).
+ * The sum is taken in double here, so the result is the exact value up to the final rounding. */
+KSQO_API void ksqo_fp8_tensor_gemm(const uint8_t* a, float a_scale, const uint8_t* b, float b_scale, float* out, size_t m,
+                                   size_t n, size_t k) {
+  float lut[256];
+  for (int i = 0; i < 256; ++i) lut[i] = ksqo_e4m3_to_f32((uint8_t)i);
+#pragma omp parallel for schedule(static)
+  for (size_t i = 0; i < m; ++i)
+    for (size_t j = 0; j < n; ++j) {
+      double acc = 0.0;
+      for (size_t kk = 0; kk < k; ++kk) acc += (double)lut[a[i * k + kk]] * (double)lut[b[j * k + kk]];
+      out[i * n + j] = (float)(acc * (double)a_scale * (double)b_scale);
+    }
+}
+
+/* ------------------------------------------------------------------------------------------------
  * Blockwise FP8 GEMM
  * ---------------------------------------------------------------------------------------------- */
 

@@ -252,6 +252,29 @@ def fp8_group_quant(x_bits, k, group, column_major, fuse_silu_mul, dtype):
     return q, s
 
 
+def fp8_channel_quant(x_bits, dtype, scale=None):
+    """[channels, size] T bits -> (codes, scales); scale given = static quantization."""
+    x = _c(x_bits, _store_dt(dtype))
+    channels, size = x.shape
+    q = np.empty((channels, size), np.uint8)
+    static = scale is not None
+    s = _c(scale, np.float32).copy() if static else np.empty(channels, np.float32)
+    lib().ksqo_fp8_channel_quant(_p(x), _p(q), _p(s), _sz(channels), _sz(size), ctypes.c_int(int(static)),
+                                 ctypes.c_int(dtype))
+    return q, s
+
+
+def fp8_tensor_gemm(a, a_scale, b, b_scale):
+    a = _c(a, np.uint8)
+    b = _c(b, np.uint8)
+    m, k = a.shape
+    n = b.shape[0]
+    out = np.empty((m, n), np.float32)
+    lib().ksqo_fp8_tensor_gemm(_p(a), ctypes.c_float(float(a_scale)), _p(b), ctypes.c_float(float(b_scale)), _p(out),
+                               _sz(m), _sz(n), _sz(k))
+    return out
+
+
 def fp8_blockwise_gemm(a, a_s, b, b_s, a_s_column_major=True):
     a = _c(a, np.uint8)
     b = _c(b, np.uint8)

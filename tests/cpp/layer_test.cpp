@@ -4,6 +4,7 @@
 //
 //   layer_test w4a16     <dir> <gptq|awq> <f16|bf16> <cutlass|marlin|machete> m n k group
 //   layer_test blockwise <dir> <f16|bf16> m n k fuse_silu_mul
+//   layer_test fp8_tensor <dir> <f16|bf16> m n k static
 //   layer_test moe       <dir> <f16|bf16> tokens experts hidden inter topk renorm scaling [groups topk_group scoring use_bias]
 //   layer_test moe_fp8   <dir> <f16|bf16> tokens experts hidden inter topk renorm scaling
 //   layer_test errors
@@ -17,6 +18,7 @@
 
 #include "blockwise_matmul_layer.h"
 #include "layer_factory.h"
+#include "fp8_matmul_layer.h"
 #include "moe_layer.h"
 #include "quant_weight_repack.h"
 #include "w4a16_matmul_layer.h"
@@ -136,6 +138,34 @@ static int RunBlockwise(int argc, char** argv) {
   MatMulLayerFactory factory(mc, rc, 0, context);
   auto layer = factory.CreateLayer(TYPE_FP8_E4M3, T, T, params, QUANT_BLOCK_FP8_E4M3, DEFAULT_LINEAR_BACKEND);
   Tensor x = Upload(dir + "/x.bin", T, {m, fuse ? 2 * k : k});
+  std::vector<Tensor> outputs{Tensor(MemoryLocation::LOCATION_DEVICE, T, {m, n}, 0)};
+  Drive(layer, mc, rc, {x, weight}, outputs);
+  HIP_OK(hipStreamSynchronize(stream));
+  Download(outputs[0], dir + "/y.bin");
+  return 0;
+}
+
+// per-tensor fp8: w.bin [n, k] e4m3, w_scale.bin 1 fp32, optional in_scale.bin 1 fp32 (static activation scale)
+static int RunFp8Tensor(int argc, char** argv) {
+  if (argc < 8) return 2;
+  const std::string dir = argv[2];
+  const DataType T = ParseT(argv[3]);
+  const size_t m = std::atol(argv[4]), n = std::atol(argv[5]), k = std::atol(argv[6]);
+  const bool is_static = std::atoi(argv[7]) != 0;
+  hipStream_t stream;
+  HIP_OK(hipStreamCreate(&stream));
+  auto context = std::make_shared<Context>(1, stream);
+  ModelConfig mc;
+  RuntimeConfig rc;
+  rc.inter_data_type = T;
+  rc.max_step_token_num = m;
+  Tensor weight = Upload(dir + "/w.bin", TYPE_FP8_E4M3, {n, k});
+  weight.weight_scales = std::make_shared<Tensor>(Upload(dir + "/w_scale.bin", TYPE_FP32, {1}));
+  if (is_static) weight.input_scales = std::make_shared<Tensor>(Upload(dir + "/in_scale.bin", TYPE_FP32, {1}));
+  std::vector<std::any> params{rc.max_step_token_num, k};
+  MatMulLayerFactory factory(mc, rc, 0, context);
+  auto layer = factory.CreateLayer(TYPE_FP8_E4M3, T, T, params, QUANT_FP8_E4M3, DEFAULT_LINEAR_BACKEND);
+  Tensor x = Upload(dir + "/x.bin", T, {m, k});
   std::vector<Tensor> outputs{Tensor(MemoryLocation::LOCATION_DEVICE, T, {m, n}, 0)};
   Drive(layer, mc, rc, {x, weight}, outputs);
   HIP_OK(hipStreamSynchronize(stream));
@@ -307,6 +337,19 @@ static int RunErrors() {
     Tensor x(MemoryLocation::LOCATION_DEVICE, TYPE_FP16, {16, 256}, 0, reinterpret_cast<void*>(0x1000));
     expect(throws([&] { layer2.Forward({x, Tensor()}, out); }), "Forward without a workspace buffer throws");
   }
+  // per-tensor fp8
+  {
+    Fp8MatMulLayer layer, bad;
+    std::vector<std::any> p{size_t(64), size_t(512)};
+    expect(layer.Init(p, rc, context, 0).OK(), "fp8 per-tensor init");
+    expect(layer.GetWorkspaceSize() >= Fp8MatMulLayer::kGemmWorkspaceBytes + 64 * 512 + 4, "fp8 per-tensor workspace");
+    std::vector<std::any> q{size_t(64), size_t(200)};
+    expect(!bad.Init(q, rc, context, 0).OK(), "k = 200 is rejected");
+    std::vector<Tensor> out{Tensor()};
+    Tensor x(MemoryLocation::LOCATION_DEVICE, TYPE_FP16, {16, 512}, 0, reinterpret_cast<void*>(0x1000));
+    Tensor w(MemoryLocation::LOCATION_DEVICE, TYPE_FP8_E4M3, {64, 512}, 0, reinterpret_cast<void*>(0x1000));
+    expect(throws([&] { layer.Forward({x, w}, out); }), "Forward without a workspace buffer throws");
+  }
   // moe: fp8 experts / impossible expert groups rejected, int4 and grouped routing accepted
   {
     MoeLayer a, b, c;
@@ -349,6 +392,7 @@ int main(int argc, char** argv) {
   try {
     if (mode == "w4a16") return RunW4A16(argc, argv);
     if (mode == "blockwise") return RunBlockwise(argc, argv);
+    if (mode == "fp8_tensor") return RunFp8Tensor(argc, argv);
     if (mode == "moe") return RunMoe(argc, argv);
     if (mode == "moe_fp8") return RunMoeFp8(argc, argv);
     if (mode == "errors") return RunErrors();

@@ -169,3 +169,46 @@ def test_blockwise_gemm_partial_scale_row_and_fp16_out(ops, oracle):
     out = ops.fp8_blockwise_gemm(q, s, torch.from_numpy(bq).cuda(), torch.from_numpy(bs).cuda(), torch.float16)
     ref = oracle.fp8_blockwise_gemm(q.cpu().numpy(), s.cpu().numpy(), bq, bs, True)
     H.check_gemm(out, ref, H.F16, "fp8 partial")
+
+
+# ---- per-tensor / per-channel fp8 ------------------------------------------------------------------------------------
+
+# the reference test's shapes (3rdparty/LLM_kernels/csrc/utils/nvidia/utils_test.cu:107) plus ragged / unaligned ones
+@pytest.mark.parametrize("dtype", [H.F16, H.BF16])
+@pytest.mark.parametrize("channels,size", [(1, 31), (1, 16383), (1, 5120), (1, 12800), (1, 4096), (64, 5120), (3, 77),
+                                           (1, 4096 * 7168)])
+def test_channel_quant_bit_exact(ops, oracle, dtype, channels, size):
+    g = H.gen(channels + size)
+    x = (torch.randn((channels, size), generator=g) * 2.5).to(H.TORCH_DT[dtype])
+    q, s = ops.fp8_e4m3_quantize(x.cuda())
+    qo, so = oracle.fp8_channel_quant(H.bits_of(x), dtype)
+    np.testing.assert_array_equal(s.cpu().numpy(), so)
+    np.testing.assert_array_equal(q.cpu().numpy(), qo)
+    # static: given scales (values far outside the range saturate at +-448)
+    given = torch.full((channels,), 0.004, dtype=torch.float32)
+    q2, _ = ops.fp8_e4m3_quantize(x.cuda(), given.cuda())
+    qo2, _ = oracle.fp8_channel_quant(H.bits_of(x), dtype, scale=given.numpy())
+    np.testing.assert_array_equal(q2.cpu().numpy(), qo2)
+
+
+def test_channel_quant_zero_tensor_takes_minimum_scale(ops):
+    x = torch.zeros((2, 64), dtype=torch.bfloat16, device="cuda")
+    q, s = ops.fp8_e4m3_quantize(x)
+    assert torch.all(s == 1.0 / 448.0 / 512.0) and torch.all(q == 0)
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 512, 1024), (16, 2304, 7168), (130, 4096, 1024), (1030, 13328, 512)])
+def test_fp8_quantized_matmul(ops, oracle, m, n, k):
+    g = H.gen(5100 + m + n)
+    w = (torch.randn((n, k), generator=g) * 0.02).to(torch.bfloat16)
+    x = make_act(5200 + m, m, k, H.BF16)
+    wq, ws = ops.fp8_e4m3_quantize(w.reshape(1, -1).cuda())
+    xq, xs = ops.fp8_e4m3_quantize(x.reshape(1, -1).cuda())
+    out = ops.fp8_quantized_matmul(xq.view(m, k), xs, wq.view(n, k), ws, torch.bfloat16)
+    ref = oracle.fp8_tensor_gemm(xq.view(m, k).cpu().numpy(), xs.item(), wq.view(n, k).cpu().numpy(), ws.item())
+    H.check_gemm(out, ref, H.BF16, "fp8 per-tensor m=%d n=%d k=%d" % (m, n, k))
+    small = torch.empty(256, dtype=torch.uint8, device="cuda")
+    from ksanallm_amd import lib as L
+    with pytest.raises(L.KsqError) as e:
+        ops.fp8_quantized_matmul(xq.view(m, k), xs, wq.view(n, k), ws, torch.bfloat16, workspace=small)
+    assert e.value.code == 3

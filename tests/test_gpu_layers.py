@@ -137,3 +137,22 @@ def test_moe_layer_block_fp8(tmp_path, oracle, dtype, tokens, renorm, scaling):
     ref = oracle.from_bits(oracle.moe_fp8_forward(H.bits_of(x), w13, s13, w2, s2, ids, tw, dtype), dtype)
     # GEMM tolerance, as for the block test in tests/test_gpu_moe.py (the fused silu*mul quantizer is not bit-pinned)
     H.check_gemm(y, ref, dtype, "block-fp8 moe layer")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,m,n,k,static", [(H.BF16, 1, 512, 1024, 0), (H.F16, 77, 2304, 512, 1), (H.BF16, 300, 1024, 2048, 0)])
+def test_fp8_per_tensor_layer(tmp_path, oracle, dtype, m, n, k, static):
+    g = H.gen(9600 + m)
+    w = (torch.randn((n, k), generator=g) * 0.02).to(torch.bfloat16)
+    wq, ws = oracle.fp8_channel_quant(H.bits_of(w).reshape(1, -1), H.BF16)
+    x = torch.randn((m, k), generator=g).to(H.TORCH_DT[dtype])
+    wq.tofile(tmp_path / "w.bin")
+    ws.tofile(tmp_path / "w_scale.bin")
+    H.bits_of(x).tofile(tmp_path / "x.bin")
+    in_scale = np.array([0.012], np.float32)
+    in_scale.tofile(tmp_path / "in_scale.bin")
+    run_driver("fp8_tensor", tmp_path, TNAME[dtype], m, n, k, static)
+    y = read_out(tmp_path / "y.bin", dtype, (m, n))
+    xq, xs = oracle.fp8_channel_quant(H.bits_of(x).reshape(1, -1), dtype, scale=in_scale if static else None)
+    ref = oracle.fp8_tensor_gemm(xq.reshape(m, k), xs[0], wq.reshape(n, k), ws[0])
+    H.check_gemm(y, ref, dtype, "fp8 per-tensor layer")

@@ -4,6 +4,8 @@ import numpy as np
 import pytest
 import torch
 
+from tests import helpers as H
+
 
 # ----------------------------------------------------------------------------- scalar formats
 def test_f16_roundtrip_all_codes(oracle):
@@ -404,3 +406,34 @@ def test_grouped_topk_ties_and_group_rank(oracle):
     w, ids = oracle.moe_grouped_topk(logits, bias, 1, 1, 1, True, False, 1.0, oracle.F32)
     assert ids[0, 0] == 3
     np.testing.assert_allclose(w[0, 0], 1 / (1 + np.exp(5.0)), rtol=1e-6)
+
+
+@pytest.mark.parametrize("channels,size", [(1, 31), (1, 5120), (3, 4096)])
+def test_fp8_channel_quant_vs_torch_float8(oracle, channels, size):
+    g = torch.Generator().manual_seed(size)
+    x = (torch.randn((channels, size), generator=g) * 3).to(torch.bfloat16)
+    x[0, 0] = 0.0
+    q, s = oracle.fp8_channel_quant(H.bits_of(x), H.BF16)
+    # the reference test's own formula for the scale (utils_test.cu:48-56)
+    amax = x.float().abs().amax(-1).numpy()
+    np.testing.assert_array_equal(s, np.maximum(amax / np.float32(448.0), np.float32(1.0 / 448.0 / 512.0)).astype(np.float32))
+    # codes: torch's float8_e4m3fn conversion (round to nearest even) of the clamped quotient
+    r = torch.clamp(x.float() / torch.from_numpy(s)[:, None], -448.0, 448.0)
+    np.testing.assert_array_equal(q, r.to(torch.float8_e4m3fn).view(torch.uint8).numpy())
+    # static: a given scale is used as is; an all-zero tensor takes the minimum scale
+    q2, s2 = oracle.fp8_channel_quant(H.bits_of(x), H.BF16, scale=np.full(channels, 0.05, np.float32))
+    r2 = torch.clamp(x.float() / 0.05, -448.0, 448.0)
+    np.testing.assert_array_equal(q2, r2.to(torch.float8_e4m3fn).view(torch.uint8).numpy())
+    _, s0 = oracle.fp8_channel_quant(np.zeros((1, 16), np.uint16), H.BF16)
+    assert s0[0] == np.float32(1.0 / 448.0 / 512.0)
+
+
+def test_fp8_tensor_gemm_vs_torch(oracle):
+    g = torch.Generator().manual_seed(9)
+    a = torch.randint(0, 256, (5, 256), generator=g, dtype=torch.uint8)
+    b = torch.randint(0, 256, (7, 256), generator=g, dtype=torch.uint8)
+    a = torch.where((a & 0x7f) == 0x7f, a & 0xfe, a)
+    b = torch.where((b & 0x7f) == 0x7f, b & 0xfe, b)
+    out = oracle.fp8_tensor_gemm(a.numpy(), 0.01, b.numpy(), 0.002)
+    ref = (a.view(torch.float8_e4m3fn).double() @ b.view(torch.float8_e4m3fn).double().T) * np.float32(0.01) * np.float32(0.002)
+    np.testing.assert_allclose(out, ref.numpy(), rtol=1e-6)
