@@ -32,17 +32,17 @@ CACHE_BYTES = 320 << 20                            # rotate through more than th
 # (`--calibrate-copy`): FETCH_SIZE reads half the bytes moved (x2.0), WRITE_SIZE reads them exactly (x1.0).
 # Keyed by (config, kernel variant); None where no counter run has been made for the current kernel.
 MEASURED_TRAFFIC = {
-    (2, "w4a16_splitk_kernel<16x16,w4>"): 31874075,
-    (2, "w4a16_splitk_kernel<16x64,w4>"): 31246449,
-    (2, "w4a16_splitk_kernel<32x16,w4>"): 38395318,
-    (2, "w4a16_splitk_kernel<32x64,w4>"): 33821620,
-    (2, "w4a16_tile_kernel<128x256,w8>"): 84562638,
-    (2, "w4a16_tile_kernel<256x256,w8>"): 221588892,
-    (3, "w4a16_tile_kernel<256x256,w8>"): 1246797628,
-    (4, "fp8_group_quant"): 27623708,
-    (4, "fp8_splitk_kernel<16x16,w16>"): 134519524,
-    (4, "fp8_splitk_kernel<16x16,w8>"): 134076218,
-    (4, "fp8_tile_kernel<256x256,w8>"): 261946688,
+    (2, "w4a16_splitk_kernel<16x16,w4>"): 31880000,
+    (2, "w4a16_splitk_kernel<16x64,w4>"): 31250000,
+    (2, "w4a16_splitk_kernel<32x16,w4>"): 38390000,
+    (2, "w4a16_splitk_kernel<32x64,w4>"): 33820000,
+    (2, "w4a16_tile_kernel<128x256,w8>"): 84610000,
+    (2, "w4a16_tile_kernel<256x256,w8>"): 216470000,
+    (3, "w4a16_tile_kernel<256x256,w8>"): 1591160000,
+    (4, "fp8_group_quant"): 27630000,
+    (4, "fp8_splitk_kernel<16x16,w4>"): 134810000,
+    (4, "fp8_splitk_kernel<16x32,w4>"): 134820000,
+    (4, "fp8_tile_kernel<256x256,w8>"): 258550000,
 }
 
 
