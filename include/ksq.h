@@ -82,6 +82,16 @@ int ksq_w4a16_repack(const void* src, int src_layout, void* dst_packed, size_t E
 /* exact inverse of ksq_w4a16_repack for every src_layout */
 int ksq_w4a16_unpack(const void* packed, int dst_layout, void* dst, size_t E, size_t K, size_t N, void* stream);
 
+/* GPTQ act-order (desc_act) checkpoints: g_idx[k] names the quantization group of input channel k.  With
+ * perm = stable argsort(g_idx) (host side, once), packed row j takes checkpoint row perm[j]; every group's rows are
+ * then adjacent, scales / zeros apply as for a checkpoint without act-order, and the GEMM reads x[:, perm]
+ * (ksq_permute_columns) - together y = x . W exactly as with g_idx.  src [K/8, N] int32 (KSQ_SRC_GPTQ), perm int32 [K].
+ * Replaces gptq_marlin_repack with has_perm (K/gptq_marlin/gptq_marlin_repack.cu:276-295), MarlinSortGIdx
+ * (S/models/quant/marlin_utils.cpp:106-122) and the activation permutation inside gptq_marlin_gemm. */
+int ksq_w4a16_repack_act_order(const void* src_gptq, const void* perm, void* dst_packed, size_t K, size_t N, void* stream);
+/* out[r, j] = x[r, perm[j]], x and out [m, k] T, perm int32 [k]; out must not alias x. */
+int ksq_permute_columns(const void* x, const void* perm, void* out, size_t m, size_t k, int dtype, void* stream);
+
 int ksq_w4a16_repack_scales(const void* src, int src_layout, void* dst_packed, size_t E, size_t K, size_t N,
                             size_t group, int dtype, void* stream);
 int ksq_w4a16_unpack_scales(const void* packed, int dst_layout, void* dst, size_t E, size_t K, size_t N, size_t group,

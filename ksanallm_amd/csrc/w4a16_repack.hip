@@ -74,6 +74,47 @@ __global__ void __launch_bounds__(256) repack_weight_kernel(const void* __restri
   dst[o] = out;
 }
 
+// GPTQ act-order: packed row k takes checkpoint row perm[k] (perm = stable argsort of g_idx, so that the rows of a
+// quantization group become adjacent); E = 1
+__global__ void __launch_bounds__(256) repack_act_order_kernel(const uint32_t* __restrict__ src,
+                                                               const int32_t* __restrict__ perm,
+                                                               uint32_t* __restrict__ dst, Geometry g) {
+  size_t o = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  size_t total = g.K * g.N / 8;
+  if (o >= total) return;
+  size_t tile = o / 256;
+  int within = static_cast<int>(o % 256);
+  int lane = within / 4, d = within % 4;
+  size_t kt = tile % g.k_tiles;
+  size_t nt = tile / g.k_tiles;
+  size_t n = nt * 16 + (lane % 16);
+  size_t kbase = kt * 128 + d * 32 + (lane / 16) * 8;
+  uint32_t out = 0;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    uint32_t row = static_cast<uint32_t>(perm[kbase + j]);
+    row = row < g.K ? row : static_cast<uint32_t>(g.K - 1);  // the host checks perm; never read outside the weight
+    const uint32_t w = src[static_cast<size_t>(row / 8) * g.N + n];
+    out |= ((w >> (4 * (row % 8))) & 15u) << (4 * packed_nibble(j));
+  }
+  dst[o] = out;
+}
+
+// out[r, j] = x[r, perm[j]]: the activation side of act-order
+__global__ void __launch_bounds__(256) permute_columns_kernel(const uint16_t* __restrict__ x, const int32_t* __restrict__ perm,
+                                                              uint16_t* __restrict__ out, size_t m, uint32_t k) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;  // one thread per 2 output columns
+  const size_t per_row = k / 2;
+  if (i >= m * per_row) return;
+  const size_t r = i / per_row;
+  const uint32_t c = static_cast<uint32_t>(i % per_row) * 2;
+  uint32_t p0 = static_cast<uint32_t>(perm[c]), p1 = static_cast<uint32_t>(perm[c + 1]);
+  p0 = p0 < k ? p0 : k - 1;
+  p1 = p1 < k ? p1 : k - 1;
+  const uint16_t* row = x + r * k;
+  reinterpret_cast<uint32_t*>(out + r * k)[c / 2] = static_cast<uint32_t>(row[p0]) | (static_cast<uint32_t>(row[p1]) << 16);
+}
+
 // one thread per 8 codes of the destination
 template <int DST>
 __global__ void __launch_bounds__(256) unpack_weight_kernel(const uint32_t* __restrict__ packed,
@@ -215,6 +256,37 @@ KSQ_EXPORT int ksq_w4a16_repack(const void* src, int src_layout, void* dst, size
       return fail(KSQ_ERR_INVALID_ARGUMENT, "ksq_w4a16_repack: unknown source layout %d", src_layout);
   }
   return check_launch("ksq_w4a16_repack");
+}
+
+KSQ_EXPORT int ksq_w4a16_repack_act_order(const void* src_gptq, const void* perm, void* dst, size_t K, size_t N,
+                                          void* stream) {
+  const char* fn = "ksq_w4a16_repack_act_order";
+  if (int rc = check_weight_args(src_gptq, dst, 1, K, N, fn)) return rc;
+  if (!perm || (reinterpret_cast<uintptr_t>(perm) & 3u)) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: perm must be a 4-byte aligned pointer", fn);
+  Geometry g{1, K, N, K / 128, N / 16};
+  unsigned blocks = static_cast<unsigned>(div_up(K * N / 8, 256));
+  repack_act_order_kernel<<<blocks, 256, 0, as_stream(stream)>>>(static_cast<const uint32_t*>(src_gptq),
+                                                                  static_cast<const int32_t*>(perm),
+                                                                  static_cast<uint32_t*>(dst), g);
+  return check_launch(fn);
+}
+
+KSQ_EXPORT int ksq_permute_columns(const void* x, const void* perm, void* out, size_t m, size_t k, int dtype,
+                                   void* stream) {
+  const char* fn = "ksq_permute_columns";
+  if (!x || !perm || !out) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: null pointer", fn);
+  if ((reinterpret_cast<uintptr_t>(x) & 1u) || (reinterpret_cast<uintptr_t>(out) & 3u) || (reinterpret_cast<uintptr_t>(perm) & 3u))
+    return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: x must be 2-byte, out and perm 4-byte aligned", fn);
+  if (dtype != KSQ_F16 && dtype != KSQ_BF16) return fail(KSQ_ERR_UNSUPPORTED, "%s: dtype must be f16 or bf16", fn);
+  if (k == 0 || k % 2 != 0 || k > 0x7fffffffull) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: k must be positive and even", fn);
+  if (x == out) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: cannot permute in place", fn);
+  if (m == 0) return KSQ_OK;
+  const size_t blocks = div_up(m * (k / 2), 256);
+  if (blocks > 0x7fffffffull) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: tensor too large", fn);
+  permute_columns_kernel<<<static_cast<unsigned>(blocks), 256, 0, as_stream(stream)>>>(
+      static_cast<const uint16_t*>(x), static_cast<const int32_t*>(perm), static_cast<uint16_t*>(out), m,
+      static_cast<uint32_t>(k));
+  return check_launch(fn);
 }
 
 KSQ_EXPORT int ksq_w4a16_unpack(const void* packed, int dst_layout, void* dst, size_t E, size_t K, size_t N,

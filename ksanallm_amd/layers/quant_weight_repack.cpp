@@ -1,9 +1,12 @@
 #include "quant_weight_repack.h"
 
+#include <algorithm>
+#include <vector>
+
 namespace ksana_llm {
 
 Tensor PackGroupQuantWeight(const Tensor& qweight, const Tensor& scales, const Tensor* qzeros, QuantMode method,
-                            size_t group_size, int rank, hipStream_t stream) {
+                            size_t group_size, int rank, hipStream_t stream, const Tensor* g_idx) {
   const char* who = "PackGroupQuantWeight";
   if (method != QUANT_GPTQ && method != QUANT_AWQ) KLLM_THROW("PackGroupQuantWeight: method must be GPTQ or AWQ");
   if (qweight.shape.size() != 2 || scales.shape.size() != 2) KLLM_THROW("PackGroupQuantWeight: 2-D tensors expected");
@@ -15,7 +18,32 @@ Tensor PackGroupQuantWeight(const Tensor& qweight, const Tensor& scales, const T
   const int dtype = KsqDtype(scales.dtype, who);
 
   Tensor packed(MemoryLocation::LOCATION_DEVICE, TYPE_I4_GROUP, {K, N / 2}, rank);
-  KsqCheck(ksq_w4a16_repack(qweight.GetPtr<void>(), awq ? KSQ_SRC_AWQ : KSQ_SRC_GPTQ, packed.GetPtr<void>(), 1, K, N, stream), who);
+  if (g_idx) {
+    if (awq) KLLM_THROW("PackGroupQuantWeight: g_idx (act-order) belongs to GPTQ checkpoints");
+    if (g_idx->GetElementNumber() != K) KLLM_THROW("PackGroupQuantWeight: g_idx must have K entries");
+    std::vector<int32_t> groups(K), perm(K);
+    if (hipStreamSynchronize(stream) != hipSuccess ||
+        hipMemcpy(groups.data(), g_idx->GetPtr<void>(), K * sizeof(int32_t), hipMemcpyDeviceToHost) != hipSuccess) {
+      KLLM_THROW("PackGroupQuantWeight: cannot read g_idx");
+    }
+    for (size_t i = 0; i < K; ++i) perm[i] = static_cast<int32_t>(i);
+    std::stable_sort(perm.begin(), perm.end(), [&](int32_t a, int32_t b) { return groups[a] < groups[b]; });
+    std::vector<int32_t> sorted(K);
+    for (size_t i = 0; i < K; ++i) {
+      sorted[i] = groups[perm[i]];
+      // sorted, every group must cover exactly its group_size rows: only then do the scales apply by position
+      if (sorted[i] != static_cast<int32_t>(i / group_size)) KLLM_THROW("PackGroupQuantWeight: g_idx does not hold group_size rows per group");
+    }
+    packed.perm = std::make_shared<Tensor>(MemoryLocation::LOCATION_DEVICE, TYPE_INT32, std::vector<size_t>{K}, rank);
+    packed.g_idx = std::make_shared<Tensor>(MemoryLocation::LOCATION_DEVICE, TYPE_INT32, std::vector<size_t>{K}, rank);
+    if (hipMemcpy(packed.perm->GetPtr<void>(), perm.data(), K * sizeof(int32_t), hipMemcpyHostToDevice) != hipSuccess ||
+        hipMemcpy(packed.g_idx->GetPtr<void>(), sorted.data(), K * sizeof(int32_t), hipMemcpyHostToDevice) != hipSuccess) {
+      KLLM_THROW("PackGroupQuantWeight: cannot upload perm");
+    }
+    KsqCheck(ksq_w4a16_repack_act_order(qweight.GetPtr<void>(), packed.perm->GetPtr<void>(), packed.GetPtr<void>(), K, N, stream), who);
+  } else {
+    KsqCheck(ksq_w4a16_repack(qweight.GetPtr<void>(), awq ? KSQ_SRC_AWQ : KSQ_SRC_GPTQ, packed.GetPtr<void>(), 1, K, N, stream), who);
+  }
   packed.scales = std::make_shared<Tensor>(MemoryLocation::LOCATION_DEVICE, scales.dtype, scales.shape, rank);
   KsqCheck(ksq_w4a16_repack_scales(scales.GetPtr<void>(), KSQ_SCALE_GN, packed.scales->GetPtr<void>(), 1, K, N, group_size, dtype, stream), who);
   if (awq) {

@@ -13,9 +13,12 @@ namespace ksana_llm {
 
 // qweight: GPTQ [K/8, N] int32 or AWQ [K, N/8] int32 (device).  scales: [K/group, N] in T.  qzeros: AWQ only,
 // [K/group, N/8] int32 (nullptr for GPTQ, whose symmetric zero point 8 is implicit).
+// g_idx: GPTQ act-order only, int32 [K] (device): quantization group of every input channel.  The rows are then
+// packed in the order perm = stable argsort(g_idx) (MarlinSortGIdx, src/ksana_llm/models/quant/marlin_utils.cpp:106-122;
+// computed on the host, which synchronizes `stream`) and `perm` and the sorted `g_idx` are bound to the result.
 // Returns a TYPE_I4_GROUP tensor of logical shape {K, N/2} with `scales` (and `zeros`) bound.
 Tensor PackGroupQuantWeight(const Tensor& qweight, const Tensor& scales, const Tensor* qzeros, QuantMode method,
-                            size_t group_size, int rank, hipStream_t stream);
+                            size_t group_size, int rank, hipStream_t stream, const Tensor* g_idx = nullptr);
 
 // experts: [E, N, K/2] uint8, low nibble = even k.  scales: [E, N, K/group] in T.
 // Returns a TYPE_UINT4x2 tensor of logical shape {E, N, K/2} with `scales` bound.

@@ -19,9 +19,10 @@ Status W4A16MatMulLayer::Init(const std::vector<std::any>& parameters, const Run
   [[maybe_unused]] bool use_gemv_cuda_core = std::any_cast<const bool>(parameters[parameter_index++]);  // no analogue
   weight_data_type_ = std::any_cast<const DataType>(parameters[parameter_index++]);
   is_k_full_ = is_gptq_desc_ ? is_k_full_ : true;
-  if (is_gptq_desc_) {
-    // act-order checkpoints need the activation columns gathered through `perm`; not built yet
-    return Status(RET_INVALID_ARGUMENT, std::string(Name()) + ": desc_act (act-order) weights are not supported");
+  if (is_gptq_desc_ && is_awq_) return Status(RET_INVALID_ARGUMENT, std::string(Name()) + ": desc_act belongs to GPTQ, not AWQ");
+  if (is_gptq_desc_ && !is_k_full_) {
+    // a K range cut out of an act-order weight does not hold whole quantization groups
+    return Status(RET_INVALID_ARGUMENT, std::string(Name()) + ": desc_act (act-order) weights split along K are not supported");
   }
   return Status();
 }
@@ -31,7 +32,11 @@ size_t W4A16MatMulLayer::GetWorkspaceSize() {
     KLLM_THROW(std::string("Not supported weight data type: ") + std::to_string(weight_data_type_) + ". " + Name() +
                " only supports TYPE_I4_GROUP.");
   }
-  workspace_size_ = ksq_w4a16_workspace_size(max_m_, max_n_, max_k_, groupsize_, KsqDtype(inter_data_type_, Name()));
+  gemm_workspace_size_ = ksq_w4a16_workspace_size(max_m_, max_n_, max_k_, groupsize_, KsqDtype(inter_data_type_, Name()));
+  gemm_workspace_size_ = (gemm_workspace_size_ + 255) & ~static_cast<size_t>(255);
+  // act-order: the activations with their columns permuted, behind the GEMM's scratch
+  permuted_input_size_ = is_gptq_desc_ ? max_m_ * max_k_ * GetTypeSize(inter_data_type_) : 0;
+  workspace_size_ = gemm_workspace_size_ + permuted_input_size_;
   return workspace_size_;
 }
 
@@ -65,11 +70,25 @@ Status W4A16MatMulLayer::Forward(const std::vector<Tensor>& input_tensors, std::
   if (input_tensors[0].shape.size() < 2 || input_tensors[0].shape[1] != k) {
     KLLM_THROW(std::string(Name()) + ": activation inner dimension does not match k");
   }
-  void* ws = workspace_buffer_ ? workspace_buffer_->GetPtr<void>() : nullptr;
-  const size_t ws_bytes = workspace_buffer_ ? workspace_buffer_->GetTotalBytes() : 0;
-  KsqCheck(ksq_w4a16_gemm(output_tensors[0].GetPtr<void>(), input_tensors[0].GetPtr<void>(), p_qweight, p_scales,
-                          p_zeros, ws, ws_bytes, m, n, k, groupsize_, KsqDtype(inter_data_type_, Name()),
-                          context_->GetComputeStreams()[rank_].Get()),
+  char* ws = workspace_buffer_ ? workspace_buffer_->GetPtr<char>() : nullptr;
+  size_t ws_bytes = workspace_buffer_ ? workspace_buffer_->GetTotalBytes() : 0;
+  const void* x = input_tensors[0].GetPtr<void>();
+  const int dtype = KsqDtype(inter_data_type_, Name());
+  hipStream_t stream = context_->GetComputeStreams()[rank_].Get();
+  if (is_gptq_desc_) {
+    // rows of the packed weight are sorted by quantization group (perm): read the activation columns the same way
+    if (!weight_tensor.perm) KLLM_THROW(std::string(Name()) + ": act-order weight tensor has no perm bound");
+    if (m > max_m_) KLLM_THROW(std::string(Name()) + ": m exceeds max_m");
+    if (!ws || ws_bytes < gemm_workspace_size_ + m * k * GetTypeSize(inter_data_type_)) {
+      KLLM_THROW(std::string(Name()) + ": workspace buffer missing or smaller than GetWorkspaceSize()");
+    }
+    void* permuted = ws + gemm_workspace_size_;
+    KsqCheck(ksq_permute_columns(x, weight_tensor.perm->GetPtr<void>(), permuted, m, k, dtype, stream), Name());
+    x = permuted;
+    ws_bytes = gemm_workspace_size_;
+  }
+  KsqCheck(ksq_w4a16_gemm(output_tensors[0].GetPtr<void>(), x, p_qweight, p_scales, p_zeros, ws, ws_bytes, m, n, k,
+                          groupsize_, dtype, stream),
            Name());
   output_tensors[0].shape = {m, n};
   output_tensors[0].dtype = input_tensors[0].dtype;

@@ -7,6 +7,9 @@
 //
 // Forward inputs: [0] activations [m, k] in T, [1] the weight in the CDNA4 packed layout with `scales` (and, for AWQ,
 // `zeros`) bound to it by PackGroupQuantWeight() (quant_weight_repack.h).  Output [0] is [m, n] in T.
+// GPTQ act-order (is_gptq_desc): the packed rows are sorted by quantization group and the weight carries `perm`; the
+// layer gathers the activation columns through it into its workspace in front of the GEMM (the reference's Marlin
+// kernel does the same gather internally).
 #pragma once
 
 #include "base_layer.h"
@@ -35,6 +38,7 @@ class W4A16MatMulLayer : public BaseLayer {
   size_t max_m_ = 0, max_n_ = 0, max_k_ = 0;
   size_t groupsize_ = 0;
   size_t workspace_size_ = 0;
+  size_t gemm_workspace_size_ = 0, permuted_input_size_ = 0;
 };
 
 class CutlassMatMulLayer : public W4A16MatMulLayer {

@@ -302,3 +302,24 @@ def fp8_quantized_matmul(a_q, a_scale, b, b_scale, out_dtype=torch.bfloat16, out
     _l.check(_lib.ksq_fp8_tensor_gemm(_ptr(a_q), _ptr(a_scale), _ptr(b), _ptr(b_scale), _ptr(out), m, n, k, _dt(out),
                                       _ptr(workspace), workspace.numel(), _stream()))
     return out
+
+
+def sort_g_idx(g_idx):
+    """MarlinSortGIdx: perm = stable argsort of the act-order group index (int32 [K], same device)."""
+    return torch.argsort(g_idx.to(torch.int64), stable=True).to(torch.int32)
+
+
+def repack_weight_act_order(qweight, perm, K, N):
+    """gptq_marlin_repack with a permutation: qweight [K/8, N] int32 (GPTQ), perm int32 [K] -> packed weight."""
+    out = torch.empty(_lib.ksq_w4a16_packed_weight_bytes(1, K, N), dtype=torch.uint8, device=qweight.device)
+    _l.check(_lib.ksq_w4a16_repack_act_order(_ptr(qweight), _ptr(perm), _ptr(out), K, N, _stream()))
+    return out
+
+
+def permute_columns(x, perm, out=None):
+    """out[r, j] = x[r, perm[j]]."""
+    m, k = x.shape
+    if out is None:
+        out = torch.empty_like(x)
+    _l.check(_lib.ksq_permute_columns(_ptr(x), _ptr(perm), _ptr(out), m, k, _dt(x), _stream()))
+    return out

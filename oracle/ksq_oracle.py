@@ -400,3 +400,17 @@ def moe_fp8_forward(x_bits, w13, w13_scale, w2, w2_scale, topk_ids, topk_w, dtyp
             c3[slots] = fp8_blockwise_gemm(a2_q[slots], a2_s[slots], w2[e], w2_scale[e], False) * tw[slots, None]
     c3b = to_bits(c3, dtype).reshape(T, topk, -1)
     return moe_sum(c3b, dtype)
+
+
+def gptq_act_order_gemm(x_bits, codes, scales_bits, g_idx, dtype, zeros=None):
+    """GPTQ with act-order, by its definition: input channel k belongs to quantization group g_idx[k], so
+    W[k, n] = (code[k, n] - zp[g_idx[k], n]) * scale[g_idx[k], n] (zp = 8 without zero points) and y = x . W.
+    The reference reaches the same product by sorting the rows by g_idx and permuting the activations
+    (S/models/quant/marlin_utils.cpp:106-122, K/gptq_marlin/gptq_marlin.cu act_order path); this function does neither.
+    numpy, double accumulation: for test sizes."""
+    x = from_bits(np.asarray(x_bits), dtype).astype(np.float64)
+    sc = from_bits(np.asarray(scales_bits), dtype).astype(np.float64)
+    g = np.asarray(g_idx).astype(np.int64)
+    z = 8.0 if zeros is None else np.asarray(zeros).astype(np.float64)[g]
+    w = (np.asarray(codes).astype(np.float64) - z) * sc[g]
+    return (x @ w).astype(np.float32)

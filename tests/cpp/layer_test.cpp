@@ -4,6 +4,7 @@
 //
 //   layer_test w4a16     <dir> <gptq|awq> <f16|bf16> <cutlass|marlin|machete> m n k group
 //   layer_test blockwise <dir> <f16|bf16> m n k fuse_silu_mul
+//   (w4a16: an optional trailing 1 = GPTQ act-order, g_idx.bin int32 [k])
 //   layer_test fp8_tensor <dir> <f16|bf16> m n k static
 //   layer_test moe       <dir> <f16|bf16> tokens experts hidden inter topk renorm scaling [groups topk_group scoring use_bias]
 //   layer_test moe_fp8   <dir> <f16|bf16> tokens experts hidden inter topk renorm scaling
@@ -87,6 +88,7 @@ static int RunW4A16(int argc, char** argv) {
   const std::string be = argv[5];
   const size_t m = std::atol(argv[6]), n = std::atol(argv[7]), k = std::atol(argv[8]), group = std::atol(argv[9]);
   LinearComputeBackend backend = be == "marlin" ? MARLIN_LINEAR_BACKEND : be == "machete" ? MACHETE_LINEAR_BACKEND : CUTLASS_LINEAR_BACKEND;
+  const bool desc_act = argc > 10 && std::atoi(argv[10]) != 0;  // GPTQ act-order: g_idx.bin int32 [k]
 
   hipStream_t stream;
   HIP_OK(hipStreamCreate(&stream));
@@ -95,6 +97,7 @@ static int RunW4A16(int argc, char** argv) {
   mc.is_quant = true;
   mc.quant_config.method = awq ? QUANT_AWQ : QUANT_GPTQ;
   mc.quant_config.group_size = group;
+  mc.quant_config.desc_act = desc_act;
   RuntimeConfig rc;
   rc.inter_data_type = T;
   rc.max_step_token_num = m;
@@ -103,7 +106,10 @@ static int RunW4A16(int argc, char** argv) {
   Tensor scales = Upload(dir + "/scales.bin", T, {k / group, n});
   Tensor qzeros;
   if (awq) qzeros = Upload(dir + "/qzeros.bin", TYPE_INT32, {k / group, n / 8});
-  Tensor weight = PackGroupQuantWeight(qweight, scales, awq ? &qzeros : nullptr, mc.quant_config.method, group, 0, stream);
+  Tensor g_idx;
+  if (desc_act) g_idx = Upload(dir + "/g_idx.bin", TYPE_INT32, {k});
+  Tensor weight = PackGroupQuantWeight(qweight, scales, awq ? &qzeros : nullptr, mc.quant_config.method, group, 0, stream,
+                                       desc_act ? &g_idx : nullptr);
 
   MatMulLayerFactory factory(mc, rc, 0, context);
   auto layer = factory.CreateLayer(TYPE_I4_GROUP, T, T, factory.GroupMatMulParams(n, k, true), mc.quant_config.method, backend);
@@ -304,11 +310,21 @@ static int RunErrors() {
     CutlassMatMulLayer layer;
     expect(!layer.Init({size_t(1)}, rc, context, 0).OK(), "short parameter list is rejected");
   }
-  // act-order rejected
+  // act-order: accepted with the whole K range, rejected for a K slice and for AWQ; its workspace holds the
+  // permuted activations
   {
-    MarlinMatMulLayer layer;
+    MarlinMatMulLayer layer, sliced, awq, plain;
     std::vector<std::any> p{size_t(16), size_t(256), size_t(256), size_t(128), false, true, true, true, TYPE_I4_GROUP};
-    expect(!layer.Init(p, rc, context, 0).OK(), "desc_act is rejected");
+    expect(layer.Init(p, rc, context, 0).OK(), "desc_act init");
+    p[5] = false;
+    expect(plain.Init(p, rc, context, 0).OK(), "plain gptq init");
+    expect(layer.GetWorkspaceSize() >= plain.GetWorkspaceSize() + 16 * 256 * 2, "desc_act workspace holds permuted x");
+    p[5] = true;
+    p[6] = false;
+    expect(!sliced.Init(p, rc, context, 0).OK(), "desc_act with a K slice is rejected");
+    p[6] = true;
+    p[4] = true;
+    expect(!awq.Init(p, rc, context, 0).OK(), "desc_act with AWQ is rejected");
   }
   // wrong weight data type surfaces in GetWorkspaceSize, as in the reference
   {

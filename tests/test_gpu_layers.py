@@ -56,6 +56,21 @@ def test_w4a16_layers(tmp_path, method, dtype, backend, m, n, k, group):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("dtype,backend,m,n,k", [(H.F16, "marlin", 3, 512, 1024), (H.BF16, "machete", 100, 1024, 512)])
+def test_w4a16_layer_act_order(tmp_path, oracle, dtype, backend, m, n, k):
+    d = H.make_w4a16(9050 + m, m, n, k, 128, dtype, False)
+    g_idx = (torch.randperm(k, generator=H.gen(9060 + k)) // 128).to(torch.int32)
+    d["qweight"].numpy().tofile(tmp_path / "qweight.bin")
+    H.bits_of(d["scales"]).tofile(tmp_path / "scales.bin")
+    H.bits_of(d["x"]).tofile(tmp_path / "x.bin")
+    g_idx.numpy().tofile(tmp_path / "g_idx.bin")
+    run_driver("w4a16", tmp_path, "gptq", TNAME[dtype], backend, m, n, k, 128, 1)
+    y = read_out(tmp_path / "y.bin", dtype, (m, n))
+    ref = oracle.gptq_act_order_gemm(H.bits_of(d["x"]), d["codes"], H.bits_of(d["scales"]), g_idx.numpy(), dtype)
+    H.check_gemm(y, ref, dtype, "%s act-order layer" % backend, weights_rounded=m > 32)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("dtype,m,n,k,fuse", [(H.BF16, 5, 512, 1024, 0), (H.F16, 33, 256, 512, 0), (H.BF16, 16, 512, 1024, 1)])
 def test_blockwise_layer(tmp_path, oracle, dtype, m, n, k, fuse):
     g = H.gen(9100 + m)

@@ -147,3 +147,25 @@ def test_bad_arguments(ops):
     with pytest.raises(L.KsqError) as e:
         ops.w4a16_gemm(x, w, w, None, 16, 128, 100)
     assert e.value.code == 2
+
+
+# GPTQ act-order (desc_act): rows sorted by g_idx at repack time, activations permuted in front of the GEMM
+@pytest.mark.parametrize("dtype", [H.F16, H.BF16])
+@pytest.mark.parametrize("M,N,K", [(1, 256, 512), (16, 4096, 1024), (70, 512, 2048)])
+def test_gptq_act_order(ops, oracle, dtype, M, N, K):
+    from ksanallm_amd import lib as L
+    d = H.make_w4a16(3500 + M + N, M, N, K, 128, dtype, awq=False)
+    g = H.gen(3600 + K)
+    g_idx = (torch.randperm(K, generator=g) // 128).to(torch.int32)
+    perm = ops.sort_g_idx(g_idx.cuda())
+    assert torch.equal(g_idx.cuda()[perm.long()], (torch.arange(K, device="cuda") // 128).to(torch.int32))
+    wp = ops.repack_weight_act_order(d["qweight"].cuda(), perm, K, N)
+    # the packed weight is the plain repack of the row-sorted checkpoint, bit for bit
+    sorted_q = torch.from_numpy(oracle.gptq_pack(d["codes"][perm.cpu().numpy()]).view(np.int32))
+    assert torch.equal(wp, ops.repack_weight(sorted_q.cuda(), L.SRC_GPTQ, 1, K, N))
+    sp = ops.repack_scales(d["scales"].cuda(), L.SCALE_GN, 1, K, N, 128)
+    xp = ops.permute_columns(d["x"].cuda(), perm)
+    assert torch.equal(xp.cpu(), d["x"][:, perm.cpu().long()])
+    y = ops.w4a16_gemm(xp, wp, sp, None, N, K, 128)
+    ref = oracle.gptq_act_order_gemm(H.bits_of(d["x"]), d["codes"], H.bits_of(d["scales"]), g_idx.numpy(), dtype)
+    H.check_gemm(y, ref, dtype, "act-order M=%d" % M, weights_rounded=M > 32)

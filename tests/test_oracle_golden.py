@@ -437,3 +437,29 @@ def test_fp8_tensor_gemm_vs_torch(oracle):
     out = oracle.fp8_tensor_gemm(a.numpy(), 0.01, b.numpy(), 0.002)
     ref = (a.view(torch.float8_e4m3fn).double() @ b.view(torch.float8_e4m3fn).double().T) * np.float32(0.01) * np.float32(0.002)
     np.testing.assert_allclose(out, ref.numpy(), rtol=1e-6)
+
+
+def test_act_order_definition(oracle):
+    g = torch.Generator().manual_seed(11)
+    K, N, M, group = 256, 32, 3, 128
+    codes = torch.randint(0, 16, (K, N), generator=g, dtype=torch.uint8).numpy()
+    scales = H.uniform(g, (K // group, N), 0.004, 0.02, H.F16)
+    x = torch.randn((M, K), generator=g).to(torch.float16)
+    # without act-order (g_idx = k // group) the definition is the plain group-wise GEMM
+    plain = oracle.w4a16_gemm(H.bits_of(x), codes, H.bits_of(scales), None, group, H.F16)
+    same = oracle.gptq_act_order_gemm(H.bits_of(x), codes, H.bits_of(scales), np.arange(K) // group, H.F16)
+    np.testing.assert_allclose(same, plain, rtol=2e-5, atol=2e-5)
+    # with a shuffled g_idx: brute force, element by element
+    g_idx = (torch.randperm(K, generator=g) // group).numpy()
+    y = oracle.gptq_act_order_gemm(H.bits_of(x), codes, H.bits_of(scales), g_idx, H.F16)
+    xs, ss = x.double().numpy(), scales.double().numpy()
+    brute = np.zeros((M, N))
+    for m in range(M):
+        for n in range(N):
+            brute[m, n] = sum(xs[m, k] * (float(codes[k, n]) - 8.0) * ss[g_idx[k], n] for k in range(K))
+    np.testing.assert_allclose(y, brute, rtol=1e-6, atol=1e-6)
+    # sorting the rows by g_idx and permuting x the same way (what the GPU path does) gives the same product
+    perm = np.argsort(g_idx, kind="stable")
+    assert np.array_equal(g_idx[perm], np.arange(K) // group)
+    moved = oracle.w4a16_gemm(H.bits_of(x[:, torch.from_numpy(perm)].contiguous()), codes[perm], H.bits_of(scales), None, group, H.F16)
+    np.testing.assert_allclose(moved, y, rtol=2e-5, atol=2e-5)
