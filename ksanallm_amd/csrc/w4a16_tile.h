@@ -69,11 +69,15 @@ struct Dequant<F16, HAS_ZP> {
   }
   __device__ __forceinline__ F16::frag operator()(uint32_t w) const {
     const h2 sixteenth{static_cast<_Float16>(0.0625f), static_cast<_Float16>(0.0625f)};
-    const uint32_t lo0 = (w & 0x000f000fu) | 0x64006400u;   // k = 0,1 : 1024 + code
-    const uint32_t hi0 = (w & 0x00f000f0u) | 0x64006400u;   // k = 2,3 : 1024 + 16*code
+    // (x & mask) | magic in one instruction: on this ISA the three-operand form takes no literal, so the mask comes
+    // from a scalar register and the magic from a vector register
+    const uint32_t magic = 0x64006400u;
     const uint32_t w8 = w >> 8;
-    const uint32_t lo1 = (w8 & 0x000f000fu) | 0x64006400u;  // k = 4,5
-    const uint32_t hi1 = (w8 & 0x00f000f0u) | 0x64006400u;  // k = 6,7
+    uint32_t lo0, hi0, lo1, hi1;
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(lo0) : "v"(w), "s"(0x000f000fu), "v"(magic));   // k = 0,1 : 1024 + code
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(hi0) : "v"(w), "s"(0x00f000f0u), "v"(magic));   // k = 2,3 : 1024 + 16*code
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(lo1) : "v"(w8), "s"(0x000f000fu), "v"(magic));  // k = 4,5
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(hi1) : "v"(w8), "s"(0x00f000f0u), "v"(magic));  // k = 6,7
     h2 r0 = (__builtin_bit_cast(h2, lo0) - c1) * s2;
     h2 r1 = (__builtin_bit_cast(h2, hi0) * sixteenth - c16) * s2;
     h2 r2 = (__builtin_bit_cast(h2, lo1) - c1) * s2;
@@ -99,14 +103,23 @@ struct Dequant<BF16, HAS_ZP> {
     b2 r = __builtin_convertvector(f2{a, c}, b2);
     return __builtin_bit_cast(uint32_t, r);
   }
+  // byte j of a dword as a float: one instruction (written out, because from `(e >> 8) & 0xff` the compiler builds a
+  // bit-field extract per code plus a conversion, twice the instructions)
+  template <int J>
+  static __device__ __forceinline__ float byte_to_float(uint32_t v) {
+    float f;
+    if (J == 0) asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(f) : "v"(v));
+    if (J == 1) asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(f) : "v"(v));
+    if (J == 2) asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(f) : "v"(v));
+    if (J == 3) asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(f) : "v"(v));
+    return f;
+  }
   __device__ __forceinline__ BF16::frag operator()(uint32_t w) const {
     // nibble p holds k = {0,2,4,6,1,3,5,7}[p]: even nibbles p=0,2,4,6 -> k=0,4,1,5 ; odd p=1,3,5,7 -> k=2,6,3,7
     const uint32_t e = w & 0x0f0f0f0fu;
     const uint32_t o = (w >> 4) & 0x0f0f0f0fu;
-    const float k0 = static_cast<float>(e & 0xffu), k4 = static_cast<float>((e >> 8) & 0xffu);
-    const float k1 = static_cast<float>((e >> 16) & 0xffu), k5 = static_cast<float>(e >> 24);
-    const float k2 = static_cast<float>(o & 0xffu), k6 = static_cast<float>((o >> 8) & 0xffu);
-    const float k3 = static_cast<float>((o >> 16) & 0xffu), k7 = static_cast<float>(o >> 24);
+    const float k0 = byte_to_float<0>(e), k4 = byte_to_float<1>(e), k1 = byte_to_float<2>(e), k5 = byte_to_float<3>(e);
+    const float k2 = byte_to_float<0>(o), k6 = byte_to_float<1>(o), k3 = byte_to_float<2>(o), k7 = byte_to_float<3>(o);
     u32x4 v;
     v.x = pk(__builtin_fmaf(k0, s, b), __builtin_fmaf(k1, s, b));
     v.y = pk(__builtin_fmaf(k2, s, b), __builtin_fmaf(k3, s, b));
@@ -300,12 +313,15 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
   constexpr int DEPTH = 4;
   static_assert(WM % DEPTH == 0, "the A prefetch ring must divide the row tiles");
   u32x4 abuf[DEPTH];
-  typename T::frag bcur[WN], bnext[WN];
+  typename T::frag bfrag[2][WN];  // weight fragments of the current step [g % 2] and the next one
   Dequant<T, HAS_ZP> dq[WN];
 
   auto frag_ptr = [&](uint32_t slot, int ks) { return lds + slot * STAGE_BYTES + ks * 1024 + a_rd; };
   // `wn`/`dn`: weight slot and dword (32-k block of its k-tile) the NEXT step uses
-  auto step = [&](uint32_t slot, int ks, WSlot (&wn)[WN], int dn) {
+  auto step = [&](auto parity, uint32_t slot, int ks, WSlot (&wn)[WN], int dn) {
+    constexpr int P = decltype(parity)::value;
+    typename T::frag(&bcur)[WN] = bfrag[P];
+    typename T::frag(&bnext)[WN] = bfrag[P ^ 1];
     const char* cur = frag_ptr(slot, ks);
     const char* nxt = ks == 0 ? frag_ptr(slot, 1) : frag_ptr((slot + 1) % NS, 0);
     if (dn == 0) {
@@ -324,9 +340,9 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
       if (i == WM / 2 + 1) bnext[1] = dq[1](wn[1].wq[dn]);
       __builtin_amdgcn_sched_barrier(0x6);  // VALU / SALU may move; LDS reads and MFMAs keep this order
     }
-#pragma unroll
-    for (int t = 0; t < WN; ++t) bcur[t] = bnext[t];
   };
+  using Even = std::integral_constant<int, 0>;
+  using Odd = std::integral_constant<int, 1>;
 
   // ---- schedule.  One synchronisation point per stage, in its middle ("sync c" sits between the two steps of
   // stage c): wait for x stage c+1, barrier, then issue [weights of k-tile c/2+2 when c is even][x stage c+3] - the LDS
@@ -346,7 +362,7 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
 #pragma unroll
   for (int t = 0; t < WN; ++t) {
     dq[t].set(ring[0][t].sc, ring[0][t].zp);
-    bcur[t] = dq[t](ring[0][t].wq[0]);
+    bfrag[0][t] = dq[t](ring[0][t].wq[0]);
   }
 #pragma unroll
   for (int j = 0; j < DEPTH; ++j) abuf[j] = *reinterpret_cast<const u32x4*>(frag_ptr(0, 0) + j * 2048);
@@ -359,7 +375,7 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
       constexpr int kDummy = 0;
       (void)kDummy;
       // first step of the stage: k block 2*(u%2) of k-tile u/2; the next step uses block 2*(u%2)+1 of the same tile
-      if (s < stages) step(slot, 0, ring[(u / 2) % 3], 2 * (u % 2) + 1);
+      if (s < stages) step(Even{}, slot, 0, ring[(u / 2) % 3], 2 * (u % 2) + 1);
       // sync s
       if (u % 2 == 0) {
         wait_tie(WaitEven{}, ring[(u / 2 + 1) % 3]);  // k-tile s/2+1, issued at sync s-2
@@ -372,9 +388,9 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
       // second step: the next step is block 2 of this k-tile (u even) or block 0 of the next k-tile (u odd)
       if (s < stages) {
         if (u % 2 == 0)
-          step(slot, 1, ring[(u / 2) % 3], 2);
+          step(Odd{}, slot, 1, ring[(u / 2) % 3], 2);
         else
-          step(slot, 1, ring[(u / 2 + 1) % 3], 0);
+          step(Odd{}, slot, 1, ring[(u / 2 + 1) % 3], 0);
       }
     }
   }
