@@ -35,4 +35,19 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float* __restr
   *reinterpret_cast<u32x4*>(y + static_cast<size_t>(row) * N + col) = o;
 }
 
+// Second pass of the decode kernel when K is cut over workgroups: y[i] = T(sum over parts of partial[s][i]), parts in
+// order, 4 outputs per thread (m*n is a multiple of 16).
+template <typename T>
+__global__ void __launch_bounds__(256) parts_reduce_kernel(const float* __restrict__ partial, uint16_t* __restrict__ y,
+                                                           size_t mn, uint32_t parts) {
+  const size_t i = (static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x) * 4;
+  if (i >= mn) return;
+  f32x4 a = *reinterpret_cast<const f32x4*>(partial + i);
+  for (uint32_t s = 1; s < parts; ++s) a += *reinterpret_cast<const f32x4*>(partial + s * mn + i);
+  u32x2 o;
+  o.x = pack2(T::from_float(a[0]), T::from_float(a[1]));
+  o.y = pack2(T::from_float(a[2]), T::from_float(a[3]));
+  *reinterpret_cast<u32x2*>(y + i) = o;
+}
+
 }  // namespace ksq

@@ -8,6 +8,7 @@ struct SplitKChoice {
   int mt;     // 16-row tiles of x per workgroup
   int nt;     // 16-column tiles per workgroup
   int waves;  // wavefronts per workgroup; wavefront w takes every waves-th k-tile
+  int parts;  // workgroups along K (1: the whole of K in one workgroup); > 1 needs parts*m*n fp32 of workspace
 };
 
 // m rows in one dense GEMM

@@ -13,9 +13,30 @@ static constexpr int kNumCU = 256;
 // - NT, the column tiles a wavefront streams per k-tile, as wide as the register file allows (8 for one 16-row tile
 //   of x, 4 for two) while the grid still has about one workgroup per CU: the x fragments and the sum-of-x MFMA are
 //   shared by the NT tiles, which also divides the x traffic out of L2 by NT.
+// Dense form only: with a long K and few columns (k >= 2n: down / o projections) the grid-fill rule ends at narrow
+// workgroups, every one of which fetches all of x - more bytes out of the L2 than the weights out of HBM once there are
+// several rows.  Then 4 column tiles share the x fragments and K is cut over 2..8 workgroups to bring the workgroup
+// count back to 160 or more (fp32 partial sums through the workspace, one small second pass).  The same helps when a
+// wavefront's share of K is very long (k > 16384).  Measured on MI355X, e.g. n=4096 k=14336 m=32: 28 -> 16 us.
 SplitKChoice select_splitk(size_t m, size_t n, size_t k) {
   const int mt = m <= 16 ? 1 : 2;
-  return select_splitk_blocks(mt, div_up(m, 16 * mt), n, k);
+  const size_t m_blocks = div_up(m, 16 * mt);
+  SplitKChoice c = select_splitk_blocks(mt, m_blocks, n, k);
+  const size_t strips = n / 16;
+  if (k >= 2 * n && strips % 4 == 0 && c.nt < 4) {
+    const size_t rows = m < static_cast<size_t>(16 * mt) ? m : static_cast<size_t>(16 * mt);
+    const size_t x_bytes = rows * k * 2 * (strips / c.nt) * m_blocks;
+    if (x_bytes > k * n / 2 || k > 16384) {
+      int parts = 2;
+      while (parts < 8 && strips / 4 * m_blocks * parts < 160) parts *= 2;
+      while (parts > 1 && k / 128 / parts < 8) parts /= 2;
+      if (parts > 1) {
+        c.nt = 4;
+        c.parts = parts;
+      }
+    }
+  }
+  return c;
 }
 
 SplitKChoice select_splitk_blocks(int mt, size_t m_blocks, size_t n, size_t k) {
@@ -23,6 +44,7 @@ SplitKChoice select_splitk_blocks(int mt, size_t m_blocks, size_t n, size_t k) {
   c.mt = mt;
   c.waves = 4;
   c.nt = 1;
+  c.parts = 1;
   const size_t n_tiles = n / 16;
   for (int nt = (mt == 1 ? 8 : 4); nt > 1; nt >>= 1) {
     if (n_tiles % nt == 0 && n_tiles / nt * m_blocks >= static_cast<size_t>(kNumCU) * 3 / 4) {
@@ -162,8 +184,8 @@ KSQ_EXPORT int ksq_select_tile(int kind, size_t m, size_t n, size_t k, int dtype
       d->block_n = 16 * c.nt;
       d->block_k = 128;
       d->waves = c.waves;
-      d->split_k = c.waves;
-      d->grid = static_cast<int32_t>((n / 16 / c.nt) * div_up(m, 16 * c.mt));
+      d->split_k = c.waves * c.parts;
+      d->grid = static_cast<int32_t>((n / 16 / c.nt) * div_up(m, 16 * c.mt) * c.parts);
       return KSQ_OK;
     }
     case KSQ_KIND_FP8_BLOCKWISE: {

@@ -14,7 +14,8 @@ namespace {
 
 template <typename T, int MT, int NT, int WAVES, int GROUP, bool HAS_ZP, bool GROUPED>
 void launch_splitk(const SplitKParams& p, uint32_t m_blocks, hipStream_t s) {
-  dim3 grid(p.N / 16 / NT, m_blocks, 1);
+  const uint32_t parts = (GROUPED || !p.partial) ? 1u : static_cast<uint32_t>(div_up(p.K / 128, p.kt_per_part));
+  dim3 grid(p.N / 16 / NT, m_blocks, parts);
   // ring depth in k-tiles and the wavefronts per SIMD the register budget is cut for
   constexpr int LOOK = GROUP != 128 ? 2 : (MT == 1 ? (NT == 1 ? 4 : (NT == 2 ? 3 : 2)) : (NT <= 2 ? 2 : 1));
   constexpr int OCC = (GROUP == 128 && MT == 1 && NT == 1) ? 4 : ((GROUP == 128 && MT == 1 && NT == 2) ? 3 : 2);
@@ -153,9 +154,19 @@ using namespace ksq;
 
 KSQ_EXPORT size_t ksq_w4a16_workspace_size(size_t max_m, size_t n, size_t k, size_t group, int dtype) {
   (void)dtype;
-  // the decode kernel reduces inside a workgroup; only the split-K form of the tile kernel needs fp32 partials
+  // fp32 partials: the decode kernel when it cuts K over workgroups, the tile kernel for the tiles it cuts along K
   if (n == 0 || k == 0 || k % 128 != 0) return 0;
   size_t need = 0;
+  // decode kernel: partial sums when K is cut over workgroups
+  if (group == 128) {
+    for (size_t m = 1; m <= max_m && m <= 32; ++m) {
+      const SplitKChoice c = select_splitk(m, n, k);
+      if (c.parts > 1) {
+        const size_t bytes = static_cast<size_t>(c.parts) * m * n * sizeof(float);
+        need = bytes > need ? bytes : need;
+      }
+    }
+  }
   // the plan is the same for all m of a band of 128 rows
   for (size_t band_end = 128; max_m > 32; band_end += 128) {
     const size_t m = band_end < max_m ? band_end : max_m;
@@ -211,12 +222,30 @@ KSQ_EXPORT int ksq_w4a16_gemm(void* y, const void* x, const void* w_packed, cons
     return check_launch(fn);
   }
   SplitKChoice c = select_splitk(m, n, k);
-  if (const char* f = getenv("KSQ_FORCE_SPLITK")) sscanf(f, "%d,%d,%d", &c.mt, &c.nt, &c.waves);
   const size_t m_blocks = div_up(m, 16 * c.mt);
   if (m_blocks > 65535) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: m too large for the decode kernel", fn);
+  p.partial = nullptr;
+  p.kt_per_part = static_cast<uint32_t>(k / 128);
+  if (c.parts > 1 && group == 128) {
+    const size_t need = static_cast<size_t>(c.parts) * m * n * sizeof(float);
+    if (!workspace || workspace_bytes < need || !aligned16(workspace))
+      return fail(KSQ_ERR_WORKSPACE, "%s: m=%zu n=%zu k=%zu needs %zu bytes of 16-byte aligned workspace, got %zu", fn, m, n,
+                  k, need, workspace ? workspace_bytes : size_t(0));
+    p.partial = static_cast<float*>(workspace);
+    p.kt_per_part = static_cast<uint32_t>(div_up(k / 128, c.parts));
+  }
   int rc = dtype == KSQ_F16 ? dispatch_tile<F16, false>(p, c, static_cast<uint32_t>(m_blocks), group, as_stream(stream))
                             : dispatch_tile<BF16, false>(p, c, static_cast<uint32_t>(m_blocks), group, as_stream(stream));
   if (rc) return rc;
+  if (p.partial) {
+    const size_t mn = m * n;
+    const uint32_t parts = static_cast<uint32_t>(div_up(k / 128, p.kt_per_part));
+    const unsigned blocks = static_cast<unsigned>(div_up(mn, 256 * 4));
+    if (dtype == KSQ_F16)
+      parts_reduce_kernel<F16><<<blocks, 256, 0, as_stream(stream)>>>(p.partial, static_cast<uint16_t*>(y), mn, parts);
+    else
+      parts_reduce_kernel<BF16><<<blocks, 256, 0, as_stream(stream)>>>(p.partial, static_cast<uint16_t*>(y), mn, parts);
+  }
   return check_launch(fn);
 }
 

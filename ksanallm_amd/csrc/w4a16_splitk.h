@@ -3,6 +3,8 @@
 // Work decomposition
 //   grid.x : groups of NT column tiles (16 output columns each)
 //   grid.y : blocks of MT*16 rows of x (MoE: aligned blocks of sorted slots, one expert each)
+//   grid.z : parts of K (dense form, shapes with few columns and a long K: wide workgroups share the x fragments over
+//            NT column tiles, and the parts of K bring the number of workgroups back up)
 // Wavefront w of a workgroup takes the 128-wide k-tiles w, w+WAVES, ...
 // Per k-tile a wavefront loads the x operand once (MT*4 fragments of 16 bytes per lane) and streams the NT weight
 // tiles of that k-tile, one coalesced 1 KiB wavefront load each.  Every packed dword becomes an MFMA operand holding
@@ -40,6 +42,10 @@ struct SplitKParams {
   const int32_t* num_post_pad;
   const float* topk_w;
   uint32_t numel, top_k;
+  // K cut over grid.z workgroups as well (dense form): part z covers k-tiles [z*kt_per_part, ...) and writes fp32
+  // partial sums [z][M][N] instead of the output; a second pass adds them up
+  float* partial;
+  uint32_t kt_per_part;
   uint32_t x_bytes;  // extent of x, below 1 GiB
   uint32_t nibble_mask, magic2;  // 0x000f000f and T::kMagic2, passed in so that they live in registers
 };
@@ -141,8 +147,8 @@ __global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKPar
   struct KOff {
     uint32_t w, s, z, x;
   };
-  const uint32_t kt_begin = 0;
-  const uint32_t kt_end = KT;
+  const uint32_t kt_begin = GROUPED ? 0 : blockIdx.z * p.kt_per_part;
+  const uint32_t kt_end = GROUPED ? KT : ((KT - kt_begin) < p.kt_per_part ? KT : kt_begin + p.kt_per_part);
   auto koff = [&](uint32_t round) {
     const uint32_t kt = kt_begin + wave + round * WAVES;
     const bool ok = kt < kt_end;
@@ -271,7 +277,12 @@ __global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKPar
         orow = blockIdx.y * (16 * MT) + r;
         valid = orow < p.M;
       }
-      if (valid) static_cast<uint16_t*>(p.y)[static_cast<size_t>(orow) * p.N + col] = T::from_float(v[i] * rw);
+      if (valid) {
+        if (!GROUPED && p.partial)
+          p.partial[(static_cast<size_t>(blockIdx.z) * p.M + orow) * p.N + col] = v[i];
+        else
+          static_cast<uint16_t*>(p.y)[static_cast<size_t>(orow) * p.N + col] = T::from_float(v[i] * rw);
+      }
     }
   }
 }

@@ -169,3 +169,25 @@ def test_gptq_act_order(ops, oracle, dtype, M, N, K):
     y = ops.w4a16_gemm(xp, wp, sp, None, N, K, 128)
     ref = oracle.gptq_act_order_gemm(H.bits_of(d["x"]), d["codes"], H.bits_of(d["scales"]), g_idx.numpy(), dtype)
     H.check_gemm(y, ref, dtype, "act-order M=%d" % M, weights_rounded=M > 32)
+
+
+# decode regime, long K and few columns: four column tiles per workgroup and K cut over workgroups (fp32 partials
+# through the workspace, second pass)
+@pytest.mark.parametrize("dtype,awq", [(H.F16, False), (H.BF16, True)])
+@pytest.mark.parametrize("M,N,K", [(8, 256, 2048), (16, 4096, 14336), (32, 1024, 4096), (1, 512, 25600)])
+def test_decode_k_parts(ops, dtype, awq, M, N, K):
+    from ksanallm_amd import lib as L
+    desc = L.select_tile(L.KIND_W4A16, M, N, K, dtype)
+    assert desc["kernel"] == 0 and desc["block_n"] == 64 and desc["split_k"] > desc["waves"]
+    parts = desc["split_k"] // desc["waves"]
+    assert L.load().ksq_w4a16_workspace_size(M, N, K, 128, dtype) >= parts * M * N * 4
+    d = H.make_w4a16(3700 + M + N, M, N, K, 128, dtype, awq=awq, z_lo=0, z_hi=15)
+    y = run_case(ops, d)
+    H.check_gemm(y, H.w4a16_oracle(d), dtype, "decode K parts M=%d N=%d K=%d" % (M, N, K))
+    if awq:
+        wp = ops.repack_weight(d["qweight"].cuda(), L.SRC_AWQ, 1, K, N)
+        sp = ops.repack_scales(d["scales"].cuda(), L.SCALE_GN, 1, K, N, 128)
+        zp = ops.repack_zeros(d["qzeros"].cuda(), L.ZERO_AWQ_PACKED, K, N, 128)
+        with pytest.raises(L.KsqError) as e:
+            ops.w4a16_gemm(d["x"].cuda(), wp, sp, zp, N, K, 128, workspace=torch.empty(64, dtype=torch.uint8, device="cuda"))
+        assert e.value.code == 3
