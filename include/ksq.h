@@ -187,13 +187,16 @@ int ksq_moe_w4a16_gemm(void* out, const void* x, const void* w_packed, const voi
                        const void* num_post_pad, size_t numel, size_t top_k, size_t E, size_t n, size_t k,
                        size_t group, size_t block_m, int dtype, void* stream);
 
-/* Grouped blockwise-FP8 GEMM over the aligned blocks (block_m 16 or 32): for every valid sorted slot id s (< numel)
+/* Grouped blockwise-FP8 GEMM over the aligned blocks: for every valid sorted slot id s (< numel)
  *   out[s, :] = sum_kb (a_q[s / top_k, kb] . b[e, :, kb]) * a_s[kb, s / top_k] * b_s[e, :/128, kb] * (topk_w ? topk_w[s] : 1)
  * with e the expert of s's block.  a_q [a_rows, k] e4m3, a_s fp32 [a_rows, k/128] (the reference's layout) or, when
  * a_s_column_major, [k/128, a_rows] - the two layouts ksq_fp8_group_quant writes; b [E, n, k] e4m3 and b_s fp32 [E, ceil(n/128), k/128] in
  * checkpoint layout, out [numel, n] in out_dtype.  top_k = 1 reads a_q rows by slot (second MoE GEMM).
+ * block_m is the block size the permutation was aligned with: 16 or 32 run the streaming (decode) kernel, 256 the MFMA
+ * tile kernel; ksq_moe_fp8_block_m() gives the choice for a problem size.
  * Replaces the fp8_w8a8 block-quantized branch of InvokeFusedMoe's fused_moe_kernel launches
  * (S/kernels/nvidia/moe_kernel_wrapper.cpp:435-456, 498-522, 560-600). */
+size_t ksq_moe_fp8_block_m(size_t numel, size_t E);
 int ksq_moe_fp8_blockwise_gemm(void* out, const void* a_q, const void* a_s, int a_s_column_major, size_t a_rows, const void* b,
                                const void* b_s, const void* topk_w, const void* sorted_ids, const void* expert_ids,
                                const void* num_post_pad, size_t numel, size_t top_k, size_t E, size_t n, size_t k,

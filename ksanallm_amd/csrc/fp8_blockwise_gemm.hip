@@ -245,12 +245,54 @@ int launch_fp8_tile(const Fp8Params& q, const TilePlan& plan, float* partial, hi
   p.main_items = plan.main_items;
   p.splits = plan.splits;
   p.kb_per_split = plan.kt_per_split;
+  p.as_row_bytes = 4;
+  p.as_kb_bytes = 4 * q.M;
   fp8_tile_kernel<TO><<<plan.grid, 512, lds, s>>>(p);
   if (plan.splits > 1) {
     const unsigned cut = plan.tiles_m * plan.tiles_n - plan.main_items;
     splitk_reduce_kernel<TO, 256><<<cut * 32, 256, 0, s>>>(partial, static_cast<uint16_t*>(p.out), p.M, p.N, p.tiles_m, p.tiles_n,
                                                           p.main_items, p.splits);
   }
+  return KSQ_OK;
+}
+
+// grouped (MoE) form of the tile kernel: one 256-slot block of the aligned permutation per row tile
+template <typename TO>
+int launch_fp8_tile_grouped(const Fp8Params& q, unsigned blocks, hipStream_t s) {
+  constexpr int kLdsMax = 160 * 1024;
+  const size_t lds = 2 * 32 * 2048 + 2 * 1024 + 2 * static_cast<size_t>(q.K / 128) * 4;
+  if (lds > kLdsMax) return fail(KSQ_ERR_UNSUPPORTED, "k range of %u blocks per workgroup does not fit the LDS", q.K / 128);
+  static std::atomic<bool> configured{false};
+  if (!configured.load(std::memory_order_acquire)) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&fp8_tile_kernel<TO, true>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLdsMax);
+    if (e != hipSuccess) return fail(KSQ_ERR_LAUNCH, "hipFuncSetAttribute(LDS %d): %s", kLdsMax, hipGetErrorString(e));
+    configured.store(true, std::memory_order_release);
+  }
+  Fp8TileParams p{};
+  p.a = q.a;
+  p.a_s = q.a_s;
+  p.b = q.b;
+  p.b_s = q.b_s;
+  p.out = q.out;
+  p.M = q.M;
+  p.N = q.N;
+  p.K = q.K;
+  p.tiles_m = blocks;
+  p.tiles_n = static_cast<uint32_t>(div_up(q.N, 256));
+  p.main_items = 0;
+  p.splits = 1;
+  p.kb_per_split = q.K / 128;
+  p.as_row_bytes = q.as_row_stride * 4;
+  p.as_kb_bytes = q.as_kb_stride * 4;
+  p.sorted_ids = q.sorted_ids;
+  p.expert_ids = q.expert_ids;
+  p.num_post_pad = q.num_post_pad;
+  p.topk_w = q.topk_w;
+  p.numel = q.numel;
+  p.top_k = q.top_k;
+  p.scale_rows = q.scale_rows;
+  fp8_tile_kernel<TO, true><<<p.tiles_m * p.tiles_n, 512, lds, s>>>(p);
   return KSQ_OK;
 }
 
@@ -337,7 +379,8 @@ KSQ_EXPORT int ksq_moe_fp8_blockwise_gemm(void* out, const void* a_q, const void
   if (out_dtype != KSQ_F16 && out_dtype != KSQ_BF16)
     return fail(KSQ_ERR_UNSUPPORTED, "%s: output dtype must be f16 or bf16", fn);
   if (top_k == 0 || E == 0) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: top_k and E must be positive", fn);
-  if (block_m != 16 && block_m != 32) return fail(KSQ_ERR_UNSUPPORTED, "%s: block_m %zu not in {16,32}", fn, block_m);
+  if (block_m != 16 && block_m != 32 && block_m != 256)
+    return fail(KSQ_ERR_UNSUPPORTED, "%s: block_m %zu not in {16,32,256}", fn, block_m);
   if (numel == 0) return KSQ_OK;
   if (a_rows < (numel + top_k - 1) / top_k)
     return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: %zu activation rows cannot serve %zu slots of top_k %zu", fn, a_rows, numel, top_k);
@@ -359,8 +402,16 @@ KSQ_EXPORT int ksq_moe_fp8_blockwise_gemm(void* out, const void* a_q, const void
   p.scale_rows = static_cast<uint32_t>(div_up(n, 128));
   const int mt = block_m == 16 ? 1 : 2;
   const unsigned blocks = static_cast<unsigned>(cap_blocks);
-  int rc = out_dtype == KSQ_F16 ? dispatch_grouped<F16>(p, mt, blocks, as_stream(stream))
-                                : dispatch_grouped<BF16>(p, mt, blocks, as_stream(stream));
+  int rc;
+  if (block_m == 256) {  // prefill regime: MFMA tile kernel, rows gathered / scattered through the permutation
+    if (a_rows * k > 0xffffffffull || a_rows * (k / 128) * 4 > 0xffffffffull)
+      return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: activations too large", fn);
+    rc = out_dtype == KSQ_F16 ? launch_fp8_tile_grouped<F16>(p, blocks, as_stream(stream))
+                              : launch_fp8_tile_grouped<BF16>(p, blocks, as_stream(stream));
+  } else {
+    rc = out_dtype == KSQ_F16 ? dispatch_grouped<F16>(p, mt, blocks, as_stream(stream))
+                              : dispatch_grouped<BF16>(p, mt, blocks, as_stream(stream));
+  }
   if (rc) return rc;
   return check_launch(fn);
 }

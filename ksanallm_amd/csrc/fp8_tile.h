@@ -31,13 +31,24 @@ struct Fp8TileParams {
   uint32_t M, N, K;
   uint32_t tiles_m, tiles_n;
   uint32_t main_items, splits, kb_per_split;  // tile_work.h
+  uint32_t as_row_bytes, as_kb_bytes;  // a_s[row, kb] at row * as_row_bytes + kb * as_kb_bytes: (4, 4*M) in the dense form
+  // grouped (MoE) form: row block b = tile_m holds the slots sorted_ids[b*256 ..] of expert expert_ids[b]
+  const int32_t* sorted_ids;
+  const int32_t* expert_ids;
+  const int32_t* num_post_pad;
+  const float* topk_w;
+  uint32_t numel, top_k, scale_rows;  // scale_rows = ceil(N/128): rows of one expert's b_s
 };
 
 __device__ __forceinline__ f32x4 mfma_fp8_k128(i32x8 a, i32x8 b, f32x4 c) {
   return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
 }
 
-template <typename TO>
+// GROUPED: the MoE form.  Row block tile_m is one 256-slot block of the aligned permutation: slot s reads activation
+// row s / top_k (pad slots carry s >= numel) and that row's scales, weights and weight scales are those of expert
+// expert_ids[tile_m], results go to out[s, :] (times topk_w[s] when given).  Blocks past num_post_pad leave at once;
+// there is no cut along K in this form.
+template <typename TO, bool GROUPED = false>
 __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
   constexpr int WAVES_N = 4;
   constexpr int WM = 8, WN = 4;  // 16x16 tiles per wavefront: 128 tokens x 64 weight rows
@@ -70,16 +81,28 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
   // the memory pipeline runs at full rate).  Load lane j lands at 1024h + 16j = 1024h + 64*(j/4) + 16*(j%4) and
   // fetches piece (j%4) ^ (j/16) of row j/4, so that MFMA lane (row r, k slot q) finds its two pieces 2(q%2)+p at
   // 1024*(q/2) + 64r + 16*((2(q%2)+p) ^ (r/4)): the sixteen lanes that read together hit different bank groups.
+  size_t expert = 0;
+  if (GROUPED) {
+    if (m0 >= static_cast<uint32_t>(p.num_post_pad[0])) return;  // uniform: the whole workgroup leaves
+    expert = static_cast<size_t>(__builtin_amdgcn_readfirstlane(p.expert_ids[tile_m]));
+  }
   const bool stage_act = wave < 4;
   const uint32_t frag0 = (wave & 3) * 4;
-  const uint8_t* g_tile = stage_act ? p.a + static_cast<size_t>(m0) * p.K : p.b + static_cast<size_t>(n0) * p.K;
+  const uint8_t* g_tile = stage_act ? p.a + static_cast<size_t>(GROUPED ? 0 : m0) * p.K
+                                    : p.b + (expert * p.N + n0) * p.K;
   g_tile += static_cast<size_t>(kb_begin) * 128;
   const uint32_t row_limit = stage_act ? p.M - m0 : p.N - n0;  // rows of this tile inside the matrix
   uint32_t d_voff[4];
 #pragma unroll
   for (int f = 0; f < 4; ++f) {
     uint32_t row = (frag0 + f) * 16 + (lane >> 2);
-    row = row < row_limit ? row : row_limit - 1;  // rows past the edge repeat the last row; their results are dropped
+    if (GROUPED && stage_act) {
+      uint32_t sid = static_cast<uint32_t>(p.sorted_ids[m0 + row]);
+      sid = sid < p.numel ? sid : p.numel - 1;  // pad slots read some valid row; their results are dropped
+      row = sid / p.top_k;
+    } else {
+      row = row < row_limit ? row : row_limit - 1;  // rows past the edge repeat the last row; their results are dropped
+    }
     d_voff[f] = row * p.K + 16 * ((lane & 3) ^ (lane >> 4));
   }
   const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<size_t>((__attribute__((address_space(3))) char*)lds));
@@ -93,12 +116,19 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
   constexpr int BS_BASE = SCALE_BASE + 2 * 1024;
   // M % 4 == 0: wavefront 0 copies all 256 with one 16-byte-per-lane load (lanes whose four tokens lie past M repeat
   // the last four).  Otherwise wavefronts 0..3 copy 64 each, 4 bytes per lane, every lane clamped on its own.
-  const bool s_vec = (p.M & 3) == 0;
+  // (the one-load form needs the 256 scales of a k-block contiguous: dense form with token-contiguous scales)
+  const bool s_vec = !GROUPED && (p.M & 3) == 0 && p.as_row_bytes == 4;
   uint32_t s_row = s_vec ? m0 + 4 * lane : m0 + (wave & 3) * 64 + lane;
-  const uint32_t s_last = s_vec ? p.M - 4 : p.M - 1;
-  s_row = s_row < s_last ? s_row : s_last;
-  const uint32_t s_voff = s_row * 4;
-  const char* as_base = reinterpret_cast<const char*>(p.a_s) + static_cast<size_t>(kb_begin) * p.M * 4;
+  if (GROUPED) {
+    uint32_t sid = static_cast<uint32_t>(p.sorted_ids[s_row]);
+    sid = sid < p.numel ? sid : p.numel - 1;
+    s_row = sid / p.top_k;
+  } else {
+    const uint32_t s_last = s_vec ? p.M - 4 : p.M - 1;
+    s_row = s_row < s_last ? s_row : s_last;
+  }
+  const uint32_t s_voff = s_row * p.as_row_bytes;
+  const char* as_base = reinterpret_cast<const char*>(p.a_s) + static_cast<size_t>(kb_begin) * p.as_kb_bytes;
   const uint32_t s_lds = lds_base + SCALE_BASE + (s_vec ? 0 : (wave & 3) * 256);
   const uint32_t n_wave = n0 + wn * 64;
   {
@@ -107,7 +137,7 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
       const uint32_t blk = t / kb_count, kb = t - blk * kb_count;
       uint32_t nb = n0 / 128 + blk;
       nb = nb < nb_last ? nb : nb_last;
-      reinterpret_cast<float*>(lds + BS_BASE)[t] = p.b_s[static_cast<size_t>(nb) * KB + kb_begin + kb];
+      reinterpret_cast<float*>(lds + BS_BASE)[t] = p.b_s[(expert * p.scale_rows + nb) * KB + kb_begin + kb];
     }
   }
   const float* bs_lds = reinterpret_cast<const float*>(lds + BS_BASE) + (wn >> 1) * kb_count;
@@ -118,7 +148,7 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
   // passed whatever produced them.
   auto load_scales = [&](uint32_t kb) {
     const uint32_t k = kb < kb_count ? kb : kb_count - 1;
-    const char* ap = as_base + static_cast<size_t>(k) * p.M * 4;
+    const char* ap = as_base + static_cast<size_t>(k) * p.as_kb_bytes;
     const uint32_t d = __builtin_amdgcn_readfirstlane(s_lds + (kb & 1) * 1024);
     if (s_vec) {
       if (wave == 0)
@@ -232,16 +262,26 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
   // ---- store: lane holds token m = l%16 of the tile and weight rows (output columns) 4*(l/16) .. +3
 #pragma unroll
   for (int i = 0; i < WM; ++i) {
-    const uint32_t row = m0 + wm * 128 + i * 16 + lrow;
-    if (row < p.M) {
+    uint32_t row = m0 + wm * 128 + i * 16 + lrow;
+    bool live = row < p.M;
+    float rw = 1.0f;
+    if (GROUPED) {
+      const uint32_t sid = static_cast<uint32_t>(p.sorted_ids[row]);
+      live = sid < p.numel;
+      row = sid;
+      if (live && p.topk_w) rw = p.topk_w[sid];
+    }
+    if (live) {
 #pragma unroll
       for (int t = 0; t < WN; ++t) {
         const uint32_t ncol = n_wave + t * 16 + 4 * lq;
         if (ncol < p.N) {
-          if (direct) {
+          if (GROUPED || direct) {
+            f32x4 v = acc[t][i];
+            if (GROUPED) v *= rw;
             u32x2 o;
-            o.x = pack2(TO::from_float(acc[t][i][0]), TO::from_float(acc[t][i][1]));
-            o.y = pack2(TO::from_float(acc[t][i][2]), TO::from_float(acc[t][i][3]));
+            o.x = pack2(TO::from_float(v[0]), TO::from_float(v[1]));
+            o.y = pack2(TO::from_float(v[2]), TO::from_float(v[3]));
             *reinterpret_cast<u32x2*>(static_cast<uint16_t*>(p.out) + static_cast<size_t>(row) * p.N + ncol) = o;
           } else {
             float* dst = p.partial + ((static_cast<size_t>(slot) * p.splits + part) * BM + (row - m0)) * BN + (ncol - n0);

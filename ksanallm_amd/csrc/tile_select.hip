@@ -147,6 +147,15 @@ TilePlan plan_fp8_tile(size_t m, size_t n, size_t k) {
 
 using namespace ksq;
 
+// The same for block-fp8 experts (ksq_moe_fp8_blockwise_gemm): 16- and 32-row blocks stream through the split-K
+// kernel, from about 96 rows per expert 256-row blocks feed the MFMA tile kernel.
+KSQ_EXPORT size_t ksq_moe_fp8_block_m(size_t numel, size_t E) {
+  if (E == 0) return 16;
+  const size_t per_expert = numel / E;
+  if (per_expert >= 96) return 256;
+  return per_expert < 16 ? 16 : 32;
+}
+
 // Rows per expert block for numel routed (token, slot) pairs over E experts.  Replaces the M thresholds of
 // InvokeFusedMoe (16 / 32 / 64 rows by token count): below about 48 rows per expert the weights are streamed once per
 // 16- or 32-row block (HBM-bound); above, 128-row blocks feed the MFMA tile kernel.

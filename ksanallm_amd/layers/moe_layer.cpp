@@ -75,7 +75,7 @@ size_t MoeLayer::GetWorkspaceSize() {
   const size_t m = std::min(kChunk, max_token_num_);
   const size_t numel = m * expert_topk_;
   size_t capacity = 0;
-  for (size_t bm : {size_t(16), size_t(32), size_t(128)}) capacity = std::max(capacity, ksq_moe_align_capacity(numel, expert_num_per_node_, bm));
+  for (size_t bm : {size_t(16), size_t(32), size_t(128), size_t(256)}) capacity = std::max(capacity, ksq_moe_align_capacity(numel, expert_num_per_node_, bm));
   topk_weights_size_ = AlignAddress(max_token_num_ * expert_topk_ * sizeof(float));
   topk_ids_size_ = AlignAddress(max_token_num_ * expert_topk_ * sizeof(int32_t));
   // sorted_ids [capacity] + expert_ids [capacity / 16] + num_tokens_post_pad [1]

@@ -34,8 +34,8 @@ class MoeLayer : public BaseLayer {
   // rows per expert block for a chunk (InvokeFusedMoe picks 16 / 32 / 64 by token count; here the library decides by
   // rows per expert, which changes no result)
   size_t BlockM(size_t tokens) const {
-    const size_t bm = ksq_moe_block_m(tokens * expert_topk_, expert_num_per_node_);
-    return IsFp8() && bm > 32 ? 32 : bm;  // the grouped fp8 GEMM has 16- and 32-row blocks
+    if (IsFp8()) return ksq_moe_fp8_block_m(tokens * expert_topk_, expert_num_per_node_);
+    return ksq_moe_block_m(tokens * expert_topk_, expert_num_per_node_);
   }
   bool IsFp8() const { return compute_dtype_ == TYPE_BLOCK_FP8_E4M3; }
 

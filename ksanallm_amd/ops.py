@@ -269,7 +269,7 @@ def fused_moe_fp8_blockwise(x, w13, w13_scale, w2, w2_scale, topk_ids, topk_w, b
     inter = two_inter // 2
     numel = T * topk
     if block_m is None:
-        block_m = min(_lib.ksq_moe_block_m(numel, E), 32)
+        block_m = _lib.ksq_moe_fp8_block_m(numel, E)
     sorted_ids, expert_ids, npp = moe_align_block_size(topk_ids, E, block_m)
     tw = topk_w.reshape(-1).to(torch.float32).contiguous()
     a1_q, a1_s = per_token_group_quant_fp8(x, hidden, 128, False)

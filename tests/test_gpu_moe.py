@@ -236,7 +236,9 @@ def _fp8_experts(oracle, seed, E, n, k):
 
 @pytest.mark.parametrize("T,E,topk,n,k,bm,colmajor,with_w", [
     (1, 8, 2, 256, 256, 16, False, False), (70, 8, 2, 208, 384, 16, True, True), (300, 6, 3, 512, 1024, 32, False, True),
-    (33, 16, 4, 4096, 7168, 32, False, False)])
+    (33, 16, 4, 4096, 7168, 32, False, False),
+    # 256-slot blocks: the MFMA tile kernel in its grouped form (ragged n, both scale layouts, routing weight)
+    (300, 6, 3, 512, 1024, 256, False, True), (700, 4, 2, 784, 512, 256, True, False), (130, 2, 1, 256, 128, 256, False, True)])
 def test_grouped_fp8_gemm_stage(ops, oracle, T, E, topk, n, k, bm, colmajor, with_w):
     """One grouped blockwise-fp8 GEMM launch against the per-expert oracle GEMM on the codes the GPU quantizer wrote."""
     g = H.gen(7000 + T + n)
@@ -265,7 +267,8 @@ def test_grouped_fp8_gemm_stage(ops, oracle, T, E, topk, n, k, bm, colmajor, wit
 
 
 @pytest.mark.parametrize("dtype", [H.F16, H.BF16])
-@pytest.mark.parametrize("T,E,topk,hidden,inter", [(1, 8, 2, 256, 128), (48, 16, 4, 512, 256), (200, 8, 2, 384, 640)])
+@pytest.mark.parametrize("T,E,topk,hidden,inter", [(1, 8, 2, 256, 128), (48, 16, 4, 512, 256), (200, 8, 2, 384, 640),
+                                                   (1200, 8, 2, 512, 256)])   # the last: 300 slots per expert, 256-slot blocks
 def test_moe_fp8_block(ops, oracle, dtype, T, E, topk, hidden, inter):
     """Whole block-fp8 MoE block.  The silu*mul front end of the second quantization rounds through T once more than
     the oracle may (see the quantizer's fused test), so the block is compared at GEMM tolerance, not bit for bit."""
