@@ -32,10 +32,10 @@ CACHE_BYTES = 320 << 20                            # rotate through more than th
 # (`--calibrate-copy`): FETCH_SIZE reads half the bytes moved (x2.0), WRITE_SIZE reads them exactly (x1.0).
 # Keyed by (config, kernel variant); None where no counter run has been made for the current kernel.
 MEASURED_TRAFFIC = {
-    (2, "w4a16_splitk_kernel<16x16,w4>"): 31880000,
-    (2, "w4a16_splitk_kernel<16x64,w4>"): 31250000,
-    (2, "w4a16_splitk_kernel<32x16,w4>"): 38390000,
-    (2, "w4a16_splitk_kernel<32x64,w4>"): 33820000,
+    (1, "w4a16_splitk_kernel<16x16,w4>"): 9350000,
+    (2, "w4a16_splitk_kernel<16x16,w4>"): 31050000,
+    (2, "w4a16_splitk_kernel<16x64,w4>"): 31900000,
+    (2, "w4a16_splitk_kernel<32x64,w4>"): 37040000,
     (2, "w4a16_tile_kernel<128x256,w8>"): 84610000,
     (2, "w4a16_tile_kernel<256x256,w8>"): 216470000,
     (3, "w4a16_tile_kernel<256x256,w8>"): 1591160000,
