@@ -1,11 +1,11 @@
 // Prefill-regime W4A16 kernel (MFMA-bound): a workgroup of 8 wavefronts computes a BM x 256 output tile
-// (BM = 256 or 128) over a contiguous range of k-tiles (split-K across workgroups when the grid would not fill the chip).
+// (BM = 256 or 128) over all of K or, for tiles that are cut along K (tile_work.h), over a contiguous range of k-tiles.
 //
 //   - x (activations) goes global -> LDS without touching registers: every wavefront issues global_load_lds_dwordx4
 //     for whole 1 KiB MFMA fragments (16 rows x 32 k, four lanes per row so that every load touches 64 contiguous
 //     bytes per row, pieces swizzled so that the read-back is free of bank conflicts), into a ring of NS stages of
-//     64 k each.  The fragment is read back with one ds_read_b128 per lane, DEPTH fragments ahead of the MFMAs that use it.  Two to three stages are in flight
-//     while one is consumed; the one barrier per stage sits in the middle of the stage, so the fragment reads never
+//     64 k each.  The fragment is read back with one ds_read_b128 per lane, DEPTH fragments ahead of the MFMAs that
+//     use it.  Two to three stages are in flight while one is consumed; the one barrier per stage sits in the middle of the stage, so the fragment reads never
 //     drain at a stage boundary.
 //   - packed int4 weights never touch LDS: the 8 wavefronts split the 256 columns (2 column tiles of 16 each), so
 //     every weight fragment belongs to exactly one wavefront and no weight is dequantized twice.  A wavefront loads
@@ -18,8 +18,8 @@
 //   - the weights are the row operand of v_mfma_f32_16x16x32 and x the column operand, so a lane ends up with four
 //     consecutive output columns of one row and stores them as one 8-byte word (or 16 bytes of fp32 partials).
 //
-// Workgroup ids are remapped so that the workgroups running on one XCD at the same time form a compact block of
-// row tiles x column tiles: both operands are then shared through that XCD's L2.
+// Workgroup ids are remapped (tile_work.h) so that the workgroups running on one XCD at the same time form a compact
+// block of row tiles x column tiles: both operands are then shared through that XCD's L2.
 #pragma once
 
 #include <type_traits>
