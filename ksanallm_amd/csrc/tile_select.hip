@@ -157,12 +157,12 @@ KSQ_EXPORT size_t ksq_moe_fp8_block_m(size_t numel, size_t E) {
 }
 
 // Rows per expert block for numel routed (token, slot) pairs over E experts.  Replaces the M thresholds of
-// InvokeFusedMoe (16 / 32 / 64 rows by token count): below about 48 rows per expert the weights are streamed once per
+// InvokeFusedMoe (16 / 32 / 64 rows by token count): below about 64 rows per expert the weights are streamed once per
 // 16- or 32-row block (HBM-bound); above, 128-row blocks feed the MFMA tile kernel.
 KSQ_EXPORT size_t ksq_moe_block_m(size_t numel, size_t E) {
   if (E == 0) return 16;
   const size_t per_expert = numel / E;
-  if (per_expert >= 48) return 128;
+  if (per_expert >= 64) return 128;
   return per_expert < 16 ? 16 : 32;
 }
 
