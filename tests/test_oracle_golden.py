@@ -61,7 +61,7 @@ def test_e4m3_encode_rne_satfinite(oracle):
     np.testing.assert_array_equal(enc, expect)
     np.testing.assert_array_equal(oracle.f32_to_e4m3(np.nextafter(mid.astype(np.float32), np.float32(0))), lo)
     np.testing.assert_array_equal(oracle.f32_to_e4m3(np.nextafter(mid.astype(np.float32), np.float32(1e9))), lo + 1)
-    # SURVEY-noted library cross-check: 17->16, 19->20, 2^-10 -> 0, 1.5*2^-9 -> code 2
+    # round-to-nearest-even boundaries: 17->16, 19->20, 2^-10 -> 0, 1.5*2^-9 -> code 2
     got = oracle.e4m3_to_f32(oracle.f32_to_e4m3(np.float32([17, 19, 2.0**-10, 1.5 * 2.0**-9])))
     np.testing.assert_array_equal(got, np.float32([16, 20, 0, 2 * 2.0**-9]))
     # saturation instead of NaN, both signs; inf saturates, NaN stays NaN
