@@ -133,7 +133,7 @@ def fp8_cases(ops, L, cfg, shapes, Ms):
         b = wn.to(torch.float8_e4m3fn).view(torch.uint8)
         b_s = torch.full(((N + 127) // 128, K // 128), 0.02 * 4.2 / 448.0, dtype=torch.float32)
         R = copies_needed(b.numel())
-        bs_ = [b.to(dev)]
+        bs_ = [ops.fp8_repack_weight(b.to(dev))]   # the load-time repack into 2 KiB MFMA fragments
         bs_ += [bs_[0].clone() for _ in range(R - 1)]
         b_sd = b_s.to(dev)
         state = {"i": 0}
@@ -212,7 +212,7 @@ def moe_fp8_cases(ops, L, cfg, Ts, E=256, hidden=7168, inter=2048, topk=8, disti
         q = torch.randint(0, 256, (distinct, n, k), generator=g, dtype=torch.uint8)
         q = torch.where((q & 0x7f) == 0x7f, q & 0xfe, q)
         s = torch.rand((distinct, n // 128, k // 128), generator=g) * 1e-4 + 1e-4
-        return q.to(dev).repeat(rep, 1, 1), s.to(dev).repeat(rep, 1, 1)
+        return ops.fp8_repack_weight(q.to(dev)).repeat(rep, 1, 1), s.to(dev).repeat(rep, 1, 1)
 
     w13, s13 = experts(2 * inter, hidden)
     w2, s2 = experts(hidden, inter)

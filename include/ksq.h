@@ -101,6 +101,17 @@ int ksq_w4a16_repack_zeros(const void* src, int src_layout, void* dst_packed, si
 int ksq_w4a16_unpack_zeros(const void* packed, int dst_layout, void* dst, size_t K, size_t N, size_t group,
                            void* stream);
 
+/* FP8 (e4m3) weights: checkpoint layout [E, N, K] row-major <-> 2 KiB MFMA fragments of 16 rows x 128 k.  Fragment
+ * (e, n/16, k/128) lies at ((e*N/16 + n/16)*(K/128) + k/128) * 2048; inside, half h (0/1), then wavefront lane
+ * l = 16*((k%128)/32) + n%16, then the 16 bytes k%32 in [16h, 16h+16): one 1 KiB load per half is the MFMA operand of
+ * v_mfma_f32_16x16x128_f8f6f4, contiguous over the wavefront.  Same size as the source; the scales keep their layout.
+ * Every FP8 GEMM below takes its weights in this layout.  N % 16 == 0, K % 128 == 0; exact inverse provided.
+ * The reference's FP8 kernels read the checkpoint layout directly (cuBLASLt / DeepGEMM / CUTLASS); this is the FP8
+ * counterpart of the int4 repack above and belongs in the loader at the same place
+ * (S/models/quant/quant_weight.cpp:817-861, where ConvertFp8E4m3Tensor and the block-scale binding run). */
+int ksq_fp8_repack_weight(const void* src, void* dst_packed, size_t E, size_t N, size_t K, void* stream);
+int ksq_fp8_unpack_weight(const void* packed, void* dst, size_t E, size_t N, size_t K, void* stream);
+
 /* ------------------------------------------------------------------------------------------------------------------
  * W4A16 group-wise GEMM: y[m,n] = x[m,k] . ((code - zp) * scale), zp = 8 when zeros_packed == NULL (GPTQ symmetric),
  * else the per-(group,n) zero point (AWQ).  x, y row-major T; weights / scales / zeros in the packed layout above.
@@ -128,7 +139,7 @@ int ksq_fp8_group_quant(const void* x, void* q, void* s, size_t m, size_t k, siz
 
 /* ------------------------------------------------------------------------------------------------------------------
  * Blockwise FP8 GEMM: out[m,n] = sum_kb (a_q[m,kb] . b[n,kb]) * a_s[kb,m] * b_s[n/128,kb], fp32 accumulate.
- * a_q [m,k] e4m3 row-major, a_s fp32 column-major [k/128, m], b [n,k] e4m3 row-major (checkpoint layout, no repack),
+ * a_q [m,k] e4m3 row-major, a_s fp32 column-major [k/128, m], b [n,k] e4m3 in the packed fragment layout (ksq_fp8_repack_weight),
  * b_s fp32 [ceil(n/128), k/128], out [m,n] in out_dtype.  k must be a multiple of 128, n of 16.
  * Replaces InvokeBlockGemm / InvokeGetBlockGemmWorkspaceSize (K/blockwise_gemm/blockwise_gemm.cu:17-33) and
  * DeepGEMMWrapper::Gemm / GemmSwapAB (K/gemm/deepgemm/deepgemm_wrapper.cu:33-103).
@@ -149,7 +160,8 @@ int ksq_fp8_channel_quant(const void* x, void* q, void* scale, size_t channels, 
                           void* stream);
 
 /* Per-tensor-scaled FP8 GEMM: out[m,n] = T((sum_k a_q[m,k] . b[n,k]) * a_scale[0] * b_scale[0]), fp32 accumulation.
- * a_q [m,k], b [n,k] e4m3 row-major; a_scale, b_scale: one fp32 each in device memory.  k % 128 == 0, n % 16 == 0.
+ * a_q [m,k] e4m3 row-major, b [n,k] e4m3 packed by ksq_fp8_repack_weight; a_scale, b_scale: one fp32 each in device
+ * memory.  k % 128 == 0, n % 16 == 0.
  * The workspace (256-byte aligned) holds the scales spread into the blockwise layouts and the split-K partials of
  * the blockwise kernels, which do the work.
  * Replaces Fp8QuantizedMatMul (S/kernels/nvidia/basic_kernel_wrapper.cpp:1042-1052, cuBLASLt with scale pointers). */
@@ -190,8 +202,8 @@ int ksq_moe_w4a16_gemm(void* out, const void* x, const void* w_packed, const voi
 /* Grouped blockwise-FP8 GEMM over the aligned blocks: for every valid sorted slot id s (< numel)
  *   out[s, :] = sum_kb (a_q[s / top_k, kb] . b[e, :, kb]) * a_s[kb, s / top_k] * b_s[e, :/128, kb] * (topk_w ? topk_w[s] : 1)
  * with e the expert of s's block.  a_q [a_rows, k] e4m3, a_s fp32 [a_rows, k/128] (the reference's layout) or, when
- * a_s_column_major, [k/128, a_rows] - the two layouts ksq_fp8_group_quant writes; b [E, n, k] e4m3 and b_s fp32 [E, ceil(n/128), k/128] in
- * checkpoint layout, out [numel, n] in out_dtype.  top_k = 1 reads a_q rows by slot (second MoE GEMM).
+ * a_s_column_major, [k/128, a_rows] - the two layouts ksq_fp8_group_quant writes; b [E, n, k] e4m3 packed by
+ * ksq_fp8_repack_weight(E = experts), b_s fp32 [E, ceil(n/128), k/128] as in the checkpoint, out [numel, n] in out_dtype.  top_k = 1 reads a_q rows by slot (second MoE GEMM).
  * block_m is the block size the permutation was aligned with: 16 or 32 run the streaming (decode) kernel, 256 the MFMA
  * tile kernel; ksq_moe_fp8_block_m() gives the choice for a problem size.
  * Replaces the fp8_w8a8 block-quantized branch of InvokeFusedMoe's fused_moe_kernel launches

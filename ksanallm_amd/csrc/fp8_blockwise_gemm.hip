@@ -1,8 +1,12 @@
 // Blockwise-scaled FP8 (OCP e4m3) GEMM:  out[m,n] = sum_kb (a_q[m,kb] . b[n,kb]) * a_s[kb,m] * b_s[n/128,kb]
 //
-// Both operands are K-contiguous bytes, which is what v_mfma_f32_16x16x128_f8f6f4 wants: lane l supplies the 32
-// bytes k = 32*(l/16) .. +31 of row l%16.  Weights are the row operand, activations the column operand, so a lane's
-// four results are four consecutive output columns of one token.
+// v_mfma_f32_16x16x128_f8f6f4 wants from lane l the 32 bytes k = 32*(l/16) .. +31 of row l%16.  Activations are read
+// from their row-major [m, k] bytes; weights come in the packed fragment layout (ksq_fp8_repack_weight): a fragment of
+// 16 weight rows x 128 k is 2 KiB, two 1 KiB halves of 16 bytes per lane in lane order, so that every wavefront load is
+// one contiguous KiB (rows of the checkpoint layout lie K bytes apart, and 16-byte pieces of 16 different rows per
+// load run the memory pipeline at a quarter of its rate: 52 % of the HBM rate against 75-80 % from fragments).
+// Weights are the row operand, activations the column operand, so a lane's four results are four consecutive output
+// columns of one token.
 #include <atomic>
 #include <cstdio>
 #include <cstdlib>
@@ -18,7 +22,7 @@ namespace {
 struct Fp8Params {
   const uint8_t* a;   // [m, k]
   const float* a_s;   // [k/128, m]
-  const uint8_t* b;   // [n, k]
+  const uint8_t* b;   // [n, k] in 2 KiB fragments (ksq_fp8_repack_weight)
   const float* b_s;   // [ceil(n/128), k/128]
   void* out;          // [m, n]
   uint32_t M, N, K;
@@ -65,7 +69,8 @@ __global__ void __launch_bounds__(WAVES * 64) fp8_splitk_kernel(Fp8Params p) {
     if (m0 >= static_cast<uint32_t>(p.num_post_pad[0])) return;  // uniform: the whole workgroup leaves
     expert = static_cast<size_t>(p.expert_ids[blockIdx.y]);
   }
-  const uint8_t* bptr = p.b + (expert * p.N + n0 + lrow) * p.K + lq * 32;
+  // fragment (strip, k-block) at ((expert*N/16 + strip)*KB + kb) * 2048; this lane's two 16-byte halves at 16*lane, +1024
+  const uint8_t* bptr = p.b + ((expert * (p.N / 16) + n0 / 16) * KB) * 2048 + lane * 16;
   const float* bs = p.b_s + (expert * p.scale_rows + n0 / 128) * KB;  // 16*NT <= 128 rows: one scale block
   const uint8_t* aptr[MT];
   const float* asptr[MT];
@@ -101,9 +106,9 @@ __global__ void __launch_bounds__(WAVES * 64) fp8_splitk_kernel(Fp8Params p) {
     kb = live ? kb : KB - 1;
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
-      const i32x4* wp = reinterpret_cast<const i32x4*>(bptr + static_cast<size_t>(nt) * 16 * p.K + static_cast<size_t>(kb) * 128);
-      s.w0[nt] = __builtin_nontemporal_load(wp);
-      s.w1[nt] = __builtin_nontemporal_load(wp + 1);
+      const uint8_t* wp = bptr + (static_cast<size_t>(nt) * KB + kb) * 2048;
+      s.w0[nt] = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(wp));
+      s.w1[nt] = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(wp + 1024));
     }
     s.ws = live ? bs[kb] : 0.f;
 #pragma unroll

@@ -24,7 +24,7 @@ namespace ksq {
 struct Fp8TileParams {
   const uint8_t* a;   // [m, k]
   const float* a_s;   // [k/128, m]
-  const uint8_t* b;   // [n, k]
+  const uint8_t* b;   // [n, k] in packed 2 KiB fragments (ksq_fp8_repack_weight)
   const float* b_s;   // [ceil(n/128), k/128]
   void* out;          // [m, n]
   float* partial;     // [slot][part][256][256] fp32 tiles of the workgroups that compute a part of K
@@ -76,7 +76,7 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
   const uint32_t kb_count = direct ? KB : ((KB - kb_begin) < p.kb_per_split ? (KB - kb_begin) : p.kb_per_split);
 
   // ---- operand staging.  Wavefronts 0..3 fetch the activation fragments 4w..4w+3, wavefronts 4..7 the weight
-  // fragments 4(w-4)..+3.  A fragment (16 rows x 128 bytes) is two loads, one per 64-byte half h of the rows; in a
+  // fragments 4(w-4)..+3.  An activation fragment (16 rows x 128 bytes) is two loads, one per 64-byte half h of the rows; in a
   // load four consecutive lanes take the four 16-byte pieces of one row (64 contiguous bytes: the granularity at which
   // the memory pipeline runs at full rate).  Load lane j lands at 1024h + 16j = 1024h + 64*(j/4) + 16*(j%4) and
   // fetches piece (j%4) ^ (j/16) of row j/4, so that MFMA lane (row r, k slot q) finds its two pieces 2(q%2)+p at
@@ -88,22 +88,36 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
   }
   const bool stage_act = wave < 4;
   const uint32_t frag0 = (wave & 3) * 4;
+  // Weights come as packed 2 KiB fragments (ksq_fp8_repack_weight), fragment (strip, k-block) at (strip*KB + kb)*2048:
+  // a half of a fragment is one contiguous KiB, fetched by one load with lane j taking bytes 16j, and lands in LDS as
+  // it lies in memory - MFMA lane l then reads 16 bytes at 16l of each half, consecutive lanes consecutive addresses,
+  // the one pattern the LDS serves at its full rate.
+  const uint32_t k_step = stage_act ? 128u : 2048u;  // bytes from one k-block to the next
+  const uint32_t strip0 = n0 / 16;
   const uint8_t* g_tile = stage_act ? p.a + static_cast<size_t>(GROUPED ? 0 : m0) * p.K
-                                    : p.b + (expert * p.N + n0) * p.K;
-  g_tile += static_cast<size_t>(kb_begin) * 128;
-  const uint32_t row_limit = stage_act ? p.M - m0 : p.N - n0;  // rows of this tile inside the matrix
-  uint32_t d_voff[4];
+                                    : p.b + ((expert * (p.N / 16) + strip0) * KB) * 2048;
+  g_tile += static_cast<size_t>(kb_begin) * k_step;
+  const uint32_t row_limit = p.M - m0;  // token rows of this tile inside the matrix
+  uint32_t d_voff[4], d_voff_hi[4];     // per fragment: first load, and second load minus its instruction offset of 64
 #pragma unroll
   for (int f = 0; f < 4; ++f) {
-    uint32_t row = (frag0 + f) * 16 + (lane >> 2);
-    if (GROUPED && stage_act) {
-      uint32_t sid = static_cast<uint32_t>(p.sorted_ids[m0 + row]);
-      sid = sid < p.numel ? sid : p.numel - 1;  // pad slots read some valid row; their results are dropped
-      row = sid / p.top_k;
+    if (stage_act) {
+      uint32_t row = (frag0 + f) * 16 + (lane >> 2);
+      if (GROUPED) {
+        uint32_t sid = static_cast<uint32_t>(p.sorted_ids[m0 + row]);
+        sid = sid < p.numel ? sid : p.numel - 1;  // pad slots read some valid row; their results are dropped
+        row = sid / p.top_k;
+      } else {
+        row = row < row_limit ? row : row_limit - 1;  // rows past the edge repeat the last row; their results are dropped
+      }
+      d_voff[f] = row * p.K + 16 * ((lane & 3) ^ (lane >> 4));
+      d_voff_hi[f] = d_voff[f];
     } else {
-      row = row < row_limit ? row : row_limit - 1;  // rows past the edge repeat the last row; their results are dropped
+      uint32_t strip = strip0 + frag0 + f;
+      strip = strip < p.N / 16 ? strip : p.N / 16 - 1;  // strips past N repeat the last one; their results are dropped
+      d_voff[f] = (strip - strip0) * KB * 2048 + 16 * lane;
+      d_voff_hi[f] = d_voff[f] + 1024 - 64;
     }
-    d_voff[f] = row * p.K + 16 * ((lane & 3) ^ (lane >> 4));
   }
   const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<size_t>((__attribute__((address_space(3))) char*)lds));
   const uint32_t d_lds = lds_base + ((stage_act ? 0 : W_FRAG0) + frag0) * FRAG;
@@ -163,7 +177,7 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
   // address as well as to the global one: the second half's 64-byte global offset is taken out of its LDS base.
   auto load_operands = [&](uint32_t kb) {
     const uint32_t k = kb < kb_count ? kb : kb_count - 1;
-    const uint8_t* src = g_tile + static_cast<size_t>(k) * 128;
+    const uint8_t* src = g_tile + static_cast<size_t>(k) * k_step;
     const uint32_t f0 = __builtin_amdgcn_readfirstlane(d_lds + (kb & 1) * STAGE_BYTES);
     const uint32_t f0h = f0 + 1024 - 64;
     const uint32_t f1 = f0 + FRAG, f1h = f0h + FRAG;
@@ -171,17 +185,18 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
     const uint32_t f3 = f2 + FRAG, f3h = f2h + FRAG;
     asm volatile(
         "s_nop 4\n\t"
-        "s_mov_b32 m0, %4\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %12\n\t"
-        "s_mov_b32 m0, %5\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %12 offset:64\n\t"
-        "s_mov_b32 m0, %6\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %12\n\t"
-        "s_mov_b32 m0, %7\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %12 offset:64\n\t"
-        "s_mov_b32 m0, %8\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %12\n\t"
-        "s_mov_b32 m0, %9\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %12 offset:64\n\t"
-        "s_mov_b32 m0, %10\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %3, %12\n\t"
-        "s_mov_b32 m0, %11\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %3, %12 offset:64"
+        "s_mov_b32 m0, %8\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %16\n\t"
+        "s_mov_b32 m0, %9\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %4, %16 offset:64\n\t"
+        "s_mov_b32 m0, %10\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %16\n\t"
+        "s_mov_b32 m0, %11\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %5, %16 offset:64\n\t"
+        "s_mov_b32 m0, %12\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %16\n\t"
+        "s_mov_b32 m0, %13\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %6, %16 offset:64\n\t"
+        "s_mov_b32 m0, %14\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %3, %16\n\t"
+        "s_mov_b32 m0, %15\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %7, %16 offset:64"
         :
-        : "v"(d_voff[0]), "v"(d_voff[1]), "v"(d_voff[2]), "v"(d_voff[3]), "s"(f0), "s"(f0h), "s"(f1), "s"(f1h),
-          "s"(f2), "s"(f2h), "s"(f3), "s"(f3h), "s"(src)
+        : "v"(d_voff[0]), "v"(d_voff[1]), "v"(d_voff[2]), "v"(d_voff[3]), "v"(d_voff_hi[0]), "v"(d_voff_hi[1]),
+          "v"(d_voff_hi[2]), "v"(d_voff_hi[3]), "s"(f0), "s"(f0h), "s"(f1), "s"(f1h), "s"(f2), "s"(f2h), "s"(f3),
+          "s"(f3h), "s"(src)
         : "memory");
   };
   // everything this wavefront issued so far has landed
@@ -200,6 +215,12 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
     const i32x4 hi = *reinterpret_cast<const i32x4*>(base + rd_hi);
     return i32x8{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
   };
+  // weight fragments lie in LDS as packed: 16 bytes per lane in lane order, second half 1 KiB further
+  auto read_wfrag = [&](const char* base) {
+    const i32x4 lo = *reinterpret_cast<const i32x4*>(base + 16 * lane);
+    const i32x4 hi = *reinterpret_cast<const i32x4*>(base + 1024 + 16 * lane);
+    return i32x8{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+  };
 
   // one k-block: 32 MFMAs; the scale FMAs of MFMA j are placed after MFMA j+2 so that they run in its shadow, and the
   // loads of k-block `next` (scales, then operands into the LDS slot the previous stage used) are issued after the
@@ -215,10 +236,10 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
     const char* wgt = lds + slot * STAGE_BYTES + (W_FRAG0 + wn * WN) * FRAG;
     i32x8 wf[WN];
     i32x8 af[2];
-    wf[0] = read_frag(wgt);
+    wf[0] = read_wfrag(wgt);
     af[0] = read_frag(act);
 #pragma unroll
-    for (int t = 1; t < WN; ++t) wf[t] = read_frag(wgt + t * FRAG);
+    for (int t = 1; t < WN; ++t) wf[t] = read_wfrag(wgt + t * FRAG);
     __builtin_amdgcn_sched_barrier(0x4);
     f32x4 tmp[3];
     const f32x4 zero{0.f, 0.f, 0.f, 0.f};

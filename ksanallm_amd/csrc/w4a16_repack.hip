@@ -115,6 +115,29 @@ __global__ void __launch_bounds__(256) permute_columns_kernel(const uint16_t* __
   reinterpret_cast<uint32_t*>(out + r * k)[c / 2] = static_cast<uint32_t>(row[p0]) | (static_cast<uint32_t>(row[p1]) << 16);
 }
 
+// FP8 weights [E, N, K] (checkpoint, row-major) <-> 2 KiB fragments of 16 rows x 128 k, fragment (e, n/16, k/128) at
+// ((e*N/16 + n/16)*(K/128) + k/128): half h, then lane l = 16*((k%128)/32) + n%16, then the 16 bytes
+// k%32 in [16h, 16h+16) - the two 16-byte halves of the lane's operand of v_mfma_f32_16x16x128_f8f6f4.
+// One thread moves 16 bytes; TO_PACKED selects the direction.
+template <bool TO_PACKED>
+__global__ void __launch_bounds__(256) fp8_repack_kernel(const u32x4* __restrict__ src, u32x4* __restrict__ dst,
+                                                         size_t E, size_t N, size_t K) {
+  const size_t o = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;  // 16-byte piece of the packed tensor
+  if (o >= E * N * K / 16) return;
+  const size_t KB = K / 128;
+  const size_t frag = o / 128;
+  const uint32_t within = static_cast<uint32_t>(o % 128);
+  const uint32_t h = within / 64, lane = within % 64;
+  const size_t kb = frag % KB;
+  const size_t nt = (frag / KB) % (N / 16);
+  const size_t e = frag / (KB * (N / 16));
+  const size_t row = nt * 16 + (lane % 16);
+  const size_t kbyte = kb * 128 + (lane / 16) * 32 + h * 16;
+  const size_t plain = ((e * N + row) * K + kbyte) / 16;
+  if (TO_PACKED) dst[o] = src[plain];
+  else dst[plain] = src[o];
+}
+
 // one thread per 8 codes of the destination
 template <int DST>
 __global__ void __launch_bounds__(256) unpack_weight_kernel(const uint32_t* __restrict__ packed,
@@ -269,6 +292,30 @@ KSQ_EXPORT int ksq_w4a16_repack_act_order(const void* src_gptq, const void* perm
                                                                   static_cast<const int32_t*>(perm),
                                                                   static_cast<uint32_t*>(dst), g);
   return check_launch(fn);
+}
+
+static int fp8_repack_common(const void* src, void* dst, size_t E, size_t N, size_t K, void* stream, bool to_packed,
+                             const char* fn) {
+  if (!src || !dst) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: null pointer", fn);
+  if (!aligned16(src) || !aligned16(dst)) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: pointers must be 16-byte aligned", fn);
+  if (src == dst) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: cannot repack in place", fn);
+  if (E == 0 || N == 0 || K == 0 || K % 128 != 0 || N % 16 != 0)
+    return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: need E>0, K %% 128 == 0, N %% 16 == 0 (E=%zu N=%zu K=%zu)", fn, E, N, K);
+  const size_t blocks = div_up(E * N * K / 16, 256);
+  if (blocks > 0x7fffffffull) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: tensor too large", fn);
+  const u32x4* s = static_cast<const u32x4*>(src);
+  u32x4* d = static_cast<u32x4*>(dst);
+  if (to_packed) fp8_repack_kernel<true><<<static_cast<unsigned>(blocks), 256, 0, as_stream(stream)>>>(s, d, E, N, K);
+  else fp8_repack_kernel<false><<<static_cast<unsigned>(blocks), 256, 0, as_stream(stream)>>>(s, d, E, N, K);
+  return check_launch(fn);
+}
+
+KSQ_EXPORT int ksq_fp8_repack_weight(const void* src, void* dst_packed, size_t E, size_t N, size_t K, void* stream) {
+  return fp8_repack_common(src, dst_packed, E, N, K, stream, true, "ksq_fp8_repack_weight");
+}
+
+KSQ_EXPORT int ksq_fp8_unpack_weight(const void* packed, void* dst, size_t E, size_t N, size_t K, void* stream) {
+  return fp8_repack_common(packed, dst, E, N, K, stream, false, "ksq_fp8_unpack_weight");
 }
 
 KSQ_EXPORT int ksq_permute_columns(const void* x, const void* perm, void* out, size_t m, size_t k, int dtype,

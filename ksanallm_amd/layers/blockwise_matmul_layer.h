@@ -1,7 +1,8 @@
 // Blockwise-FP8 (e4m3, 128x128 weight scales) matmul layer.
 // Mirrors src/ksana_llm/layers/blockwise_matmul_layer.h:15 and nvidia/blockwise_matmul_layer.cpp:16-299:
 // activations are quantized per token / per 128 channels into the head of the workspace (a_q at offset 0, a_s right
-// after the cur_m*k quantized bytes, column-major), then multiplied with the checkpoint-layout weight.
+// after the cur_m*k quantized bytes, column-major), then multiplied with the weight, which the loader has put into the
+// packed fragment layout (PackFp8Weight, quant_weight_repack.h).
 // The reference picks between Cutlass / DeepGEMM / DeepGEMM-swapAB by timing them in Preprocess; here the variant is a
 // pure function of (m, n, k), so Preprocess has nothing to search and the m -> RoundUp(m, 4) padding DeepGEMM needs
 // does not exist.
@@ -19,7 +20,8 @@ class BlockwiseMatMulLayer : public BaseLayer {
   size_t GetWorkspaceSize() override;
   Status Preprocess(const ModelConfig& model_config, const RuntimeConfig& runtime_config) override;
   // inputs: [0] activations [m, k] (or [m, 2k]: silu(x[:, :k]) * x[:, k:] is fused into the quantizer),
-  //         [1] weight [n, k] e4m3 with weight_scales [ceil(n/128), k/128] fp32.  output [0]: [m, n] in T.
+  //         [1] weight [n, k] e4m3 packed by PackFp8Weight, with weight_scales [ceil(n/128), k/128] fp32.
+  // output [0]: [m, n] in T.
   Status Forward(const std::vector<Tensor>& input_tensors, std::vector<Tensor>& output_tensors) override;
 
  private:

@@ -19,7 +19,8 @@ class Fp8MatMulLayer : public BaseLayer {
   // reference's cuBLAS workspace is: n is not known before Forward)
   size_t GetWorkspaceSize(const int m, const int k);
   size_t GetWorkspaceSize() override;
-  // inputs: [0] activations [m, k] T, [1] weight [n, k] e4m3 with weight_scales (1 fp32) and optionally input_scales
+  // inputs: [0] activations [m, k] T, [1] weight [n, k] e4m3 packed by PackFp8Weight (quant_weight_repack.h), with
+  // weight_scales (1 fp32) and optionally input_scales
   // (1 fp32, static activation scale).  output [0]: [m, n] in T.
   Status Forward(const std::vector<Tensor>& input_tensors, std::vector<Tensor>& output_tensors) override;
 

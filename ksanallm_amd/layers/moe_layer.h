@@ -1,6 +1,7 @@
 // Fused MoE layer for int4 group-quantized experts (the "moe-int4" path: weights [E, N, K/2] uint4x2 with per-group
 // scales, activations in T) and for block-quantized fp8 experts (weights [E, N, K] e4m3 with fp32 scales per 128 x 128
-// block bound as weight_scales, activations quantized per token and 128 channels in front of each GEMM).  Mirrors src/ksana_llm/layers/moe_layer.h:42 and nvidia/moe_layer.cpp:38-380 together with
+// block bound as weight_scales, packed by PackFp8Weight; activations quantized per token and 128 channels in front of
+// each GEMM).  Mirrors src/ksana_llm/layers/moe_layer.h:42 and nvidia/moe_layer.cpp:38-380 together with
 // InvokeFusedMoe (src/ksana_llm/kernels/nvidia/moe_kernel_wrapper.cpp:466-657):
 //   router (softmax top-k, or grouped / sigmoid / bias-corrected top-k with the bias as input tensor 5) -> align/permute -> grouped GEMM gate_up -> silu*mul -> grouped GEMM down (x routing
 //   weight) -> sum over top-k, processed in chunks of 32768 tokens, all scratch carved out of one workspace buffer.

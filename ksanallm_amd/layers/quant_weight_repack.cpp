@@ -68,4 +68,21 @@ Tensor PackMoeExpertWeight(const Tensor& experts, const Tensor& scales, size_t g
   return packed;
 }
 
+Tensor PackFp8Weight(const Tensor& weight, int rank, hipStream_t stream) {
+  const char* who = "PackFp8Weight";
+  if (weight.dtype != TYPE_FP8_E4M3) KLLM_THROW("PackFp8Weight: weight must be TYPE_FP8_E4M3");
+  if (weight.shape.size() != 2 && weight.shape.size() != 3) KLLM_THROW("PackFp8Weight: [N, K] or [E, N, K] expected");
+  const size_t E = weight.shape.size() == 3 ? weight.shape[0] : 1;
+  const size_t N = weight.shape[weight.shape.size() - 2], K = weight.shape.back();
+  Tensor packed(MemoryLocation::LOCATION_DEVICE, TYPE_FP8_E4M3, weight.shape, rank);
+  KsqCheck(ksq_fp8_repack_weight(weight.GetPtr<void>(), packed.GetPtr<void>(), E, N, K, stream), who);
+  packed.scales = weight.scales;
+  packed.zeros = weight.zeros;
+  packed.input_scales = weight.input_scales;
+  packed.weight_scales = weight.weight_scales;
+  packed.pre_quant_scales = weight.pre_quant_scales;
+  packed.input_alpha = weight.input_alpha;
+  return packed;
+}
+
 }  // namespace ksana_llm

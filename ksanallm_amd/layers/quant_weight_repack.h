@@ -24,4 +24,10 @@ Tensor PackGroupQuantWeight(const Tensor& qweight, const Tensor& scales, const T
 // Returns a TYPE_UINT4x2 tensor of logical shape {E, N, K/2} with `scales` bound.
 Tensor PackMoeExpertWeight(const Tensor& experts, const Tensor& scales, size_t group_size, int rank, hipStream_t stream);
 
+// FP8 (e4m3) weights, [N, K] or an expert stack [E, N, K] in checkpoint layout: returns the same shape and dtype in the
+// packed 2 KiB fragment layout every FP8 layer here consumes (BlockwiseMatMulLayer, Fp8MatMulLayer, MoeLayer with
+// block-fp8 experts); the side tensors of `weight` (weight_scales, input_scales, ...) are carried over unchanged.
+// Stands where the reference binds the scales of FP8 weights after loading (quant_weight.cpp:817-861).
+Tensor PackFp8Weight(const Tensor& weight, int rank, hipStream_t stream);
+
 }  // namespace ksana_llm

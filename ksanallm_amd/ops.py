@@ -135,7 +135,8 @@ def per_token_group_quant_fp8(x, k, group=128, column_major=True, fuse_silu_mul=
 
 
 def fp8_blockwise_gemm(a_q, a_s, b, b_s, out_dtype=torch.bfloat16, out=None, workspace=None):
-    """InvokeBlockGemm / DeepGEMMWrapper::Gemm: a_q [m,k] e4m3 bytes, a_s [k/128,m], b [n,k], b_s [n/128,k/128]."""
+    """InvokeBlockGemm / DeepGEMMWrapper::Gemm: a_q [m,k] e4m3 bytes, a_s [k/128,m], b [n,k] packed by
+    fp8_repack_weight, b_s [n/128,k/128]."""
     m, k = a_q.shape
     n = b.shape[0]
     if out is None:
@@ -246,8 +247,8 @@ def fused_moe_w4a16(x, w13_packed, s13_packed, w2_packed, s2_packed, topk_ids, t
 
 def moe_fp8_blockwise_gemm(a_q, a_s, a_s_column_major, b, b_s, topk_w, sorted_ids, expert_ids, num_post_pad, numel,
                            top_k, block_m, out_dtype=torch.bfloat16, out=None):
-    """fp8_w8a8 block-quantized fused_moe_kernel launch: a_q [rows,k] e4m3 bytes, b [E,n,k], b_s [E,n/128,k/128];
-    out [numel, n]."""
+    """fp8_w8a8 block-quantized fused_moe_kernel launch: a_q [rows,k] e4m3 bytes, b [E,n,k] packed by fp8_repack_weight,
+    b_s [E,n/128,k/128]; out [numel, n]."""
     rows, k = a_q.shape
     E, n = b.shape[0], b.shape[1]
     if out is None:
@@ -263,7 +264,7 @@ def fused_moe_fp8_blockwise(x, w13, w13_scale, w2, w2_scale, topk_ids, topk_w, b
     """InvokeFusedMoe<T,false> for block-quantized fp8 experts (S/kernels/nvidia/moe_kernel_wrapper.cpp:463-654 with
     compute_dtype TYPE_BLOCK_FP8_E4M3): quantize x per token and 128 channels -> align -> GEMM1 -> silu*mul fused into
     the second quantization -> GEMM2 (* routed weight) -> sum over top-k.  w13 [E, 2*inter, hidden], w2 [E, hidden, inter]
-    e4m3 bytes, scales fp32 per 128 x 128 block."""
+    e4m3 bytes packed by fp8_repack_weight, scales fp32 per 128 x 128 block."""
     T, topk = topk_ids.shape
     E, two_inter, hidden = w13.shape
     inter = two_inter // 2
@@ -292,7 +293,7 @@ def fp8_e4m3_quantize(x, scale=None):
 
 
 def fp8_quantized_matmul(a_q, a_scale, b, b_scale, out_dtype=torch.bfloat16, out=None, workspace=None):
-    """Fp8QuantizedMatMul: a_q [m,k], b [n,k] e4m3 bytes, one fp32 device scale each."""
+    """Fp8QuantizedMatMul: a_q [m,k] e4m3 bytes, b [n,k] packed by fp8_repack_weight, one fp32 device scale each."""
     m, k = a_q.shape
     n = b.shape[0]
     if out is None:
@@ -322,4 +323,22 @@ def permute_columns(x, perm, out=None):
     if out is None:
         out = torch.empty_like(x)
     _l.check(_lib.ksq_permute_columns(_ptr(x), _ptr(perm), _ptr(out), m, k, _dt(x), _stream()))
+    return out
+
+
+def fp8_repack_weight(w):
+    """Checkpoint-layout e4m3 weight [N, K] or [E, N, K] (uint8) -> the packed fragment layout the FP8 GEMMs read."""
+    E = w.shape[0] if w.dim() == 3 else 1
+    N, K = w.shape[-2], w.shape[-1]
+    out = torch.empty_like(w)
+    _l.check(_lib.ksq_fp8_repack_weight(_ptr(w), _ptr(out), E, N, K, _stream()))
+    return out
+
+
+def fp8_unpack_weight(packed):
+    """Inverse of :func:`fp8_repack_weight` (the tensor keeps the logical shape [N, K] / [E, N, K])."""
+    E = packed.shape[0] if packed.dim() == 3 else 1
+    N, K = packed.shape[-2], packed.shape[-1]
+    out = torch.empty_like(packed)
+    _l.check(_lib.ksq_fp8_unpack_weight(_ptr(packed), _ptr(out), E, N, K, _stream()))
     return out

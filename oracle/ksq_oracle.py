@@ -414,3 +414,16 @@ def gptq_act_order_gemm(x_bits, codes, scales_bits, g_idx, dtype, zeros=None):
     z = 8.0 if zeros is None else np.asarray(zeros).astype(np.float64)[g]
     w = (np.asarray(codes).astype(np.float64) - z) * sc[g]
     return (x @ w).astype(np.float32)
+
+
+def fp8_repack_weight(w):
+    """Packed fragment layout of an e4m3 weight [N, K] or [E, N, K] (uint8), as include/ksq.h defines it: fragments of
+    16 rows x 128 k in (e, n/16, k/128) order; inside, half h, lane l = 16*((k%128)/32) + n%16, 16 bytes k%32 in
+    [16h, 16h+16).  Written as an index permutation in numpy (the layout has no counterpart in the reference)."""
+    w = np.asarray(w, np.uint8)
+    shape = w.shape
+    w3 = w.reshape((-1,) + shape[-2:])
+    E, N, K = w3.shape
+    # axes: e, nt, r(16), kb, q(4), h(2), byte(16)  ->  e, nt, kb, h, q, r, byte
+    v = w3.reshape(E, N // 16, 16, K // 128, 4, 2, 16).transpose(0, 1, 3, 5, 4, 2, 6)
+    return np.ascontiguousarray(v).reshape(shape)

@@ -138,8 +138,9 @@ static int RunBlockwise(int argc, char** argv) {
   rc.inter_data_type = T;
   rc.max_step_token_num = (m + 3) / 4 * 4;
 
-  Tensor weight = Upload(dir + "/w.bin", TYPE_FP8_E4M3, {n, k});
-  weight.weight_scales = std::make_shared<Tensor>(Upload(dir + "/w_scale.bin", TYPE_FP32, {(n + 127) / 128, k / 128}));
+  Tensor loaded = Upload(dir + "/w.bin", TYPE_FP8_E4M3, {n, k});
+  loaded.weight_scales = std::make_shared<Tensor>(Upload(dir + "/w_scale.bin", TYPE_FP32, {(n + 127) / 128, k / 128}));
+  Tensor weight = PackFp8Weight(loaded, 0, stream);
   std::vector<std::any> params{rc.max_step_token_num, n, k, size_t(128), weight};
   MatMulLayerFactory factory(mc, rc, 0, context);
   auto layer = factory.CreateLayer(TYPE_FP8_E4M3, T, T, params, QUANT_BLOCK_FP8_E4M3, DEFAULT_LINEAR_BACKEND);
@@ -165,9 +166,10 @@ static int RunFp8Tensor(int argc, char** argv) {
   RuntimeConfig rc;
   rc.inter_data_type = T;
   rc.max_step_token_num = m;
-  Tensor weight = Upload(dir + "/w.bin", TYPE_FP8_E4M3, {n, k});
-  weight.weight_scales = std::make_shared<Tensor>(Upload(dir + "/w_scale.bin", TYPE_FP32, {1}));
-  if (is_static) weight.input_scales = std::make_shared<Tensor>(Upload(dir + "/in_scale.bin", TYPE_FP32, {1}));
+  Tensor loaded = Upload(dir + "/w.bin", TYPE_FP8_E4M3, {n, k});
+  loaded.weight_scales = std::make_shared<Tensor>(Upload(dir + "/w_scale.bin", TYPE_FP32, {1}));
+  if (is_static) loaded.input_scales = std::make_shared<Tensor>(Upload(dir + "/in_scale.bin", TYPE_FP32, {1}));
+  Tensor weight = PackFp8Weight(loaded, 0, stream);
   std::vector<std::any> params{rc.max_step_token_num, k};
   MatMulLayerFactory factory(mc, rc, 0, context);
   auto layer = factory.CreateLayer(TYPE_FP8_E4M3, T, T, params, QUANT_FP8_E4M3, DEFAULT_LINEAR_BACKEND);
@@ -264,10 +266,12 @@ static int RunMoeFp8(int argc, char** argv) {
   ModelConfig mc;
   RuntimeConfig rc;
   rc.inter_data_type = T;
-  Tensor w13 = Upload(dir + "/w13.bin", TYPE_FP8_E4M3, {E, 2 * inter, hidden});
-  w13.weight_scales = std::make_shared<Tensor>(Upload(dir + "/s13.bin", TYPE_FP32, {E, (2 * inter + 127) / 128, hidden / 128}));
-  Tensor w2 = Upload(dir + "/w2.bin", TYPE_FP8_E4M3, {E, hidden, inter});
-  w2.weight_scales = std::make_shared<Tensor>(Upload(dir + "/s2.bin", TYPE_FP32, {E, (hidden + 127) / 128, inter / 128}));
+  Tensor w13_loaded = Upload(dir + "/w13.bin", TYPE_FP8_E4M3, {E, 2 * inter, hidden});
+  w13_loaded.weight_scales = std::make_shared<Tensor>(Upload(dir + "/s13.bin", TYPE_FP32, {E, (2 * inter + 127) / 128, hidden / 128}));
+  Tensor w2_loaded = Upload(dir + "/w2.bin", TYPE_FP8_E4M3, {E, hidden, inter});
+  w2_loaded.weight_scales = std::make_shared<Tensor>(Upload(dir + "/s2.bin", TYPE_FP32, {E, (hidden + 127) / 128, inter / 128}));
+  Tensor w13 = PackFp8Weight(w13_loaded, 0, stream);
+  Tensor w2 = PackFp8Weight(w2_loaded, 0, stream);
   auto params = MoeParams(tokens, E, hidden, inter, topk, renorm, scaling, TYPE_INVALID);
   params[17] = TYPE_BLOCK_FP8_E4M3;
   MoeLayerFactory factory(mc, rc, 0, context);

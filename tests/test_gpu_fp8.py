@@ -109,6 +109,11 @@ def test_quant_fused_silu_mul(ops, oracle, dtype):
     assert np.linalg.norm(a - b) / np.linalg.norm(b) < 2e-2
 
 
+def packed(ops, bq):
+    """checkpoint-layout e4m3 weight (numpy) -> device tensor in the packed fragment layout the GEMMs read"""
+    return ops.fp8_repack_weight(torch.from_numpy(bq).cuda())
+
+
 def make_fp8_problem(oracle, seed, m, n, k, dtype=H.BF16):
     g = H.gen(seed)
     w = (torch.randn((n, k), generator=g) * 0.02).to(torch.bfloat16).float().numpy()
@@ -122,7 +127,7 @@ def make_fp8_problem(oracle, seed, m, n, k, dtype=H.BF16):
 def test_blockwise_gemm(ops, oracle, m, n, k):
     x, bq, bs = make_fp8_problem(oracle, 4100 + m + n, m, n, k)
     q, s = ops.per_token_group_quant_fp8(x.cuda(), k, 128, True)
-    out = ops.fp8_blockwise_gemm(q, s, torch.from_numpy(bq).cuda(), torch.from_numpy(bs).cuda(), torch.bfloat16)
+    out = ops.fp8_blockwise_gemm(q, s, packed(ops, bq), torch.from_numpy(bs).cuda(), torch.bfloat16)
     # the oracle consumes the very codes and scales the GPU quantizer produced
     ref = oracle.fp8_blockwise_gemm(q.cpu().numpy(), s.cpu().numpy(), bq, bs, True)
     H.check_gemm(out, ref, H.BF16, "fp8 m=%d n=%d k=%d" % (m, n, k))
@@ -137,13 +142,13 @@ def test_blockwise_gemm_tile_kernel(ops, oracle, m, n, k):
     assert desc["kernel"] == 1
     x, bq, bs = make_fp8_problem(oracle, 4400 + m + n, m, n, k)
     q, s = ops.per_token_group_quant_fp8(x.cuda(), k, 128, True)
-    out = ops.fp8_blockwise_gemm(q, s, torch.from_numpy(bq).cuda(), torch.from_numpy(bs).cuda(), torch.bfloat16)
+    out = ops.fp8_blockwise_gemm(q, s, packed(ops, bq), torch.from_numpy(bs).cuda(), torch.bfloat16)
     ref = oracle.fp8_blockwise_gemm(q.cpu().numpy(), s.cpu().numpy(), bq, bs, True)
     H.check_gemm(out, ref, H.BF16, "fp8 tile m=%d n=%d k=%d split=%d" % (m, n, k, desc["split_k"]))
     if desc["split_k"] > 1:
         small = torch.empty(64, dtype=torch.uint8, device="cuda")
         with pytest.raises(L.KsqError) as e:
-            ops.fp8_blockwise_gemm(q, s, torch.from_numpy(bq).cuda(), torch.from_numpy(bs).cuda(), torch.bfloat16,
+            ops.fp8_blockwise_gemm(q, s, packed(ops, bq), torch.from_numpy(bs).cuda(), torch.bfloat16,
                                    workspace=small)
         assert e.value.code == 3
 
@@ -157,7 +162,7 @@ def test_blockwise_gemm_whole_and_cut_tiles(ops, oracle):
     assert desc["kernel"] == 1 and desc["split_k"] > 1 and desc["grid"] == 256 + (tiles - 256) * desc["split_k"]
     x, bq, bs = make_fp8_problem(oracle, 4500, m, n, k)
     q, s = ops.per_token_group_quant_fp8(x.cuda(), k, 128, True)
-    out = ops.fp8_blockwise_gemm(q, s, torch.from_numpy(bq).cuda(), torch.from_numpy(bs).cuda(), torch.bfloat16)
+    out = ops.fp8_blockwise_gemm(q, s, packed(ops, bq), torch.from_numpy(bs).cuda(), torch.bfloat16)
     ref = oracle.fp8_blockwise_gemm(q.cpu().numpy(), s.cpu().numpy(), bq, bs, True)
     H.check_gemm(out, ref, H.BF16, "fp8 whole + cut tiles")
 
@@ -166,7 +171,7 @@ def test_blockwise_gemm_partial_scale_row_and_fp16_out(ops, oracle):
     m, n, k = 7, 208, 384  # n not a multiple of 128: the last scale row covers 80 weight rows
     x, bq, bs = make_fp8_problem(oracle, 4321, m, n, k, H.F16)
     q, s = ops.per_token_group_quant_fp8(x.cuda(), k, 128, True)
-    out = ops.fp8_blockwise_gemm(q, s, torch.from_numpy(bq).cuda(), torch.from_numpy(bs).cuda(), torch.float16)
+    out = ops.fp8_blockwise_gemm(q, s, packed(ops, bq), torch.from_numpy(bs).cuda(), torch.float16)
     ref = oracle.fp8_blockwise_gemm(q.cpu().numpy(), s.cpu().numpy(), bq, bs, True)
     H.check_gemm(out, ref, H.F16, "fp8 partial")
 
@@ -204,11 +209,31 @@ def test_fp8_quantized_matmul(ops, oracle, m, n, k):
     x = make_act(5200 + m, m, k, H.BF16)
     wq, ws = ops.fp8_e4m3_quantize(w.reshape(1, -1).cuda())
     xq, xs = ops.fp8_e4m3_quantize(x.reshape(1, -1).cuda())
-    out = ops.fp8_quantized_matmul(xq.view(m, k), xs, wq.view(n, k), ws, torch.bfloat16)
+    wp = ops.fp8_repack_weight(wq.view(n, k))
+    out = ops.fp8_quantized_matmul(xq.view(m, k), xs, wp, ws, torch.bfloat16)
     ref = oracle.fp8_tensor_gemm(xq.view(m, k).cpu().numpy(), xs.item(), wq.view(n, k).cpu().numpy(), ws.item())
     H.check_gemm(out, ref, H.BF16, "fp8 per-tensor m=%d n=%d k=%d" % (m, n, k))
     small = torch.empty(256, dtype=torch.uint8, device="cuda")
     from ksanallm_amd import lib as L
     with pytest.raises(L.KsqError) as e:
-        ops.fp8_quantized_matmul(xq.view(m, k), xs, wq.view(n, k), ws, torch.bfloat16, workspace=small)
+        ops.fp8_quantized_matmul(xq.view(m, k), xs, wp, ws, torch.bfloat16, workspace=small)
     assert e.value.code == 3
+
+
+# ---- packed fragment layout of fp8 weights ---------------------------------------------------------------------------
+
+@pytest.mark.parametrize("shape", [(16, 128), (48, 384), (3, 32, 256), (2320, 1152)])
+def test_fp8_weight_repack_bit_exact_and_round_trip(ops, oracle, shape):
+    g = H.gen(sum(shape))
+    w = torch.randint(0, 256, shape, generator=g, dtype=torch.uint8)
+    p = ops.fp8_repack_weight(w.cuda())
+    np.testing.assert_array_equal(p.cpu().numpy(), oracle.fp8_repack_weight(w.numpy()))
+    assert torch.equal(ops.fp8_unpack_weight(p).cpu(), w)
+
+
+def test_fp8_weight_repack_rejects_bad_shapes(ops):
+    from ksanallm_amd import lib as L
+    for shape in ((8, 128), (16, 100)):
+        with pytest.raises(L.KsqError) as e:
+            ops.fp8_repack_weight(torch.zeros(shape, dtype=torch.uint8, device="cuda"))
+        assert e.value.code == 1

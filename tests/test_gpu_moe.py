@@ -249,7 +249,7 @@ def test_grouped_fp8_gemm_stage(ops, oracle, T, E, topk, n, k, bm, colmajor, wit
     numel = T * topk
     q, s = ops.per_token_group_quant_fp8(x.cuda(), k, 128, colmajor)
     sorted_ids, expert_ids, npp = ops.moe_align_block_size(ids.cuda(), E, bm)
-    out = ops.moe_fp8_blockwise_gemm(q, s, colmajor, torch.from_numpy(bq).cuda(), torch.from_numpy(bs).cuda(),
+    out = ops.moe_fp8_blockwise_gemm(q, s, colmajor, ops.fp8_repack_weight(torch.from_numpy(bq).cuda()), torch.from_numpy(bs).cuda(),
                                      tw.reshape(-1).cuda() if with_w else None, sorted_ids, expert_ids, npp, numel, topk,
                                      bm, torch.bfloat16)
     qh, sh = q.cpu().numpy(), s.cpu().numpy()
@@ -278,7 +278,7 @@ def test_moe_fp8_block(ops, oracle, dtype, T, E, topk, hidden, inter):
     x = torch.randn((T, hidden), generator=g).to(H.TORCH_DT[dtype])
     logits = torch.randn((T, E), generator=g)
     tw, ids = ops.moe_topk_softmax(logits.cuda(), topk, True, 1.0)
-    y = ops.fused_moe_fp8_blockwise(x.cuda(), torch.from_numpy(w13).cuda(), torch.from_numpy(s13).cuda(),
-                                    torch.from_numpy(w2).cuda(), torch.from_numpy(s2).cuda(), ids, tw)
+    y = ops.fused_moe_fp8_blockwise(x.cuda(), ops.fp8_repack_weight(torch.from_numpy(w13).cuda()), torch.from_numpy(s13).cuda(),
+                                    ops.fp8_repack_weight(torch.from_numpy(w2).cuda()), torch.from_numpy(s2).cuda(), ids, tw)
     ref = oracle.moe_fp8_forward(H.bits_of(x), w13, s13, w2, s2, ids.cpu().numpy(), tw.cpu().numpy(), dtype)
     H.check_gemm(y, oracle.from_bits(ref, dtype), dtype, "fp8 moe block")

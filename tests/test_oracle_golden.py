@@ -463,3 +463,22 @@ def test_act_order_definition(oracle):
     assert np.array_equal(g_idx[perm], np.arange(K) // group)
     moved = oracle.w4a16_gemm(H.bits_of(x[:, torch.from_numpy(perm)].contiguous()), codes[perm], H.bits_of(scales), None, group, H.F16)
     np.testing.assert_allclose(moved, y, rtol=2e-5, atol=2e-5)
+
+
+def test_fp8_weight_fragment_layout_by_definition(oracle):
+    """The packed fp8 layout, element by element from its definition: fragment (e, n/16, k/128) of 2 KiB; inside, half h,
+    lane l = 16*((k%128)/32) + n%16, byte k%16 - against the oracle's vectorised permutation."""
+    g = torch.Generator().manual_seed(21)
+    E, N, K = 2, 32, 256
+    w = torch.randint(0, 256, (E, N, K), generator=g, dtype=torch.uint8).numpy()
+    p = oracle.fp8_repack_weight(w).reshape(-1)
+    KB = K // 128
+    for e in range(E):
+        for n in range(N):
+            for k in range(K):
+                frag = (e * (N // 16) + n // 16) * KB + k // 128
+                h = (k % 32) // 16
+                lane = 16 * ((k % 128) // 32) + n % 16
+                assert p[frag * 2048 + h * 1024 + lane * 16 + k % 16] == w[e, n, k]
+    # 2-D input is the E = 1 case
+    np.testing.assert_array_equal(oracle.fp8_repack_weight(w[0]), oracle.fp8_repack_weight(w[:1])[0])
