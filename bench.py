@@ -40,9 +40,9 @@ MEASURED_TRAFFIC = {
     (2, "w4a16_tile_kernel<256x256,w8>"): 216470000,
     (3, "w4a16_tile_kernel<256x256,w8>"): 1591160000,
     (4, "fp8_group_quant"): 27630000,
-    (4, "fp8_splitk_kernel<16x16,w4>"): 134810000,
-    (4, "fp8_splitk_kernel<16x32,w4>"): 134820000,
-    (4, "fp8_tile_kernel<256x256,w8>"): 258550000,
+    (4, "fp8_splitk_kernel<16x16,w4>"): 133550000,
+    (4, "fp8_splitk_kernel<16x32,w4>"): 134270000,
+    (4, "fp8_tile_kernel<256x256,w8>"): 258430000,
 }
 
 
