@@ -237,3 +237,25 @@ def test_fp8_weight_repack_rejects_bad_shapes(ops):
         with pytest.raises(L.KsqError) as e:
             ops.fp8_repack_weight(torch.zeros(shape, dtype=torch.uint8, device="cuda"))
         assert e.value.code == 1
+
+
+def test_blockwise_gemm_full_size_properties(ops, oracle):
+    """Size-independent properties of the fp8 tile kernel at a full benchmark shape (M = 4096, N = 7168, K = 18432):
+    doubling the activations doubles the scales and leaves the codes alone, so every output doubles exactly; permuting
+    the rows of x permutes the rows of the output bit for bit."""
+    m, n, k = 4096, 7168, 18432
+    g = H.gen(4700)
+    b = torch.randint(0, 256, (n, k), generator=g, dtype=torch.uint8)
+    b = torch.where((b & 0x7f) == 0x7f, b & 0xfe, b)          # no NaN codes
+    bs = (torch.rand((n // 128, k // 128), generator=g) * 1e-4 + 1e-4).cuda()
+    bp = ops.fp8_repack_weight(b.cuda())
+    x = torch.randn((m, k), generator=g).to(torch.bfloat16).cuda()
+    q, s = ops.per_token_group_quant_fp8(x, k, 128, True)
+    y = ops.fp8_blockwise_gemm(q, s, bp, bs, torch.bfloat16)
+    assert torch.all(torch.isfinite(y)) and y.abs().max() > 0
+    q2, s2 = ops.per_token_group_quant_fp8(x * 2, k, 128, True)
+    assert torch.equal(q2, q) and torch.equal(s2, s * 2)
+    assert torch.equal(ops.fp8_blockwise_gemm(q2, s2, bp, bs, torch.bfloat16), y * 2)
+    perm = torch.randperm(m, generator=g).cuda()
+    qp, sp = ops.per_token_group_quant_fp8(x[perm].contiguous(), k, 128, True)
+    assert torch.equal(ops.fp8_blockwise_gemm(qp, sp, bp, bs, torch.bfloat16), y[perm])

@@ -191,3 +191,28 @@ def test_decode_k_parts(ops, dtype, awq, M, N, K):
         with pytest.raises(L.KsqError) as e:
             ops.w4a16_gemm(d["x"].cuda(), wp, sp, zp, N, K, 128, workspace=torch.empty(64, dtype=torch.uint8, device="cuda"))
         assert e.value.code == 3
+
+
+@pytest.mark.parametrize("N,K", [(25600, 5120), (5120, 25600)])
+def test_prefill_full_size_properties(ops, N, K):
+    """Size-independent properties of the MFMA tile kernel at the full prefill benchmark shapes (M = 2048; for
+    N = 5120 the launch holds whole tiles and tiles cut along K): doubling the activations doubles every output
+    exactly (outside fp16's subnormal range), a zero row gives a zero row, and permuting the rows of x permutes the rows of y bit for bit."""
+    from ksanallm_amd import lib as L
+    M = 2048
+    d = H.make_w4a16(4100 + N, 8, N, K, 128, H.F16, awq=False, x_std=0.5, s_lo=0.002, s_hi=0.01)
+    wp = ops.repack_weight(d["qweight"].cuda(), L.SRC_GPTQ, 1, K, N)
+    sp = ops.repack_scales(d["scales"].cuda(), L.SCALE_GN, 1, K, N, 128)
+    g = H.gen(4200 + K)
+    x = (torch.randn((M, K), generator=g) * 0.5).to(torch.float16).cuda()
+    x[5] = 0
+    y = ops.w4a16_gemm(x, wp, sp, None, N, K, 128)
+    assert torch.all(torch.isfinite(y)) and torch.all(y[5] == 0) and y.abs().max() > 0
+    y2 = ops.w4a16_gemm(x * 2, wp, sp, None, N, K, 128)
+    # (outputs in fp16's subnormal range round on an absolute grid, where rounding and doubling do not commute)
+    normal = y.abs() >= 2.0 ** -13
+    assert torch.equal(y2[normal], (y * 2)[normal])
+    assert (y2.float() - 2 * y.float())[~normal].abs().max() <= 2.0 ** -23
+    perm = torch.randperm(M, generator=g).cuda()
+    yp = ops.w4a16_gemm(x[perm].contiguous(), wp, sp, None, N, K, 128)
+    assert torch.equal(yp, y[perm])
