@@ -1,11 +1,12 @@
 // Prefill-regime blockwise-FP8 kernel (MFMA-bound): a workgroup of 8 wavefronts (2 along M x 4 along N) computes a
 // 256 x 256 output tile over a contiguous range of 128-deep k-blocks.
 //
-//   - both operands are e4m3 bytes, K-contiguous, and need no conversion, so both go global -> LDS without touching
-//     registers (global_load_lds_dwordx4), one 128-deep k-block (32 KiB of activations + 32 KiB of weights) per stage,
-//     two stages.  A 16-row x 128-byte MFMA operand is kept as a 2 KiB fragment filled by two loads of 64 contiguous
-//     bytes per row, its 16-byte pieces swizzled so that a lane reads its operand back with two ds_read_b128 free of
-//     bank conflicts.
+//   - both operands are e4m3 bytes and need no conversion, so both go global -> LDS without touching registers
+//     (global_load_lds_dwordx4), one 128-deep k-block (32 KiB of activations + 32 KiB of weights) per stage, two
+//     stages.  A 16-row x 128-byte MFMA operand is a 2 KiB fragment read back with two ds_read_b128 per lane.
+//     Activation fragments are filled from the row-major [m, k] bytes by two loads of 64 contiguous bytes per row,
+//     their 16-byte pieces swizzled so that the read-back is free of bank conflicts; weight fragments arrive packed
+//     (ksq_fp8_repack_weight) as two contiguous KiB and are read back in lane order.
 //   - one v_mfma_f32_16x16x128_f8f6f4 covers exactly one scale block: its result goes to a scratch tile and is folded
 //     into the accumulator with a_s[kb, m] * b_s[n/128, kb] by four fp32 FMAs, issued under the following MFMA.
 //   - activation scales reach the lanes through LDS as well (one small LDS-targeted load per stage), the weight
@@ -76,8 +77,8 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
   const uint32_t kb_count = direct ? KB : ((KB - kb_begin) < p.kb_per_split ? (KB - kb_begin) : p.kb_per_split);
 
   // ---- operand staging.  Wavefronts 0..3 fetch the activation fragments 4w..4w+3, wavefronts 4..7 the weight
-  // fragments 4(w-4)..+3.  An activation fragment (16 rows x 128 bytes) is two loads, one per 64-byte half h of the rows; in a
-  // load four consecutive lanes take the four 16-byte pieces of one row (64 contiguous bytes: the granularity at which
+  // fragments 4(w-4)..+3.  An activation fragment (16 rows x 128 bytes) is two loads, one per 64-byte half h of the
+  // rows; in a load four consecutive lanes take the four 16-byte pieces of one row (64 contiguous bytes: the granularity at which
   // the memory pipeline runs at full rate).  Load lane j lands at 1024h + 16j = 1024h + 64*(j/4) + 16*(j%4) and
   // fetches piece (j%4) ^ (j/16) of row j/4, so that MFMA lane (row r, k slot q) finds its two pieces 2(q%2)+p at
   // 1024*(q/2) + 64r + 16*((2(q%2)+p) ^ (r/4)): the sixteen lanes that read together hit different bank groups.
