@@ -25,6 +25,12 @@
  *                                     K/blockwise_gemm/blockwise_gemm_test.cu:138-177
  *   moe_align ....................... worked example in K/moe_utils/moe_utils.cu:150-156, invariants
  *   silu_mul / moe_sum .............. closed forms (K/moe_utils/moe_utils.cu:597-606,549-562)
+ *   moe_gemm ........................ equals the dense dequantize-then-multiply of each expert's rows
+ *   moe_topk_softmax ................ torch softmax + topk
+ *   moe_grouped_topk ................ the published DeepSeek-V2/V3 formula in torch tensor ops, and the reference's own
+ *                                     host implementation compiled from the reference tree (oracle/_ref)
+ *   fp8_channel_quant ............... torch float8_e4m3fn conversion, every rounding boundary
+ *   fp8_tensor_gemm ................. torch fp32 matmul of the decoded operands
  */
 #include <math.h>
 #include <stdint.h>
@@ -686,7 +692,8 @@ KSQO_API void ksqo_moe_topk_softmax(const void* gating, float* topk_w, int32_t* 
  * tensor-op form of S/kernels/nvidia/moe_kernel_wrapper.cpp:286-347 for the other options (softmax scoring, no
  * bias -> group rank = largest, renormalize off, experts outside the kept groups excluded outright).
  * Picks are by repeated arg-max, the lower index winning ties.
- * Pinned by tests/test_oracle_golden.py against the published DeepSeek-V3 formula written with torch tensor ops. */
+ * Pinned by tests/test_oracle_golden.py against the published DeepSeek-V3 formula written with torch tensor ops and
+ * against that reference header itself, compiled from the reference tree into oracle/_ref (ref_grouped_topk.cpp). */
 KSQO_API void ksqo_moe_grouped_topk(const void* gating, const float* bias, float* topk_w, int32_t* topk_ids,
                                     size_t tokens, size_t E, size_t top_k, size_t groups, size_t topk_group,
                                     int sigmoid, int renorm, float scaling, int dtype) {

@@ -25,6 +25,39 @@ def build(force=False):
     return _SO
 
 
+_REF_SO = os.path.join(_HERE, "_ref", "libksq_ref.so")
+_REF_HEADER = "/root/reference/3rdparty/LLM_kernels/tests/references/deepseek_v3_grouped_topk.h"
+
+
+def build_ref():
+    """Compile the reference's own host router (oracle/ref_grouped_topk.cpp around its header) into oracle/_ref/ where
+    the reference tree is present; returns the library path or None."""
+    if os.path.exists(_REF_HEADER):
+        subprocess.check_call(["make", "-C", _HERE, "-B", "ref"], stdout=subprocess.DEVNULL)
+    return _REF_SO if os.path.exists(_REF_SO) else None
+
+
+_ref = None
+
+
+def ref_grouped_topk(gating_f32, bias_f32, top_k, groups, topk_group, scaling):
+    """RunDeepSeekV3GroupedTopkRef<float> of the reference (sigmoid scores, bias-corrected choice, top-2 group rank,
+    renormalized weights times `scaling`) from oracle/_ref; None when that library has not been built."""
+    global _ref
+    if _ref is None:
+        if not os.path.exists(_REF_SO):
+            return None
+        _ref = ctypes.CDLL(_REF_SO)
+    g = np.ascontiguousarray(gating_f32, np.float32)
+    b = np.ascontiguousarray(bias_f32, np.float32)
+    T, E = g.shape
+    w = np.zeros((T, top_k), np.float32)
+    ids = np.zeros((T, top_k), np.int32)
+    _ref.ksq_ref_grouped_topk(_p(g), _p(b), ctypes.c_float(scaling), _p(w), _p(ids), ctypes.c_int(T), ctypes.c_int(E),
+                              ctypes.c_int(top_k), ctypes.c_int(groups), ctypes.c_int(topk_group))
+    return w, ids
+
+
 _lib = None
 
 

@@ -110,6 +110,29 @@ def test_grouped_topk(ops, oracle, T, E, topk, groups, topk_group, scoring, use_
             np.testing.assert_allclose(w.cpu().numpy().sum(-1), 2.5, rtol=1e-5)
 
 
+# the HIP router against the reference's own host implementation (oracle/_ref, built beforehand from the reference tree)
+@pytest.mark.parametrize("T,E,topk,groups,topk_group", [(2048, 256, 8, 8, 4), (333, 128, 4, 4, 2)])
+def test_grouped_topk_vs_reference_host_code(ops, oracle, T, E, topk, groups, topk_group):
+    g = H.gen(3 * T + E)
+    logits = torch.rand((T, E), generator=g) * 1.98 - 0.99
+    bias = torch.rand(E, generator=g) * 0.009 - 0.01
+    ref = oracle.ref_grouped_topk(logits.numpy(), bias.numpy(), topk, groups, topk_group, 2.5)
+    if ref is None:
+        pytest.skip("oracle/_ref is not built")
+    rw, ri = ref
+    w, ids = ops.moe_grouped_topk(logits.cuda(), topk, groups, topk_group, "sigmoid", bias.cuda(), True, 2.5)
+    w, ids = w.cpu().numpy(), ids.cpu().numpy()
+    swapped = 0
+    for t in range(T):
+        if sorted(ids[t].tolist()) != sorted(ri[t].tolist()):
+            swapped += 1      # GPU and host expf may order two near-equal scores differently
+            continue
+        mine = dict(zip(ids[t].tolist(), w[t].tolist()))
+        for e, x in zip(ri[t].tolist(), rw[t].tolist()):
+            assert abs(mine[e] - x) <= 3e-4, (t, e, mine[e], x)
+    assert swapped <= T // 200, swapped
+
+
 def test_grouped_topk_matches_plain_softmax_router(ops):
     g = H.gen(5)
     logits = torch.randn((33, 256), generator=g).cuda()

@@ -391,6 +391,27 @@ def test_grouped_topk_vs_torch(oracle, E, top_k, groups, topk_group, sigmoid, us
     assert max(len(set((row // per).tolist())) for row in ids) <= topk_group
 
 
+# The reference's own host implementation of the router (compiled from the reference tree into oracle/_ref by
+# `make -C oracle ref`; it exists for fp32 logits, sigmoid scoring with a correction bias and renormalized weights):
+# same picks per token, same weight per pick.  Its heap returns a token's picks in another order, so picks are compared
+# as sets and weights by expert id.
+@pytest.mark.parametrize("T,E,top_k,groups,topk_group", [(301, 256, 8, 8, 4), (64, 128, 4, 4, 2), (17, 64, 6, 4, 3)])
+def test_grouped_topk_vs_reference_host_code(oracle, T, E, top_k, groups, topk_group):
+    g = torch.Generator().manual_seed(7 * E + T)
+    logits = (torch.rand((T, E), generator=g) * 1.98 - 0.99).numpy()
+    bias = (torch.rand(E, generator=g) * 0.009 - 0.01).numpy()
+    ref = oracle.ref_grouped_topk(logits, bias, top_k, groups, topk_group, 2.5)
+    if ref is None:
+        pytest.skip("oracle/_ref is not built (the reference tree is not on this machine)")
+    rw, ri = ref
+    w, ids = oracle.moe_grouped_topk(logits, bias, top_k, groups, topk_group, True, True, 2.5, oracle.F32)
+    for t in range(T):
+        assert sorted(ids[t].tolist()) == sorted(ri[t].tolist()), t
+        mine = dict(zip(ids[t].tolist(), w[t].tolist()))
+        for e, x in zip(ri[t].tolist(), rw[t].tolist()):
+            assert abs(mine[e] - x) <= 2e-6 * 2.5, (t, e, mine[e], x)
+
+
 def test_grouped_topk_ties_and_group_rank(oracle):
     # 2 groups of 4; group 1 holds the single largest value but group 0 the larger top-2 sum: with a bias the rank is
     # the top-2 sum (group 0 kept), without it the maximum (group 1 kept)
