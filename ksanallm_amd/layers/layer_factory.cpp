@@ -3,6 +3,7 @@
 #include "blockwise_matmul_layer.h"
 #include "fp8_matmul_layer.h"
 #include "moe_layer.h"
+#include "marlin_moe_layer.h"
 #include "w4a16_matmul_layer.h"
 
 namespace ksana_llm {
@@ -59,6 +60,8 @@ MoeLayerFactory::MoeLayerFactory(const ModelConfig& model_config, const RuntimeC
   // "deepseek moe-int4" rows of the reference
   builder_map_[{TYPE_UINT8, TYPE_FP16, TYPE_FP16, MOE_QUANT_GPTQ, TRITON_MOE_BACKEND}] = &MoeLayerFactory::BuildLayer<MoeLayer>;
   builder_map_[{TYPE_UINT8, TYPE_BF16, TYPE_BF16, MOE_QUANT_GPTQ, TRITON_MOE_BACKEND}] = &MoeLayerFactory::BuildLayer<MoeLayer>;
+  // "hunyuan-large int4" row
+  builder_map_[{TYPE_I4_GROUP, TYPE_FP16, TYPE_FP16, MOE_QUANT_GPTQ, MARLIN_MOE_BACKEND}] = &MoeLayerFactory::BuildLayer<MarlinMoeLayer>;
   // "deepseek fp8 blockwise" rows
   builder_map_[{TYPE_FP8_E4M3, TYPE_FP16, TYPE_FP16, MOE_QUANT_BLOCK_FP8_E4M3, TRITON_MOE_BACKEND}] = &MoeLayerFactory::BuildLayer<MoeLayer>;
   builder_map_[{TYPE_FP8_E4M3, TYPE_BF16, TYPE_BF16, MOE_QUANT_BLOCK_FP8_E4M3, TRITON_MOE_BACKEND}] = &MoeLayerFactory::BuildLayer<MoeLayer>;

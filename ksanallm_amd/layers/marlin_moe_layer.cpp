@@ -1,0 +1,48 @@
+#include "marlin_moe_layer.h"
+
+namespace ksana_llm {
+
+Status MarlinMoeLayer::Init(const std::vector<std::any>& parameters, const RuntimeConfig& runtime_config,
+                            std::shared_ptr<Context> context, int rank) {
+  if (parameters.size() < 20) return Status(RET_INVALID_ARGUMENT, "MarlinMoeLayer: expects 20 init parameters");
+  // the same values in MoeLayer's order: the layer index is the one this interface does not carry
+  std::vector<std::any> p(parameters.begin(), parameters.begin() + 2);
+  p.push_back(static_cast<int>(0));
+  p.insert(p.end(), parameters.begin() + 2, parameters.begin() + 20);
+  // fused_marlin_moe routes with a plain softmax top-k whatever the routing fields say, and never scales the weights
+  p[9] = static_cast<uint32_t>(1);    // num_expert_group
+  p[10] = static_cast<uint32_t>(1);   // expert_groups_topk
+  p[11] = std::string("softmax");     // scoring_func
+  p[12] = std::string("greedy");      // topk_method
+  p[13] = false;                      // norm_topk_prob: the norm mode alone decides
+  p[14] = 1.0f;                       // routed_scaling_factor
+  p[15] = false;                      // use_e_score_correction_bias
+  p[8] = true;                        // the aligned-block flow is the only one here
+  if (std::any_cast<DataType>(parameters[16]) != TYPE_INVALID)
+    return Status(RET_INVALID_ARGUMENT, "MarlinMoeLayer: fp8 expert weights do not belong to this layer");
+  p[18] = TYPE_UINT4x2;               // int_weight_dtype: 4-bit codes, two per byte
+  if (runtime_config.inter_data_type != TYPE_FP16)
+    return Status(RET_INVALID_ARGUMENT, "MarlinMoeLayer: only fp16 activations (marlin_moe_layer.cpp:96-99)");
+  return MoeLayer::Init(p, runtime_config, context, rank);
+}
+
+Status MarlinMoeLayer::Forward(const std::vector<Tensor>& input_tensors, std::vector<Tensor>& output_tensors) {
+  if (input_tensors.size() < 4) KLLM_THROW("MarlinMoeLayer: expects hidden_states, gating_output, up_gate weight, down weight");
+  if (input_tensors[0].dtype != TYPE_FP16) {
+    KLLM_THROW("marlin moe only support input type " + std::to_string(TYPE_FP16) + ", not support input type " +
+               std::to_string(input_tensors[0].dtype));
+  }
+  for (int i : {2, 3}) {
+    if (input_tensors[i].GetPtr<void>() == nullptr) KLLM_THROW("w1 or w2 is nullptr.");
+    if (!input_tensors[i].scales || input_tensors[i].scales->GetPtr<void>() == nullptr)
+      KLLM_THROW("w1_scales or w2_scales is nullptr.");
+    if (input_tensors[i].g_idx || input_tensors[i].perm)
+      KLLM_THROW("MarlinMoeLayer: act-order experts (g_idx / perm) are not built");
+    if (input_tensors[i].zeros) KLLM_THROW("MarlinMoeLayer: expert zero points are not built");
+  }
+  // hidden_states, gating_output, w1, w2 only: the router of this layer takes no bias and no expert map
+  std::vector<Tensor> inputs(input_tensors.begin(), input_tensors.begin() + 4);
+  return MoeLayer::Forward(inputs, output_tensors);
+}
+
+}  // namespace ksana_llm

@@ -53,6 +53,21 @@ Tensor PackGroupQuantWeight(const Tensor& qweight, const Tensor& scales, const T
   return packed;
 }
 
+Tensor PackGptqExpertWeight(const Tensor& qweight, const Tensor& scales, size_t group_size, int rank, hipStream_t stream) {
+  const char* who = "PackGptqExpertWeight";
+  if (qweight.shape.size() != 3 || scales.shape.size() != 3) KLLM_THROW("PackGptqExpertWeight: 3-D tensors expected");
+  const size_t E = qweight.shape[0], K = qweight.shape[1] * 8, N = qweight.shape[2];
+  if (scales.shape[0] != E || scales.shape[1] * group_size != K || scales.shape[2] != N) {
+    KLLM_THROW("PackGptqExpertWeight: scales shape mismatch");
+  }
+  const int dtype = KsqDtype(scales.dtype, who);
+  Tensor packed(MemoryLocation::LOCATION_DEVICE, TYPE_I4_GROUP, {E, K, N / 2}, rank);
+  KsqCheck(ksq_w4a16_repack(qweight.GetPtr<void>(), KSQ_SRC_GPTQ, packed.GetPtr<void>(), E, K, N, stream), who);
+  packed.scales = std::make_shared<Tensor>(MemoryLocation::LOCATION_DEVICE, scales.dtype, scales.shape, rank);
+  KsqCheck(ksq_w4a16_repack_scales(scales.GetPtr<void>(), KSQ_SCALE_GN, packed.scales->GetPtr<void>(), E, K, N, group_size, dtype, stream), who);
+  return packed;
+}
+
 Tensor PackMoeExpertWeight(const Tensor& experts, const Tensor& scales, size_t group_size, int rank, hipStream_t stream) {
   const char* who = "PackMoeExpertWeight";
   if (experts.shape.size() != 3 || scales.shape.size() != 3) KLLM_THROW("PackMoeExpertWeight: 3-D tensors expected");

@@ -24,6 +24,11 @@ Tensor PackGroupQuantWeight(const Tensor& qweight, const Tensor& scales, const T
 // Returns a TYPE_UINT4x2 tensor of logical shape {E, N, K/2} with `scales` bound.
 Tensor PackMoeExpertWeight(const Tensor& experts, const Tensor& scales, size_t group_size, int rank, hipStream_t stream);
 
+// GPTQ expert stack as the Marlin MoE loader holds it before its own repack: qweight [E, K/8, N] int32, scales
+// [E, K/group, N] in T (symmetric, no act-order).  Returns a TYPE_I4_GROUP tensor of logical shape {E, K, N/2} with
+// `scales` bound: the same packed tiles PackMoeExpertWeight produces, for MarlinMoeLayer.
+Tensor PackGptqExpertWeight(const Tensor& qweight, const Tensor& scales, size_t group_size, int rank, hipStream_t stream);
+
 // FP8 (e4m3) weights, [N, K] or an expert stack [E, N, K] in checkpoint layout: returns the same shape and dtype in the
 // packed 2 KiB fragment layout every FP8 layer here consumes (BlockwiseMatMulLayer, Fp8MatMulLayer, MoeLayer with
 // block-fp8 experts); the side tensors of `weight` (weight_scales, input_scales, ...) are carried over unchanged.

@@ -8,6 +8,7 @@
 //   layer_test fp8_tensor <dir> <f16|bf16> m n k static
 //   layer_test moe       <dir> <f16|bf16> tokens experts hidden inter topk renorm scaling [groups topk_group scoring use_bias]
 //   layer_test moe_fp8   <dir> <f16|bf16> tokens experts hidden inter topk renorm scaling
+//   layer_test marlin_moe <dir> f16 tokens experts hidden inter topk renorm
 //   layer_test errors
 #include <hip/hip_runtime.h>
 
@@ -21,6 +22,7 @@
 #include "layer_factory.h"
 #include "fp8_matmul_layer.h"
 #include "moe_layer.h"
+#include "marlin_moe_layer.h"
 #include "quant_weight_repack.h"
 #include "w4a16_matmul_layer.h"
 
@@ -251,6 +253,56 @@ static int RunMoe(int argc, char** argv) {
   return 0;
 }
 
+// GPTQ experts behind the Marlin MoE interface (fp16): qw13.bin int32 [E, hidden/8, 2*inter], s13.bin [E, hidden/128,
+// 2*inter], qw2.bin int32 [E, inter/8, hidden], s2.bin [E, inter/128, hidden], gating.bin fp16 [tokens, E]
+static int RunMarlinMoe(int argc, char** argv) {
+  if (argc < 10) return 2;
+  const std::string dir = argv[2];
+  const DataType T = ParseT(argv[3]);
+  const size_t tokens = std::atol(argv[4]), E = std::atol(argv[5]), hidden = std::atol(argv[6]), inter = std::atol(argv[7]),
+               topk = std::atol(argv[8]);
+  const bool renorm = std::atoi(argv[9]) != 0;
+  hipStream_t stream;
+  HIP_OK(hipStreamCreate(&stream));
+  auto context = std::make_shared<Context>(1, stream);
+  ModelConfig mc;
+  RuntimeConfig rc;
+  rc.inter_data_type = T;
+  Tensor w13 = PackGptqExpertWeight(Upload(dir + "/qw13.bin", TYPE_INT32, {E, hidden / 8, 2 * inter}),
+                                    Upload(dir + "/s13.bin", T, {E, hidden / 128, 2 * inter}), 128, 0, stream);
+  Tensor w2 = PackGptqExpertWeight(Upload(dir + "/qw2.bin", TYPE_INT32, {E, inter / 8, hidden}),
+                                   Upload(dir + "/s2.bin", T, {E, inter / 128, hidden}), 128, 0, stream);
+  HIP_OK(hipStreamSynchronize(stream));
+  // the reference's 20 positional values (marlin_moe_layer.cpp:16-36); the routing fields are ignored by this layer
+  std::vector<std::any> params{renorm ? MoeScaleNormMode::RE_NORM : MoeScaleNormMode::NO_NORM,
+                               tokens, E, hidden, inter, topk, size_t(1), false, uint32_t(1), uint32_t(1),
+                               std::string("softmax"), std::string("greedy"), false, 1.0f, false, false,
+                               TYPE_INVALID, TYPE_I4_GROUP, int(128), false};
+  MoeLayerFactory factory(mc, rc, 0, context);
+  auto layer = factory.CreateLayer(TYPE_I4_GROUP, T, T, params, MOE_QUANT_GPTQ, MARLIN_MOE_BACKEND);
+  Tensor x = Upload(dir + "/x.bin", T, {tokens, hidden});
+  Tensor gating = Upload(dir + "/gating.bin", T, {tokens, E});
+  std::vector<Tensor> outputs{Tensor(MemoryLocation::LOCATION_DEVICE, T, {tokens, hidden}, 0)};
+  Drive(layer, mc, rc, {x, gating, w13, w2}, outputs);
+  HIP_OK(hipStreamSynchronize(stream));
+  Download(outputs[0], dir + "/y.bin");
+  // act-order experts are refused with a message, not run wrongly
+  Tensor w13_act = w13;
+  w13_act.perm = std::make_shared<Tensor>(MemoryLocation::LOCATION_DEVICE, TYPE_INT32, std::vector<size_t>{E, hidden}, 0);
+  bool threw = false;
+  try {
+    std::vector<Tensor> in2{x, gating, w13_act, w2};
+    layer->Forward(in2, outputs);
+  } catch (const std::exception&) {
+    threw = true;
+  }
+  if (!threw) {
+    std::fprintf(stderr, "FAILED: act-order experts were accepted\n");
+    return 1;
+  }
+  return 0;
+}
+
 // block-fp8 experts: w13.bin [E, 2*inter, hidden] e4m3, s13.bin fp32 [E, 2*inter/128, hidden/128], w2.bin, s2.bin alike
 static int RunMoeFp8(int argc, char** argv) {
   if (argc < 11) return 2;
@@ -370,6 +422,21 @@ static int RunErrors() {
     Tensor w(MemoryLocation::LOCATION_DEVICE, TYPE_FP8_E4M3, {64, 512}, 0, reinterpret_cast<void*>(0x1000));
     expect(throws([&] { layer.Forward({x, w}, out); }), "Forward without a workspace buffer throws");
   }
+  // marlin moe: fp16 only, 20 parameters
+  {
+    std::vector<std::any> p{MoeScaleNormMode::RE_NORM, size_t(8), size_t(8), size_t(256), size_t(128), size_t(2), size_t(1),
+                            true, uint32_t(1), uint32_t(1), std::string("softmax"), std::string("greedy"), false, 1.0f,
+                            false, false, TYPE_INVALID, TYPE_I4_GROUP, int(128), false};
+    MarlinMoeLayer ok, bf, shortp;
+    RuntimeConfig half = rc, bf16 = rc;
+    half.inter_data_type = TYPE_FP16;
+    bf16.inter_data_type = TYPE_BF16;
+    expect(ok.Init(p, half, context, 0).OK(), "marlin moe fp16 init");
+    expect(ok.GetWorkspaceSize() > 0, "marlin moe workspace size");
+    expect(!bf.Init(p, bf16, context, 0).OK(), "marlin moe rejects bf16");
+    p.pop_back();
+    expect(!shortp.Init(p, half, context, 0).OK(), "marlin moe rejects a short parameter list");
+  }
   // moe: fp8 experts / impossible expert groups rejected, int4 and grouped routing accepted
   {
     MoeLayer a, b, c;
@@ -415,6 +482,7 @@ int main(int argc, char** argv) {
     if (mode == "fp8_tensor") return RunFp8Tensor(argc, argv);
     if (mode == "moe") return RunMoe(argc, argv);
     if (mode == "moe_fp8") return RunMoeFp8(argc, argv);
+    if (mode == "marlin_moe") return RunMarlinMoe(argc, argv);
     if (mode == "errors") return RunErrors();
   } catch (const std::exception& e) {
     std::fprintf(stderr, "exception: %s\n", e.what());

@@ -126,6 +126,39 @@ def test_moe_layer(tmp_path, oracle, dtype, tokens, renorm, scaling, routing):
     H.check_gemm(y, ref, dtype, "moe layer", weights_rounded=rounded, rel_l2_max=5e-3 * (2 ** 0.5 if rounded else 1.0))
 
 
+# GPTQ experts behind the Marlin MoE interface: checkpoint-layout int32 words, fp16 gating output, plain softmax router
+@pytest.mark.gpu
+@pytest.mark.parametrize("tokens,renorm", [(1, 0), (37, 1), (400, 1)])
+def test_marlin_moe_layer(tmp_path, oracle, tokens, renorm):
+    E, hidden, inter, topk = 16, 256, 128, 4
+    dtype = H.F16
+    g = H.gen(9300 + tokens)
+
+    def experts(n, k):
+        codes = torch.randint(0, 16, (E, n, k), generator=g, dtype=torch.uint8).numpy()
+        moe_bytes = (codes[:, :, 0::2] | (codes[:, :, 1::2] << 4)).astype(np.uint8)          # [E, n, k/2], low nibble = even k
+        c = codes.transpose(0, 2, 1).reshape(E, k // 8, 8, n).astype(np.uint32)              # [E, k/8, 8, n]
+        words = np.zeros((E, k // 8, n), np.uint32)
+        for j in range(8):
+            words |= c[:, :, j, :] << np.uint32(4 * j)                                          # GPTQ: nibble j = row 8i+j
+        scales = H.uniform(g, (E, n, k // 128), 0.002, 0.01, dtype)
+        return moe_bytes, words.view(np.int32), scales
+
+    w13, qw13, s13 = experts(2 * inter, hidden)
+    w2, qw2, s2 = experts(hidden, inter)
+    x = torch.randn((tokens, hidden), generator=g).to(H.TORCH_DT[dtype])
+    gating = torch.randn((tokens, E), generator=g).to(torch.float16)
+    for name, arr in (("qw13", qw13), ("qw2", qw2), ("s13", H.bits_of(s13.transpose(1, 2).contiguous())),
+                      ("s2", H.bits_of(s2.transpose(1, 2).contiguous())), ("x", H.bits_of(x)), ("gating", H.bits_of(gating))):
+        np.ascontiguousarray(arr).tofile(tmp_path / (name + ".bin"))
+    run_driver("marlin_moe", tmp_path, TNAME[dtype], tokens, E, hidden, inter, topk, renorm)
+    y = read_out(tmp_path / "y.bin", dtype, (tokens, hidden))
+    tw, ids = oracle.moe_topk_softmax(H.bits_of(gating), topk, bool(renorm), 1.0, H.F16)
+    ref = oracle.from_bits(oracle.moe_forward(H.bits_of(x), w13, H.bits_of(s13), w2, H.bits_of(s2), ids, tw, 128, dtype), dtype)
+    rounded = tokens * topk // E >= 64
+    H.check_gemm(y, ref, dtype, "marlin moe layer", weights_rounded=rounded, rel_l2_max=5e-3 * (2 ** 0.5 if rounded else 1.0))
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype,tokens,renorm,scaling", [(H.BF16, 1, 0, 2.5), (H.F16, 40, 1, 1.0), (H.BF16, 300, 1, 1.0)])
 def test_moe_layer_block_fp8(tmp_path, oracle, dtype, tokens, renorm, scaling):
