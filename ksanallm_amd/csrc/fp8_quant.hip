@@ -2,6 +2,16 @@
 //   amax = max(1e-10, max|x|),  s = amax / 448,  q = e4m3_rne_satfinite(x / s)      (IEEE fp32 divisions)
 // Each lane owns 8 consecutive channels (one 16-byte load, one 8-byte store); a group of `GROUP` channels is
 // GROUP/8 adjacent lanes, reduced with cross-lane shuffles, so a wavefront covers 512 contiguous channels.
+//
+// The kernels are HBM-bound only if the arithmetic stays small: a full IEEE division is about ten instructions, eight
+// of them per lane were more than the memory pipeline leaves time for.  x / s is therefore formed from ONE correctly
+// rounded reciprocal per lane, y = 1 / s, and a residual correction per element,
+//     q0 = x * y,   r = fma(-q0, s, x)  (exact),   q = fma(r, y, q0),
+// which is the correctly rounded quotient (Markstein's theorem) as long as r stays in the normal range;
+// tests/cpp/exact_div_test.c checks it against the division for every one of the 2^23 mantissas of s and every
+// mantissa a 16-bit input can have.  The sign of x is put back afterwards (x = -0 would otherwise come out as +0).
+// Scales outside [2^-80, 2^100] take the division itself; inside, r is exact whenever |x / s| >= 2^-20, and a smaller
+// quotient that is one unit in the last place off still converts to the same signed zero.
 #include "ksq_common.h"
 
 namespace ksq {
@@ -18,16 +28,40 @@ __device__ __forceinline__ uint32_t cvt2_e4m3(float a, float b, uint32_t old, bo
             : static_cast<uint32_t>(__builtin_amdgcn_cvt_pk_fp8_f32(ca, cb, static_cast<int>(old), false));
 }
 
-template <typename T, int GROUP, bool COLMAJOR, bool FUSE>
-__global__ void __launch_bounds__(256) fp8_group_quant_kernel(const uint16_t* __restrict__ x, uint8_t* __restrict__ q,
-                                                              float* __restrict__ s, uint32_t m, uint32_t k) {
+// x / s, correctly rounded, for many x and one s (see the head of this file)
+struct ExactDiv {
+  float s, y;
+  bool fast;
+  __device__ __forceinline__ explicit ExactDiv(float scale)
+      : s(scale), y(1.0f / scale), fast(scale >= 0x1p-80f && scale <= 0x1p100f) {}
+  // |x| finite or NaN; an infinite x needs the caller's attention (r would be NaN)
+  __device__ __forceinline__ float operator()(float x) const {
+    if (!fast) return x / s;
+    const float q0 = x * y;
+    const float r = __builtin_fmaf(-q0, s, x);
+    return __builtin_copysignf(__builtin_fmaf(r, y, q0), x);
+  }
+};
+
+// two quotients that are known to lie within +-448 * (1 + 2^-23), or NaN: no clamp in front of the conversion
+__device__ __forceinline__ uint32_t cvt2_e4m3_in_range(float a, float b, uint32_t old, bool hi) {
+  return hi ? static_cast<uint32_t>(__builtin_amdgcn_cvt_pk_fp8_f32(a, b, static_cast<int>(old), true))
+            : static_cast<uint32_t>(__builtin_amdgcn_cvt_pk_fp8_f32(a, b, static_cast<int>(old), false));
+}
+
+// Grid: x = chunks of BLOCK*8 channels of a row, y and z = the row (token) as z * gridDim.y + y, so that no index needs
+// an integer division (about fifty instructions on this ISA, more than the rest of the kernel).  Lanes past the end of
+// the row in its last chunk idle; groups never straddle a chunk.
+template <typename T, int GROUP, bool COLMAJOR, bool FUSE, int BLOCK>
+__global__ void __launch_bounds__(BLOCK) fp8_group_quant_kernel(const uint16_t* __restrict__ x, uint8_t* __restrict__ q,
+                                                                float* __restrict__ s, uint32_t m, uint32_t k) {
   constexpr int LPG = GROUP / 8;  // lanes per group
-  const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
-  const size_t total = static_cast<size_t>(m) * k / 8;
-  const bool live = i < total;
-  const size_t e0 = (live ? i : 0) * 8;
-  const uint32_t t = static_cast<uint32_t>(e0 / k);
-  const uint32_t col = static_cast<uint32_t>(e0 % k);
+  const uint32_t row = blockIdx.z * gridDim.y + blockIdx.y;
+  const uint32_t col0 = (blockIdx.x * BLOCK + threadIdx.x) * 8;
+  const bool live = row < m && col0 < k;
+  const uint32_t t = live ? row : 0;
+  const uint32_t col = live ? col0 : 0;
+  const size_t e0 = static_cast<size_t>(t) * k + col;
 
   float v[8];
   {
@@ -60,7 +94,17 @@ __global__ void __launch_bounds__(256) fp8_group_quant_kernel(const uint16_t* __
 #pragma unroll
   for (int off = LPG / 2; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, LPG));
 
-  const float scale = amax / 448.0f;
+  // amax / 448, correctly rounded, by the same reciprocal-and-correction (amax has at most 11 significant bits, or is
+  // the floor 1e-10, whose quotient is a constant)
+  float scale;
+  {
+    constexpr float y448 = 1.0f / 448.0f;
+    const float q0 = amax * y448;
+    const float r = __builtin_fmaf(-q0, 448.0f, amax);
+    scale = __builtin_fmaf(r, y448, q0);
+    scale = amax == 1e-10f ? 1e-10f / 448.0f : scale;
+    scale = (amax >= 0x1p-60f && amax <= 0x1p100f) ? scale : amax / 448.0f;
+  }
   if (!live) return;
   if ((threadIdx.x % LPG) == 0) {
     const uint32_t g = col / GROUP;
@@ -68,27 +112,45 @@ __global__ void __launch_bounds__(256) fp8_group_quant_kernel(const uint16_t* __
     s[COLMAJOR ? static_cast<size_t>(g) * m + t : static_cast<size_t>(t) * ng + g] = scale;
   }
   u32x2 out{0u, 0u};
-  out.x = cvt2_e4m3(v[0] / scale, v[1] / scale, out.x, false);
-  out.x = cvt2_e4m3(v[2] / scale, v[3] / scale, out.x, true);
-  out.y = cvt2_e4m3(v[4] / scale, v[5] / scale, out.y, false);
-  out.y = cvt2_e4m3(v[6] / scale, v[7] / scale, out.y, true);
+  const ExactDiv div(scale);
+  if (div.fast) {
+    // every |v| <= amax (an infinite v makes amax, hence the scale, infinite: not this branch), so the quotients stay
+    // within 448 * (1 + 2^-23), which the conversion rounds to 448 by itself
+    out.x = cvt2_e4m3_in_range(div(v[0]), div(v[1]), out.x, false);
+    out.x = cvt2_e4m3_in_range(div(v[2]), div(v[3]), out.x, true);
+    out.y = cvt2_e4m3_in_range(div(v[4]), div(v[5]), out.y, false);
+    out.y = cvt2_e4m3_in_range(div(v[6]), div(v[7]), out.y, true);
+  } else {
+    out.x = cvt2_e4m3(v[0] / scale, v[1] / scale, out.x, false);
+    out.x = cvt2_e4m3(v[2] / scale, v[3] / scale, out.x, true);
+    out.y = cvt2_e4m3(v[4] / scale, v[5] / scale, out.y, false);
+    out.y = cvt2_e4m3(v[6] / scale, v[7] / scale, out.y, true);
+  }
   *reinterpret_cast<u32x2*>(q + e0) = out;
 }
 
-template <typename T, int GROUP>
-void launch(const void* x, void* q, void* s, uint32_t m, uint32_t k, bool col, bool fuse, hipStream_t st) {
-  const size_t total = static_cast<size_t>(m) * k / 8;
-  const unsigned blocks = static_cast<unsigned>(div_up(total, 256));
+template <typename T, int GROUP, int BLOCK>
+void launch_block(const void* x, void* q, void* s, uint32_t m, uint32_t k, bool col, bool fuse, hipStream_t st) {
+  const unsigned gy = m < 32768u ? m : 32768u;
+  const dim3 grid(static_cast<unsigned>(div_up(k, BLOCK * 8)), gy, static_cast<unsigned>(div_up(m, gy)));
   const uint16_t* xp = static_cast<const uint16_t*>(x);
   uint8_t* qp = static_cast<uint8_t*>(q);
   float* sp = static_cast<float*>(s);
   if (col) {
-    if (fuse) fp8_group_quant_kernel<T, GROUP, true, true><<<blocks, 256, 0, st>>>(xp, qp, sp, m, k);
-    else fp8_group_quant_kernel<T, GROUP, true, false><<<blocks, 256, 0, st>>>(xp, qp, sp, m, k);
+    if (fuse) fp8_group_quant_kernel<T, GROUP, true, true, BLOCK><<<grid, BLOCK, 0, st>>>(xp, qp, sp, m, k);
+    else fp8_group_quant_kernel<T, GROUP, true, false, BLOCK><<<grid, BLOCK, 0, st>>>(xp, qp, sp, m, k);
   } else {
-    if (fuse) fp8_group_quant_kernel<T, GROUP, false, true><<<blocks, 256, 0, st>>>(xp, qp, sp, m, k);
-    else fp8_group_quant_kernel<T, GROUP, false, false><<<blocks, 256, 0, st>>>(xp, qp, sp, m, k);
+    if (fuse) fp8_group_quant_kernel<T, GROUP, false, true, BLOCK><<<grid, BLOCK, 0, st>>>(xp, qp, sp, m, k);
+    else fp8_group_quant_kernel<T, GROUP, false, false, BLOCK><<<grid, BLOCK, 0, st>>>(xp, qp, sp, m, k);
   }
+}
+
+template <typename T, int GROUP>
+void launch(const void* x, void* q, void* s, uint32_t m, uint32_t k, bool col, bool fuse, hipStream_t st) {
+  // workgroup width by row length: a short row would leave most of a wide workgroup idle
+  if (k <= 512) launch_block<T, GROUP, 64>(x, q, s, m, k, col, fuse, st);
+  else if (k <= 1024) launch_block<T, GROUP, 128>(x, q, s, m, k, col, fuse, st);
+  else launch_block<T, GROUP, 256>(x, q, s, m, k, col, fuse, st);
 }
 
 
@@ -135,6 +197,9 @@ __global__ void __launch_bounds__(256) fp8_channel_quant_kernel(const uint16_t* 
                                                                 const float* __restrict__ scale, size_t size, bool vec) {
   const size_t base = static_cast<size_t>(blockIdx.y) * size;
   const float sc = scale[blockIdx.y];
+  const ExactDiv div(sc);
+  // with a scale handed in by the caller an input may be infinite where the scale is not: that one keeps the division
+  auto quot = [&](float a) { return __builtin_fabsf(a) == __builtin_inff() ? a / sc : div(a); };
   const size_t tid = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
   const size_t stride = static_cast<size_t>(gridDim.x) * 256;
   if (vec) {
@@ -143,8 +208,8 @@ __global__ void __launch_bounds__(256) fp8_channel_quant_kernel(const uint16_t* 
       float v[8];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        v[2 * j] = T::to_float(static_cast<uint16_t>(raw[j] & 0xffffu)) / sc;
-        v[2 * j + 1] = T::to_float(static_cast<uint16_t>(raw[j] >> 16)) / sc;
+        v[2 * j] = quot(T::to_float(static_cast<uint16_t>(raw[j] & 0xffffu)));
+        v[2 * j + 1] = quot(T::to_float(static_cast<uint16_t>(raw[j] >> 16)));
       }
       u32x2 out{0u, 0u};
       out.x = cvt2_e4m3(v[0], v[1], out.x, false);
