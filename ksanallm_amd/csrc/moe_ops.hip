@@ -79,6 +79,71 @@ __global__ void __launch_bounds__(kAlignThreads) moe_align_kernel(const int32_t*
   }
 }
 
+// ---- the same sort for up to 1024 ids (decode batches), one id per thread, everything in LDS: no counter ever makes
+// a round trip through global memory, which is what the launch above spends most of its microseconds on.
+//   r        = lower lanes of the wavefront with the same id (64 readlanes)
+//   wcnt[w][e] = ids == e in wavefront w, then, scanned over w, ids == e in the wavefronts before w
+//   position = first[e] + wcnt[w][e] + r : ascending with the flat index inside an expert, as above
+__global__ void __launch_bounds__(1024) moe_align_small_kernel(const int32_t* __restrict__ ids, uint32_t numel, uint32_t E,
+                                                               uint32_t block_m, uint32_t capacity,
+                                                               int32_t* __restrict__ sorted, int32_t* __restrict__ expert_ids,
+                                                               int32_t* __restrict__ num_post_pad) {
+  extern __shared__ int32_t lds[];  // wcnt[W][E], then [2][E + 1] ping-pong scan buffers
+  const uint32_t tid = threadIdx.x, threads = blockDim.x;
+  const uint32_t lane = tid & 63, wave = tid >> 6;
+  const uint32_t W = (numel + 63) / 64;
+  const uint32_t EP = E + 1;
+  int32_t* wcnt = lds;
+  int32_t* scan_a = lds + W * E;
+  int32_t* scan_b = scan_a + EP;
+
+  for (uint32_t i = tid; i < capacity; i += threads) sorted[i] = static_cast<int32_t>(numel);  // every slot starts as padding
+  for (uint32_t i = tid; i < W * E; i += threads) wcnt[i] = 0;
+
+  const uint32_t id = tid < numel ? static_cast<uint32_t>(ids[tid]) : 0xffffffffu;
+  const bool valid = id < E;
+  uint32_t r = 0;
+  bool last = true;
+#pragma unroll
+  for (int l = 0; l < 64; ++l) {
+    const uint32_t v = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(id), l));
+    const bool same = v == id;
+    r += (same && static_cast<uint32_t>(l) < lane) ? 1u : 0u;
+    last = last && !(same && static_cast<uint32_t>(l) > lane);
+  }
+  __syncthreads();
+  if (valid && last) wcnt[wave * E + id] = static_cast<int32_t>(r + 1);
+  __syncthreads();
+
+  for (uint32_t e = tid; e < E; e += threads) {
+    int32_t run = 0;
+    for (uint32_t w = 0; w < W; ++w) {
+      const int32_t c = wcnt[w * E + e];
+      wcnt[w * E + e] = run;
+      run += c;
+    }
+    scan_a[e + 1] = (run + static_cast<int32_t>(block_m) - 1) / static_cast<int32_t>(block_m) * static_cast<int32_t>(block_m);
+  }
+  if (tid == 0) scan_a[0] = 0;
+  __syncthreads();
+
+  int32_t* src = scan_a;
+  int32_t* dst = scan_b;
+  for (uint32_t off = 1; off < EP; off <<= 1) {
+    for (uint32_t i = tid; i < EP; i += threads) dst[i] = src[i] + (i >= off ? src[i - off] : 0);
+    __syncthreads();
+    int32_t* t = src;
+    src = dst;
+    dst = t;
+  }
+  const int32_t* first = src;
+
+  if (tid == 0) num_post_pad[0] = first[E];
+  for (uint32_t e = tid; e < E; e += threads)
+    for (int32_t p = first[e]; p < first[e + 1]; p += static_cast<int32_t>(block_m)) expert_ids[p / static_cast<int32_t>(block_m)] = static_cast<int32_t>(e);
+  if (valid) sorted[first[id] + wcnt[wave * E + id] + static_cast<int32_t>(r)] = static_cast<int32_t>(tid);
+}
+
 // ---- the same sort for many ids: two launches over `chunks` workgroups ---------------------------------------------
 constexpr int kChunkThreads = 256;
 constexpr uint32_t kMaxChunks = 128;
@@ -230,12 +295,25 @@ __global__ void __launch_bounds__(256) moe_sum_kernel(const uint16_t* __restrict
   float acc[8];
 #pragma unroll
   for (int j = 0; j < 8; ++j) acc[j] = 0.f;
-  for (uint32_t s = 0; s < topk; ++s) {
-    u32x4 r = *reinterpret_cast<const u32x4*>(in + (t * topk + s) * d + c);
+  // four rows are fetched before the first of them is added: the sums form a chain (each is rounded to T), the loads
+  // need not wait for it
+  const uint16_t* src = in + t * topk * d + c;
+  for (uint32_t s0 = 0; s0 < topk; s0 += 4) {
+    u32x4 r[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      acc[2 * j] = T::to_float(T::from_float(acc[2 * j] + T::to_float(static_cast<uint16_t>(r[j] & 0xffffu))));
-      acc[2 * j + 1] = T::to_float(T::from_float(acc[2 * j + 1] + T::to_float(static_cast<uint16_t>(r[j] >> 16))));
+    for (int u = 0; u < 4; ++u) {
+      const uint32_t sr = s0 + u < topk ? s0 + u : topk - 1;  // rows past the end repeat the last one and are not added
+      r[u] = *reinterpret_cast<const u32x4*>(src + static_cast<size_t>(sr) * d);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (s0 + u < topk) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          acc[2 * j] = T::to_float(T::from_float(acc[2 * j] + T::to_float(static_cast<uint16_t>(r[u][j] & 0xffffu))));
+          acc[2 * j + 1] = T::to_float(T::from_float(acc[2 * j + 1] + T::to_float(static_cast<uint16_t>(r[u][j] >> 16))));
+        }
+      }
     }
   }
   u32x4 o;
@@ -502,6 +580,15 @@ KSQ_EXPORT int ksq_moe_align(const void* topk_ids, size_t numel, size_t E, size_
         static_cast<const int32_t*>(topk_ids), static_cast<uint32_t>(numel), static_cast<uint32_t>(E),
         static_cast<uint32_t>(block_m), static_cast<int32_t*>(sorted_ids), static_cast<int32_t*>(expert_ids),
         static_cast<int32_t*>(num_post_pad), static_cast<const int32_t*>(scratch), chunks, per);
+    return check_launch(fn);
+  }
+  if (numel <= 1024 && div_up(numel, 64) * E <= 12288) {  // one id per thread, counters in LDS (at most 48 KiB of them)
+    const size_t small_lds = (div_up(numel, 64) * E + 2 * (E + 1)) * sizeof(int32_t);
+    const unsigned threads = numel <= 256 ? 256u : 1024u;
+    moe_align_small_kernel<<<1, threads, small_lds, as_stream(stream)>>>(
+        static_cast<const int32_t*>(topk_ids), static_cast<uint32_t>(numel), static_cast<uint32_t>(E),
+        static_cast<uint32_t>(block_m), static_cast<uint32_t>(cap), static_cast<int32_t*>(sorted_ids),
+        static_cast<int32_t*>(expert_ids), static_cast<int32_t*>(num_post_pad));
     return check_launch(fn);
   }
   align_geometry(numel, &chunks, &per);

@@ -44,6 +44,21 @@ def test_align_out_of_range_ids_dropped(ops, oracle):
     np.testing.assert_array_equal(s.cpu().numpy(), so)
 
 
+@pytest.mark.parametrize("numel,E,bm", [(1, 256, 16), (8, 256, 16), (63, 5, 32), (64, 1, 16), (65, 192, 128), (256, 7, 16),
+                                        (257, 64, 256), (1000, 12, 32), (1024, 192, 16), (1024, 1000, 16)])
+def test_align_few_ids(ops, oracle, numel, E, bm):
+    # decode batches (one id per thread, counters in LDS): every wavefront count around 64, one expert taking all ids,
+    # ids outside [0, E), and a shape whose counters do not fit and falls back to the general kernel
+    g = H.gen(7 * numel + E)
+    ids = torch.randint(-2, E + 2, (numel,), generator=g, dtype=torch.int32)
+    s, e, npp = ops.moe_align_block_size(ids.cuda(), E, bm)
+    so, eo, nppo = oracle.moe_align(ids.numpy(), E, bm)
+    assert npp.item() == nppo
+    np.testing.assert_array_equal(s.cpu().numpy(), so)
+    nb = nppo // bm
+    np.testing.assert_array_equal(e.cpu().numpy()[:nb], eo[:nb])
+
+
 @pytest.mark.parametrize("numel,E,bm", [(2048, 7, 128), (2049, 4096, 16), (33333, 300, 32), (70001, 1, 128)])
 def test_align_many_ids_ragged(ops, oracle, numel, E, bm):
     # the sort over several workgroups: ragged chunk ends, ids outside [0, E), one expert, the largest expert count
