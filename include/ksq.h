@@ -204,8 +204,8 @@ int ksq_moe_w4a16_gemm(void* out, const void* x, const void* w_packed, const voi
  * with e the expert of s's block.  a_q [a_rows, k] e4m3, a_s fp32 [a_rows, k/128] (the reference's layout) or, when
  * a_s_column_major, [k/128, a_rows] - the two layouts ksq_fp8_group_quant writes; b [E, n, k] e4m3 packed by
  * ksq_fp8_repack_weight(E = experts), b_s fp32 [E, ceil(n/128), k/128] as in the checkpoint, out [numel, n] in out_dtype.  top_k = 1 reads a_q rows by slot (second MoE GEMM).
- * block_m is the block size the permutation was aligned with: 16 or 32 run the streaming (decode) kernel, 256 the MFMA
- * tile kernel; ksq_moe_fp8_block_m() gives the choice for a problem size.
+ * block_m is the block size the permutation was aligned with: 16 or 32 run the streaming (decode) kernel, 128 or 256
+ * the MFMA tile kernel; ksq_moe_fp8_block_m() gives the choice for a problem size.
  * Replaces the fp8_w8a8 block-quantized branch of InvokeFusedMoe's fused_moe_kernel launches
  * (S/kernels/nvidia/moe_kernel_wrapper.cpp:435-456, 498-522, 560-600). */
 size_t ksq_moe_fp8_block_m(size_t numel, size_t E);

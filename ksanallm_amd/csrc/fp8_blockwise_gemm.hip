@@ -222,16 +222,16 @@ int dispatch(const Fp8Params& p, hipStream_t s) {
 namespace ksq {
 namespace {
 
-template <typename TO>
+template <typename TO, int WM>
 int launch_fp8_tile(const Fp8Params& q, const TilePlan& plan, float* partial, hipStream_t s) {
   // two operand stages, two stages of activation scales, the weight scales of the k range
   constexpr int kLdsMax = 160 * 1024;
   const size_t kb_max = (plan.main_items || plan.splits == 1) ? q.K / 128 : plan.kt_per_split;  // whole tiles span all of K
-  const size_t lds = 2 * 32 * 2048 + 2 * 1024 + 2 * kb_max * 4;
+  const size_t lds = fp8_tile_lds_bytes(WM, kb_max);
   if (lds > kLdsMax) return fail(KSQ_ERR_UNSUPPORTED, "k range of %zu blocks per workgroup does not fit the LDS", kb_max);
   static std::atomic<bool> configured{false};
   if (!configured.load(std::memory_order_acquire)) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&fp8_tile_kernel<TO>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&fp8_tile_kernel<TO, false, WM>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, kLdsMax);
     if (e != hipSuccess) return fail(KSQ_ERR_LAUNCH, "hipFuncSetAttribute(LDS %d): %s", kLdsMax, hipGetErrorString(e));
     configured.store(true, std::memory_order_release);
@@ -253,24 +253,24 @@ int launch_fp8_tile(const Fp8Params& q, const TilePlan& plan, float* partial, hi
   p.kb_per_split = plan.kt_per_split;
   p.as_row_bytes = 4;
   p.as_kb_bytes = 4 * q.M;
-  fp8_tile_kernel<TO><<<plan.grid, 512, lds, s>>>(p);
+  fp8_tile_kernel<TO, false, WM><<<plan.grid, 512, lds, s>>>(p);
   if (plan.splits > 1) {
     const unsigned cut = plan.tiles_m * plan.tiles_n - plan.main_items;
-    splitk_reduce_kernel<TO, 256><<<cut * 32, 256, 0, s>>>(partial, static_cast<uint16_t*>(p.out), p.M, p.N, p.tiles_m, p.tiles_n,
-                                                          p.main_items, p.splits);
+    splitk_reduce_kernel<TO, 32 * WM><<<cut * (4 * WM), 256, 0, s>>>(partial, static_cast<uint16_t*>(p.out), p.M, p.N, p.tiles_m,
+                                                                    p.tiles_n, p.main_items, p.splits);
   }
   return KSQ_OK;
 }
 
 // grouped (MoE) form of the tile kernel: one 256-slot block of the aligned permutation per row tile
-template <typename TO>
+template <typename TO, int WM>
 int launch_fp8_tile_grouped(const Fp8Params& q, unsigned blocks, hipStream_t s) {
   constexpr int kLdsMax = 160 * 1024;
-  const size_t lds = 2 * 32 * 2048 + 2 * 1024 + 2 * static_cast<size_t>(q.K / 128) * 4;
+  const size_t lds = fp8_tile_lds_bytes(WM, q.K / 128);
   if (lds > kLdsMax) return fail(KSQ_ERR_UNSUPPORTED, "k range of %u blocks per workgroup does not fit the LDS", q.K / 128);
   static std::atomic<bool> configured{false};
   if (!configured.load(std::memory_order_acquire)) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&fp8_tile_kernel<TO, true>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&fp8_tile_kernel<TO, true, WM>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, kLdsMax);
     if (e != hipSuccess) return fail(KSQ_ERR_LAUNCH, "hipFuncSetAttribute(LDS %d): %s", kLdsMax, hipGetErrorString(e));
     configured.store(true, std::memory_order_release);
@@ -298,7 +298,7 @@ int launch_fp8_tile_grouped(const Fp8Params& q, unsigned blocks, hipStream_t s) 
   p.numel = q.numel;
   p.top_k = q.top_k;
   p.scale_rows = q.scale_rows;
-  fp8_tile_kernel<TO, true><<<p.tiles_m * p.tiles_n, 512, lds, s>>>(p);
+  fp8_tile_kernel<TO, true, WM><<<p.tiles_m * p.tiles_n, 512, lds, s>>>(p);
   return KSQ_OK;
 }
 
@@ -322,8 +322,8 @@ KSQ_EXPORT size_t ksq_fp8_blockwise_workspace_size(size_t max_m, size_t n, size_
   // only the split-K form of the tile kernel needs scratch: fp32 partial tiles
   if (n == 0 || k == 0 || k % 128 != 0) return 0;
   size_t need = 0;
-  // the plan is the same for all m of a band of 256 rows
-  for (size_t band_end = 256; max_m > 32; band_end += 256) {
+  // the plan is the same for all m of a band of 128 rows
+  for (size_t band_end = 128; max_m > 32; band_end += 128) {
     const size_t m = band_end < max_m ? band_end : max_m;
     const TilePlan t = plan_fp8_tile(m, n, k);
     need = t.workspace_bytes > need ? t.workspace_bytes : need;
@@ -361,8 +361,12 @@ KSQ_EXPORT int ksq_fp8_blockwise_gemm(const void* a_q, const void* a_s, const vo
                   n, k, plan.workspace_bytes, workspace ? workspace_bytes : size_t(0));
     if (256 * k > 0xffffffffull) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: k too large", fn);
     float* partial = plan.splits > 1 ? static_cast<float*>(workspace) : nullptr;
-    rc = out_dtype == KSQ_F16 ? launch_fp8_tile<F16>(p, plan, partial, as_stream(stream))
-                              : launch_fp8_tile<BF16>(p, plan, partial, as_stream(stream));
+    if (plan.block_m == 128)
+      rc = out_dtype == KSQ_F16 ? launch_fp8_tile<F16, 4>(p, plan, partial, as_stream(stream))
+                                : launch_fp8_tile<BF16, 4>(p, plan, partial, as_stream(stream));
+    else
+      rc = out_dtype == KSQ_F16 ? launch_fp8_tile<F16, 8>(p, plan, partial, as_stream(stream))
+                                : launch_fp8_tile<BF16, 8>(p, plan, partial, as_stream(stream));
   } else {
     rc = out_dtype == KSQ_F16 ? dispatch<F16>(p, as_stream(stream)) : dispatch<BF16>(p, as_stream(stream));
   }
@@ -385,8 +389,8 @@ KSQ_EXPORT int ksq_moe_fp8_blockwise_gemm(void* out, const void* a_q, const void
   if (out_dtype != KSQ_F16 && out_dtype != KSQ_BF16)
     return fail(KSQ_ERR_UNSUPPORTED, "%s: output dtype must be f16 or bf16", fn);
   if (top_k == 0 || E == 0) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: top_k and E must be positive", fn);
-  if (block_m != 16 && block_m != 32 && block_m != 256)
-    return fail(KSQ_ERR_UNSUPPORTED, "%s: block_m %zu not in {16,32,256}", fn, block_m);
+  if (block_m != 16 && block_m != 32 && block_m != 128 && block_m != 256)
+    return fail(KSQ_ERR_UNSUPPORTED, "%s: block_m %zu not in {16,32,128,256}", fn, block_m);
   if (numel == 0) return KSQ_OK;
   if (a_rows < (numel + top_k - 1) / top_k)
     return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: %zu activation rows cannot serve %zu slots of top_k %zu", fn, a_rows, numel, top_k);
@@ -409,11 +413,15 @@ KSQ_EXPORT int ksq_moe_fp8_blockwise_gemm(void* out, const void* a_q, const void
   const int mt = block_m == 16 ? 1 : 2;
   const unsigned blocks = static_cast<unsigned>(cap_blocks);
   int rc;
-  if (block_m == 256) {  // prefill regime: MFMA tile kernel, rows gathered / scattered through the permutation
+  if (block_m >= 128) {  // prefill regime: MFMA tile kernel, rows gathered / scattered through the permutation
     if (a_rows * k > 0xffffffffull || a_rows * (k / 128) * 4 > 0xffffffffull)
       return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: activations too large", fn);
-    rc = out_dtype == KSQ_F16 ? launch_fp8_tile_grouped<F16>(p, blocks, as_stream(stream))
-                              : launch_fp8_tile_grouped<BF16>(p, blocks, as_stream(stream));
+    if (block_m == 128)
+      rc = out_dtype == KSQ_F16 ? launch_fp8_tile_grouped<F16, 4>(p, blocks, as_stream(stream))
+                                : launch_fp8_tile_grouped<BF16, 4>(p, blocks, as_stream(stream));
+    else
+      rc = out_dtype == KSQ_F16 ? launch_fp8_tile_grouped<F16, 8>(p, blocks, as_stream(stream))
+                                : launch_fp8_tile_grouped<BF16, 8>(p, blocks, as_stream(stream));
   } else {
     rc = out_dtype == KSQ_F16 ? dispatch_grouped<F16>(p, mt, blocks, as_stream(stream))
                               : dispatch_grouped<BF16>(p, mt, blocks, as_stream(stream));

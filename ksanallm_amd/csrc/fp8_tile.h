@@ -49,16 +49,30 @@ __device__ __forceinline__ f32x4 mfma_fp8_k128(i32x8 a, i32x8 b, f32x4 c) {
 // row s / top_k (pad slots carry s >= numel) and that row's scales, weights and weight scales are those of expert
 // expert_ids[tile_m], results go to out[s, :] (times topk_w[s] when given).  Blocks past num_post_pad leave at once;
 // there is no cut along K in this form.
-template <typename TO, bool GROUPED = false>
-__global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
-  constexpr int WAVES_N = 4;
-  constexpr int WM = 8, WN = 4;  // 16x16 tiles per wavefront: 128 tokens x 64 weight rows
-  constexpr int BM = 256, BN = 256;
-  constexpr int FRAG = 2048;                  // bytes of one 16 x 128 operand fragment
-  constexpr int STAGE_BYTES = 32 * FRAG;      // 16 activation + 16 weight fragments
-  constexpr int W_FRAG0 = 16;                 // first weight fragment of a stage
+// WM = 8: 256-token tiles.  WM = 4: 128-token tiles (each wavefront 64 tokens x 64 weight rows) for row counts that
+// would leave half of a 256-token tile to padding; a stage then holds 8 activation fragments.
+constexpr int fp8_tile_stage_bytes(int wm) { return (2 * wm + 16) * 2048; }
+// LDS stages: the 48 KiB stages of the 128-token tile fit three times, and need it - a stage of that tile is over in
+// less time than a load takes to come back
+constexpr int fp8_tile_stages(int wm) { return wm == 4 ? 3 : 2; }
+constexpr size_t fp8_tile_lds_bytes(int wm, size_t kb_max) {
+  return static_cast<size_t>(fp8_tile_stages(wm)) * (fp8_tile_stage_bytes(wm) + 1024) + 2 * kb_max * 4;
+}
 
-  extern __shared__ __attribute__((aligned(16))) char lds[];  // 2 * STAGE_BYTES
+template <typename TO, bool GROUPED = false, int WM = 8>
+__global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
+  static_assert(WM == 8 || WM == 4, "256- or 128-token tiles");
+  constexpr int WAVES_N = 4;
+  constexpr int WN = 4;  // 16x16 tiles per wavefront: 16*WM tokens x 64 weight rows
+  constexpr int BM = 2 * WM * 16, BN = 256;
+  constexpr int FRAG = 2048;                  // bytes of one 16 x 128 operand fragment
+  constexpr int AF = BM / 16;                 // activation fragments of a stage
+  constexpr int AFW = AF / 4;                 // ... fetched by each of the wavefronts 0..3
+  constexpr int STAGE_BYTES = fp8_tile_stage_bytes(WM);  // AF activation + 16 weight fragments
+  constexpr int W_FRAG0 = AF;                 // first weight fragment of a stage
+  constexpr int NS = fp8_tile_stages(WM);     // LDS stages
+
+  extern __shared__ __attribute__((aligned(16))) char lds[];  // fp8_tile_lds_bytes
 
   const int lane = threadIdx.x & 63;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -88,7 +102,7 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
     expert = static_cast<size_t>(__builtin_amdgcn_readfirstlane(p.expert_ids[tile_m]));
   }
   const bool stage_act = wave < 4;
-  const uint32_t frag0 = (wave & 3) * 4;
+  const uint32_t frag0 = (wave & 3) * (stage_act ? AFW : 4);
   // Weights come as packed 2 KiB fragments (ksq_fp8_repack_weight), fragment (strip, k-block) at (strip*KB + kb)*2048:
   // a half of a fragment is one contiguous KiB, fetched by one load with lane j taking bytes 16j, and lands in LDS as
   // it lies in memory - MFMA lane l then reads 16 bytes at 16l of each half, consecutive lanes consecutive addresses,
@@ -102,7 +116,9 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
   uint32_t d_voff[4], d_voff_hi[4];     // per fragment: first load, and second load minus its instruction offset of 64
 #pragma unroll
   for (int f = 0; f < 4; ++f) {
-    if (stage_act) {
+    if (stage_act && f >= AFW) {
+      d_voff[f] = d_voff_hi[f] = 0;  // not fetched
+    } else if (stage_act) {
       uint32_t row = (frag0 + f) * 16 + (lane >> 2);
       if (GROUPED) {
         uint32_t sid = static_cast<uint32_t>(p.sorted_ids[m0 + row]);
@@ -127,13 +143,14 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
   // copy 64 of them each into LDS with one 4-byte-per-lane LDS-targeted load per stage.  The weight scales of the
   // workgroup's two 128-row scale blocks, for its whole k range, are copied into LDS once.  A lane needs one activation
   // scale per row tile (token = column l%16 of the MFMA result) and one weight scale per k-block.
-  constexpr int SCALE_BASE = 2 * STAGE_BYTES;    // [2 slots][256] activation scales, then [2][kb_count] weight scales
-  constexpr int BS_BASE = SCALE_BASE + 2 * 1024;
+  constexpr int SCALE_BASE = NS * STAGE_BYTES;    // [NS slots][256] activation scales, then [2][kb_count] weight scales
+  constexpr int BS_BASE = SCALE_BASE + NS * 1024;
   // M % 4 == 0: wavefront 0 copies all 256 with one 16-byte-per-lane load (lanes whose four tokens lie past M repeat
   // the last four).  Otherwise wavefronts 0..3 copy 64 each, 4 bytes per lane, every lane clamped on its own.
   // (the one-load form needs the 256 scales of a k-block contiguous: dense form with token-contiguous scales)
   const bool s_vec = !GROUPED && (p.M & 3) == 0 && p.as_row_bytes == 4;
   uint32_t s_row = s_vec ? m0 + 4 * lane : m0 + (wave & 3) * 64 + lane;
+  if (!s_vec && (wave & 3) * 64 >= BM) s_row = m0;  // this wavefront copies no scales (128-token tiles)
   if (GROUPED) {
     uint32_t sid = static_cast<uint32_t>(p.sorted_ids[s_row]);
     sid = sid < p.numel ? sid : p.numel - 1;
@@ -156,7 +173,7 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
     }
   }
   const float* bs_lds = reinterpret_cast<const float*>(lds + BS_BASE) + (wn >> 1) * kb_count;
-  const float* as_lds = reinterpret_cast<const float*>(lds + SCALE_BASE) + wm * 128 + lrow;
+  const float* as_lds = reinterpret_cast<const float*>(lds + SCALE_BASE) + wm * (WM * 16) + lrow;
 
   // Every group of loads is one assembly statement opening with `s_nop 4`: its scalar operands are in place before
   // it starts, and the wait states a vector memory instruction needs after a VALU write of a scalar register have
@@ -164,12 +181,12 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
   auto load_scales = [&](uint32_t kb) {
     const uint32_t k = kb < kb_count ? kb : kb_count - 1;
     const char* ap = as_base + static_cast<size_t>(k) * p.as_kb_bytes;
-    const uint32_t d = __builtin_amdgcn_readfirstlane(s_lds + (kb & 1) * 1024);
+    const uint32_t d = __builtin_amdgcn_readfirstlane(s_lds + (kb % NS) * 1024);
     if (s_vec) {
       if (wave == 0)
         asm volatile("s_nop 4\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %2" ::"v"(s_voff), "s"(d), "s"(ap)
                      : "memory");
-    } else if (wave < 4) {
+    } else if (wave < BM / 64) {
       asm volatile("s_nop 4\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, %2" ::"v"(s_voff), "s"(d), "s"(ap)
                    : "memory");
     }
@@ -179,9 +196,22 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
   auto load_operands = [&](uint32_t kb) {
     const uint32_t k = kb < kb_count ? kb : kb_count - 1;
     const uint8_t* src = g_tile + static_cast<size_t>(k) * k_step;
-    const uint32_t f0 = __builtin_amdgcn_readfirstlane(d_lds + (kb & 1) * STAGE_BYTES);
+    const uint32_t f0 = __builtin_amdgcn_readfirstlane(d_lds + (kb % NS) * STAGE_BYTES);
     const uint32_t f0h = f0 + 1024 - 64;
     const uint32_t f1 = f0 + FRAG, f1h = f0h + FRAG;
+    if (AFW == 2 && stage_act) {  // two activation fragments per wavefront (128-token tiles)
+      asm volatile(
+          "s_nop 4\n\t"
+          "s_mov_b32 m0, %4\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %8\n\t"
+          "s_mov_b32 m0, %5\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %8 offset:64\n\t"
+          "s_mov_b32 m0, %6\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %8\n\t"
+          "s_mov_b32 m0, %7\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %3, %8 offset:64"
+          :
+          : "v"(d_voff[0]), "v"(d_voff[1]), "v"(d_voff_hi[0]), "v"(d_voff_hi[1]), "s"(f0), "s"(f0h), "s"(f1), "s"(f1h),
+            "s"(src)
+          : "memory");
+      return;
+    }
     const uint32_t f2 = f1 + FRAG, f2h = f1h + FRAG;
     const uint32_t f3 = f2 + FRAG, f3h = f2h + FRAG;
     asm volatile(
@@ -200,8 +230,21 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
           "s"(f3h), "s"(src)
         : "memory");
   };
-  // everything this wavefront issued so far has landed
-  auto wait_all = [&]() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
+  // Everything this wavefront issued has landed, except the loads of the youngest stage when three stages are in use
+  // (vmcnt retires in issue order; a wavefront issues the same loads every stage: 8 weight loads, or 2*AFW activation
+  // loads with or without the one scale load in front of them).
+  const bool has_scale_load = s_vec ? wave == 0 : wave < BM / 64;
+  auto wait_stage = [&]() {
+    if (NS == 2) {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    } else if (!stage_act) {
+      asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    } else if (has_scale_load) {
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * AFW + 1) : "memory");
+    } else {
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * AFW) : "memory");
+    }
+  };
 
   f32x4 acc[WN][WM];
 #pragma unroll
@@ -266,17 +309,21 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
     }
   };
 
-  // ---- schedule: stage c computes k-block c out of LDS slot c%2 and, a quarter of the way in, issues the loads of
-  // k-block c+1 into the other slot (every wavefront left it at the previous barrier).  At the end of the stage they
-  // have to have landed (vmcnt(0)); the barrier makes them visible to all wavefronts.
+  // ---- schedule: stage c computes k-block c out of LDS slot c % NS and, right behind its first MFMA, issues the loads
+  // of k-block c+NS-1 into the slot stage c-1 used (every wavefront left it at the previous barrier).  At the end of
+  // the stage the loads of k-block c+1 have to have landed; the barrier makes them visible to all wavefronts.
   load_scales(0);
   load_operands(0);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  if (NS == 3) {
+    load_scales(1);
+    load_operands(1);
+  }
+  wait_stage();
   __syncthreads();  // also publishes the weight-scale table written with ordinary stores above
 
   for (uint32_t c = 0; c < kb_count; ++c) {
-    compute(c & 1, c, c + 1);
-    wait_all();  // operands and scales of c+1
+    compute(c % NS, c, c + NS - 1);
+    wait_stage();  // operands and scales of c+1
     __builtin_amdgcn_s_barrier();
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // drain the clamped prefetches before the LDS is released
@@ -284,7 +331,7 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
   // ---- store: lane holds token m = l%16 of the tile and weight rows (output columns) 4*(l/16) .. +3
 #pragma unroll
   for (int i = 0; i < WM; ++i) {
-    uint32_t row = m0 + wm * 128 + i * 16 + lrow;
+    uint32_t row = m0 + wm * (WM * 16) + i * 16 + lrow;
     bool live = row < p.M;
     float rw = 1.0f;
     if (GROUPED) {

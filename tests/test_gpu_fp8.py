@@ -133,13 +133,15 @@ def test_blockwise_gemm(ops, oracle, m, n, k):
     H.check_gemm(out, ref, H.BF16, "fp8 m=%d n=%d k=%d" % (m, n, k))
 
 
-# prefill regime (256 x 256 MFMA tile kernel): ragged M and N, odd k-block counts, split-K through the workspace
-@pytest.mark.parametrize("m,n,k", [(65, 256, 128), (300, 2320, 1152), (256, 7168, 2048), (1024, 512, 4096),
-                                   (130, 4096, 7168)])
-def test_blockwise_gemm_tile_kernel(ops, oracle, m, n, k):
+# prefill regime (MFMA tile kernel, 256 x 256 or 128 x 256 tiles): ragged M and N, odd k-block counts, split-K through
+# the workspace
+@pytest.mark.parametrize("m,n,k,bm", [(65, 256, 128, 128), (300, 2320, 1152, 128), (256, 7168, 2048, 256), (1024, 512, 4096, 256),
+                                      (130, 4096, 7168, 256), (128, 7168, 2048, 128), (384, 528, 1024, 128), (100, 272, 384, 128),
+                                      (500, 768, 640, 256)])
+def test_blockwise_gemm_tile_kernel(ops, oracle, m, n, k, bm):
     from ksanallm_amd import lib as L
     desc = L.select_tile(L.KIND_FP8_BLOCKWISE, m, n, k, H.BF16)
-    assert desc["kernel"] == 1
+    assert desc["kernel"] == 1 and desc["block_m"] == bm
     x, bq, bs = make_fp8_problem(oracle, 4400 + m + n, m, n, k)
     q, s = ops.per_token_group_quant_fp8(x.cuda(), k, 128, True)
     out = ops.fp8_blockwise_gemm(q, s, packed(ops, bq), torch.from_numpy(bs).cuda(), torch.bfloat16)

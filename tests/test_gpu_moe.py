@@ -276,7 +276,10 @@ def _fp8_experts(oracle, seed, E, n, k):
     (1, 8, 2, 256, 256, 16, False, False), (70, 8, 2, 208, 384, 16, True, True), (300, 6, 3, 512, 1024, 32, False, True),
     (33, 16, 4, 4096, 7168, 32, False, False),
     # 256-slot blocks: the MFMA tile kernel in its grouped form (ragged n, both scale layouts, routing weight)
-    (300, 6, 3, 512, 1024, 256, False, True), (700, 4, 2, 784, 512, 256, True, False), (130, 2, 1, 256, 128, 256, False, True)])
+    (300, 6, 3, 512, 1024, 256, False, True), (700, 4, 2, 784, 512, 256, True, False), (130, 2, 1, 256, 128, 256, False, True),
+    # 128-slot blocks of the same kernel
+    (300, 6, 3, 512, 1024, 128, False, True), (700, 4, 2, 784, 512, 128, True, False), (130, 2, 1, 256, 128, 128, False, True),
+    (90, 3, 2, 2064, 640, 128, True, True)])
 def test_grouped_fp8_gemm_stage(ops, oracle, T, E, topk, n, k, bm, colmajor, with_w):
     """One grouped blockwise-fp8 GEMM launch against the per-expert oracle GEMM on the codes the GPU quantizer wrote."""
     g = H.gen(7000 + T + n)
