@@ -39,10 +39,11 @@ MEASURED_TRAFFIC = {
     (2, "w4a16_tile_kernel<128x256,w8>"): 84610000,
     (2, "w4a16_tile_kernel<256x256,w8>"): 216470000,
     (3, "w4a16_tile_kernel<256x256,w8>"): 1591160000,
-    (4, "fp8_group_quant"): 27630000,
-    (4, "fp8_splitk_kernel<16x16,w4>"): 133550000,
-    (4, "fp8_splitk_kernel<16x32,w4>"): 134270000,
-    (4, "fp8_tile_kernel<256x256,w8>"): 258430000,
+    (4, "fp8_group_quant"): 26940000,
+    (4, "fp8_splitk_kernel<16x16,w4>"): 133530000,
+    (4, "fp8_splitk_kernel<16x32,w4>"): 134280000,
+    (4, "fp8_tile_kernel<128x256,w8>"): 176820000,
+    (4, "fp8_tile_kernel<256x256,w8>"): 519390000,
 }
 
 

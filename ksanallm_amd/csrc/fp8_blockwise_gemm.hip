@@ -229,13 +229,9 @@ int launch_fp8_tile(const Fp8Params& q, const TilePlan& plan, float* partial, hi
   const size_t kb_max = (plan.main_items || plan.splits == 1) ? q.K / 128 : plan.kt_per_split;  // whole tiles span all of K
   const size_t lds = fp8_tile_lds_bytes(WM, kb_max);
   if (lds > kLdsMax) return fail(KSQ_ERR_UNSUPPORTED, "k range of %zu blocks per workgroup does not fit the LDS", kb_max);
-  static std::atomic<bool> configured{false};
-  if (!configured.load(std::memory_order_acquire)) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&fp8_tile_kernel<TO, false, WM>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLdsMax);
-    if (e != hipSuccess) return fail(KSQ_ERR_LAUNCH, "hipFuncSetAttribute(LDS %d): %s", kLdsMax, hipGetErrorString(e));
-    configured.store(true, std::memory_order_release);
-  }
+  // more dynamic LDS than a kernel may use without asking: once per device
+  static std::atomic<uint64_t> configured{0};
+  if (int rc = allow_dynamic_lds(configured, reinterpret_cast<const void*>(&fp8_tile_kernel<TO, false, WM>), kLdsMax)) return rc;
   Fp8TileParams p{};
   p.a = q.a;
   p.a_s = q.a_s;
@@ -268,13 +264,9 @@ int launch_fp8_tile_grouped(const Fp8Params& q, unsigned blocks, hipStream_t s) 
   constexpr int kLdsMax = 160 * 1024;
   const size_t lds = fp8_tile_lds_bytes(WM, q.K / 128);
   if (lds > kLdsMax) return fail(KSQ_ERR_UNSUPPORTED, "k range of %u blocks per workgroup does not fit the LDS", q.K / 128);
-  static std::atomic<bool> configured{false};
-  if (!configured.load(std::memory_order_acquire)) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&fp8_tile_kernel<TO, true, WM>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLdsMax);
-    if (e != hipSuccess) return fail(KSQ_ERR_LAUNCH, "hipFuncSetAttribute(LDS %d): %s", kLdsMax, hipGetErrorString(e));
-    configured.store(true, std::memory_order_release);
-  }
+  // more dynamic LDS than a kernel may use without asking: once per device
+  static std::atomic<uint64_t> configured{0};
+  if (int rc = allow_dynamic_lds(configured, reinterpret_cast<const void*>(&fp8_tile_kernel<TO, true, WM>), kLdsMax)) return rc;
   Fp8TileParams p{};
   p.a = q.a;
   p.a_s = q.a_s;

@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 
@@ -98,5 +99,20 @@ __device__ __forceinline__ uint32_t pack2(uint16_t lo, uint16_t hi) {
 }
 
 inline size_t div_up(size_t a, size_t b) { return (a + b - 1) / b; }
+
+// A kernel that asks for more dynamic LDS than the default limit needs hipFuncSetAttribute once per device (the
+// attribute belongs to the function as loaded on that device; a process that drives several GPUs from several threads
+// calls in here from each).  `done` holds one bit per device ordinal, set after the attribute has been accepted.
+// Returns 0, or the KSQ_ERR_LAUNCH code after recording the message.
+inline int allow_dynamic_lds(std::atomic<uint64_t>& done, const void* kernel, int bytes) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev > 63) return fail(KSQ_ERR_LAUNCH, "cannot tell the current device");
+  const uint64_t bit = uint64_t(1) << dev;
+  if (done.load(std::memory_order_acquire) & bit) return 0;
+  const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e != hipSuccess) return fail(KSQ_ERR_LAUNCH, "hipFuncSetAttribute(LDS %d): %s", bytes, hipGetErrorString(e));
+  done.fetch_or(bit, std::memory_order_release);
+  return 0;
+}
 
 }  // namespace ksq

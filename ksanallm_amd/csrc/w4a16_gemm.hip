@@ -81,14 +81,9 @@ int dispatch_tile(SplitKParams& p, SplitKChoice c, uint32_t m_blocks, size_t gro
 template <typename T, int WM, bool HAS_ZP>
 int launch_tile_zp(const TileParams& p, unsigned grid, hipStream_t s) {
   constexpr int kLds = 4 * WM * 2 * 1024;  // NS stages of WM*2 fragments
-  static std::atomic<bool> configured{false};
-  if (!configured.load(std::memory_order_acquire)) {
-    // more dynamic LDS than the 64 KiB a kernel may use without asking
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&w4a16_tile_kernel<T, WM, HAS_ZP>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
-    if (e != hipSuccess) return fail(KSQ_ERR_LAUNCH, "hipFuncSetAttribute(LDS %d): %s", kLds, hipGetErrorString(e));
-    configured.store(true, std::memory_order_release);
-  }
+  // more dynamic LDS than a kernel may use without asking: once per device
+  static std::atomic<uint64_t> configured{0};
+  if (int rc = allow_dynamic_lds(configured, reinterpret_cast<const void*>(&w4a16_tile_kernel<T, WM, HAS_ZP>), kLds)) return rc;
   w4a16_tile_kernel<T, WM, HAS_ZP><<<grid, 512, kLds, s>>>(p);
   return KSQ_OK;
 }
@@ -97,13 +92,9 @@ int launch_tile_zp(const TileParams& p, unsigned grid, hipStream_t s) {
 template <typename T>
 int launch_tile_grouped(const TileParams& p, hipStream_t s) {
   constexpr int kLds = 4 * 8 * 2 * 1024;
-  static std::atomic<bool> configured{false};
-  if (!configured.load(std::memory_order_acquire)) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&w4a16_tile_kernel<T, 8, false, true>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
-    if (e != hipSuccess) return fail(KSQ_ERR_LAUNCH, "hipFuncSetAttribute(LDS %d): %s", kLds, hipGetErrorString(e));
-    configured.store(true, std::memory_order_release);
-  }
+  // more dynamic LDS than a kernel may use without asking: once per device
+  static std::atomic<uint64_t> configured{0};
+  if (int rc = allow_dynamic_lds(configured, reinterpret_cast<const void*>(&w4a16_tile_kernel<T, 8, false, true>), kLds)) return rc;
   w4a16_tile_kernel<T, 8, false, true><<<p.tiles_m * p.tiles_n, 512, kLds, s>>>(p);
   return KSQ_OK;
 }
