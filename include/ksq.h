@@ -199,6 +199,18 @@ int ksq_moe_w4a16_gemm(void* out, const void* x, const void* w_packed, const voi
                        const void* num_post_pad, size_t numel, size_t top_k, size_t E, size_t n, size_t k,
                        size_t group, size_t block_m, int dtype, void* stream);
 
+/* The first MoE GEMM with the activation in its epilogue: w_packed holds [gate | up] rows (n = 2 * inter), and for every
+ * valid sorted slot id s   out[s, c] = T(silu(T(g)) * T(u)),  g = x[s / top_k, :] . W[e, c, :],  u = x[s / top_k, :] . W[e, inter + c, :],
+ * out [numel, inter] T: bit for bit what ksq_moe_w4a16_gemm into a [numel, 2 * inter] buffer followed by ksq_silu_mul
+ * gives, in one launch and without that buffer.  block_m 16 or 32 (the decode regime, where a launch is a sizeable part
+ * of the layer's time); 128 returns KSQ_ERR_UNSUPPORTED: run the two calls.
+ * Replaces the pair InvokeMoeWna16Gemm + InvokeSiluAndMul of InvokeFusedMoe
+ * (S/kernels/nvidia/moe_kernel_wrapper.cpp:616-640). */
+int ksq_moe_w4a16_gate_up_silu(void* out, const void* x, const void* w_packed, const void* scales_packed,
+                               const void* zeros_packed, const void* sorted_ids, const void* expert_ids,
+                               const void* num_post_pad, size_t numel, size_t top_k, size_t E, size_t n, size_t k,
+                               size_t group, size_t block_m, int dtype, void* stream);
+
 /* Grouped blockwise-FP8 GEMM over the aligned blocks: for every valid sorted slot id s (< numel)
  *   out[s, :] = sum_kb (a_q[s / top_k, kb] . b[e, :, kb]) * a_s[kb, s / top_k] * b_s[e, :/128, kb] * (topk_w ? topk_w[s] : 1)
  * with e the expert of s's block.  a_q [a_rows, k] e4m3, a_s fp32 [a_rows, k/128] (the reference's layout) or, when

@@ -240,13 +240,17 @@ KSQ_EXPORT int ksq_w4a16_gemm(void* y, const void* x, const void* w_packed, cons
   return check_launch(fn);
 }
 
-KSQ_EXPORT int ksq_moe_w4a16_gemm(void* out, const void* x, const void* w_packed, const void* scales_packed,
-                                  const void* zeros_packed, const void* topk_w, const void* sorted_ids,
-                                  const void* expert_ids, const void* num_post_pad, size_t numel, size_t top_k,
-                                  size_t E, size_t n, size_t k, size_t group, size_t block_m, int dtype,
-                                  void* stream) {
-  const char* fn = "ksq_moe_w4a16_gemm";
+namespace {
+int moe_w4a16_gemm_impl(const char* fn, bool fuse_silu, void* out, const void* x, const void* w_packed,
+                        const void* scales_packed, const void* zeros_packed, const void* topk_w, const void* sorted_ids,
+                        const void* expert_ids, const void* num_post_pad, size_t numel, size_t top_k, size_t E, size_t n,
+                        size_t k, size_t group, size_t block_m, int dtype, void* stream) {
   if (int rc = check_common(fn, out, x, w_packed, scales_packed, n, k, group, dtype)) return rc;
+  if (fuse_silu) {
+    if (n % 32 != 0) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: n = 2 * inter must be a multiple of 32", fn);
+    if (block_m == 128)
+      return fail(KSQ_ERR_UNSUPPORTED, "%s: 128-row blocks run the plain GEMM and ksq_silu_mul", fn);
+  }
   if (!sorted_ids || !expert_ids || !num_post_pad) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: null index buffer", fn);
   if (zeros_packed) return fail(KSQ_ERR_UNSUPPORTED, "%s: zero points are not supported for expert weights", fn);
   if (group != 128) return fail(KSQ_ERR_UNSUPPORTED, "%s: expert weights need group size 128", fn);
@@ -303,8 +307,30 @@ KSQ_EXPORT int ksq_moe_w4a16_gemm(void* out, const void* x, const void* w_packed
   // about numel/block_m + E/2 of the aligned blocks hold rows; K is never split across workgroups here
   SplitKChoice c = select_splitk_blocks(static_cast<int>(block_m / 16),
                                         std::min(cap_blocks, numel / block_m + E / 2 + 1), n, k);
+  if (fuse_silu) {
+    if (c.nt < 2) c.nt = 2;  // a workgroup holds gate and up tiles in pairs
+    p.pair_tiles = static_cast<uint32_t>(n / 32);
+  }
   int rc = dtype == KSQ_F16 ? dispatch_tile<F16, true>(p, c, static_cast<uint32_t>(cap_blocks), group, as_stream(stream))
                             : dispatch_tile<BF16, true>(p, c, static_cast<uint32_t>(cap_blocks), group, as_stream(stream));
   if (rc) return rc;
   return check_launch(fn);
+}
+}  // namespace
+
+KSQ_EXPORT int ksq_moe_w4a16_gemm(void* out, const void* x, const void* w_packed, const void* scales_packed,
+                                  const void* zeros_packed, const void* topk_w, const void* sorted_ids,
+                                  const void* expert_ids, const void* num_post_pad, size_t numel, size_t top_k,
+                                  size_t E, size_t n, size_t k, size_t group, size_t block_m, int dtype,
+                                  void* stream) {
+  return moe_w4a16_gemm_impl("ksq_moe_w4a16_gemm", false, out, x, w_packed, scales_packed, zeros_packed, topk_w, sorted_ids,
+                             expert_ids, num_post_pad, numel, top_k, E, n, k, group, block_m, dtype, stream);
+}
+
+KSQ_EXPORT int ksq_moe_w4a16_gate_up_silu(void* out, const void* x, const void* w_packed, const void* scales_packed,
+                                          const void* zeros_packed, const void* sorted_ids, const void* expert_ids,
+                                          const void* num_post_pad, size_t numel, size_t top_k, size_t E, size_t n,
+                                          size_t k, size_t group, size_t block_m, int dtype, void* stream) {
+  return moe_w4a16_gemm_impl("ksq_moe_w4a16_gate_up_silu", true, out, x, w_packed, scales_packed, zeros_packed, nullptr,
+                             sorted_ids, expert_ids, num_post_pad, numel, top_k, E, n, k, group, block_m, dtype, stream);
 }

@@ -46,6 +46,10 @@ struct SplitKParams {
   // partial sums [z][M][N] instead of the output; a second pass adds them up
   float* partial;
   uint32_t kt_per_part;
+  // grouped form, gate_up GEMM with silu*mul in the epilogue: the workgroup's first NT/2 column tiles are gate tiles
+  // g0.., the other NT/2 the up tiles pair_tiles + g0.. (pair_tiles = inter/16), and out[s, c] = T(silu(T(gate)) * T(up))
+  // is [numel, N/2].  0: plain GEMM.
+  uint32_t pair_tiles;
   uint32_t x_bytes;  // extent of x, below 1 GiB
   uint32_t nibble_mask, magic2;  // 0x000f000f and T::kMagic2, passed in so that they live in registers
 };
@@ -77,7 +81,10 @@ __global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKPar
   const int lq = lane >> 4;
   const uint32_t KT = p.K / 128;
   const uint32_t G = p.K / GROUP;
-  const uint32_t nt0 = blockIdx.x * NT;
+  const bool fused = GROUPED && NT > 1 && p.pair_tiles != 0;
+  const uint32_t nt0 = fused ? blockIdx.x * (NT / 2) : blockIdx.x * NT;
+  // tiles skipped between the workgroup's column tile NT/2-1 and its column tile NT/2 (0 unless fused)
+  const uint32_t pair_extra = fused ? p.pair_tiles - NT / 2 : 0;
 
   __shared__ f32x4 red[WAVES][NT * MT][64];
 
@@ -110,12 +117,13 @@ __global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKPar
   const uint32_t s_tile_stride = G * 32;
   const uint32_t z_tile_stride = G * 16;
   const __amdgpu_buffer_rsrc_t wr = make_rsrc(
-      static_cast<const char*>(p.w) + (tile_base + static_cast<size_t>(nt0) * KT) * 1024, NT * w_tile_stride);
+      static_cast<const char*>(p.w) + (tile_base + static_cast<size_t>(nt0) * KT) * 1024, (NT + pair_extra) * w_tile_stride);
   const __amdgpu_buffer_rsrc_t sr = make_rsrc(
-      static_cast<const char*>(p.scales) + (sz_base + static_cast<size_t>(nt0) * G * 16) * 2, NT * s_tile_stride);
+      static_cast<const char*>(p.scales) + (sz_base + static_cast<size_t>(nt0) * G * 16) * 2, (NT + pair_extra) * s_tile_stride);
   const __amdgpu_buffer_rsrc_t zr = make_rsrc(
       HAS_ZP ? static_cast<const char*>(p.zeros) + sz_base + static_cast<size_t>(nt0) * G * 16 : nullptr,
-      HAS_ZP ? NT * z_tile_stride : 0);
+      HAS_ZP ? (NT + pair_extra) * z_tile_stride : 0);
+  const uint32_t pair_w = pair_extra * w_tile_stride, pair_s = pair_extra * s_tile_stride, pair_z = pair_extra * z_tile_stride;
   // x spans less than 1 GiB (checked on the host), so offset kOutOfRange is past this constant extent
   const __amdgpu_buffer_rsrc_t xr = make_rsrc(p.x, 0x3fffffffu);
   const uint32_t w_off = lane * 16;
@@ -162,11 +170,12 @@ __global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKPar
   };
 
   auto load_slot = [&](Slot& s, int t, const KOff& o) {
-    s.wq = __builtin_amdgcn_raw_buffer_load_b128(wr, w_off, t * w_tile_stride + o.w, 2);
+    const bool upper = NT > 1 && t >= NT / 2;  // the up tiles of a fused gate_up workgroup lie pair_extra tiles further
+    s.wq = __builtin_amdgcn_raw_buffer_load_b128(wr, w_off, t * w_tile_stride + (upper ? pair_w : 0) + o.w, 2);
 #pragma unroll
     for (int gi = 0; gi < GPT; ++gi) {
-      s.sc[gi] = __builtin_amdgcn_raw_buffer_load_b16(sr, s_off, t * s_tile_stride + o.s + gi * 32, 0);
-      if (HAS_ZP) s.zp[gi] = __builtin_amdgcn_raw_buffer_load_b8(zr, z_off, t * z_tile_stride + o.z + gi * 16, 0);
+      s.sc[gi] = __builtin_amdgcn_raw_buffer_load_b16(sr, s_off, t * s_tile_stride + (upper ? pair_s : 0) + o.s + gi * 32, 0);
+      if (HAS_ZP) s.zp[gi] = __builtin_amdgcn_raw_buffer_load_b8(zr, z_off, t * z_tile_stride + (upper ? pair_z : 0) + o.z + gi * 16, 0);
     }
   };
   auto load_x = [&](XBuf& b, const KOff& o) {
@@ -253,6 +262,36 @@ __global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKPar
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) red[wave][t * MT + mt][lane] = acc[t][mt];
   __syncthreads();
+
+  if (GROUPED && NT > 1 && fused) {
+    // gate_up with silu*mul: both sums are rounded to T as the unfused GEMM would store them, then
+    // silu(g) * u in fp32 and one more rounding, the arithmetic of silu_mul_kernel
+    constexpr int HALF = NT > 1 ? NT / 2 : 1;
+    const uint32_t out_n = p.N / 2;
+    for (int idx = threadIdx.x; idx < HALF * MT * 64; idx += WAVES * 64) {
+      const int l = idx & 63;
+      const int tm = idx >> 6;
+      const int t = tm / MT, mt = tm % MT;
+      f32x4 g = red[0][t * MT + mt][l], u = red[0][(t + HALF) * MT + mt][l];
+#pragma unroll
+      for (int w = 1; w < WAVES; ++w) {
+        g += red[w][t * MT + mt][l];
+        u += red[w][(t + HALF) * MT + mt][l];
+      }
+      const uint32_t col = (nt0 + t) * 16 + (l & 15);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t r = mt * 16 + 4 * (l >> 4) + i;
+        const uint32_t sid = static_cast<uint32_t>(p.sorted_ids[blockIdx.y * (16 * MT) + r]);
+        if (sid < p.numel) {
+          const float gv = T::to_float(T::from_float(g[i])), uv = T::to_float(T::from_float(u[i]));
+          const float y = gv / (1.0f + expf(-gv)) * uv;
+          static_cast<uint16_t*>(p.y)[static_cast<size_t>(sid) * out_n + col] = T::from_float(y);
+        }
+      }
+    }
+    return;
+  }
 
   for (int idx = threadIdx.x; idx < NT * MT * 64; idx += WAVES * 64) {
     const int l = idx & 63;

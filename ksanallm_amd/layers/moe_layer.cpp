@@ -216,11 +216,18 @@ Status MoeLayer::Forward(const std::vector<Tensor>& input_tensors, std::vector<T
       continue;
     }
     // gate_up: every (token, slot) row reads hidden[token]
-    KsqCheck(ksq_moe_w4a16_gemm(cache1, hidden + begin * hidden_size * elem, w1, w1_scale, nullptr, nullptr, sorted_ids,
-                                expert_ids, num_post_pad, numel, topk, E, 2 * inter, hidden_size, group_size_, block_m,
-                                dtype, stream),
-             "MoeLayer");
-    KsqCheck(ksq_moe_silu_mul(cache1, cache2, numel, inter, dtype, stream), "MoeLayer");
+    if (block_m <= 32 && (2 * inter) % 32 == 0) {  // decode regime: the activation runs in the GEMM's epilogue
+      KsqCheck(ksq_moe_w4a16_gate_up_silu(cache2, hidden + begin * hidden_size * elem, w1, w1_scale, nullptr, sorted_ids,
+                                          expert_ids, num_post_pad, numel, topk, E, 2 * inter, hidden_size, group_size_,
+                                          block_m, dtype, stream),
+               "MoeLayer");
+    } else {
+      KsqCheck(ksq_moe_w4a16_gemm(cache1, hidden + begin * hidden_size * elem, w1, w1_scale, nullptr, nullptr, sorted_ids,
+                                  expert_ids, num_post_pad, numel, topk, E, 2 * inter, hidden_size, group_size_, block_m,
+                                  dtype, stream),
+               "MoeLayer");
+      KsqCheck(ksq_moe_silu_mul(cache1, cache2, numel, inter, dtype, stream), "MoeLayer");
+    }
     // down: row s reads cache2[s]; the routing weight is applied in the epilogue
     KsqCheck(ksq_moe_w4a16_gemm(cache3, cache2, w2, w2_scale, nullptr, weights, sorted_ids, expert_ids, num_post_pad,
                                 numel, 1, E, hidden_size, inter, group_size_, block_m, dtype, stream),

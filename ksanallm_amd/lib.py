@@ -44,6 +44,8 @@ SIGNATURES = {
     "ksq_moe_align": (c_i, [c_p, c_sz, c_sz, c_sz, c_p, c_p, c_p, c_p, c_p]),
     "ksq_moe_w4a16_gemm": (c_i, [c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_sz, c_sz, c_sz, c_sz, c_sz, c_sz,
                                  c_sz, c_i, c_p]),
+    "ksq_moe_w4a16_gate_up_silu": (c_i, [c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_sz, c_sz, c_sz, c_sz, c_sz, c_sz, c_sz,
+                                         c_i, c_p]),
     "ksq_w4a16_repack_act_order": (c_i, [c_p, c_p, c_p, c_sz, c_sz, c_p]),
     "ksq_permute_columns": (c_i, [c_p, c_p, c_p, c_sz, c_sz, c_i, c_p]),
     "ksq_fp8_repack_weight": (c_i, [c_p, c_p, c_sz, c_sz, c_sz, c_p]),

@@ -180,6 +180,18 @@ def moe_w4a16_gemm(x, w_packed, scales_packed, topk_w, sorted_ids, expert_ids, n
     return out
 
 
+def moe_w4a16_gate_up_silu(x, w_packed, scales_packed, sorted_ids, expert_ids, num_post_pad, numel, top_k, E, n, k, group,
+                           block_m, out=None):
+    """The first MoE GEMM with silu*mul in its epilogue (block_m 16 or 32): out [numel, n/2], bit for bit what
+    moe_w4a16_gemm followed by silu_and_mul gives."""
+    if out is None:
+        out = torch.empty((numel, n // 2), dtype=x.dtype, device=x.device)
+    _l.check(_lib.ksq_moe_w4a16_gate_up_silu(_ptr(out), _ptr(x), _ptr(w_packed), _ptr(scales_packed), None,
+                                             _ptr(sorted_ids), _ptr(expert_ids), _ptr(num_post_pad), numel, top_k, E, n,
+                                             k, group, block_m, _dt(x), _stream()))
+    return out
+
+
 def moe_topk_softmax(gating, top_k, norm_topk_prob=False, routed_scaling_factor=1.0):
     """InvokeBasicSoftmaxTopk: (topk_weights fp32 [T, top_k], topk_ids int32 [T, top_k])."""
     tokens, E = gating.shape
@@ -237,9 +249,13 @@ def fused_moe_w4a16(x, w13_packed, s13_packed, w2_packed, s2_packed, topk_ids, t
         block_m = _lib.ksq_moe_block_m(numel, E)
     sorted_ids, expert_ids, npp = moe_align_block_size(topk_ids, E, block_m)
     tw = topk_w.reshape(-1).to(torch.float32).contiguous()
-    c1 = moe_w4a16_gemm(x, w13_packed, s13_packed, None, sorted_ids, expert_ids, npp, numel, topk, E, 2 * inter,
-                        hidden, group, block_m)
-    c2 = silu_and_mul(c1)
+    if block_m <= 32 and (2 * inter) % 32 == 0:  # decode regime: the activation runs in the GEMM's epilogue
+        c2 = moe_w4a16_gate_up_silu(x, w13_packed, s13_packed, sorted_ids, expert_ids, npp, numel, topk, E, 2 * inter,
+                                    hidden, group, block_m)
+    else:
+        c1 = moe_w4a16_gemm(x, w13_packed, s13_packed, None, sorted_ids, expert_ids, npp, numel, topk, E, 2 * inter,
+                            hidden, group, block_m)
+        c2 = silu_and_mul(c1)
     c3 = moe_w4a16_gemm(c2, w2_packed, s2_packed, tw, sorted_ids, expert_ids, npp, numel, 1, E, hidden, inter, group,
                         block_m)
     return moe_sum(c3.view(T, topk, hidden))

@@ -187,6 +187,31 @@ def test_silu_mul_and_sum(ops, oracle, dtype):
     np.testing.assert_array_equal(H.bits_of(got.cpu()), ref)
 
 
+@pytest.mark.parametrize("dtype", [H.F16, H.BF16])
+@pytest.mark.parametrize("T,E,topk,hidden,inter,bm", [(1, 8, 2, 256, 128, 16), (5, 16, 4, 512, 256, 16), (70, 8, 2, 384, 80 * 16, 32),
+                                                      (33, 256, 8, 7168, 2048, 16), (300, 16, 4, 256, 16, 32)])
+def test_gate_up_with_silu_in_the_epilogue_equals_the_two_launches(ops, dtype, T, E, topk, hidden, inter, bm):
+    """ksq_moe_w4a16_gate_up_silu against ksq_moe_w4a16_gemm + ksq_silu_mul on the same inputs: the same bits."""
+    from ksanallm_amd import lib as L
+    g = H.gen(8800 + T + inter)
+    td = H.TORCH_DT[dtype]
+    w13 = torch.randint(0, 256, (E, 2 * inter, hidden // 2), generator=g, dtype=torch.uint8)
+    s13 = H.uniform(g, (E, 2 * inter, hidden // 128), 0.002, 0.01, dtype)
+    x = torch.randn((T, hidden), generator=g).to(td).cuda()
+    ids = torch.stack([torch.randperm(E, generator=g)[:topk] for _ in range(T)]).to(torch.int32).cuda()
+    wp = ops.repack_weight(w13.cuda(), L.SRC_MOE_NK, E, hidden, 2 * inter)
+    sp = ops.repack_scales(s13.cuda(), L.SCALE_NG, E, hidden, 2 * inter, 128)
+    numel = T * topk
+    s, e, npp = ops.moe_align_block_size(ids, E, bm)
+    two = ops.silu_and_mul(ops.moe_w4a16_gemm(x, wp, sp, None, s, e, npp, numel, topk, E, 2 * inter, hidden, 128, bm))
+    one = ops.moe_w4a16_gate_up_silu(x, wp, sp, s, e, npp, numel, topk, E, 2 * inter, hidden, 128, bm)
+    torch.cuda.synchronize()
+    assert torch.equal(one.view(torch.int16), two.view(torch.int16))
+    with pytest.raises(L.KsqError) as err:
+        ops.moe_w4a16_gate_up_silu(x, wp, sp, s, e, npp, numel, topk, E, 2 * inter, hidden, 128, 128)
+    assert err.value.code == 2
+
+
 def make_moe(oracle, seed, E, hidden, inter, T, topk, group, dtype):
     g = H.gen(seed)
     td = H.TORCH_DT[dtype]
