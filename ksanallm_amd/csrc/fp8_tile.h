@@ -97,10 +97,22 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
   // fetches piece (j%4) ^ (j/16) of row j/4, so that MFMA lane (row r, k slot q) finds its two pieces 2(q%2)+p at
   // 1024*(q/2) + 64r + 16*((2(q%2)+p) ^ (r/4)): the sixteen lanes that read together hit different bank groups.
   size_t expert = 0;
+  // Row tiles (16 tokens) of this block that hold tokens at all.  In the grouped form an expert's last block is padded
+  // to the block size and the pad slots lie at its end: a wavefront all of whose tokens are pad slots (the upper half
+  // of a block that is at most half full) only takes its part in the loads and barriers.
+  uint32_t live_tiles = AF;
   if (GROUPED) {
     if (m0 >= static_cast<uint32_t>(p.num_post_pad[0])) return;  // uniform: the whole workgroup leaves
     expert = static_cast<size_t>(__builtin_amdgcn_readfirstlane(p.expert_ids[tile_m]));
+    uint32_t rows = 0;
+#pragma unroll
+    for (int h = 0; h < BM / 64; ++h) {
+      const bool is_row = static_cast<uint32_t>(p.sorted_ids[m0 + h * 64 + lane]) < p.numel;
+      rows += static_cast<uint32_t>(__builtin_popcountll(__builtin_amdgcn_ballot_w64(is_row)));
+    }
+    live_tiles = __builtin_amdgcn_readfirstlane((rows + 15) / 16);
   }
+  const bool idle = GROUPED && live_tiles <= wm * WM;  // none of this wavefront's row tiles wm*WM .. holds a token
   const bool stage_act = wave < 4;
   const uint32_t frag0 = (wave & 3) * (stage_act ? AFW : 4);
   // Weights come as packed 2 KiB fragments (ksq_fp8_repack_weight), fragment (strip, k-block) at (strip*KB + kb)*2048:
@@ -322,7 +334,12 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
   __syncthreads();  // also publishes the weight-scale table written with ordinary stores above
 
   for (uint32_t c = 0; c < kb_count; ++c) {
-    compute(c % NS, c, c + NS - 1);
+    if (idle) {
+      load_scales(c + NS - 1);
+      load_operands(c + NS - 1);
+    } else {
+      compute(c % NS, c, c + NS - 1);
+    }
     wait_stage();  // operands and scales of c+1
     __builtin_amdgcn_s_barrier();
   }

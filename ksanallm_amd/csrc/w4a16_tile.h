@@ -176,9 +176,19 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
   const uint32_t kt_count = direct ? KT : ((KT - kt_begin) < p.kt_per_split ? (KT - kt_begin) : p.kt_per_split);
   const uint32_t stages = kt_count * 2;
   uint32_t expert = 0;
+  // Row tiles (16 rows) of this block that hold rows at all.  In the grouped form an expert's last block is padded to
+  // the block size and the pad slots lie at its end.
+  uint32_t live_tiles = WM;
   if (GROUPED) {
     if (m0 >= static_cast<uint32_t>(p.num_post_pad[0])) return;  // uniform: the whole workgroup leaves
     expert = static_cast<uint32_t>(p.expert_ids[tile_m]);
+    uint32_t rows = 0;
+#pragma unroll
+    for (int h = 0; h < BM / 64; ++h) {
+      const bool is_row = static_cast<uint32_t>(p.sorted_ids[m0 + h * 64 + lane]) < p.numel;
+      rows += static_cast<uint32_t>(__builtin_popcountll(__builtin_amdgcn_ballot_w64(is_row)));
+    }
+    live_tiles = __builtin_amdgcn_readfirstlane((rows + 15) / 16);
   }
 
   // ---- x staging: this wavefront fetches fragments f = wave*AP + 2j + {0,1}: row block f/2, k half f%2.
@@ -308,91 +318,106 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
   };
   auto wait_only = [&](auto n) { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(decltype(n)::value) : "memory"); };
 
-  // ---- compute pipeline, in steps of 32 k (two per stage).  A fragments are read DEPTH ahead of the MFMAs that use
-  // them, across step and stage boundaries; the weight fragments of step g+1 are dequantized while step g multiplies.
-  constexpr int DEPTH = 4;
-  static_assert(WM % DEPTH == 0, "the A prefetch ring must divide the row tiles");
-  u32x4 abuf[DEPTH];
-  typename T::frag bfrag[2][WN];  // weight fragments of the current step [g % 2] and the next one
-  Dequant<T, HAS_ZP> dq[WN];
+  // Everything from here to the end of the main loop exists once per number of row tiles that are multiplied (WMV):
+  // all WM of them, or - grouped form, block at most half full - the lower WM/2 only.  The choice is made once per
+  // workgroup, outside the scheduled loop; guarding single row tiles inside it would split the loop body into basic
+  // blocks and lose the interleaving of LDS reads, conversions and MFMAs (measured: 20 % slower, not faster).
+  auto run = [&](auto wmv_c) {
+    constexpr int WMV = decltype(wmv_c)::value;
+    // ---- compute pipeline, in steps of 32 k (two per stage).  A fragments are read DEPTH ahead of the MFMAs that use
+    // them, across step and stage boundaries; the weight fragments of step g+1 are dequantized while step g multiplies.
+    constexpr int DEPTH = 4;
+    static_assert(WMV % DEPTH == 0, "the A prefetch ring must divide the row tiles");
+    u32x4 abuf[DEPTH];
+    typename T::frag bfrag[2][WN];  // weight fragments of the current step [g % 2] and the next one
+    Dequant<T, HAS_ZP> dq[WN];
 
-  auto frag_ptr = [&](uint32_t slot, int ks) { return lds + slot * STAGE_BYTES + ks * 1024 + a_rd; };
-  // `wn`/`dn`: weight slot and dword (32-k block of its k-tile) the NEXT step uses
-  auto step = [&](auto parity, uint32_t slot, int ks, WSlot (&wn)[WN], int dn) {
-    constexpr int P = decltype(parity)::value;
-    typename T::frag(&bcur)[WN] = bfrag[P];
-    typename T::frag(&bnext)[WN] = bfrag[P ^ 1];
-    const char* cur = frag_ptr(slot, ks);
-    const char* nxt = ks == 0 ? frag_ptr(slot, 1) : frag_ptr((slot + 1) % NS, 0);
-    if (dn == 0) {
-#pragma unroll
-      for (int t = 0; t < WN; ++t) dq[t].set(wn[t].sc, wn[t].zp);
+    auto frag_ptr = [&](uint32_t slot, int ks) { return lds + slot * STAGE_BYTES + ks * 1024 + a_rd; };
+    // `wn`/`dn`: weight slot and dword (32-k block of its k-tile) the NEXT step uses
+    auto step = [&](auto parity, uint32_t slot, int ks, WSlot (&wn)[WN], int dn) {
+      constexpr int P = decltype(parity)::value;
+      typename T::frag(&bcur)[WN] = bfrag[P];
+      typename T::frag(&bnext)[WN] = bfrag[P ^ 1];
+      const char* cur = frag_ptr(slot, ks);
+      const char* nxt = ks == 0 ? frag_ptr(slot, 1) : frag_ptr((slot + 1) % NS, 0);
+      if (dn == 0) {
+  #pragma unroll
+        for (int t = 0; t < WN; ++t) dq[t].set(wn[t].sc, wn[t].zp);
+      }
+  #pragma unroll
+      for (int i = 0; i < WMV; ++i) {
+        const u32x4 a = abuf[i % DEPTH];
+        const int ni = i + DEPTH;
+        abuf[i % DEPTH] = ni < WMV ? *reinterpret_cast<const u32x4*>(cur + ni * 2048)
+                                   : *reinterpret_cast<const u32x4*>(nxt + (ni - WMV) * 2048);
+  #pragma unroll
+        for (int t = 0; t < WN; ++t) acc[t][i] = T::mfma(bcur[t], as_frag<T>(a), acc[t][i]);
+        if (i == 1) bnext[0] = dq[0](wn[0].wq[dn]);
+        if (i == WMV / 2 + 1) bnext[1] = dq[1](wn[1].wq[dn]);
+        __builtin_amdgcn_sched_barrier(0x6);  // VALU / SALU may move; LDS reads and MFMAs keep this order
+      }
+    };
+    using Even = std::integral_constant<int, 0>;
+    using Odd = std::integral_constant<int, 1>;
+
+    // ---- schedule.  One synchronisation point per stage, in its middle ("sync c" sits between the two steps of
+    // stage c): wait for x stage c+1, barrier, then issue [weights of k-tile c/2+2 when c is even][x stage c+3] - the LDS
+    // slot of stage c+3 is the one stage c-1 used, and every wavefront is past that.  Weights of k-tile kt are issued at
+    // sync 2kt-4, complete at sync 2kt-2 and are first dequantized during the last step of k-tile kt-1.
+    // Loads outstanding after x stage c+1 at sync c: those of sync c-1, i.e. AP, plus 2*WL when c-1 is even.
+    using WaitEven = std::integral_constant<int, AP>;
+    using WaitOdd = std::integral_constant<int, AP + WN * WL>;
+    using WaitFirst = std::integral_constant<int, 2 * AP + WN * WL>;
+    load_w(ring[0], 0);  // sync -4
+    load_a(0);           // sync -3
+    load_w(ring[1], 1);  // sync -2
+    load_a(1);
+    load_a(2);           // sync -1
+    wait_tie(WaitFirst{}, ring[0]);  // x stage 0 and k-tile 0 are in
+    __builtin_amdgcn_s_barrier();
+  #pragma unroll
+    for (int t = 0; t < WN; ++t) {
+      dq[t].set(ring[0][t].sc, ring[0][t].zp);
+      bfrag[0][t] = dq[t](ring[0][t].wq[0]);
     }
-#pragma unroll
-    for (int i = 0; i < WM; ++i) {
-      const u32x4 a = abuf[i % DEPTH];
-      const int ni = i + DEPTH;
-      abuf[i % DEPTH] = ni < WM ? *reinterpret_cast<const u32x4*>(cur + ni * 2048)
-                                : *reinterpret_cast<const u32x4*>(nxt + (ni - WM) * 2048);
-#pragma unroll
-      for (int t = 0; t < WN; ++t) acc[t][i] = T::mfma(bcur[t], as_frag<T>(a), acc[t][i]);
-      if (i == 1) bnext[0] = dq[0](wn[0].wq[dn]);
-      if (i == WM / 2 + 1) bnext[1] = dq[1](wn[1].wq[dn]);
-      __builtin_amdgcn_sched_barrier(0x6);  // VALU / SALU may move; LDS reads and MFMAs keep this order
+  #pragma unroll
+    for (int j = 0; j < DEPTH; ++j) abuf[j] = *reinterpret_cast<const u32x4*>(frag_ptr(0, 0) + j * 2048);
+
+    for (uint32_t base = 0; base < stages; base += 6) {
+  #pragma unroll
+      for (int u = 0; u < 6; ++u) {
+        const uint32_t s = base + u;
+        const uint32_t slot = s % NS;
+        constexpr int kDummy = 0;
+        (void)kDummy;
+        // first step of the stage: k block 2*(u%2) of k-tile u/2; the next step uses block 2*(u%2)+1 of the same tile
+        if (s < stages) step(Even{}, slot, 0, ring[(u / 2) % 3], 2 * (u % 2) + 1);
+        // sync s
+        if (u % 2 == 0) {
+          wait_tie(WaitEven{}, ring[(u / 2 + 1) % 3]);  // k-tile s/2+1, issued at sync s-2
+        } else {
+          wait_only(WaitOdd{});
+        }
+        __builtin_amdgcn_s_barrier();
+        if (u % 2 == 0) load_w(ring[(u / 2 + 2) % 3], s / 2 + 2);
+        load_a(s + 3);
+        // second step: the next step is block 2 of this k-tile (u even) or block 0 of the next k-tile (u odd)
+        if (s < stages) {
+          if (u % 2 == 0)
+            step(Odd{}, slot, 1, ring[(u / 2) % 3], 2);
+          else
+            step(Odd{}, slot, 1, ring[(u / 2 + 1) % 3], 0);
+        }
+      }
     }
   };
-  using Even = std::integral_constant<int, 0>;
-  using Odd = std::integral_constant<int, 1>;
-
-  // ---- schedule.  One synchronisation point per stage, in its middle ("sync c" sits between the two steps of
-  // stage c): wait for x stage c+1, barrier, then issue [weights of k-tile c/2+2 when c is even][x stage c+3] - the LDS
-  // slot of stage c+3 is the one stage c-1 used, and every wavefront is past that.  Weights of k-tile kt are issued at
-  // sync 2kt-4, complete at sync 2kt-2 and are first dequantized during the last step of k-tile kt-1.
-  // Loads outstanding after x stage c+1 at sync c: those of sync c-1, i.e. AP, plus 2*WL when c-1 is even.
-  using WaitEven = std::integral_constant<int, AP>;
-  using WaitOdd = std::integral_constant<int, AP + WN * WL>;
-  using WaitFirst = std::integral_constant<int, 2 * AP + WN * WL>;
-  load_w(ring[0], 0);  // sync -4
-  load_a(0);           // sync -3
-  load_w(ring[1], 1);  // sync -2
-  load_a(1);
-  load_a(2);           // sync -1
-  wait_tie(WaitFirst{}, ring[0]);  // x stage 0 and k-tile 0 are in
-  __builtin_amdgcn_s_barrier();
-#pragma unroll
-  for (int t = 0; t < WN; ++t) {
-    dq[t].set(ring[0][t].sc, ring[0][t].zp);
-    bfrag[0][t] = dq[t](ring[0][t].wq[0]);
-  }
-#pragma unroll
-  for (int j = 0; j < DEPTH; ++j) abuf[j] = *reinterpret_cast<const u32x4*>(frag_ptr(0, 0) + j * 2048);
-
-  for (uint32_t base = 0; base < stages; base += 6) {
-#pragma unroll
-    for (int u = 0; u < 6; ++u) {
-      const uint32_t s = base + u;
-      const uint32_t slot = s % NS;
-      constexpr int kDummy = 0;
-      (void)kDummy;
-      // first step of the stage: k block 2*(u%2) of k-tile u/2; the next step uses block 2*(u%2)+1 of the same tile
-      if (s < stages) step(Even{}, slot, 0, ring[(u / 2) % 3], 2 * (u % 2) + 1);
-      // sync s
-      if (u % 2 == 0) {
-        wait_tie(WaitEven{}, ring[(u / 2 + 1) % 3]);  // k-tile s/2+1, issued at sync s-2
-      } else {
-        wait_only(WaitOdd{});
-      }
-      __builtin_amdgcn_s_barrier();
-      if (u % 2 == 0) load_w(ring[(u / 2 + 2) % 3], s / 2 + 2);
-      load_a(s + 3);
-      // second step: the next step is block 2 of this k-tile (u even) or block 0 of the next k-tile (u odd)
-      if (s < stages) {
-        if (u % 2 == 0)
-          step(Odd{}, slot, 1, ring[(u / 2) % 3], 2);
-        else
-          step(Odd{}, slot, 1, ring[(u / 2 + 1) % 3], 0);
-      }
-    }
+  if constexpr (GROUPED) {
+    if (live_tiles <= WM / 2)
+      run(std::integral_constant<int, WM / 2>{});
+    else
+      run(std::integral_constant<int, WM>{});
+  } else {
+    run(std::integral_constant<int, WM>{});
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // drain the clamped prefetches before the LDS is released
 
