@@ -162,12 +162,13 @@ KSQ_EXPORT size_t ksq_moe_fp8_block_m(size_t numel, size_t E) {
 }
 
 // Rows per expert block for numel routed (token, slot) pairs over E experts.  Replaces the M thresholds of
-// InvokeFusedMoe (16 / 32 / 64 rows by token count): below about 64 rows per expert the weights are streamed once per
-// 16- or 32-row block (HBM-bound); above, 128-row blocks feed the MFMA tile kernel.
+// InvokeFusedMoe (16 / 32 / 64 rows by token count): below about 40 rows per expert the weights are streamed once per
+// 16- or 32-row block (HBM-bound); above, 128-row blocks feed the MFMA tile kernel (E = 256, hidden 7168, inter 2048,
+// top-8: 2.52 against 2.70 ms at 32 rows per expert, 3.37 against 3.00 ms at 48).
 KSQ_EXPORT size_t ksq_moe_block_m(size_t numel, size_t E) {
   if (E == 0) return 16;
   const size_t per_expert = numel / E;
-  if (per_expert >= 64) return 128;
+  if (per_expert >= 40) return 128;
   return per_expert < 16 ? 16 : 32;
 }
 
