@@ -97,10 +97,15 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
   // fetches piece (j%4) ^ (j/16) of row j/4, so that MFMA lane (row r, k slot q) finds its two pieces 2(q%2)+p at
   // 1024*(q/2) + 64r + 16*((2(q%2)+p) ^ (r/4)): the sixteen lanes that read together hit different bank groups.
   size_t expert = 0;
-  // Row tiles (16 tokens) of this block that hold tokens at all.  In the grouped form an expert's last block is padded
-  // to the block size and the pad slots lie at its end: a wavefront all of whose tokens are pad slots (the upper half
-  // of a block that is at most half full) only takes its part in the loads and barriers.
+  // Row tiles (16 tokens) of this block that hold tokens at all: the last block of the matrix may be short, and in the
+  // grouped form an expert's last block is padded to the block size with the pad slots at its end.  A wavefront none
+  // of whose row tiles holds a token (the upper half of a block that is at most half full) only takes its part in the
+  // loads and barriers.
   uint32_t live_tiles = AF;
+  if (!GROUPED) {
+    const uint32_t rows = p.M - m0;
+    live_tiles = rows < static_cast<uint32_t>(BM) ? (rows + 15) / 16 : AF;
+  }
   if (GROUPED) {
     if (m0 >= static_cast<uint32_t>(p.num_post_pad[0])) return;  // uniform: the whole workgroup leaves
     expert = static_cast<size_t>(__builtin_amdgcn_readfirstlane(p.expert_ids[tile_m]));
@@ -112,7 +117,7 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
     }
     live_tiles = __builtin_amdgcn_readfirstlane((rows + 15) / 16);
   }
-  const bool idle = GROUPED && live_tiles <= wm * WM;  // none of this wavefront's row tiles wm*WM .. holds a token
+  const bool idle = live_tiles <= wm * WM;  // none of this wavefront's row tiles wm*WM .. holds a token
   const bool stage_act = wave < 4;
   const uint32_t frag0 = (wave & 3) * (stage_act ? AFW : 4);
   // Weights come as packed 2 KiB fragments (ksq_fp8_repack_weight), fragment (strip, k-block) at (strip*KB + kb)*2048:

@@ -176,9 +176,13 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
   const uint32_t kt_count = direct ? KT : ((KT - kt_begin) < p.kt_per_split ? (KT - kt_begin) : p.kt_per_split);
   const uint32_t stages = kt_count * 2;
   uint32_t expert = 0;
-  // Row tiles (16 rows) of this block that hold rows at all.  In the grouped form an expert's last block is padded to
-  // the block size and the pad slots lie at its end.
+  // Row tiles (16 rows) of this block that hold rows at all: the last row block of the matrix may be short, and in the
+  // grouped form an expert's last block is padded to the block size with the pad slots at its end.
   uint32_t live_tiles = WM;
+  if (!GROUPED) {
+    const uint32_t rows = p.M - m0;
+    live_tiles = rows < static_cast<uint32_t>(BM) ? (rows + 15) / 16 : WM;
+  }
   if (GROUPED) {
     if (m0 >= static_cast<uint32_t>(p.num_post_pad[0])) return;  // uniform: the whole workgroup leaves
     expert = static_cast<uint32_t>(p.expert_ids[tile_m]);
@@ -319,7 +323,7 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
   auto wait_only = [&](auto n) { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(decltype(n)::value) : "memory"); };
 
   // Everything from here to the end of the main loop exists once per number of row tiles that are multiplied (WMV):
-  // all WM of them, or - grouped form, block at most half full - the lower WM/2 only.  The choice is made once per
+  // all WM of them, or - block at most half full - the lower WM/2 only.  The choice is made once per
   // workgroup, outside the scheduled loop; guarding single row tiles inside it would split the loop body into basic
   // blocks and lose the interleaving of LDS reads, conversions and MFMAs (measured: 20 % slower, not faster).
   auto run = [&](auto wmv_c) {
@@ -411,14 +415,10 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
       }
     }
   };
-  if constexpr (GROUPED) {
-    if (live_tiles <= WM / 2)
-      run(std::integral_constant<int, WM / 2>{});
-    else
-      run(std::integral_constant<int, WM>{});
-  } else {
+  if (live_tiles <= WM / 2)
+    run(std::integral_constant<int, WM / 2>{});
+  else
     run(std::integral_constant<int, WM>{});
-  }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // drain the clamped prefetches before the LDS is released
 
   // ---- store: lane holds row m = l%16 of the 16x16 tile and columns 4*(l/16) .. +3
