@@ -1,10 +1,17 @@
-"""Pins the CPU oracle against the known-answer vectors the reference's own tests hold, and against what the
+"""Pins the CPU oracle against the known-answer vectors the reference's own tests hold (tests/golden/
+reference_known_answers.json, each entry with the reference file:line it was taken from), and against what the
 mathematics fixes.  No GPU."""
+import json
+import os
+
 import numpy as np
 import pytest
 import torch
 
 from tests import helpers as H
+
+with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_known_answers.json")) as _f:
+    GOLDEN = json.load(_f)
 
 
 # ----------------------------------------------------------------------------- scalar formats
@@ -79,12 +86,13 @@ def test_e4m3_encode_rne_satfinite(oracle):
 # ----------------------------------------------------------------------------- checkpoint layouts
 def test_unpack_known_answer_0x66666666(oracle):
     """S/models/quant/cutlass_utils_test.cpp:80-108: int32 1717986918 everywhere -> every packed byte == -18."""
-    q = np.full((64, 128), 1717986918, dtype=np.uint32)
+    fx = GOLDEN["unpack_0x66666666"]
+    q = np.full(tuple(fx["shape"]), fx["input_word"], dtype=np.uint32)
     for unpack in (oracle.gptq_unpack, oracle.awq_unpack):
         codes = unpack(q)
         signed = (codes.astype(np.int16) - 8).astype(np.int8)
         packed = oracle.pack_int8_to_int4x2(signed)
-        assert np.all(packed == -18)
+        assert np.all(packed == fx["expected_packed_int8"])
 
 
 def test_gptq_awq_unpack_positions(oracle):
@@ -106,23 +114,24 @@ def test_marlin_repack_golden(oracle):
     t = np.arange(1024 * 1024, dtype=np.uint32).reshape(1024, 1024)
     awq = oracle.marlin_awq_repack(t)    # k=1024, n=8192
     gptq = oracle.marlin_gptq_repack(t)  # k=8192, n=1024
-    assert gptq.shape == (512, 2048) and awq.shape == (64, 16384)
+    fx = GOLDEN["marlin_repack_arange"]
+    assert gptq.shape == tuple(fx["gptq_shape"]) and awq.shape == tuple(fx["awq_shape"])
     g, a = gptq.reshape(-1).view(np.int32), awq.reshape(-1).view(np.int32)
-    np.testing.assert_array_equal(g[:10], [34816, 286361600, 572688384, 859015168, 16448, 16448, 16448, 16448, 0, 0])
-    np.testing.assert_array_equal(a[:10], [285217024, 857879330, 1430541636, 2003203942, 285217024, 857879330,
-                                           1430541636, 2003203942, 285217024, 857879330])
-    np.testing.assert_array_equal(g[-10:], [-1029, -1029, 65535, 65535, 65535, 65535, 0, 0, 0, 0])
-    np.testing.assert_array_equal(a[-10:], [0] * 10)
+    np.testing.assert_array_equal(g[:10], fx["gptq_first10"])
+    np.testing.assert_array_equal(a[:10], fx["awq_first10"])
+    np.testing.assert_array_equal(g[-10:], fx["gptq_last10"])
+    np.testing.assert_array_equal(a[-10:], fx["awq_last10"])
 
 
 def test_marlin_awq_zero_points_golden(oracle):
     """S/models/quant/marlin_utils_test.cpp:149-173."""
     t = np.arange(1024 * 128, dtype=np.uint32).reshape(1024, 128)
     zp = oracle.marlin_awq_zero_points(t)
-    assert zp.shape == (1024, 128)
+    fx = GOLDEN["marlin_awq_zero_points_arange"]
+    assert zp.shape == tuple(fx["shape"])
     z = zp.reshape(-1).view(np.int32)
-    np.testing.assert_array_equal(z[:10], [1966171168, 0, 0, 0, 0, 0, 0, 0, -38146904, 0])
-    np.testing.assert_array_equal(z[-10:], [-1, 0, -38146904, 286331153, -1, 0, -1, 0, -1, 0])
+    np.testing.assert_array_equal(z[:10], fx["first10"])
+    np.testing.assert_array_equal(z[-10:], fx["last10"])
 
 
 def test_moe_layout_roundtrip_and_nibble_order(oracle):
@@ -141,7 +150,7 @@ def test_dequant_all_zero_codes_is_minus_8(oracle):
     codes = np.zeros((256, 32), np.uint8)
     s = oracle.to_bits(np.ones((2, 32), np.float32), oracle.F16)
     w = oracle.w4a16_dequant(codes, s, None, 128, oracle.F16)
-    assert np.all(w == -8.0)
+    assert np.all(w == GOLDEN["dequant_all_zero_codes"]["expected"])
 
 
 @pytest.mark.parametrize("dtype", [0, 1])
@@ -167,19 +176,7 @@ def test_w4a16_gemm_vs_float64(oracle, dtype):
 
 
 # ----------------------------------------------------------------------------- fp8 quantizer
-TARGET_Q = [
-    0, 70, 78, 83, 86, 89, 91, 92, 94, 96, 97, 98, 99, 99, 100, 101, 102, 103, 104, 104, 105, 105,
-    106, 106, 107, 107, 107, 108, 108, 109, 109, 110, 110, 111, 111, 111, 112, 112, 112, 113, 113, 113, 113, 113,
-    114, 114, 114, 114, 115, 115, 115, 115, 115, 116, 116, 116, 116, 117, 117, 117, 117, 117, 118, 118, 118, 118,
-    119, 119, 119, 119, 119, 119, 120, 120, 120, 120, 120, 120, 121, 121, 121, 121, 121, 121, 121, 121, 121, 122,
-    122, 122, 122, 122, 122, 122, 122, 122, 123, 123, 123, 123, 123, 123, 123, 123, 123, 124, 124, 124, 124, 124,
-    124, 124, 124, 124, 125, 125, 125, 125, 125, 125, 125, 125, 125, 126, 126, 126, 126, 126, 118, 118, 118, 118,
-    118, 119, 119, 119, 119, 119, 119, 119, 119, 119, 120, 120, 120, 120, 120, 120, 120, 120, 120, 120, 120, 120,
-    120, 121, 121, 121, 121, 121, 121, 121, 121, 121, 121, 121, 121, 121, 121, 121, 121, 121, 121, 121, 122, 122,
-    122, 122, 122, 122, 122, 122, 122, 122, 122, 122, 122, 122, 122, 122, 122, 122, 123, 123, 123, 123, 123, 123,
-    123, 123, 123, 123, 123, 123, 123, 123, 123, 123, 123, 123, 123, 124, 124, 124, 124, 124, 124, 124, 124, 124,
-    124, 124, 124, 124, 124, 124, 124, 124, 124, 125, 125, 125, 125, 125, 125, 125, 125, 125, 125, 125, 125, 125,
-    125, 125, 125, 125, 125, 126, 126, 126, 126, 126, 126, 126, 126, 126]
+TARGET_Q = GOLDEN["fp8_group_quant_i_over_100"]["codes"]
 
 
 @pytest.mark.parametrize("dtype", [0, 1])
@@ -192,9 +189,10 @@ def test_fp8_group_quant_known_answer(oracle, dtype, n, colmajor):
     xb = oracle.to_bits(x, dtype)
     q, s = oracle.fp8_group_quant(xb, n, 128, colmajor, False, dtype)
     s = s.reshape(-1)
-    np.testing.assert_allclose(s, [0.0028, 0.0057][: n // 128], atol=1e-4)
+    fx = GOLDEN["fp8_group_quant_i_over_100"]
+    np.testing.assert_allclose(s, fx["scales"][: n // 128], atol=fx["scale_atol"])
     diff = np.abs(q.reshape(-1).astype(int) - np.array(TARGET_Q[:n]))
-    assert diff.max() <= 1
+    assert diff.max() <= fx["code_tolerance"]
     assert (diff == 0).mean() > 0.95
 
 
@@ -263,12 +261,11 @@ def test_fp8_blockwise_gemm_vs_float64(oracle):
 # ----------------------------------------------------------------------------- MoE
 def test_moe_align_worked_example(oracle):
     """K/moe_utils/moe_utils.cu:150-156."""
-    ids = [0, 1, 2, 1, 2, 3, 0, 3, 4]
-    sorted_ids, expert_ids, npp = oracle.moe_align(ids, 5, 4)
-    P = 9
-    np.testing.assert_array_equal(sorted_ids[:20], [0, 6, P, P, 1, 3, P, P, 2, 4, P, P, 5, 7, P, P, 8, P, P, P])
-    assert npp == 20
-    np.testing.assert_array_equal(expert_ids[:5], [0, 1, 2, 3, 4])
+    fx = GOLDEN["moe_align_worked_example"]
+    sorted_ids, expert_ids, npp = oracle.moe_align(fx["topk_ids"], fx["experts"], fx["block"])
+    np.testing.assert_array_equal(sorted_ids[:20], fx["sorted_ids_first20"])   # 9 = the pad value numel
+    assert npp == fx["num_tokens_post_pad"]
+    np.testing.assert_array_equal(expert_ids[:5], fx["expert_ids_first5"])
 
 
 def test_moe_align_invariants(oracle):
