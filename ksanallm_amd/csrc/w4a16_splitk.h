@@ -21,8 +21,8 @@
 // The wavefronts' partials meet in LDS and are summed in wavefront order: the summation order is fixed, so the
 // output does not depend on timing.
 //
-// Rows of x beyond M are read from the last valid row instead of being masked: an MFMA output row depends only on
-// its own row of x, and those rows are never stored.
+// Rows of x beyond M are not fetched at all (buffer loads past the extent of the resource return zero): an MFMA output
+// row depends only on its own row of x, and those rows are never stored.
 #pragma once
 
 #include "ksq_common.h"
@@ -88,7 +88,10 @@ __global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKPar
 
   __shared__ f32x4 red[WAVES][NT * MT][64];
 
-  // ---- rows of x this lane feeds (row operand: lane l supplies row l%16, k = 8*(l/16)..+7 of each k-step)
+  // ---- rows of x this lane feeds (row operand: lane l supplies row l%16, k = 8*(l/16)..+7 of each k-step).  A lane
+  // whose row lies past M (or is a pad slot) gets an offset beyond the extent of x's buffer resource: its loads fetch
+  // nothing and return zero, and its MFMA output rows, which depend on no other row, are never stored.
+  constexpr uint32_t kNoRow = 0xffffffffu;
   uint32_t xrow[MT];
   size_t tile_base = 0;  // first weight tile of the expert, in tiles
   size_t sz_base = 0;    // first scale / zero element of the expert
@@ -100,15 +103,14 @@ __global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKPar
     sz_base = static_cast<size_t>(e) * G * p.N;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-      uint32_t sid = static_cast<uint32_t>(p.sorted_ids[pos0 + mt * 16 + lrow]);
-      sid = sid < p.numel ? sid : p.numel - 1;
-      xrow[mt] = sid / p.top_k;
+      const uint32_t sid = static_cast<uint32_t>(p.sorted_ids[pos0 + mt * 16 + lrow]);
+      xrow[mt] = sid < p.numel ? sid / p.top_k : kNoRow;
     }
   } else {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-      uint32_t r = blockIdx.y * (16 * MT) + mt * 16 + lrow;
-      xrow[mt] = r < p.M ? r : p.M - 1;
+      const uint32_t r = blockIdx.y * (16 * MT) + mt * 16 + lrow;
+      xrow[mt] = r < p.M ? r : kNoRow;
     }
   }
 
@@ -131,7 +133,7 @@ __global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKPar
   const uint32_t z_off = lrow;
   uint32_t x_off[MT];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) x_off[mt] = (xrow[mt] * p.K + lq * 8) * 2;
+  for (int mt = 0; mt < MT; ++mt) x_off[mt] = xrow[mt] != kNoRow ? (xrow[mt] * p.K + lq * 8) * 2 : 0x40000000u;
 
   // acc[t][mt][i]: column (nt0+t)*16 + lrow, row mt*16 + 4*lq + i
   f32x4 acc[NT][MT];
