@@ -348,3 +348,64 @@ def test_moe_fp8_block(ops, oracle, dtype, T, E, topk, hidden, inter):
                                     ops.fp8_repack_weight(torch.from_numpy(w2).cuda()), torch.from_numpy(s2).cuda(), ids, tw)
     ref = oracle.moe_fp8_forward(H.bits_of(x), w13, s13, w2, s2, ids.cpu().numpy(), tw.cpu().numpy(), dtype)
     H.check_gemm(y, oracle.from_bits(ref, dtype), dtype, "fp8 moe block")
+
+
+# ---- full-size properties (DeepSeek-V3 expert shapes: 256 experts, hidden 7168, inter 2048, top-8), no oracle needed:
+# a token's output depends on its own row, its experts and its routing weights only, so a permutation of the tokens
+# permutes the outputs bit for bit (whatever blocks, tiles and kernels the sizes select), a token routed with zero
+# weights comes out as exact zeros, and the same token repeated gives the same row every time.
+def _full_size_experts(ops, kind, distinct=16):
+    from ksanallm_amd import lib as L
+    E, hidden, inter = 256, 7168, 2048
+    g = H.gen(9900)
+    rep = E // distinct
+    if kind == "int4":
+        w13 = torch.randint(0, 256, (distinct, 2 * inter, hidden // 2), generator=g, dtype=torch.uint8)
+        w2 = torch.randint(0, 256, (distinct, hidden, inter // 2), generator=g, dtype=torch.uint8)
+        s13 = H.uniform(g, (distinct, 2 * inter, hidden // 128), 0.002, 0.01, H.BF16)
+        s2 = H.uniform(g, (distinct, hidden, inter // 128), 0.002, 0.01, H.BF16)
+        return (ops.repack_weight(w13.cuda(), L.SRC_MOE_NK, distinct, hidden, 2 * inter).repeat(rep),
+                ops.repack_scales(s13.cuda(), L.SCALE_NG, distinct, hidden, 2 * inter, 128).repeat(rep),
+                ops.repack_weight(w2.cuda(), L.SRC_MOE_NK, distinct, inter, hidden).repeat(rep),
+                ops.repack_scales(s2.cuda(), L.SCALE_NG, distinct, inter, hidden, 128).repeat(rep))
+
+    def experts(n, k):
+        q = torch.randint(0, 256, (distinct, n, k), generator=g, dtype=torch.uint8)
+        q = torch.where((q & 0x7f) == 0x7f, q & 0xfe, q)     # no NaN codes
+        s = torch.rand((distinct, n // 128, k // 128), generator=g) * 1e-4 + 1e-4
+        return ops.fp8_repack_weight(q.cuda()).repeat(rep, 1, 1), s.cuda().repeat(rep, 1, 1)
+
+    w13, s13 = experts(2 * inter, hidden)
+    w2, s2 = experts(hidden, inter)
+    return w13, s13, w2, s2
+
+
+@pytest.mark.parametrize("kind", ["int4", "fp8"])
+@pytest.mark.parametrize("T", [24, 700, 2304])      # 16-row, 32-row and tile-kernel blocks
+def test_moe_full_size_properties(ops, kind, T):
+    E, hidden, inter, topk = 256, 7168, 2048, 8
+    w13, s13, w2, s2 = _full_size_experts(ops, kind)
+    g = H.gen(9950 + T)
+    x = torch.randn((T, hidden), generator=g).to(torch.bfloat16)
+    x[T // 2] = x[0]                                    # a repeated token
+    logits = torch.randn((T, E), generator=g)
+    logits[T // 2] = logits[0]
+    tw, ids = torch.topk(torch.softmax(logits, -1), topk, dim=-1)
+    tw = tw.float().contiguous()
+    tw[1] = 0.0                                         # a token whose routing weights are all zero
+    ids = ids.to(torch.int32)
+
+    def run(xx, ii, ww):
+        if kind == "int4":
+            return ops.fused_moe_w4a16(xx.cuda(), w13, s13, w2, s2, ii.cuda(), ww.cuda(), E, hidden, inter, 128)
+        return ops.fused_moe_fp8_blockwise(xx.cuda(), w13, s13, w2, s2, ii.cuda(), ww.cuda())
+
+    y = run(x, ids, tw)
+    torch.cuda.synchronize()
+    assert torch.isfinite(y.float()).all()
+    assert torch.count_nonzero(y[1]) == 0
+    assert torch.equal(y[0].view(torch.int16), y[T // 2].view(torch.int16))
+    perm = torch.randperm(T, generator=g)
+    yp = run(x[perm], ids[perm], tw[perm])
+    torch.cuda.synchronize()
+    assert torch.equal(yp.view(torch.int16), y[perm.cuda()].view(torch.int16))
