@@ -170,6 +170,38 @@ int ksq_fp8_tensor_gemm(const void* a_q, const void* a_scale, const void* b, con
                         size_t n, size_t k, int out_dtype, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------------------------------------------------
+ * W4A8: int4 weights (group 128, fp16 scales, no zero points) against statically quantized e4m3 activations,
+ *   out[m,n] = T(alpha * sum_g scale[g,n] * sum_{k in g} a_q[m,k] * w[k,n]),  w in -8..7, fp32 accumulation.
+ * The path of FinegrainedMixedDtypeGemmLayer (S/layers/nvidia/finegrained_mixed_dtype_gemm_layer.cpp:15-183) over
+ * FinegrainedMixedDtypeGemmWrapper (K/gemm/finegrained_mixed_dtype_gemm/finegrained_mixed_dtype_gemm_wrapper.cpp).
+ *
+ * ksq_w4a8_repack_weight: src int8 [k, n/2], two's-complement nibbles, low nibble = even column - the tensor the
+ *   reference gives to PreprocessWeightsForMixedGemm (S/models/weight_method/w4a8_awq_method.cpp:176-181) - into
+ *   the 1 KiB fragment layout of the fp8 matrix instruction (n*k/2 bytes).  n % 16 == 0, k % 128 == 0.
+ *   ksq_w4a8_unpack_weight is its inverse (bit-exact round trip).
+ * ksq_w4a8_static_quant: q[m,k] = e4m3(x[m,k] / s), IEEE fp32 division, round to nearest even, saturating;
+ *   s = scale[0] (KSQ_W4A8_PER_TENSOR) or scale[channel] (KSQ_W4A8_PER_CHANNEL), fp32 in device memory; and
+ *   xsum[m, k/128] fp32 = the sum of each group of 128 quantized values, which the GEMM needs.  KSQ_W4A8_SUMS_ONLY
+ *   takes x that is e4m3 already and writes xsum only (q and scale unused).
+ *   Replaces StaticQuantizeE4M3PerTensor / PerChannel (wrapper.cpp:128-153 -> scaleMatrix,
+ *   K/others/tensorrt-llm/dev/common/cudaFp8Utils.cu:38-52).
+ * ksq_w4a8_gemm: a_q [m,k] e4m3 row-major, xsum [m,k/128], w_packed from ksq_w4a8_repack_weight, scales fp16
+ *   [k/128, n] as the reference holds them (weight_scale / weight_scale_2), alpha = input_scale * weight_scale_2.
+ *   Replaces FinegrainedMixedDtypeGemmWrapper::Forward (wrapper.cpp:68-100); no tactic argument: the kernel is
+ *   chosen from the shape.
+ * ------------------------------------------------------------------------------------------------------------------ */
+enum { KSQ_W4A8_PER_TENSOR = 0, KSQ_W4A8_PER_CHANNEL = 1, KSQ_W4A8_SUMS_ONLY = 2 };
+size_t ksq_w4a8_packed_weight_bytes(size_t n, size_t k);
+int ksq_w4a8_repack_weight(const void* src, void* dst_packed, size_t n, size_t k, void* stream);
+int ksq_w4a8_unpack_weight(const void* packed, void* dst, size_t n, size_t k, void* stream);
+int ksq_w4a8_static_quant(const void* x, const void* scale, void* q, void* xsum, size_t m, size_t k, int mode,
+                          int dtype, void* stream);
+size_t ksq_w4a8_workspace_size(size_t max_m, size_t n, size_t k);
+int ksq_w4a8_gemm(const void* a_q, const void* xsum, const void* w_packed, const void* scales, float alpha, void* out,
+                  size_t m, size_t n, size_t k, size_t group, int out_dtype, void* workspace, size_t workspace_bytes,
+                  void* stream);
+
+/* ------------------------------------------------------------------------------------------------------------------
  * MoE: expert-offset / permutation build, grouped W4A16 GEMM, silu*mul, top-k sum.
  * ------------------------------------------------------------------------------------------------------------------ */
 

@@ -10,6 +10,7 @@ SRC_GPTQ, SRC_AWQ, SRC_MOE_NK, SRC_INT4X2_KN = 0, 1, 2, 3
 SCALE_GN, SCALE_NG = 0, 1
 ZERO_AWQ_PACKED, ZERO_U8_GN = 0, 1
 KIND_W4A16, KIND_FP8_BLOCKWISE, KIND_MOE_W4A16 = 0, 1, 2
+W4A8_PER_TENSOR, W4A8_PER_CHANNEL, W4A8_SUMS_ONLY = 0, 1, 2
 
 c_sz = ctypes.c_size_t
 c_p = ctypes.c_void_p
@@ -61,6 +62,12 @@ SIGNATURES = {
     "ksq_moe_grouped_topk": (c_i, [c_p, c_p, c_p, c_p, c_sz, c_sz, c_sz, c_sz, c_sz, c_i, c_i, ctypes.c_float, c_i, c_p]),
     "ksq_moe_silu_mul": (c_i, [c_p, c_p, c_sz, c_sz, c_i, c_p]),
     "ksq_moe_sum": (c_i, [c_p, c_p, c_sz, c_sz, c_sz, c_i, c_p]),
+    "ksq_w4a8_packed_weight_bytes": (c_sz, [c_sz, c_sz]),
+    "ksq_w4a8_repack_weight": (c_i, [c_p, c_p, c_sz, c_sz, c_p]),
+    "ksq_w4a8_unpack_weight": (c_i, [c_p, c_p, c_sz, c_sz, c_p]),
+    "ksq_w4a8_static_quant": (c_i, [c_p, c_p, c_p, c_p, c_sz, c_sz, c_i, c_i, c_p]),
+    "ksq_w4a8_workspace_size": (c_sz, [c_sz, c_sz, c_sz]),
+    "ksq_w4a8_gemm": (c_i, [c_p, c_p, c_p, c_p, ctypes.c_float, c_p, c_sz, c_sz, c_sz, c_sz, c_i, c_p, c_sz, c_p]),
     "ksq_select_tile": (c_i, [c_i, c_sz, c_sz, c_sz, c_i, ctypes.POINTER(TileDesc)]),
 }
 

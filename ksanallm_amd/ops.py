@@ -358,3 +358,53 @@ def fp8_unpack_weight(packed):
     out = torch.empty_like(packed)
     _l.check(_lib.ksq_fp8_unpack_weight(_ptr(packed), _ptr(out), E, N, K, _stream()))
     return out
+
+
+# ----------------------------------------------------------------------------------------------- W4A8
+def w4a8_repack_weight(w):
+    """W4A8 weight [K, N/2] (int8/uint8, two's-complement nibbles, low nibble = even column: the input of the
+    reference's PreprocessWeightsForMixedGemm) -> the packed fragment layout ksq_w4a8_gemm reads."""
+    K, half = w.shape
+    out = torch.empty(_lib.ksq_w4a8_packed_weight_bytes(2 * half, K), dtype=torch.uint8, device=w.device)
+    _l.check(_lib.ksq_w4a8_repack_weight(_ptr(w), _ptr(out), 2 * half, K, _stream()))
+    return out
+
+
+def w4a8_unpack_weight(packed, K, N):
+    """Inverse of :func:`w4a8_repack_weight`: uint8 [K, N/2]."""
+    out = torch.empty((K, N // 2), dtype=torch.uint8, device=packed.device)
+    _l.check(_lib.ksq_w4a8_unpack_weight(_ptr(packed), _ptr(out), N, K, _stream()))
+    return out
+
+
+def w4a8_static_quant(x, scale, per_channel=False):
+    """StaticQuantizeE4M3PerTensor / PerChannel: x [m,k] T, scale fp32 [1] or [k] -> (codes uint8 [m,k], group sums
+    fp32 [m, k/128])."""
+    m, k = x.shape
+    q = torch.empty((m, k), dtype=torch.uint8, device=x.device)
+    xsum = torch.empty((m, k // 128), dtype=torch.float32, device=x.device)
+    mode = _l.W4A8_PER_CHANNEL if per_channel else _l.W4A8_PER_TENSOR
+    _l.check(_lib.ksq_w4a8_static_quant(_ptr(x), _ptr(scale), _ptr(q), _ptr(xsum), m, k, mode, _dt(x), _stream()))
+    return q, xsum
+
+
+def w4a8_group_sums(a_q):
+    """Group sums of activations that are e4m3 already (uint8 [m,k]) -> fp32 [m, k/128]."""
+    m, k = a_q.shape
+    xsum = torch.empty((m, k // 128), dtype=torch.float32, device=a_q.device)
+    _l.check(_lib.ksq_w4a8_static_quant(_ptr(a_q), None, None, _ptr(xsum), m, k, _l.W4A8_SUMS_ONLY, F16, _stream()))
+    return xsum
+
+
+def w4a8_gemm(a_q, xsum, w_packed, scales, alpha, n, out_dtype=torch.bfloat16, out=None, workspace=None):
+    """FinegrainedMixedDtypeGemmWrapper::Forward: a_q [m,k] e4m3 bytes, scales fp16 [k/128, n]."""
+    m, k = a_q.shape
+    if out is None:
+        out = torch.empty((m, n), dtype=out_dtype, device=a_q.device)
+    if workspace is None:
+        need = _lib.ksq_w4a8_workspace_size(m, n, k)
+        workspace = torch.empty(max(need, 1), dtype=torch.uint8, device=a_q.device)
+    assert scales.dtype == torch.float16
+    _l.check(_lib.ksq_w4a8_gemm(_ptr(a_q), _ptr(xsum), _ptr(w_packed), _ptr(scales), float(alpha), _ptr(out), m, n, k,
+                                128, _dt(out), _ptr(workspace), workspace.numel(), _stream()))
+    return out

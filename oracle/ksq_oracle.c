@@ -31,6 +31,12 @@
  *                                     host implementation compiled from the reference tree (oracle/_ref)
  *   fp8_channel_quant ............... torch float8_e4m3fn conversion, every rounding boundary
  *   fp8_tensor_gemm ................. torch fp32 matmul of the decoded operands
+ *   w4a8_unpack_int4 ................ hand-written known answers of the sign-extending nibble split
+ *                                     (K/others/tensorrt-llm/dev/thop/finegrained_mixed_dtype_gemm_thop_test.cu:53-80)
+ *   w4a8_static_quant ............... torch float8_e4m3fn conversion of the fp32 quotient
+ *   w4a8_group_sums ................. numpy float64 sums of the decoded values
+ *   w4a8_gemm ....................... torch float64 matmul of the reference test's own formula
+ *                                     (finegrained_mixed_dtype_gemm_thop_test.cu:186-206) on the decoded operands
  */
 #include <math.h>
 #include <stdint.h>
@@ -777,4 +783,68 @@ KSQO_API void ksqo_moe_sum(const void* in, void* out, size_t tokens, size_t topk
       for (size_t j = 0; j < topk; ++j) acc = round_t(acc + load_t(in, (t * topk + j) * d + i, dtype), dtype);
       store_t(out, t * d + i, acc, dtype);
     }
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * W4A8 (FinegrainedMixedDtypeGemmLayer)
+ * ---------------------------------------------------------------------------------------------- */
+
+/* [K, N/2] packed bytes -> [K, N] int8: low nibble = even column, both sign-extended
+ * (finegrained_mixed_dtype_gemm_thop_test.cu:53-80). */
+KSQO_API void ksqo_w4a8_unpack_int4(const int8_t* w, int8_t* out, size_t K, size_t N) {
+  for (size_t i = 0; i < K * (N / 2); ++i) {
+    const int8_t b = w[i];
+    out[2 * i] = (int8_t)((int8_t)(b << 4) >> 4);
+    out[2 * i + 1] = (int8_t)(b >> 4);
+  }
+}
+
+/* q[i] = e4m3(float(x[i]) / scale), scale = scale[0] or scale[i % k]: scaleMatrix<PER_TENSOR | PER_CHANNEL, true>
+ * (K/others/tensorrt-llm/dev/common/cudaFp8Utils.cu:33-52); the conversion saturates to +-448 (__nv_fp8_e4m3). */
+KSQO_API void ksqo_w4a8_static_quant(const void* x, const float* scale, uint8_t* q, size_t m, size_t k, int per_channel,
+                                     int dtype) {
+  for (size_t i = 0; i < m * k; ++i) {
+    volatile float sc = per_channel ? scale[i % k] : scale[0];
+    volatile float r = load_t(x, i, dtype) / sc;
+    q[i] = ksqo_f32_to_e4m3(fminf(fmaxf(r, -448.0f), 448.0f));
+  }
+}
+
+/* xsum[m, g] = sum of the 128 decoded e4m3 values of group g (in double, rounded once). */
+KSQO_API void ksqo_w4a8_group_sums(const uint8_t* q, float* xsum, size_t m, size_t k) {
+  for (size_t i = 0; i < m; ++i)
+    for (size_t g = 0; g < k / 128; ++g) {
+      double acc = 0.0;
+      for (size_t j = 0; j < 128; ++j) acc += (double)ksqo_e4m3_to_f32(q[i * k + g * 128 + j]);
+      xsum[i * (k / 128) + g] = (float)acc;
+    }
+}
+
+/* out[m,n] = alpha * sum_k a[m,k] * (w[k,n] * scale[k/group, n]): the reference test's formula
+ * (finegrained_mixed_dtype_gemm_thop_test.cu:186-206: unpack, multiply by the repeated scales, matmul of the
+ * alpha-scaled activations), taken in double here so that the result is the exact value up to the last rounding.
+ * a [m,k] e4m3, w [k,n/2] packed int4 as above, scales fp16 [k/group, n]. */
+KSQO_API void ksqo_w4a8_gemm(const uint8_t* a, const int8_t* w, const uint16_t* scales, float alpha, float* out,
+                             size_t m, size_t n, size_t k, size_t group) {
+  float lut[256];
+  for (int i = 0; i < 256; ++i) lut[i] = ksqo_e4m3_to_f32((uint8_t)i);
+  double* wd = (double*)malloc(sizeof(double) * k * n);
+  for (size_t kk = 0; kk < k; ++kk)
+    for (size_t j = 0; j < n; ++j) {
+      const int8_t b = w[kk * (n / 2) + j / 2];
+      const int v = (j & 1) ? (b >> 4) : ((int8_t)(b << 4) >> 4);
+      wd[kk * n + j] = (double)v * (double)ksqo_f16_to_f32(scales[(kk / group) * n + j]);
+    }
+#pragma omp parallel for schedule(static)
+  for (size_t i = 0; i < m; ++i) {
+    double* acc = (double*)calloc(n, sizeof(double));
+    for (size_t kk = 0; kk < k; ++kk) {
+      const double av = (double)lut[a[i * k + kk]];
+      if (av == 0.0) continue;
+      for (size_t j = 0; j < n; ++j) acc[j] += av * wd[kk * n + j];
+    }
+    for (size_t j = 0; j < n; ++j) out[i * n + j] = (float)(acc[j] * (double)alpha);
+    free(acc);
+  }
+  free(wd);
 }

@@ -460,3 +460,59 @@ def fp8_repack_weight(w):
     # axes: e, nt, r(16), kb, q(4), h(2), byte(16)  ->  e, nt, kb, h, q, r, byte
     v = w3.reshape(E, N // 16, 16, K // 128, 4, 2, 16).transpose(0, 1, 3, 5, 4, 2, 6)
     return np.ascontiguousarray(v).reshape(shape)
+
+
+# ---------------------------------------------------------------- W4A8
+def w4a8_unpack_int4(w):
+    """[K, N/2] packed bytes -> [K, N] int8 (low nibble = even column, sign-extended)."""
+    w = _c(w, np.int8)
+    K, half = w.shape
+    out = np.empty((K, 2 * half), np.int8)
+    lib().ksqo_w4a8_unpack_int4(_p(w), _p(out), _sz(K), _sz(2 * half))
+    return out
+
+
+def w4a8_static_quant(x_bits, scale, per_channel, dtype):
+    x = _c(x_bits, _store_dt(dtype))
+    m, k = x.shape
+    s = _c(np.asarray(scale, np.float32).reshape(-1), np.float32)
+    assert s.size == (k if per_channel else 1)
+    q = np.empty((m, k), np.uint8)
+    lib().ksqo_w4a8_static_quant(_p(x), _p(s), _p(q), _sz(m), _sz(k), ctypes.c_int(int(per_channel)),
+                                 ctypes.c_int(dtype))
+    return q
+
+
+def w4a8_group_sums(q):
+    q = _c(q, np.uint8)
+    m, k = q.shape
+    out = np.empty((m, k // 128), np.float32)
+    lib().ksqo_w4a8_group_sums(_p(q), _p(out), _sz(m), _sz(k))
+    return out
+
+
+def w4a8_gemm(a_q, w, scales_f16_bits, alpha, group=128):
+    a = _c(a_q, np.uint8)
+    w = _c(w, np.int8)
+    s = _c(scales_f16_bits, np.uint16)
+    m, k = a.shape
+    n = 2 * w.shape[1]
+    assert w.shape[0] == k and s.shape == (k // group, n)
+    out = np.empty((m, n), np.float32)
+    lib().ksqo_w4a8_gemm(_p(a), _p(w), _p(s), ctypes.c_float(float(alpha)), _p(out), _sz(m), _sz(n), _sz(k),
+                         _sz(group))
+    return out
+
+
+def w4a8_repack_weight(w):
+    """Packed fragment layout of a W4A8 weight ([K, N/2] packed int4) as include/ksq.h defines it, returned as uint32
+    words: fragment (n/16, k/128) of 256 words; word 4*lane + i of lane = 16*((k%128)/32) + n%16 holds the codes
+    u = w + 8 of k%32 in [8i, 8i+8): nibble 2j = element j, nibble 2j+1 = element 4+j.  numpy index arithmetic (the
+    layout has no counterpart in the reference)."""
+    u = (w4a8_unpack_int4(w).astype(np.int32) + 8).astype(np.uint32)  # [K, N]
+    K, N = u.shape
+    # axes: kb, q(4), i(4), e(8), nt, r(16)  ->  nt, kb, q, r, i, e
+    v = u.reshape(K // 128, 4, 4, 8, N // 16, 16).transpose(4, 0, 1, 5, 2, 3)
+    pos = np.array([0, 2, 4, 6, 1, 3, 5, 7], np.uint32) * 4
+    words = (v << pos).sum(axis=-1, dtype=np.uint64).astype(np.uint32)
+    return np.ascontiguousarray(words).reshape(-1)
