@@ -133,6 +133,7 @@ class Tensor {
 
   // quantization side tensors, named as in the reference
   std::shared_ptr<Tensor> scales, zeros, g_idx, perm, input_scales, weight_scales, pre_quant_scales, input_alpha;
+  float alpha = 1.0f;  // W4A8: input_scale * weight_scale_2
 
   Tensor() = default;
   Tensor(MemoryLocation location, DataType dtype, const std::vector<size_t>& shape, int device_id,
@@ -193,6 +194,8 @@ class Context {
   int tp_;
   std::vector<Stream> compute_streams_;
 };
+
+struct BaseLayerParameters {};
 
 enum QuantMode {
   QUANT_NONE,

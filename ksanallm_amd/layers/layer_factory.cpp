@@ -1,6 +1,7 @@
 #include "layer_factory.h"
 
 #include "blockwise_matmul_layer.h"
+#include "finegrained_mixed_dtype_gemm_layer.h"
 #include "fp8_matmul_layer.h"
 #include "moe_layer.h"
 #include "marlin_moe_layer.h"
@@ -18,6 +19,8 @@ MatMulLayerFactory::MatMulLayerFactory(const ModelConfig& model_config, const Ru
       builder_map_[{TYPE_I4_GROUP, t, t, q, MARLIN_LINEAR_BACKEND}] = &MatMulLayerFactory::BuildLayer<MarlinMatMulLayer>;
       builder_map_[{TYPE_I4_GROUP, t, t, q, MACHETE_LINEAR_BACKEND}] = &MatMulLayerFactory::BuildLayer<MacheteMatMulLayer>;
     }
+    builder_map_[{TYPE_I4_GROUP, t, t, QUANT_W4A8_AWQ, CUTLASS_LINEAR_BACKEND}] =
+        &MatMulLayerFactory::BuildLayer<FinegrainedMixedDtypeGemmLayer>;
     builder_map_[{TYPE_FP8_E4M3, t, t, QUANT_BLOCK_FP8_E4M3, DEFAULT_LINEAR_BACKEND}] =
         &MatMulLayerFactory::BuildLayer<BlockwiseMatMulLayer>;
     builder_map_[{TYPE_FP8_E4M3, t, t, QUANT_FP8_E4M3, DEFAULT_LINEAR_BACKEND}] = &MatMulLayerFactory::BuildLayer<Fp8MatMulLayer>;

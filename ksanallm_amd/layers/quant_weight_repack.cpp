@@ -100,4 +100,19 @@ Tensor PackFp8Weight(const Tensor& weight, int rank, hipStream_t stream) {
   return packed;
 }
 
+Tensor PackW4A8Weight(const Tensor& weight, int rank, hipStream_t stream) {
+  const char* who = "PackW4A8Weight";
+  if (weight.shape.size() != 2) KLLM_THROW("PackW4A8Weight: [K, N/2] expected");
+  if (GetTypeSize(weight.dtype) != 1) KLLM_THROW("PackW4A8Weight: one byte per two weights expected");
+  const size_t K = weight.shape[0], N = 2 * weight.shape[1];
+  Tensor packed(MemoryLocation::LOCATION_DEVICE, weight.dtype, weight.shape, rank);
+  KsqCheck(ksq_w4a8_repack_weight(weight.GetPtr<void>(), packed.GetPtr<void>(), N, K, stream), who);
+  packed.input_scales = weight.input_scales;
+  packed.weight_scales = weight.weight_scales;
+  packed.pre_quant_scales = weight.pre_quant_scales;
+  packed.input_alpha = weight.input_alpha;
+  packed.alpha = weight.alpha;
+  return packed;
+}
+
 }  // namespace ksana_llm

@@ -35,4 +35,10 @@ Tensor PackGptqExpertWeight(const Tensor& qweight, const Tensor& scales, size_t 
 // Stands where the reference binds the scales of FP8 weights after loading (quant_weight.cpp:817-861).
 Tensor PackFp8Weight(const Tensor& weight, int rank, hipStream_t stream);
 
+// W4A8 weight as the reference holds it before PreprocessWeightsForMixedGemm
+// (src/ksana_llm/models/weight_method/w4a8_awq_method.cpp:158-181): [K, N/2] bytes, two's-complement nibbles, low
+// nibble = even column -> the packed fragment layout FinegrainedMixedDtypeGemmLayer consumes.  The tensor keeps its
+// shape; input_scales, weight_scales, pre_quant_scales and alpha are carried over.
+Tensor PackW4A8Weight(const Tensor& weight, int rank, hipStream_t stream);
+
 }  // namespace ksana_llm

@@ -20,6 +20,7 @@
 
 #include "blockwise_matmul_layer.h"
 #include "layer_factory.h"
+#include "finegrained_mixed_dtype_gemm_layer.h"
 #include "fp8_matmul_layer.h"
 #include "moe_layer.h"
 #include "marlin_moe_layer.h"
@@ -175,6 +176,45 @@ static int RunFp8Tensor(int argc, char** argv) {
   std::vector<std::any> params{rc.max_step_token_num, k};
   MatMulLayerFactory factory(mc, rc, 0, context);
   auto layer = factory.CreateLayer(TYPE_FP8_E4M3, T, T, params, QUANT_FP8_E4M3, DEFAULT_LINEAR_BACKEND);
+  Tensor x = Upload(dir + "/x.bin", T, {m, k});
+  std::vector<Tensor> outputs{Tensor(MemoryLocation::LOCATION_DEVICE, T, {m, n}, 0)};
+  Drive(layer, mc, rc, {x, weight}, outputs);
+  HIP_OK(hipStreamSynchronize(stream));
+  Download(outputs[0], dir + "/y.bin");
+  return 0;
+}
+
+// w4a8 <dir> <f16|bf16> <m> <n> <k> <per_channel> <alpha>
+static int RunW4A8(int argc, char** argv) {
+  if (argc < 9) return 2;
+  const std::string dir = argv[2];
+  const DataType T = ParseT(argv[3]);
+  const size_t m = std::atol(argv[4]), n = std::atol(argv[5]), k = std::atol(argv[6]);
+  const bool per_channel = std::atoi(argv[7]) != 0;
+  const float alpha = static_cast<float>(std::atof(argv[8]));
+  hipStream_t stream;
+  HIP_OK(hipStreamCreate(&stream));
+  auto context = std::make_shared<Context>(1, stream);
+  ModelConfig mc;
+  RuntimeConfig rc;
+  rc.inter_data_type = T;
+  rc.max_step_token_num = m;
+  Tensor loaded = Upload(dir + "/w.bin", TYPE_INT8, {k, n / 2});
+  loaded.weight_scales = std::make_shared<Tensor>(Upload(dir + "/w_scale.bin", TYPE_FP16, {k / 128, n}));
+  loaded.input_scales = std::make_shared<Tensor>(Upload(dir + "/in_scale.bin", TYPE_FP32, {1}));
+  if (per_channel) loaded.pre_quant_scales = std::make_shared<Tensor>(Upload(dir + "/pqs.bin", TYPE_FP32, {k}));
+  loaded.alpha = alpha;
+  Tensor weight = PackW4A8Weight(loaded, 0, stream);
+  FinegrainedMixedDtypeGemmLayerParameters param;
+  param.m = rc.max_step_token_num;
+  param.n = n;
+  param.k = k;
+  param.group_size = 128;
+  param.has_zero = false;
+  param.activation_type = TYPE_FP8_E4M3;
+  param.output_type = T;
+  MatMulLayerFactory factory(mc, rc, 0, context);
+  auto layer = factory.CreateLayer(TYPE_I4_GROUP, T, T, {param}, QUANT_W4A8_AWQ, CUTLASS_LINEAR_BACKEND);
   Tensor x = Upload(dir + "/x.bin", T, {m, k});
   std::vector<Tensor> outputs{Tensor(MemoryLocation::LOCATION_DEVICE, T, {m, n}, 0)};
   Drive(layer, mc, rc, {x, weight}, outputs);
@@ -422,6 +462,35 @@ static int RunErrors() {
     Tensor w(MemoryLocation::LOCATION_DEVICE, TYPE_FP8_E4M3, {64, 512}, 0, reinterpret_cast<void*>(0x1000));
     expect(throws([&] { layer.Forward({x, w}, out); }), "Forward without a workspace buffer throws");
   }
+  // w4a8: group size, zero points, activation type, shapes; forward without a workspace
+  {
+    FinegrainedMixedDtypeGemmLayerParameters good;
+    good.m = 64;
+    good.n = 256;
+    good.k = 512;
+    good.group_size = 128;
+    good.activation_type = TYPE_FP8_E4M3;
+    good.output_type = TYPE_BF16;
+    FinegrainedMixedDtypeGemmLayer ok;
+    expect(ok.Init({good}, rc, context, 0).OK(), "w4a8 init");
+    expect(ok.GetWorkspaceSize() >= 64 * 512 + 64 * 4 * 4, "w4a8 workspace holds the quantized activations and their group sums");
+    expect(ok.Preprocess(mc, rc).OK(), "w4a8 preprocess");
+    auto bad = [&](auto edit, const char* what) {
+      FinegrainedMixedDtypeGemmLayerParameters p = good;
+      edit(p);
+      FinegrainedMixedDtypeGemmLayer l;
+      expect(!l.Init({p}, rc, context, 0).OK(), what);
+    };
+    bad([](auto& p) { p.group_size = 64; }, "w4a8 rejects group size 64");
+    bad([](auto& p) { p.has_zero = true; }, "w4a8 rejects zero points");
+    bad([](auto& p) { p.activation_type = TYPE_FP16; }, "w4a8 rejects a 16-bit activation type");
+    bad([](auto& p) { p.k = 200; }, "w4a8 rejects k = 200");
+    bad([](auto& p) { p.output_type = TYPE_FP32; }, "w4a8 rejects fp32 output");
+    std::vector<Tensor> out{Tensor()};
+    Tensor x(MemoryLocation::LOCATION_DEVICE, TYPE_BF16, {16, 512}, 0, reinterpret_cast<void*>(0x1000));
+    Tensor w(MemoryLocation::LOCATION_DEVICE, TYPE_INT8, {512, 128}, 0, reinterpret_cast<void*>(0x1000));
+    expect(throws([&] { ok.Forward({x, w}, out); }), "w4a8 Forward without a workspace buffer throws");
+  }
   // marlin moe: fp16 only, 20 parameters
   {
     std::vector<std::any> p{MoeScaleNormMode::RE_NORM, size_t(8), size_t(8), size_t(256), size_t(128), size_t(2), size_t(1),
@@ -483,6 +552,7 @@ int main(int argc, char** argv) {
     if (mode == "moe") return RunMoe(argc, argv);
     if (mode == "moe_fp8") return RunMoeFp8(argc, argv);
     if (mode == "marlin_moe") return RunMarlinMoe(argc, argv);
+    if (mode == "w4a8") return RunW4A8(argc, argv);
     if (mode == "errors") return RunErrors();
   } catch (const std::exception& e) {
     std::fprintf(stderr, "exception: %s\n", e.what());

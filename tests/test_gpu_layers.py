@@ -204,3 +204,28 @@ def test_fp8_per_tensor_layer(tmp_path, oracle, dtype, m, n, k, static):
     xq, xs = oracle.fp8_channel_quant(H.bits_of(x).reshape(1, -1), dtype, scale=in_scale if static else None)
     ref = oracle.fp8_tensor_gemm(xq.reshape(m, k), xs[0], wq.reshape(n, k), ws[0])
     H.check_gemm(y, ref, dtype, "fp8 per-tensor layer")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,m,n,k,per_channel", [(H.BF16, 1, 512, 1024, 0), (H.F16, 77, 2304, 512, 1),
+                                                      (H.BF16, 300, 1024, 2048, 1), (H.F16, 20, 48, 128, 0)])
+def test_w4a8_layer(tmp_path, oracle, dtype, m, n, k, per_channel):
+    """FinegrainedMixedDtypeGemmLayer through the factory: static per-tensor scale, or the per-channel divisor
+    input_scale / pre_quant_scale the reference's loader prepares (w4a8_awq_method.cpp:193-200)."""
+    g = H.gen(9700 + m)
+    w = torch.randint(0, 256, (k, n // 2), generator=g, dtype=torch.uint8).numpy()
+    ws = (torch.rand((k // 128, n), generator=g) * 0.02 + 0.002).to(torch.float16)
+    x = torch.randn((m, k), generator=g).to(H.TORCH_DT[dtype])
+    in_scale = np.array([0.03], np.float32)
+    pqs = (in_scale[0] / (torch.rand(k, generator=g) * 1.5 + 0.5).numpy()).astype(np.float32)
+    alpha = float(np.float32(0.03 * 0.8))
+    w.tofile(tmp_path / "w.bin")
+    H.bits_of(ws).tofile(tmp_path / "w_scale.bin")
+    in_scale.tofile(tmp_path / "in_scale.bin")
+    pqs.tofile(tmp_path / "pqs.bin")
+    H.bits_of(x).tofile(tmp_path / "x.bin")
+    run_driver("w4a8", tmp_path, TNAME[dtype], m, n, k, per_channel, repr(alpha))
+    y = read_out(tmp_path / "y.bin", dtype, (m, n))
+    xq = oracle.w4a8_static_quant(H.bits_of(x), pqs if per_channel else in_scale, bool(per_channel), dtype)
+    ref = oracle.w4a8_gemm(xq, w.view(np.int8), H.bits_of(ws), alpha)
+    H.check_gemm(y, ref, dtype, "w4a8 layer")
