@@ -181,11 +181,12 @@ int ksq_fp8_tensor_gemm(const void* a_q, const void* a_scale, const void* b, con
  *   ksq_w4a8_unpack_weight is its inverse (bit-exact round trip).
  * ksq_w4a8_static_quant: q[m,k] = e4m3(x[m,k] / s), IEEE fp32 division, round to nearest even, saturating;
  *   s = scale[0] (KSQ_W4A8_PER_TENSOR) or scale[channel] (KSQ_W4A8_PER_CHANNEL), fp32 in device memory; and
- *   xsum[m, k/128] fp32 = the sum of each group of 128 quantized values, which the GEMM needs.  KSQ_W4A8_SUMS_ONLY
+ *   xsum[k/128, m] fp32 (group-major, tokens contiguous) = the sum of each group of 128 quantized values, which
+ *   the GEMM needs.  KSQ_W4A8_SUMS_ONLY
  *   takes x that is e4m3 already and writes xsum only (q and scale unused).
  *   Replaces StaticQuantizeE4M3PerTensor / PerChannel (wrapper.cpp:128-153 -> scaleMatrix,
  *   K/others/tensorrt-llm/dev/common/cudaFp8Utils.cu:38-52).
- * ksq_w4a8_gemm: a_q [m,k] e4m3 row-major, xsum [m,k/128], w_packed from ksq_w4a8_repack_weight, scales fp16
+ * ksq_w4a8_gemm: a_q [m,k] e4m3 row-major, xsum [k/128,m], w_packed from ksq_w4a8_repack_weight, scales fp16
  *   [k/128, n] as the reference holds them (weight_scale / weight_scale_2), alpha = input_scale * weight_scale_2.
  *   Replaces FinegrainedMixedDtypeGemmWrapper::Forward (wrapper.cpp:68-100); no tactic argument: the kernel is
  *   chosen from the shape.

@@ -12,7 +12,12 @@
 // Packed weight layout: a fragment of 16 weight columns x 128 k is 1 KiB, 16 bytes per lane in lane order; lane l
 // (column l % 16, quarter q = l / 16) holds dwords P0..P3, nibble 2j of Pi = u(k = 32q + 8i + j), nibble 2j+1 of
 // Pi = u(k = 32q + 8i + 4 + j), j = 0..3.  Fragment (strip, kb) lies at (strip * K/128 + kb) * 1024 bytes.
+#include <atomic>
+
 #include "ksq_common.h"
+#include "splitk_reduce.h"
+#include "tile_select.h"
+#include "w4a8_tile.h"
 
 namespace ksq {
 namespace {
@@ -84,7 +89,7 @@ __device__ __forceinline__ float sum8_e4m3(u32x2 q) {
 }
 
 // MODE 0: q = e4m3(x / scale[0]); MODE 1: q = e4m3(x / scale[channel]); MODE 2: x is e4m3 already (sums only).
-// IEEE fp32 division, round to nearest even, saturating.  xsum[row, g] = sum of the 128 quantized values of group g
+// IEEE fp32 division, round to nearest even, saturating.  xsum[g, row] = sum of the 128 quantized values of group g
 // (every e4m3 value is a multiple of 2^-9, so the fp32 sum is exact, in any order, while it stays below 2^15).
 // Grid: x = chunks of 256 * 8 channels, y/z = row; a group of 128 channels is 16 adjacent lanes.
 template <typename T, int MODE>
@@ -131,13 +136,13 @@ __global__ void __launch_bounds__(256) w4a8_quant_kernel(const void* __restrict_
   for (int off = 1; off < 16; off <<= 1) sum += __shfl_xor(sum, off, 16);
   if (!live) return;
   if (MODE != 2) *reinterpret_cast<u32x2*>(q + e0) = out;
-  if ((threadIdx.x & 15) == 0) xsum[static_cast<size_t>(t) * (k / 128) + col / 128] = sum;
+  if ((threadIdx.x & 15) == 0) xsum[static_cast<size_t>(col / 128) * m + t] = sum;
 }
 
 // ------------------------------------------------------------------------------------------------ GEMM
 struct W4A8Params {
   const uint8_t* a;      // [M, K] e4m3
-  const float* xsum;     // [M, K/128]
+  const float* xsum;     // [K/128, M]
   const uint8_t* w;      // packed fragments
   const uint16_t* sc;    // fp16 [K/128, N]
   void* out;             // [M, N]
@@ -185,7 +190,7 @@ __global__ void __launch_bounds__(WAVES * 64) w4a8_splitk_kernel(W4A8Params p) {
     uint32_t row = m0 + mt * 16 + lrow;
     row = row < p.M ? row : p.M - 1;  // rows past M repeat the last token; their results are not stored
     aptr[mt] = p.a + static_cast<size_t>(row) * p.K + lq * 32;
-    xsptr[mt] = p.xsum + static_cast<size_t>(row) * KB;
+    xsptr[mt] = p.xsum + row;
   }
 
   f32x4 acc[NT][MT];
@@ -216,7 +221,7 @@ __global__ void __launch_bounds__(WAVES * 64) w4a8_splitk_kernel(W4A8Params p) {
       const i32x4* ap = reinterpret_cast<const i32x4*>(aptr[mt] + static_cast<size_t>(kb) * 128);
       s.a0[mt] = ap[0];
       s.a1[mt] = ap[1];
-      s.xs[mt] = xsptr[mt][kb];
+      s.xs[mt] = xsptr[mt][static_cast<size_t>(kb) * p.M];
     }
   };
   auto compute_stage = [&](const Stage& s) {
@@ -286,6 +291,41 @@ int dispatch_splitk(const W4A8Params& p, hipStream_t s) {
   return fail(KSQ_ERR_UNSUPPORTED, "no w4a8 kernel for mt=%d nt=%d", mt, nt);
 }
 
+// Prefill regime: the MFMA tile kernel of w4a8_tile.h on the grid the blockwise-FP8 planner lays out (same tile
+// shapes, same instruction; a k-step is one 128-deep group).
+template <typename TO, int WM>
+int launch_tile(const W4A8Params& q, const TilePlan& plan, float* partial, hipStream_t s) {
+  constexpr int kLds = static_cast<int>(w4a8_tile_lds_bytes(WM));
+  static std::atomic<uint64_t> configured{0};
+  if (int rc = allow_dynamic_lds(configured, reinterpret_cast<const void*>(&w4a8_tile_kernel<TO, WM>), kLds)) return rc;
+  W4A8TileParams p{};
+  p.a = q.a;
+  p.xsum = q.xsum;
+  p.w = q.w;
+  p.sc = q.sc;
+  p.out = q.out;
+  p.partial = partial;
+  p.M = q.M;
+  p.N = q.N;
+  p.K = q.K;
+  p.tiles_m = plan.tiles_m;
+  p.tiles_n = plan.tiles_n;
+  p.main_items = plan.main_items;
+  p.splits = plan.splits;
+  p.kb_per_split = plan.kt_per_split;
+  p.alpha512 = q.alpha512;
+  w4a8_tile_kernel<TO, WM><<<plan.grid, 512, kLds, s>>>(p);
+  if (plan.splits > 1) {
+    const unsigned cut = plan.tiles_m * plan.tiles_n - plan.main_items;
+    splitk_reduce_kernel<TO, 32 * WM><<<cut * (4 * WM), 256, 0, s>>>(partial, static_cast<uint16_t*>(p.out), p.M, p.N,
+                                                                    p.tiles_m, p.tiles_n, p.main_items, p.splits);
+  }
+  return KSQ_OK;
+}
+
+// above two 16-token tiles the tile kernel takes over, as for blockwise FP8
+inline bool use_tile(size_t m) { return m > 32; }
+
 }  // namespace
 }  // namespace ksq
 
@@ -350,23 +390,30 @@ KSQ_EXPORT int ksq_w4a8_static_quant(const void* x, const void* scale, void* q, 
 }
 
 KSQ_EXPORT size_t ksq_w4a8_workspace_size(size_t max_m, size_t n, size_t k) {
-  (void)max_m; (void)n; (void)k;
-  return 0;
+  if (n == 0 || k == 0 || k % 128 != 0) return 0;
+  // only the split-K form of the tile kernel needs scratch (fp32 partial tiles); the plan is the same for all m of a
+  // band of 128 rows
+  size_t need = 0;
+  for (size_t band_end = 128; max_m > 32; band_end += 128) {
+    const size_t m = band_end < max_m ? band_end : max_m;
+    const TilePlan t = plan_fp8_tile(m, n, k);
+    need = t.workspace_bytes > need ? t.workspace_bytes : need;
+    if (m == max_m) break;
+  }
+  return need;
 }
 
 KSQ_EXPORT int ksq_w4a8_gemm(const void* a_q, const void* xsum, const void* w_packed, const void* scales, float alpha,
                              void* out, size_t m, size_t n, size_t k, size_t group, int out_dtype, void* workspace,
                              size_t workspace_bytes, void* stream) {
   const char* fn = "ksq_w4a8_gemm";
-  (void)workspace; (void)workspace_bytes;
   if (!a_q || !xsum || !w_packed || !scales || !out) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: null pointer", fn);
   if (group != 128) return fail(KSQ_ERR_UNSUPPORTED, "%s: group size %zu (only 128)", fn, group);
   if (n == 0 || k == 0 || n % 16 != 0 || k % 128 != 0)
     return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: n must be a positive multiple of 16 and k of 128 (n=%zu k=%zu)", fn, n, k);
   if (out_dtype != KSQ_F16 && out_dtype != KSQ_BF16) return fail(KSQ_ERR_UNSUPPORTED, "%s: out dtype must be f16 or bf16", fn);
-  if (!aligned16(a_q) || !aligned16(w_packed) || (reinterpret_cast<uintptr_t>(scales) & 7u) ||
-      (reinterpret_cast<uintptr_t>(out) & 7u) || (reinterpret_cast<uintptr_t>(xsum) & 3u))
-    return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: misaligned pointer", fn);
+  if (!aligned16(a_q) || !aligned16(w_packed) || !aligned16(scales) || !aligned16(out) || !aligned16(xsum))
+    return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: every pointer must be 16-byte aligned", fn);
   if (m == 0) return KSQ_OK;
   if (m > 0x7fffffffull || n > 0x7fffffffull || k > 0x7fffffffull || div_up(m, 16) > 65535)
     return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: tensor too large", fn);
@@ -381,7 +428,21 @@ KSQ_EXPORT int ksq_w4a8_gemm(const void* a_q, const void* xsum, const void* w_pa
   p.K = static_cast<uint32_t>(k);
   p.alpha512 = alpha * 512.0f;
   hipStream_t st = as_stream(stream);
-  const int rc = out_dtype == KSQ_F16 ? dispatch_splitk<F16>(p, st) : dispatch_splitk<BF16>(p, st);
+  int rc;
+  if (use_tile(m)) {
+    const TilePlan plan = plan_fp8_tile(m, n, k);
+    if (plan.splits > 1 && (!workspace || workspace_bytes < plan.workspace_bytes || !aligned16(workspace)))
+      return fail(KSQ_ERR_WORKSPACE, "%s: m=%zu n=%zu k=%zu needs %zu bytes of 16-byte aligned workspace, got %zu", fn, m,
+                  n, k, plan.workspace_bytes, workspace ? workspace_bytes : size_t(0));
+    if (256 * k > 0xffffffffull || 16 * (k / 128) * 1024 > 0xffffffffull) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: k too large", fn);
+    float* partial = plan.splits > 1 ? static_cast<float*>(workspace) : nullptr;
+    if (plan.block_m == 128)
+      rc = out_dtype == KSQ_F16 ? launch_tile<F16, 4>(p, plan, partial, st) : launch_tile<BF16, 4>(p, plan, partial, st);
+    else
+      rc = out_dtype == KSQ_F16 ? launch_tile<F16, 8>(p, plan, partial, st) : launch_tile<BF16, 8>(p, plan, partial, st);
+  } else {
+    rc = out_dtype == KSQ_F16 ? dispatch_splitk<F16>(p, st) : dispatch_splitk<BF16>(p, st);
+  }
   if (rc != KSQ_OK) return rc;
   return check_launch(fn);
 }

@@ -379,19 +379,19 @@ def w4a8_unpack_weight(packed, K, N):
 
 def w4a8_static_quant(x, scale, per_channel=False):
     """StaticQuantizeE4M3PerTensor / PerChannel: x [m,k] T, scale fp32 [1] or [k] -> (codes uint8 [m,k], group sums
-    fp32 [m, k/128])."""
+    fp32 [k/128, m])."""
     m, k = x.shape
     q = torch.empty((m, k), dtype=torch.uint8, device=x.device)
-    xsum = torch.empty((m, k // 128), dtype=torch.float32, device=x.device)
+    xsum = torch.empty((k // 128, m), dtype=torch.float32, device=x.device)
     mode = _l.W4A8_PER_CHANNEL if per_channel else _l.W4A8_PER_TENSOR
     _l.check(_lib.ksq_w4a8_static_quant(_ptr(x), _ptr(scale), _ptr(q), _ptr(xsum), m, k, mode, _dt(x), _stream()))
     return q, xsum
 
 
 def w4a8_group_sums(a_q):
-    """Group sums of activations that are e4m3 already (uint8 [m,k]) -> fp32 [m, k/128]."""
+    """Group sums of activations that are e4m3 already (uint8 [m,k]) -> fp32 [k/128, m]."""
     m, k = a_q.shape
-    xsum = torch.empty((m, k // 128), dtype=torch.float32, device=a_q.device)
+    xsum = torch.empty((k // 128, m), dtype=torch.float32, device=a_q.device)
     _l.check(_lib.ksq_w4a8_static_quant(_ptr(a_q), None, None, _ptr(xsum), m, k, _l.W4A8_SUMS_ONLY, F16, _stream()))
     return xsum
 

@@ -55,9 +55,9 @@ def test_static_quant_bit_exact(ops, oracle, dtype, per_channel, m, k):
     q, xsum = ops.w4a8_static_quant(x.cuda(), scale.cuda(), per_channel)
     ref = oracle.w4a8_static_quant(H.bits_of(x), scale.numpy(), per_channel, dtype)
     np.testing.assert_array_equal(q.cpu().numpy(), ref)
-    np.testing.assert_array_equal(xsum.cpu().numpy(), oracle.w4a8_group_sums(ref))
+    np.testing.assert_array_equal(xsum.cpu().numpy().T, oracle.w4a8_group_sums(ref))
     # sums of activations that are quantized already
-    np.testing.assert_array_equal(ops.w4a8_group_sums(q).cpu().numpy(), oracle.w4a8_group_sums(ref))
+    np.testing.assert_array_equal(ops.w4a8_group_sums(q).cpu().numpy().T, oracle.w4a8_group_sums(ref))
 
 
 def test_static_quant_boundaries_and_specials(ops, oracle):
@@ -85,10 +85,10 @@ def test_static_quant_boundaries_and_specials(ops, oracle):
 
 
 @pytest.mark.parametrize("out_dtype", [H.F16, H.BF16])
-@pytest.mark.parametrize("m", [1, 8, 16, 17, 32, 33, 100])
+@pytest.mark.parametrize("m", [1, 8, 16, 17, 32, 33, 100, 256])
 @pytest.mark.parametrize("n,k", [(2048, 1024), (16, 128), (5120, 5120), (48, 640)])
 def test_gemm(ops, oracle, out_dtype, m, n, k):
-    if (n, k) == (5120, 5120) and m not in (1, 17, 100):
+    if (n, k) == (5120, 5120) and m not in (1, 17, 100, 256):
         pytest.skip("large shape at three token counts")
     w, scales = make_weight(n * 3 + k, k, n)
     x = make_act(m + n + k, m, k, H.BF16)
@@ -99,6 +99,73 @@ def test_gemm(ops, oracle, out_dtype, m, n, k):
     out = ops.w4a8_gemm(xq, xsum, wp, scales.cuda(), alpha, n, H.TORCH_DT[out_dtype])
     ref = oracle.w4a8_gemm(xq.cpu().numpy(), w.numpy().view(np.int8), H.bits_of(scales), alpha)
     H.check_gemm(out, ref, out_dtype, "w4a8 m=%d n=%d k=%d" % (m, n, k))
+
+
+@pytest.mark.parametrize("m,n,k", [
+    (64, 256, 8192),     # a grid far smaller than the chip: cut along K, partial tiles through the workspace
+    (33, 48, 128),       # one k-block, one short column tile
+    (130, 2064, 1024),   # N not a multiple of the 256-column tile
+    (257, 512, 640),     # M not a multiple of 4: the per-lane form of the group-sum staging
+    (300, 1024, 1024),   # 128-token tiles with a half-empty last block
+    (1024, 1024, 2048),
+    (515, 13328, 512),
+])
+@pytest.mark.parametrize("out_dtype", [H.F16, H.BF16])
+def test_gemm_tile_kernel(ops, oracle, out_dtype, m, n, k):
+    w, scales = make_weight(n + k + m, k, n)
+    x = make_act(m * 3 + n, m, k, H.F16)
+    in_scale = torch.tensor([0.04], dtype=torch.float32)
+    alpha = 0.04 * 1.3
+    xq, xsum = ops.w4a8_static_quant(x.cuda(), in_scale.cuda(), False)
+    wp = ops.w4a8_repack_weight(w.cuda())
+    out = ops.w4a8_gemm(xq, xsum, wp, scales.cuda(), alpha, n, H.TORCH_DT[out_dtype])
+    ref = oracle.w4a8_gemm(xq.cpu().numpy(), w.numpy().view(np.int8), H.bits_of(scales), alpha)
+    H.check_gemm(out, ref, out_dtype, "w4a8 tile m=%d n=%d k=%d" % (m, n, k))
+
+
+def test_gemm_workspace_is_checked(ops):
+    from ksanallm_amd import lib as L
+    m, n, k = 64, 256, 8192
+    need = L.load().ksq_w4a8_workspace_size(m, n, k)
+    assert need > 0
+    w, scales = make_weight(1, k, n)
+    xq = torch.zeros((m, k), dtype=torch.uint8, device="cuda")
+    xsum = torch.zeros((k // 128, m), dtype=torch.float32, device="cuda")
+    wp = ops.w4a8_repack_weight(w.cuda())
+    with pytest.raises(L.KsqError) as e:
+        ops.w4a8_gemm(xq, xsum, wp, scales.cuda(), 1.0, n, workspace=torch.empty(256, dtype=torch.uint8, device="cuda"))
+    assert e.value.code == 3
+    out = ops.w4a8_gemm(xq, xsum, wp, scales.cuda(), 1.0, n)
+    assert torch.all(out == 0)
+
+
+def test_gemm_full_size_properties(ops):
+    """At the reference's own performance shape (n = 25600, k = 5120; finegrained_mixed_dtype_gemm_thop_test.cu:312-321)
+    with 4096 tokens, where the oracle would take minutes:
+      * the tile kernel agrees with the streaming kernel run on 32-token chunks of the same rows (same products and
+        fp32 partial sums per group, summed in another order: one unit in the last place of the output at most, plus
+        what reordering an fp32 sum of forty terms of magnitude ~10 can move, which matters for results near zero);
+      * permuting the tokens permutes the output rows bit for bit;
+      * zero activations give zeros."""
+    m, n, k = 4096, 25600, 5120
+    w, scales = make_weight(7, k, n)
+    x = make_act(8, m, k, H.BF16)
+    in_scale = torch.tensor([0.05], dtype=torch.float32)
+    xq, xsum = ops.w4a8_static_quant(x.cuda(), in_scale.cuda(), False)
+    wp = ops.w4a8_repack_weight(w.cuda())
+    sc = scales.cuda()
+    out = ops.w4a8_gemm(xq, xsum, wp, sc, 0.03, n)
+    for r0 in (0, 2016, 4064):
+        rows = slice(r0, r0 + 32)
+        part = ops.w4a8_gemm(xq[rows].contiguous(), xsum[:, rows].contiguous(), wp, sc, 0.03, n)
+        a, b = out[rows].float(), part.float()
+        ulp = torch.from_numpy(H.ulp(b.cpu().numpy(), H.BF16)).cuda()
+        assert bool(torch.all((a - b).abs() <= ulp + 5e-5)), "rows %d..: %g" % (r0, float((a - b).abs().max()))
+    perm = torch.randperm(m, generator=H.gen(9)).cuda()
+    out_p = ops.w4a8_gemm(xq[perm].contiguous(), xsum[:, perm].contiguous(), wp, sc, 0.03, n)
+    assert torch.equal(out_p, out[perm])
+    zq = torch.zeros_like(xq)
+    assert torch.all(ops.w4a8_gemm(zq, ops.w4a8_group_sums(zq), wp, sc, 0.03, n) == 0)
 
 
 def test_gemm_extreme_codes_and_sums(ops, oracle):
