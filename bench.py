@@ -168,6 +168,57 @@ def fp8_cases(ops, L, cfg, shapes, Ms):
     return cases, keep
 
 
+def w4a8_cases(ops, L, cfg, shapes, Ms):
+    """W4A8: static per-tensor e4m3 quantization of bf16 activations (with the group sums the GEMM needs), then int4
+    weights x e4m3 activations on the fp8 matrix instruction."""
+    dev = "cuda"
+    cases, keep = [], []
+    for si, (tag, N, K) in enumerate(shapes):
+        g = seeded(cfg, si)
+        w = torch.randint(0, 256, (K, N // 2), generator=g, dtype=torch.uint8)
+        scales = (torch.rand((K // 128, N), generator=g) * 0.012 + 0.003).to(torch.float16)
+        wp1 = ops.w4a8_repack_weight(w.to(dev))
+        R = copies_needed(wp1.numel())
+        wps = [wp1] + [wp1.clone() for _ in range(R - 1)]
+        sc_d = scales.to(dev)
+        in_scale = torch.tensor([0.05], dtype=torch.float32, device=dev)
+        state = {"i": 0}
+        for mi, M in enumerate(Ms):
+            gx = seeded(cfg, 100 * si + mi + 10)
+            x = torch.randn((M, K), generator=gx)
+            x = torch.where(torch.rand((M, K), generator=gx) < 0.01, x * 20, x).to(torch.bfloat16).to(dev)
+            a_q = torch.empty((M, K), dtype=torch.uint8, device=dev)
+            xsum = torch.empty((K // 128, M), dtype=torch.float32, device=dev)
+            y = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+
+            def quant(x=x, a_q=a_q, xsum=xsum, M=M, K=K):
+                L.check(L.load().ksq_w4a8_static_quant(x.data_ptr(), in_scale.data_ptr(), a_q.data_ptr(), xsum.data_ptr(),
+                                                       M, K, L.W4A8_PER_TENSOR, L.BF16,
+                                                       torch.cuda.current_stream().cuda_stream))
+
+            need = L.load().ksq_w4a8_workspace_size(M, N, K)
+            ws = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
+
+            def gemm(a_q=a_q, xsum=xsum, y=y, wps=wps, sc_d=sc_d, state=state, R=R, ws=ws, N=N):
+                i = state["i"] = (state["i"] + 1) % R
+                ops.w4a8_gemm(a_q, xsum, wps[i], sc_d, 0.035, N, out=y, workspace=ws)
+
+            quant()
+            cases.append(Case("%s:quant:M=%d" % (tag, M), quant, 0, 2 * M * K + M * K + 4 * M * K // 128, "fp8",
+                              "w4a8_quant"))
+            nbytes = N * K // 2 + (K // 128) * N * 2 + M * K + 4 * M * K // 128 + 2 * M * N
+            if M <= 32:
+                nt = 4
+                while nt > 1 and (N % (16 * nt) or N // (16 * nt) < 128):
+                    nt //= 2
+                kern = "w4a8_splitk_kernel<%dx%d,w%d>" % (16 if M <= 16 else 32, 16 * nt, 8 if N // (16 * nt) < 256 else 4)
+            else:
+                d = L.select_tile(L.KIND_FP8_BLOCKWISE, M, N, K, L.BF16)   # the W4A8 tile kernel runs on this plan
+                kern = "w4a8_tile_kernel<%dx%d,w%d>" % (d["block_m"], d["block_n"], d["waves"])
+            cases.append(Case("%s:gemm:M=%d" % (tag, M), gemm, 2 * M * N * K, nbytes, "fp8", kern, R))
+    return cases, keep
+
+
 def moe_cases(ops, L, cfg, Ts, E=256, hidden=7168, inter=2048, topk=8, distinct=32):
     dev = "cuda"
     g = seeded(cfg, 0)
@@ -257,6 +308,10 @@ def build(cfg, ops, L):
     if cfg == 6:  # not one of the reference's five benchmark configurations: the block-fp8 expert path, same shapes as 5
         return ("DeepSeek-V3 MoE block-fp8 bf16 E=256 top-8 T in {1,64,512,4096}",) + moe_fp8_cases(
             ops, L, 6, [1, 64, 512, 4096]) + ("fp8",)
+    if cfg == 7:  # not one of the reference's five benchmark configurations: the W4A8 path on the shapes of the
+        # reference's own performance test (finegrained_mixed_dtype_gemm_thop_test.cu:312-321) plus decode and prefill
+        return ("W4A8 bf16 (5120x5120)+(25600x5120) M in {1,16,64,128,256,4096}",) + w4a8_cases(
+            ops, L, 7, [("sq", 5120, 5120), ("up", 25600, 5120)], [1, 16, 64, 128, 256, 4096]) + ("fp8",)
     raise SystemExit("unknown --config %d" % cfg)
 
 
@@ -339,7 +394,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--config", type=int, default=2, help="BASELINE.json config number 1..5 (default 2); 6 = block-fp8 MoE, same shapes as 5")
+    ap.add_argument("--config", type=int, default=2, help="BASELINE.json config number 1..5 (default 2); 6 = block-fp8 MoE, same shapes as 5; 7 = W4A8")
     ap.add_argument("--only", default="", help="substring filter on case names (for profiling one case)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-graph", action="store_true", help="launch every kernel from Python instead of replaying "

@@ -12,6 +12,7 @@
 // mantissa a 16-bit input can have.  The sign of x is put back afterwards (x = -0 would otherwise come out as +0).
 // Scales outside [2^-80, 2^100] take the division itself; inside, r is exact whenever |x / s| >= 2^-20, and a smaller
 // quotient that is one unit in the last place off still converts to the same signed zero.
+#include "exact_div.h"
 #include "ksq_common.h"
 
 namespace ksq {
@@ -27,21 +28,6 @@ __device__ __forceinline__ uint32_t cvt2_e4m3(float a, float b, uint32_t old, bo
   return hi ? static_cast<uint32_t>(__builtin_amdgcn_cvt_pk_fp8_f32(ca, cb, static_cast<int>(old), true))
             : static_cast<uint32_t>(__builtin_amdgcn_cvt_pk_fp8_f32(ca, cb, static_cast<int>(old), false));
 }
-
-// x / s, correctly rounded, for many x and one s (see the head of this file)
-struct ExactDiv {
-  float s, y;
-  bool fast;
-  __device__ __forceinline__ explicit ExactDiv(float scale)
-      : s(scale), y(1.0f / scale), fast(scale >= 0x1p-80f && scale <= 0x1p100f) {}
-  // |x| finite or NaN; an infinite x needs the caller's attention (r would be NaN)
-  __device__ __forceinline__ float operator()(float x) const {
-    if (!fast) return x / s;
-    const float q0 = x * y;
-    const float r = __builtin_fmaf(-q0, s, x);
-    return __builtin_copysignf(__builtin_fmaf(r, y, q0), x);
-  }
-};
 
 // two quotients that are known to lie within +-448 * (1 + 2^-23), or NaN: no clamp in front of the conversion
 __device__ __forceinline__ uint32_t cvt2_e4m3_in_range(float a, float b, uint32_t old, bool hi) {

@@ -14,6 +14,7 @@
 // Pi = u(k = 32q + 8i + 4 + j), j = 0..3.  Fragment (strip, kb) lies at (strip * K/128 + kb) * 1024 bytes.
 #include <atomic>
 
+#include "exact_div.h"
 #include "ksq_common.h"
 #include "splitk_reduce.h"
 #include "tile_select.h"
@@ -114,9 +115,11 @@ __global__ void __launch_bounds__(256) w4a8_quant_kernel(const void* __restrict_
       v[2 * j + 1] = T::hi_to_float(raw[j]);
     }
     if (MODE == 0) {
+      // one scale for all: the quotient from one reciprocal per lane (exact_div.h); an infinite input keeps the division
       const float s = scale[0];
+      const ExactDiv div(s);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) v[j] = v[j] / s;
+      for (int j = 0; j < 8; ++j) v[j] = __builtin_fabsf(v[j]) == __builtin_inff() ? v[j] / s : div(v[j]);
     } else {
       const f32x4 s0 = *reinterpret_cast<const f32x4*>(scale + col);
       const f32x4 s1 = *reinterpret_cast<const f32x4*>(scale + col + 4);
@@ -166,7 +169,7 @@ __device__ __forceinline__ i32x8 expand_u4(i32x4 p) {
 }
 
 // Streaming form (HBM-bound at few tokens): a workgroup owns NT strips of 16 weight columns and MT*16 tokens;
-// wavefront w takes the k-blocks w, w+WAVES, ... with LOOK of them in flight in a register ring.  Blocks past the end
+// wavefront w takes the k-blocks w, w+WAVES, ... with LOOK of them loaded ahead into registers.  Blocks past the end
 // are clamped to the last one and given zero scales, so that control flow stays uniform.  Partials are summed through
 // LDS in wavefront order.
 template <typename TO, int MT, int NT, int WAVES, int LOOK>
@@ -278,17 +281,29 @@ __global__ void __launch_bounds__(WAVES * 64) w4a8_splitk_kernel(W4A8Params p) {
   }
 }
 
+// Measured on MI355X (n = 25600 and n = 5120 at k = 5120, 1 and 16 tokens): the loads of activations, scales and group
+// sums are as many as the weight loads of one strip, so a workgroup takes as many strips as still leave the chip half
+// covered with workgroups (four strips: 19.2 -> 14.1 us at n = 25600), with no register ring at all - fewer registers,
+// more resident wavefronts, and those hide the latency better than a ring does (a ring 2, 3 or 4 deep measured 6-15 %
+// slower each step).  Grids below one workgroup per CU split K over eight wavefronts instead of four (n = 5120:
+// 8.1 -> 6.1 us).
 template <typename TO>
 int dispatch_splitk(const W4A8Params& p, hipStream_t s) {
   const int mt = p.M <= 16 ? 1 : 2;
-  int nt = (p.M > 8 || p.K > p.N) ? 2 : 1;
-  if (p.N % (16 * nt) != 0) nt = 1;
-  const dim3 grid(p.N / (16 * nt), static_cast<unsigned>(div_up(p.M, 16 * mt)), 1);
-#define KSQ_CASE(MT_, NT_) \
-  if (mt == MT_ && nt == NT_) { w4a8_splitk_kernel<TO, MT_, NT_, 4, 2><<<grid, 256, 0, s>>>(p); return KSQ_OK; }
-  KSQ_CASE(1, 1) KSQ_CASE(1, 2) KSQ_CASE(2, 1) KSQ_CASE(2, 2)
+  int nt = 4;
+  while (nt > 1 && (p.N % (16 * nt) != 0 || p.N / (16 * nt) < 128)) nt /= 2;
+  const unsigned groups = p.N / (16 * nt);
+  const int waves = groups < 256 ? 8 : 4;
+  const dim3 grid(groups, static_cast<unsigned>(div_up(p.M, 16 * mt)), 1);
+#define KSQ_CASE(MT_, NT_, W_)                                                   \
+  if (mt == MT_ && nt == NT_ && waves == W_) {                                   \
+    w4a8_splitk_kernel<TO, MT_, NT_, W_, 1><<<grid, W_ * 64, 0, s>>>(p);         \
+    return KSQ_OK;                                                               \
+  }
+  KSQ_CASE(1, 1, 4) KSQ_CASE(1, 2, 4) KSQ_CASE(1, 4, 4) KSQ_CASE(2, 1, 4) KSQ_CASE(2, 2, 4) KSQ_CASE(2, 4, 4)
+  KSQ_CASE(1, 1, 8) KSQ_CASE(1, 2, 8) KSQ_CASE(1, 4, 8) KSQ_CASE(2, 1, 8) KSQ_CASE(2, 2, 8) KSQ_CASE(2, 4, 8)
 #undef KSQ_CASE
-  return fail(KSQ_ERR_UNSUPPORTED, "no w4a8 kernel for mt=%d nt=%d", mt, nt);
+  return fail(KSQ_ERR_UNSUPPORTED, "no w4a8 kernel for mt=%d nt=%d waves=%d", mt, nt, waves);
 }
 
 // Prefill regime: the MFMA tile kernel of w4a8_tile.h on the grid the blockwise-FP8 planner lays out (same tile
