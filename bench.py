@@ -44,6 +44,11 @@ MEASURED_TRAFFIC = {
     (4, "fp8_splitk_kernel<16x32,w4>"): 134280000,
     (4, "fp8_tile_kernel<128x256,w8>"): 176820000,
     (4, "fp8_tile_kernel<256x256,w8>"): 519390000,
+    (7, "w4a8_quant"): 12690000,
+    (7, "w4a8_splitk_kernel<16x32,w8>"): 14420000,
+    (7, "w4a8_splitk_kernel<16x64,w4>"): 68990000,
+    (7, "w4a8_tile_kernel<128x256,w8>"): 51450000,
+    (7, "w4a8_tile_kernel<256x256,w8>"): 116860000,
 }
 
 

@@ -92,13 +92,13 @@ __device__ __forceinline__ float sum8_e4m3(u32x2 q) {
 // MODE 0: q = e4m3(x / scale[0]); MODE 1: q = e4m3(x / scale[channel]); MODE 2: x is e4m3 already (sums only).
 // IEEE fp32 division, round to nearest even, saturating.  xsum[g, row] = sum of the 128 quantized values of group g
 // (every e4m3 value is a multiple of 2^-9, so the fp32 sum is exact, in any order, while it stays below 2^15).
-// Grid: x = chunks of 256 * 8 channels, y/z = row; a group of 128 channels is 16 adjacent lanes.
-template <typename T, int MODE>
-__global__ void __launch_bounds__(256) w4a8_quant_kernel(const void* __restrict__ xin, const float* __restrict__ scale,
+// Grid: x = chunks of BLOCK * 8 channels, y/z = row; a group of 128 channels is 16 adjacent lanes.
+template <typename T, int MODE, int BLOCK>
+__global__ void __launch_bounds__(BLOCK) w4a8_quant_kernel(const void* __restrict__ xin, const float* __restrict__ scale,
                                                          uint8_t* __restrict__ q, float* __restrict__ xsum, uint32_t m,
                                                          uint32_t k) {
   const uint32_t row = blockIdx.z * gridDim.y + blockIdx.y;
-  const uint32_t col0 = (blockIdx.x * 256 + threadIdx.x) * 8;
+  const uint32_t col0 = (blockIdx.x * BLOCK + threadIdx.x) * 8;
   const bool live = row < m && col0 < k;
   const uint32_t t = live ? row : 0;
   const uint32_t col = live ? col0 : 0;
@@ -390,17 +390,29 @@ KSQ_EXPORT int ksq_w4a8_static_quant(const void* x, const void* scale, void* q, 
   if (m == 0) return KSQ_OK;
   if (m > 0x7fffffffull || k > 0x7fffffffull) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: tensor too large", fn);
   const unsigned gy = static_cast<unsigned>(m < 32768 ? m : 32768);
-  const dim3 grid(static_cast<unsigned>(div_up(k, 2048)), gy, static_cast<unsigned>(div_up(m, gy)));
+  const unsigned gz = static_cast<unsigned>(div_up(m, gy));
   hipStream_t st = as_stream(stream);
   const float* sp = static_cast<const float*>(scale);
   uint8_t* qp = static_cast<uint8_t*>(q);
   float* xs = static_cast<float*>(xsum);
   const uint32_t mm = static_cast<uint32_t>(m), kk = static_cast<uint32_t>(k);
-  if (sums) w4a8_quant_kernel<F16, 2><<<grid, 256, 0, st>>>(x, nullptr, nullptr, xs, mm, kk);
-  else if (dtype == KSQ_F16 && mode == KSQ_W4A8_PER_TENSOR) w4a8_quant_kernel<F16, 0><<<grid, 256, 0, st>>>(x, sp, qp, xs, mm, kk);
-  else if (dtype == KSQ_F16) w4a8_quant_kernel<F16, 1><<<grid, 256, 0, st>>>(x, sp, qp, xs, mm, kk);
-  else if (mode == KSQ_W4A8_PER_TENSOR) w4a8_quant_kernel<BF16, 0><<<grid, 256, 0, st>>>(x, sp, qp, xs, mm, kk);
-  else w4a8_quant_kernel<BF16, 1><<<grid, 256, 0, st>>>(x, sp, qp, xs, mm, kk);
+  // the largest block whose chunks tile a row without idle lanes (k is a multiple of 128 = 16 lanes)
+  const int block = k % 2048 == 0 ? 256 : (k % 1024 == 0 ? 128 : (k % 512 == 0 || k < 2048 ? 64 : 256));
+#define KSQ_Q(TT, MODE_, B_)                                                                                      \
+  w4a8_quant_kernel<TT, MODE_, B_><<<dim3(static_cast<unsigned>(div_up(k, B_ * 8)), gy, gz), B_, 0, st>>>(x, sp, qp, xs, mm, kk)
+#define KSQ_QB(TT, MODE_)                        \
+  do {                                           \
+    if (block == 256) KSQ_Q(TT, MODE_, 256);     \
+    else if (block == 128) KSQ_Q(TT, MODE_, 128);\
+    else KSQ_Q(TT, MODE_, 64);                   \
+  } while (0)
+  if (mode == KSQ_W4A8_SUMS_ONLY) KSQ_QB(F16, 2);
+  else if (dtype == KSQ_F16 && mode == KSQ_W4A8_PER_TENSOR) KSQ_QB(F16, 0);
+  else if (dtype == KSQ_F16) KSQ_QB(F16, 1);
+  else if (mode == KSQ_W4A8_PER_TENSOR) KSQ_QB(BF16, 0);
+  else KSQ_QB(BF16, 1);
+#undef KSQ_QB
+#undef KSQ_Q
   return check_launch(fn);
 }
 
