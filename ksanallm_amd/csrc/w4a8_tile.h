@@ -271,13 +271,17 @@ __global__ void __launch_bounds__(512, 1) w4a8_tile_kernel(W4A8TileParams p) {
     for (int t = 0; t < WN; ++t) wf[t] = w4a8_expand(*reinterpret_cast<const i32x4*>(wgt + t * WFRAG));
     __builtin_amdgcn_sched_barrier(0x4);
     f32x4 tmp[3];
+    f32x4 cv[2];  // the addend of a row tile, spread once over the four registers the instruction reads
+    cv[0] = f32x4{cs[0], cs[0], cs[0], cs[0]};
 #pragma unroll
     for (int j = 0; j < WM * WN + 2; ++j) {
       const int i = j / WN, t = j % WN;
       if (j < WM * WN) {
-        if (t == 0 && i + 1 < WM) af[(i + 1) & 1] = read_frag(act + (i + 1) * FRAG);
-        tmp[j % 3] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[t], af[i & 1], f32x4{cs[i], cs[i], cs[i], cs[i]}, 0,
-                                                                      0, 0, 0, 0, 0);
+        if (t == 0 && i + 1 < WM) {
+          af[(i + 1) & 1] = read_frag(act + (i + 1) * FRAG);
+          cv[(i + 1) & 1] = f32x4{cs[i + 1], cs[i + 1], cs[i + 1], cs[i + 1]};
+        }
+        tmp[j % 3] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[t], af[i & 1], cv[i & 1], 0, 0, 0, 0, 0, 0);
       }
       __builtin_amdgcn_sched_barrier(0x4);
       if (j >= 2) {  // the MFMA issued two places earlier has left the pipeline by now
