@@ -92,6 +92,14 @@ int ksq_w4a16_repack_act_order(const void* src_gptq, const void* perm, void* dst
 /* out[r, j] = x[r, perm[j]], x and out [m, k] T, perm int32 [k]; out must not alias x. */
 int ksq_permute_columns(const void* x, const void* perm, void* out, size_t m, size_t k, int dtype, void* stream);
 
+/* The same for expert stacks: out[s, j] = x[s / top_k, perm[topk_ids[s], j]] for the numel = tokens * top_k slots
+ * (top_k = 1: x holds one row per slot already, as in front of the second MoE GEMM); perm int32 [E, k], out [numel, k]
+ * T, read by the grouped GEMM with top_k = 1.  Ids outside [0, E) take expert 0's permutation; the grouped GEMM never
+ * reads those rows.  Replaces the perm / sorted-g_idx arguments of fused_marlin_moe
+ * (S/layers/nvidia/marlin_moe_layer.cpp:71-93). */
+int ksq_moe_permute_columns(const void* x, const void* perm, const void* topk_ids, void* out, size_t numel, size_t k,
+                            size_t top_k, size_t E, int dtype, void* stream);
+
 int ksq_w4a16_repack_scales(const void* src, int src_layout, void* dst_packed, size_t E, size_t K, size_t N,
                             size_t group, int dtype, void* stream);
 int ksq_w4a16_unpack_scales(const void* packed, int dst_layout, void* dst, size_t E, size_t K, size_t N, size_t group,

@@ -115,6 +115,27 @@ __global__ void __launch_bounds__(256) permute_columns_kernel(const uint16_t* __
   reinterpret_cast<uint32_t*>(out + r * k)[c / 2] = static_cast<uint32_t>(row[p0]) | (static_cast<uint32_t>(row[p1]) << 16);
 }
 
+// out[s, j] = x[s / top_k, perm[ids[s], j]]: the activation side of act-order for expert stacks, one row per
+// (token, slot); slots whose id is not an expert (masked out by an expert map) get row 0's permutation of expert 0 -
+// their rows are never read by the grouped GEMM
+__global__ void __launch_bounds__(256) moe_permute_columns_kernel(const uint16_t* __restrict__ x, const int32_t* __restrict__ perm,
+                                                                  const int32_t* __restrict__ ids, uint16_t* __restrict__ out,
+                                                                  size_t numel, uint32_t k, uint32_t top_k, uint32_t E) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;  // one thread per 2 output columns
+  const size_t per_row = k / 2;
+  if (i >= numel * per_row) return;
+  const size_t s = i / per_row;
+  const uint32_t c = static_cast<uint32_t>(i % per_row) * 2;
+  uint32_t e = static_cast<uint32_t>(ids[s]);
+  e = e < E ? e : 0;
+  const int32_t* pe = perm + static_cast<size_t>(e) * k;
+  uint32_t p0 = static_cast<uint32_t>(pe[c]), p1 = static_cast<uint32_t>(pe[c + 1]);
+  p0 = p0 < k ? p0 : k - 1;
+  p1 = p1 < k ? p1 : k - 1;
+  const uint16_t* row = x + (s / top_k) * k;
+  reinterpret_cast<uint32_t*>(out + s * k)[c / 2] = static_cast<uint32_t>(row[p0]) | (static_cast<uint32_t>(row[p1]) << 16);
+}
+
 // FP8 weights [E, N, K] (checkpoint, row-major) <-> 2 KiB fragments of 16 rows x 128 k, fragment (e, n/16, k/128) at
 // ((e*N/16 + n/16)*(K/128) + k/128): half h, then lane l = 16*((k%128)/32) + n%16, then the 16 bytes
 // k%32 in [16h, 16h+16) - the two 16-byte halves of the lane's operand of v_mfma_f32_16x16x128_f8f6f4.
@@ -333,6 +354,27 @@ KSQ_EXPORT int ksq_permute_columns(const void* x, const void* perm, void* out, s
   permute_columns_kernel<<<static_cast<unsigned>(blocks), 256, 0, as_stream(stream)>>>(
       static_cast<const uint16_t*>(x), static_cast<const int32_t*>(perm), static_cast<uint16_t*>(out), m,
       static_cast<uint32_t>(k));
+  return check_launch(fn);
+}
+
+KSQ_EXPORT int ksq_moe_permute_columns(const void* x, const void* perm, const void* topk_ids, void* out, size_t numel,
+                                       size_t k, size_t top_k, size_t E, int dtype, void* stream) {
+  const char* fn = "ksq_moe_permute_columns";
+  if (!x || !perm || !topk_ids || !out) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: null pointer", fn);
+  if ((reinterpret_cast<uintptr_t>(x) & 1u) || (reinterpret_cast<uintptr_t>(out) & 3u) ||
+      (reinterpret_cast<uintptr_t>(perm) & 3u) || (reinterpret_cast<uintptr_t>(topk_ids) & 3u))
+    return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: x must be 2-byte, out, perm and topk_ids 4-byte aligned", fn);
+  if (dtype != KSQ_F16 && dtype != KSQ_BF16) return fail(KSQ_ERR_UNSUPPORTED, "%s: dtype must be f16 or bf16", fn);
+  if (k == 0 || k % 2 != 0 || k > 0x7fffffffull) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: k must be positive and even", fn);
+  if (top_k == 0 || E == 0 || top_k > 0x7fffffffull || E > 0x7fffffffull)
+    return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: top_k and E must be positive", fn);
+  if (x == out) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: cannot permute in place", fn);
+  if (numel == 0) return KSQ_OK;
+  const size_t blocks = div_up(numel * (k / 2), 256);
+  if (blocks > 0x7fffffffull) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: tensor too large", fn);
+  moe_permute_columns_kernel<<<static_cast<unsigned>(blocks), 256, 0, as_stream(stream)>>>(
+      static_cast<const uint16_t*>(x), static_cast<const int32_t*>(perm), static_cast<const int32_t*>(topk_ids),
+      static_cast<uint16_t*>(out), numel, static_cast<uint32_t>(k), static_cast<uint32_t>(top_k), static_cast<uint32_t>(E));
   return check_launch(fn);
 }
 

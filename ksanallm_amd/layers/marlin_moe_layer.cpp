@@ -23,6 +23,7 @@ Status MarlinMoeLayer::Init(const std::vector<std::any>& parameters, const Runti
   p[18] = TYPE_UINT4x2;               // int_weight_dtype: 4-bit codes, two per byte
   if (runtime_config.inter_data_type != TYPE_FP16)
     return Status(RET_INVALID_ARGUMENT, "MarlinMoeLayer: only fp16 activations (marlin_moe_layer.cpp:96-99)");
+  reserve_act_order_ = true;  // g_idx / perm may come bound to the weights (marlin_moe_layer.cpp:71-81)
   return MoeLayer::Init(p, runtime_config, context, rank);
 }
 
@@ -36,8 +37,8 @@ Status MarlinMoeLayer::Forward(const std::vector<Tensor>& input_tensors, std::ve
     if (input_tensors[i].GetPtr<void>() == nullptr) KLLM_THROW("w1 or w2 is nullptr.");
     if (!input_tensors[i].scales || input_tensors[i].scales->GetPtr<void>() == nullptr)
       KLLM_THROW("w1_scales or w2_scales is nullptr.");
-    if (input_tensors[i].g_idx || input_tensors[i].perm)
-      KLLM_THROW("MarlinMoeLayer: act-order experts (g_idx / perm) are not built");
+    if (input_tensors[i].g_idx && !input_tensors[i].perm)
+      KLLM_THROW("MarlinMoeLayer: g_idx without perm: pack act-order experts with PackGptqExpertWeight");
     if (input_tensors[i].zeros) KLLM_THROW("MarlinMoeLayer: expert zero points are not built");
   }
   // hidden_states, gating_output, w1, w2 only: the router of this layer takes no bias and no expert map

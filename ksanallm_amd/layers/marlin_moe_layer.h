@@ -6,8 +6,8 @@
 // That is the sequence MoeLayer runs for int4 experts, on the same kernels; what differs is the interface: 20 init
 // parameters (no layer index), fp16 activations only, and no grouped / sigmoid routing.  The weights are the expert
 // stacks packed by PackMoeExpertWeight (where the reference holds Marlin tiles), with their scales bound.
-// Act-order experts (g_idx / perm bound to a weight) and zero points are rejected with a message: neither has a grouped
-// kernel here.
+// Act-order experts (perm bound to a weight by PackGptqExpertWeight) run with one extra pass per GEMM that gathers every
+// slot's activation row through its expert's permutation; zero points are rejected with a message.
 #pragma once
 
 #include "moe_layer.h"

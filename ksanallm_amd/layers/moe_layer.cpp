@@ -92,8 +92,10 @@ size_t MoeLayer::GetWorkspaceSize() {
   }
   cache3_size_ = AlignAddress(numel * expert_hidden_size_ * elem);
   cache13_size_ = std::max(cache1_size_, cache3_size_);  // cache1 is dead once silu*mul has run: cache3 reuses it
+  act_order1_size_ = reserve_act_order_ ? AlignAddress(numel * expert_hidden_size_ * elem) : 0;
+  act_order2_size_ = reserve_act_order_ ? AlignAddress(numel * expert_inter_size_ * elem) : 0;
   max_ws_bytes_ = topk_weights_size_ + topk_ids_size_ + fused_id_buffer_size_ + align_scratch_size_ + cache13_size_ +
-                  cache2_size_ + a1_size_;
+                  cache2_size_ + a1_size_ + act_order1_size_ + act_order2_size_;
   return max_ws_bytes_;
 }
 
@@ -134,6 +136,9 @@ Status MoeLayer::Forward(const std::vector<Tensor>& input_tensors, std::vector<T
   } else if (!input_tensors[2].scales || !input_tensors[3].scales) {
     KLLM_THROW("MoeLayer: expert weights have no scales bound");
   }
+  if ((input_tensors[2].perm || input_tensors[3].perm) && (IsFp8() || !reserve_act_order_)) {
+    KLLM_THROW("MoeLayer: act-order experts (perm bound to the weights) need the Marlin MoE layer");
+  }
 
   const int dtype = KsqDtype(inter_data_type_, "MoeLayer");
   const size_t elem = GetTypeSize(inter_data_type_);
@@ -154,6 +159,10 @@ Status MoeLayer::Forward(const std::vector<Tensor>& input_tensors, std::vector<T
   char* cache2 = p;
   p += cache2_size_;
   char* a1 = p;  // block-fp8 only
+  p += a1_size_;
+  char* act_order1 = p;  // act-order experts only
+  p += act_order1_size_;
+  char* act_order2 = p;
 
   const int gating_dtype = input_tensors[1].dtype == TYPE_FP32 ? KSQ_F32 : KsqDtype(input_tensors[1].dtype, "MoeLayer");
   const bool renormalize = norm_topk_prob_ || moe_scale_norm_mode_ == MoeScaleNormMode::RE_NORM;
@@ -215,21 +224,36 @@ Status MoeLayer::Forward(const std::vector<Tensor>& input_tensors, std::vector<T
       KsqCheck(ksq_moe_sum(cache3, out + begin * hidden_size * elem, tokens, topk, hidden_size, dtype, stream), "MoeLayer");
       continue;
     }
-    // gate_up: every (token, slot) row reads hidden[token]
+    // gate_up: every (token, slot) row reads hidden[token]; with act-order experts the row of a slot is gathered
+    // through its expert's permutation first (the weight rows lie in that order) and the GEMM reads it by slot
+    const void* gemm1_in = hidden + begin * hidden_size * elem;
+    size_t gemm1_topk = topk;
+    if (input_tensors[2].perm) {
+      KsqCheck(ksq_moe_permute_columns(gemm1_in, input_tensors[2].perm->GetPtr<void>(), ids, act_order1, numel, hidden_size,
+                                       topk, E, dtype, stream),
+               "MoeLayer");
+      gemm1_in = act_order1;
+      gemm1_topk = 1;
+    }
     if (block_m <= 32 && (2 * inter) % 32 == 0) {  // decode regime: the activation runs in the GEMM's epilogue
-      KsqCheck(ksq_moe_w4a16_gate_up_silu(cache2, hidden + begin * hidden_size * elem, w1, w1_scale, nullptr, sorted_ids,
-                                          expert_ids, num_post_pad, numel, topk, E, 2 * inter, hidden_size, group_size_,
-                                          block_m, dtype, stream),
+      KsqCheck(ksq_moe_w4a16_gate_up_silu(cache2, gemm1_in, w1, w1_scale, nullptr, sorted_ids, expert_ids, num_post_pad,
+                                          numel, gemm1_topk, E, 2 * inter, hidden_size, group_size_, block_m, dtype, stream),
                "MoeLayer");
     } else {
-      KsqCheck(ksq_moe_w4a16_gemm(cache1, hidden + begin * hidden_size * elem, w1, w1_scale, nullptr, nullptr, sorted_ids,
-                                  expert_ids, num_post_pad, numel, topk, E, 2 * inter, hidden_size, group_size_, block_m,
-                                  dtype, stream),
+      KsqCheck(ksq_moe_w4a16_gemm(cache1, gemm1_in, w1, w1_scale, nullptr, nullptr, sorted_ids, expert_ids, num_post_pad,
+                                  numel, gemm1_topk, E, 2 * inter, hidden_size, group_size_, block_m, dtype, stream),
                "MoeLayer");
       KsqCheck(ksq_moe_silu_mul(cache1, cache2, numel, inter, dtype, stream), "MoeLayer");
     }
     // down: row s reads cache2[s]; the routing weight is applied in the epilogue
-    KsqCheck(ksq_moe_w4a16_gemm(cache3, cache2, w2, w2_scale, nullptr, weights, sorted_ids, expert_ids, num_post_pad,
+    const void* gemm2_in = cache2;
+    if (input_tensors[3].perm) {
+      KsqCheck(ksq_moe_permute_columns(cache2, input_tensors[3].perm->GetPtr<void>(), ids, act_order2, numel, inter, 1, E,
+                                       dtype, stream),
+               "MoeLayer");
+      gemm2_in = act_order2;
+    }
+    KsqCheck(ksq_moe_w4a16_gemm(cache3, gemm2_in, w2, w2_scale, nullptr, weights, sorted_ids, expert_ids, num_post_pad,
                                 numel, 1, E, hidden_size, inter, group_size_, block_m, dtype, stream),
              "MoeLayer");
     KsqCheck(ksq_moe_sum(cache3, out + begin * hidden_size * elem, tokens, topk, hidden_size, dtype, stream), "MoeLayer");

@@ -40,6 +40,12 @@ class MoeLayer : public BaseLayer {
   }
   bool IsFp8() const { return compute_dtype_ == TYPE_BLOCK_FP8_E4M3; }
 
+ protected:
+  // act-order experts (weights with `perm` bound): the activation rows of every slot are gathered through its expert's
+  // permutation in front of each GEMM, into workspace that is reserved only when a derived layer asks for it before
+  // Init (MarlinMoeLayer does)
+  bool reserve_act_order_ = false;
+
  private:
   static constexpr size_t kChunk = 32 * 1024;
 
@@ -67,6 +73,7 @@ class MoeLayer : public BaseLayer {
   size_t topk_weights_size_ = 0, topk_ids_size_ = 0, fused_id_buffer_size_ = 0, align_scratch_size_ = 0;
   size_t cache1_size_ = 0, cache2_size_ = 0, cache3_size_ = 0, cache13_size_ = 0;
   size_t a1_q_size_ = 0, a1_size_ = 0, a2_q_size_ = 0;  // block-fp8: quantized activations
+  size_t act_order1_size_ = 0, act_order2_size_ = 0;
   size_t max_ws_bytes_ = 0;
 };
 

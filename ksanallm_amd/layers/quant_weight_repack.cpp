@@ -53,7 +53,8 @@ Tensor PackGroupQuantWeight(const Tensor& qweight, const Tensor& scales, const T
   return packed;
 }
 
-Tensor PackGptqExpertWeight(const Tensor& qweight, const Tensor& scales, size_t group_size, int rank, hipStream_t stream) {
+Tensor PackGptqExpertWeight(const Tensor& qweight, const Tensor& scales, size_t group_size, int rank, hipStream_t stream,
+                            const Tensor* g_idx) {
   const char* who = "PackGptqExpertWeight";
   if (qweight.shape.size() != 3 || scales.shape.size() != 3) KLLM_THROW("PackGptqExpertWeight: 3-D tensors expected");
   const size_t E = qweight.shape[0], K = qweight.shape[1] * 8, N = qweight.shape[2];
@@ -62,7 +63,40 @@ Tensor PackGptqExpertWeight(const Tensor& qweight, const Tensor& scales, size_t 
   }
   const int dtype = KsqDtype(scales.dtype, who);
   Tensor packed(MemoryLocation::LOCATION_DEVICE, TYPE_I4_GROUP, {E, K, N / 2}, rank);
-  KsqCheck(ksq_w4a16_repack(qweight.GetPtr<void>(), KSQ_SRC_GPTQ, packed.GetPtr<void>(), E, K, N, stream), who);
+  if (g_idx) {
+    // act-order: every expert has its own group index; its rows are sorted by group (stable), as MarlinSortGIdx and the
+    // perm form of gptq_marlin_repack do per expert, and the layer gathers the activation columns through `perm`
+    if (g_idx->GetElementNumber() != E * K) KLLM_THROW("PackGptqExpertWeight: g_idx must have E * K entries");
+    std::vector<int32_t> groups(E * K), perm(E * K), sorted(E * K);
+    if (hipStreamSynchronize(stream) != hipSuccess ||
+        hipMemcpy(groups.data(), g_idx->GetPtr<void>(), E * K * sizeof(int32_t), hipMemcpyDeviceToHost) != hipSuccess) {
+      KLLM_THROW("PackGptqExpertWeight: cannot read g_idx");
+    }
+    for (size_t e = 0; e < E; ++e) {
+      int32_t* pe = perm.data() + e * K;
+      const int32_t* ge = groups.data() + e * K;
+      for (size_t i = 0; i < K; ++i) pe[i] = static_cast<int32_t>(i);
+      std::stable_sort(pe, pe + K, [&](int32_t a, int32_t b) { return ge[a] < ge[b]; });
+      for (size_t i = 0; i < K; ++i) {
+        sorted[e * K + i] = ge[pe[i]];
+        if (sorted[e * K + i] != static_cast<int32_t>(i / group_size))
+          KLLM_THROW("PackGptqExpertWeight: g_idx does not hold group_size rows per group");
+      }
+    }
+    packed.perm = std::make_shared<Tensor>(MemoryLocation::LOCATION_DEVICE, TYPE_INT32, std::vector<size_t>{E, K}, rank);
+    packed.g_idx = std::make_shared<Tensor>(MemoryLocation::LOCATION_DEVICE, TYPE_INT32, std::vector<size_t>{E, K}, rank);
+    if (hipMemcpy(packed.perm->GetPtr<void>(), perm.data(), E * K * sizeof(int32_t), hipMemcpyHostToDevice) != hipSuccess ||
+        hipMemcpy(packed.g_idx->GetPtr<void>(), sorted.data(), E * K * sizeof(int32_t), hipMemcpyHostToDevice) != hipSuccess) {
+      KLLM_THROW("PackGptqExpertWeight: cannot upload perm");
+    }
+    for (size_t e = 0; e < E; ++e) {
+      KsqCheck(ksq_w4a16_repack_act_order(qweight.GetPtr<int32_t>() + e * (K / 8) * N, packed.perm->GetPtr<int32_t>() + e * K,
+                                          packed.GetPtr<char>() + e * (K * N / 2), K, N, stream),
+               who);
+    }
+  } else {
+    KsqCheck(ksq_w4a16_repack(qweight.GetPtr<void>(), KSQ_SRC_GPTQ, packed.GetPtr<void>(), E, K, N, stream), who);
+  }
   packed.scales = std::make_shared<Tensor>(MemoryLocation::LOCATION_DEVICE, scales.dtype, scales.shape, rank);
   KsqCheck(ksq_w4a16_repack_scales(scales.GetPtr<void>(), KSQ_SCALE_GN, packed.scales->GetPtr<void>(), E, K, N, group_size, dtype, stream), who);
   return packed;

@@ -25,9 +25,12 @@ Tensor PackGroupQuantWeight(const Tensor& qweight, const Tensor& scales, const T
 Tensor PackMoeExpertWeight(const Tensor& experts, const Tensor& scales, size_t group_size, int rank, hipStream_t stream);
 
 // GPTQ expert stack as the Marlin MoE loader holds it before its own repack: qweight [E, K/8, N] int32, scales
-// [E, K/group, N] in T (symmetric, no act-order).  Returns a TYPE_I4_GROUP tensor of logical shape {E, K, N/2} with
-// `scales` bound: the same packed tiles PackMoeExpertWeight produces, for MarlinMoeLayer.
-Tensor PackGptqExpertWeight(const Tensor& qweight, const Tensor& scales, size_t group_size, int rank, hipStream_t stream);
+// [E, K/group, N] in T (symmetric).  Returns a TYPE_I4_GROUP tensor of logical shape {E, K, N/2} with `scales` bound:
+// the same packed tiles PackMoeExpertWeight produces, for MarlinMoeLayer.  With g_idx (int32 [E, K], the checkpoint's
+// act-order group index of every expert) each expert's rows are sorted by group and `perm` / the sorted `g_idx`
+// ([E, K] each) are bound, as the reference binds them for fused_marlin_moe (S/layers/nvidia/marlin_moe_layer.cpp:71-81).
+Tensor PackGptqExpertWeight(const Tensor& qweight, const Tensor& scales, size_t group_size, int rank, hipStream_t stream,
+                            const Tensor* g_idx = nullptr);
 
 // FP8 (e4m3) weights, [N, K] or an expert stack [E, N, K] in checkpoint layout: returns the same shape and dtype in the
 // packed 2 KiB fragment layout every FP8 layer here consumes (BlockwiseMatMulLayer, Fp8MatMulLayer, MoeLayer with

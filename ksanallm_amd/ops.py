@@ -342,6 +342,17 @@ def permute_columns(x, perm, out=None):
     return out
 
 
+def moe_permute_columns(x, perm, topk_ids, top_k, out=None):
+    """out[s, j] = x[s // top_k, perm[topk_ids[s], j]]: x [rows, k], perm int32 [E, k], topk_ids int32 [numel]."""
+    k = x.shape[1]
+    numel = topk_ids.numel()
+    if out is None:
+        out = torch.empty((numel, k), dtype=x.dtype, device=x.device)
+    _l.check(_lib.ksq_moe_permute_columns(_ptr(x), _ptr(perm), _ptr(topk_ids), _ptr(out), numel, k, top_k, perm.shape[0],
+                                          _dt(x), _stream()))
+    return out
+
+
 def fp8_repack_weight(w):
     """Checkpoint-layout e4m3 weight [N, K] or [E, N, K] (uint8) -> the packed fragment layout the FP8 GEMMs read."""
     E = w.shape[0] if w.dim() == 3 else 1

@@ -516,3 +516,28 @@ def w4a8_repack_weight(w):
     pos = np.array([0, 2, 4, 6, 1, 3, 5, 7], np.uint32) * 4
     words = (v << pos).sum(axis=-1, dtype=np.uint64).astype(np.uint32)
     return np.ascontiguousarray(words).reshape(-1)
+
+
+def moe_act_order_forward(x_bits, codes13, s13_bits, g13, codes2, s2_bits, g2, topk_ids, topk_w, dtype):
+    """Int4 MoE block with act-order (desc_act) experts, by the definition of g_idx: row k of expert e belongs to
+    quantization group g[e, k], W_e[k, n] = (code[e, k, n] - 8) * scale[e, g[e, k], n] (codes [E, K, N] in checkpoint row
+    order, scales [E, K/group, N]).  The reference reaches the same products by sorting each expert's rows by group and
+    permuting the activations (S/layers/nvidia/marlin_moe_layer.cpp:71-93); this function does neither.  Rounding as in
+    moe_forward: GEMM1 -> T, silu*mul -> T, GEMM2 * routed weight -> T, sum over top-k in T.  numpy, for test sizes."""
+    ids = np.asarray(topk_ids)
+    tw = np.asarray(topk_w, np.float32)
+    T, topk = ids.shape
+    x = from_bits(np.asarray(x_bits), dtype).astype(np.float64)
+
+    def dense(codes, s_bits, g):
+        s = from_bits(np.asarray(s_bits), dtype).astype(np.float64)
+        E = codes.shape[0]
+        return [(np.asarray(codes[e]).astype(np.float64) - 8.0) * s[e][np.asarray(g[e]).astype(np.int64)] for e in range(E)]
+
+    w13, w2 = dense(codes13, s13_bits, g13), dense(codes2, s2_bits, g2)
+    c1 = np.stack([x[t] @ w13[ids[t, j]] for t in range(T) for j in range(topk)]).astype(np.float32)
+    c2b = silu_mul(to_bits(c1, dtype), dtype)
+    c2 = from_bits(c2b, dtype).astype(np.float64)
+    c3 = np.stack([(c2[t * topk + j] @ w2[ids[t, j]]).astype(np.float32) * tw[t, j]
+                   for t in range(T) for j in range(topk)]).astype(np.float32)
+    return moe_sum(to_bits(c3, dtype).reshape(T, topk, -1), dtype)

@@ -308,10 +308,19 @@ static int RunMarlinMoe(int argc, char** argv) {
   ModelConfig mc;
   RuntimeConfig rc;
   rc.inter_data_type = T;
+  // optional: act-order experts, g13.bin int32 [E, hidden] and g2.bin int32 [E, inter] (the checkpoints' g_idx)
+  const bool act_order = argc > 10 && std::atoi(argv[10]) != 0;
+  Tensor g13, g2;
+  if (act_order) {
+    g13 = Upload(dir + "/g13.bin", TYPE_INT32, {E, hidden});
+    g2 = Upload(dir + "/g2.bin", TYPE_INT32, {E, inter});
+  }
   Tensor w13 = PackGptqExpertWeight(Upload(dir + "/qw13.bin", TYPE_INT32, {E, hidden / 8, 2 * inter}),
-                                    Upload(dir + "/s13.bin", T, {E, hidden / 128, 2 * inter}), 128, 0, stream);
+                                    Upload(dir + "/s13.bin", T, {E, hidden / 128, 2 * inter}), 128, 0, stream,
+                                    act_order ? &g13 : nullptr);
   Tensor w2 = PackGptqExpertWeight(Upload(dir + "/qw2.bin", TYPE_INT32, {E, inter / 8, hidden}),
-                                   Upload(dir + "/s2.bin", T, {E, inter / 128, hidden}), 128, 0, stream);
+                                   Upload(dir + "/s2.bin", T, {E, inter / 128, hidden}), 128, 0, stream,
+                                   act_order ? &g2 : nullptr);
   HIP_OK(hipStreamSynchronize(stream));
   // the reference's 20 positional values (marlin_moe_layer.cpp:16-36); the routing fields are ignored by this layer
   std::vector<std::any> params{renorm ? MoeScaleNormMode::RE_NORM : MoeScaleNormMode::NO_NORM,
@@ -326,18 +335,19 @@ static int RunMarlinMoe(int argc, char** argv) {
   Drive(layer, mc, rc, {x, gating, w13, w2}, outputs);
   HIP_OK(hipStreamSynchronize(stream));
   Download(outputs[0], dir + "/y.bin");
-  // act-order experts are refused with a message, not run wrongly
-  Tensor w13_act = w13;
-  w13_act.perm = std::make_shared<Tensor>(MemoryLocation::LOCATION_DEVICE, TYPE_INT32, std::vector<size_t>{E, hidden}, 0);
+  // a group index without the permutation that goes with it is refused with a message, not run wrongly
+  Tensor w13_bad = w13;
+  w13_bad.perm = nullptr;
+  w13_bad.g_idx = std::make_shared<Tensor>(MemoryLocation::LOCATION_DEVICE, TYPE_INT32, std::vector<size_t>{E, hidden}, 0);
   bool threw = false;
   try {
-    std::vector<Tensor> in2{x, gating, w13_act, w2};
+    std::vector<Tensor> in2{x, gating, w13_bad, w2};
     layer->Forward(in2, outputs);
   } catch (const std::exception&) {
     threw = true;
   }
   if (!threw) {
-    std::fprintf(stderr, "FAILED: act-order experts were accepted\n");
+    std::fprintf(stderr, "FAILED: g_idx without perm was accepted\n");
     return 1;
   }
   return 0;

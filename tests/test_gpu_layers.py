@@ -159,6 +159,44 @@ def test_marlin_moe_layer(tmp_path, oracle, tokens, renorm):
     H.check_gemm(y, ref, dtype, "marlin moe layer", weights_rounded=rounded, rel_l2_max=5e-3 * (2 ** 0.5 if rounded else 1.0))
 
 
+def _act_order_experts(g, E, n, k, dtype):
+    """GPTQ act-order expert stack: codes [E, k, n] in checkpoint row order, words [E, k/8, n], scales [E, k/128, n],
+    g_idx [E, k] = a random assignment of the k rows to k/128 groups of 128 rows each."""
+    codes = torch.randint(0, 16, (E, k, n), generator=g, dtype=torch.uint8).numpy()
+    c = codes.reshape(E, k // 8, 8, n).astype(np.uint32)
+    words = np.zeros((E, k // 8, n), np.uint32)
+    for j in range(8):
+        words |= c[:, :, j, :] << np.uint32(4 * j)
+    scales = H.uniform(g, (E, k // 128, n), 0.002, 0.01, dtype)
+    g_idx = np.stack([(torch.randperm(k, generator=g).numpy() // 128) for _ in range(E)]).astype(np.int32)
+    return codes, words.view(np.int32), scales, g_idx
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("tokens,renorm", [(1, 0), (9, 1), (200, 1)])
+def test_marlin_moe_layer_act_order(tmp_path, oracle, tokens, renorm):
+    """Experts quantized with desc_act: every expert has its own g_idx.  The oracle applies the definition
+    (scale[g_idx[k]] per row), the layer sorts the rows at load time and gathers the activations per slot."""
+    E, hidden, inter, topk = 16, 256, 128, 4
+    dtype = H.F16
+    g = H.gen(9800 + tokens)
+    c13, qw13, s13, g13 = _act_order_experts(g, E, 2 * inter, hidden, dtype)
+    c2, qw2, s2, g2 = _act_order_experts(g, E, hidden, inter, dtype)
+    x = torch.randn((tokens, hidden), generator=g).to(H.TORCH_DT[dtype])
+    gating = torch.randn((tokens, E), generator=g).to(torch.float16)
+    for name, arr in (("qw13", qw13), ("qw2", qw2), ("s13", H.bits_of(s13)), ("s2", H.bits_of(s2)), ("g13", g13), ("g2", g2),
+                      ("x", H.bits_of(x)), ("gating", H.bits_of(gating))):
+        np.ascontiguousarray(arr).tofile(tmp_path / (name + ".bin"))
+    run_driver("marlin_moe", tmp_path, TNAME[dtype], tokens, E, hidden, inter, topk, renorm, 1)
+    y = read_out(tmp_path / "y.bin", dtype, (tokens, hidden))
+    tw, ids = oracle.moe_topk_softmax(H.bits_of(gating), topk, bool(renorm), 1.0, H.F16)
+    ref = oracle.from_bits(oracle.moe_act_order_forward(H.bits_of(x), c13, H.bits_of(s13), g13, c2, H.bits_of(s2), g2, ids, tw,
+                                                        dtype), dtype)
+    rounded = tokens * topk // E >= 40
+    H.check_gemm(y, ref, dtype, "marlin moe layer, act-order", weights_rounded=rounded,
+                 rel_l2_max=5e-3 * (2 ** 0.5 if rounded else 1.0))
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype,tokens,renorm,scaling", [(H.BF16, 1, 0, 2.5), (H.F16, 40, 1, 1.0), (H.BF16, 300, 1, 1.0)])
 def test_moe_layer_block_fp8(tmp_path, oracle, dtype, tokens, renorm, scaling):

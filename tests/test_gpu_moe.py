@@ -409,3 +409,21 @@ def test_moe_full_size_properties(ops, kind, T):
     yp = run(x[perm], ids[perm], tw[perm])
     torch.cuda.synchronize()
     assert torch.equal(yp.view(torch.int16), y[perm.cuda()].view(torch.int16))
+
+
+@pytest.mark.parametrize("dtype", [H.F16, H.BF16])
+@pytest.mark.parametrize("tokens,top_k,E,k", [(1, 4, 8, 128), (37, 2, 16, 384), (300, 8, 64, 2048)])
+def test_moe_permute_columns_bit_exact(ops, dtype, tokens, top_k, E, k):
+    """out[s, j] = x[s // top_k, perm[ids[s], j]] for the first MoE GEMM, and with top_k = 1 (one input row per slot)
+    for the second."""
+    g = H.gen(tokens + k)
+    x = torch.randn((tokens, k), generator=g).to(H.TORCH_DT[dtype])
+    perm = torch.stack([torch.randperm(k, generator=g) for _ in range(E)]).to(torch.int32)
+    ids = torch.randint(0, E, (tokens * top_k,), generator=g, dtype=torch.int32)
+    out = ops.moe_permute_columns(x.cuda(), perm.cuda(), ids.cuda(), top_k)
+    rows = torch.arange(tokens * top_k) // top_k
+    ref = torch.gather(x[rows], 1, perm[ids.long()].long())
+    assert torch.equal(out.cpu(), ref)
+    xs = torch.randn((tokens * top_k, k), generator=g).to(H.TORCH_DT[dtype])
+    out1 = ops.moe_permute_columns(xs.cuda(), perm.cuda(), ids.cuda(), 1)
+    assert torch.equal(out1.cpu(), torch.gather(xs, 1, perm[ids.long()].long()))

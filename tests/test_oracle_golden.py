@@ -500,3 +500,53 @@ def test_fp8_weight_fragment_layout_by_definition(oracle):
                 assert p[frag * 2048 + h * 1024 + lane * 16 + k % 16] == w[e, n, k]
     # 2-D input is the E = 1 case
     np.testing.assert_array_equal(oracle.fp8_repack_weight(w[0]), oracle.fp8_repack_weight(w[:1])[0])
+
+
+def test_moe_act_order_forward_reduces_to_the_plain_block(oracle):
+    """The act-order MoE oracle (scale[g_idx[k]] per weight row, by definition) against the pinned plain block:
+      * with g_idx[k] = k // 128 the two are the same function;
+      * with a shuffled g_idx it equals the plain block run on experts whose rows are sorted by group and on activations
+        whose columns are permuted the same way - the route the reference takes (marlin_moe_layer.cpp:71-93)."""
+    rng = np.random.default_rng(21)
+    E, hidden, inter, topk, T = 4, 256, 128, 2, 5
+    dtype = 0
+
+    def experts(n, k):
+        codes = rng.integers(0, 16, (E, k, n), dtype=np.uint8)               # [E, k, n], checkpoint row order
+        scales = oracle.to_bits((rng.random((E, k // 128, n)) * 0.01 + 0.002).astype(np.float32), dtype)
+        return codes, scales
+
+    def as_moe_bytes(codes, scales_bits):                                      # [E, n, k/2] bytes, [E, n, k/128] scales
+        c = codes.transpose(0, 2, 1)
+        return (c[:, :, 0::2] | (c[:, :, 1::2] << 4)).astype(np.uint8), np.ascontiguousarray(scales_bits.transpose(0, 2, 1))
+
+    c13, s13 = experts(2 * inter, hidden)
+    c2, s2 = experts(hidden, inter)
+    x = oracle.to_bits(rng.standard_normal((T, hidden)).astype(np.float32), dtype)
+    ids = np.stack([rng.choice(E, topk, replace=False) for _ in range(T)]).astype(np.int32)
+    tw = rng.random((T, topk)).astype(np.float32)
+    nat13 = np.tile(np.arange(hidden) // 128, (E, 1)).astype(np.int32)
+    nat2 = np.tile(np.arange(inter) // 128, (E, 1)).astype(np.int32)
+    w13b, s13b = as_moe_bytes(c13, s13)
+    w2b, s2b = as_moe_bytes(c2, s2)
+    plain = oracle.moe_forward(x, w13b, s13b, w2b, s2b, ids, tw, 128, dtype)
+    np.testing.assert_array_equal(oracle.moe_act_order_forward(x, c13, s13, nat13, c2, s2, nat2, ids, tw, dtype), plain)
+
+    # shuffled groups on the first GEMM only (the second keeps natural order so that one permutation is in play):
+    # one expert per token, so that a single column permutation of x describes the reference's route
+    g13 = np.stack([rng.permutation(hidden) // 128 for _ in range(E)]).astype(np.int32)
+    ids1 = ids[:, :1].copy()
+    tw1 = tw[:, :1].copy()
+    got = oracle.moe_act_order_forward(x, c13, s13, g13, c2, s2, nat2, ids1, tw1, dtype)
+    for t in range(T):
+        e = int(ids1[t, 0])
+        perm = np.argsort(g13[e], kind="stable")
+        c13s = c13.copy()
+        c13s[e] = c13[e][perm]
+        w13s, _ = as_moe_bytes(c13s, s13)
+        xt = np.ascontiguousarray(x[t:t + 1][:, perm])
+        ref = oracle.moe_forward(xt, w13s, s13b, w2b, s2b, ids1[t:t + 1], tw1[t:t + 1], 128, dtype)
+        # same products in another order inside each group sum: equal up to one rounding of the 16-bit results
+        a = oracle.from_bits(got[t:t + 1], dtype).astype(np.float64)
+        b = oracle.from_bits(ref, dtype).astype(np.float64)
+        assert np.max(np.abs(a - b)) <= 2e-3 * max(1.0, np.max(np.abs(b)))
