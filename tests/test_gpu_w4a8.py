@@ -123,6 +123,19 @@ def test_gemm_tile_kernel(ops, oracle, out_dtype, m, n, k):
     H.check_gemm(out, ref, out_dtype, "w4a8 tile m=%d n=%d k=%d" % (m, n, k))
 
 
+@pytest.mark.parametrize("m,n,k", [(3, 8192, 512), (20, 8192, 512), (16, 16384, 256), (32, 16384, 256), (1, 4096, 1024)])
+def test_gemm_streaming_kernel_variants(ops, oracle, m, n, k):
+    """The streaming kernel's other instantiations: four strips per workgroup with eight wavefronts (n = 8192) and with
+    four (n = 16384), one and two 16-token tiles; two strips with eight wavefronts (n = 4096)."""
+    w, scales = make_weight(n + k + m, k, n)
+    x = make_act(m * 5 + n, m, k, H.BF16)
+    in_scale = torch.tensor([0.06], dtype=torch.float32)
+    xq, xsum = ops.w4a8_static_quant(x.cuda(), in_scale.cuda(), False)
+    out = ops.w4a8_gemm(xq, xsum, ops.w4a8_repack_weight(w.cuda()), scales.cuda(), 0.02, n, torch.bfloat16)
+    ref = oracle.w4a8_gemm(xq.cpu().numpy(), w.numpy().view(np.int8), H.bits_of(scales), 0.02)
+    H.check_gemm(out, ref, H.BF16, "w4a8 streaming m=%d n=%d k=%d" % (m, n, k))
+
+
 def test_gemm_workspace_is_checked(ops):
     from ksanallm_amd import lib as L
     m, n, k = 64, 256, 8192
