@@ -188,18 +188,19 @@ int ksq_fp8_tensor_gemm(const void* a_q, const void* a_scale, const void* b, con
  *   the 1 KiB fragment layout of the fp8 matrix instruction (n*k/2 bytes).  n % 16 == 0, k % 128 == 0.
  *   ksq_w4a8_unpack_weight is its inverse (bit-exact round trip).
  * ksq_w4a8_static_quant: q[m,k] = e4m3(x[m,k] / s), IEEE fp32 division, round to nearest even, saturating;
- *   s = scale[0] (KSQ_W4A8_PER_TENSOR) or scale[channel] (KSQ_W4A8_PER_CHANNEL), fp32 in device memory; and
+ *   s = scale[0] (KSQ_W4A8_PER_TENSOR), scale[channel] (KSQ_W4A8_PER_CHANNEL) or scale[row] (KSQ_W4A8_PER_TOKEN), fp32
+ *   in device memory; and
  *   xsum[k/128, m] fp32 (group-major, tokens contiguous) = the sum of each group of 128 quantized values, which
  *   the GEMM needs.  KSQ_W4A8_SUMS_ONLY
  *   takes x that is e4m3 already and writes xsum only (q and scale unused).
- *   Replaces StaticQuantizeE4M3PerTensor / PerChannel (wrapper.cpp:128-153 -> scaleMatrix,
+ *   Replaces StaticQuantizeE4M3PerTensor / PerToken / PerChannel (wrapper.cpp:128-153 -> scaleMatrix,
  *   K/others/tensorrt-llm/dev/common/cudaFp8Utils.cu:38-52).
  * ksq_w4a8_gemm: a_q [m,k] e4m3 row-major, xsum [k/128,m], w_packed from ksq_w4a8_repack_weight, scales fp16
  *   [k/128, n] as the reference holds them (weight_scale / weight_scale_2), alpha = input_scale * weight_scale_2.
  *   Replaces FinegrainedMixedDtypeGemmWrapper::Forward (wrapper.cpp:68-100); no tactic argument: the kernel is
  *   chosen from the shape.
  * ------------------------------------------------------------------------------------------------------------------ */
-enum { KSQ_W4A8_PER_TENSOR = 0, KSQ_W4A8_PER_CHANNEL = 1, KSQ_W4A8_SUMS_ONLY = 2 };
+enum { KSQ_W4A8_PER_TENSOR = 0, KSQ_W4A8_PER_CHANNEL = 1, KSQ_W4A8_SUMS_ONLY = 2, KSQ_W4A8_PER_TOKEN = 3 };
 size_t ksq_w4a8_packed_weight_bytes(size_t n, size_t k);
 int ksq_w4a8_repack_weight(const void* src, void* dst_packed, size_t n, size_t k, void* stream);
 int ksq_w4a8_unpack_weight(const void* packed, void* dst, size_t n, size_t k, void* stream);

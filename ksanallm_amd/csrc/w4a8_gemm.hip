@@ -89,7 +89,8 @@ __device__ __forceinline__ float sum8_e4m3(u32x2 q) {
   return ((((((a.x + a.y) + b.x) + b.y) + c.x) + c.y) + d.x) + d.y;
 }
 
-// MODE 0: q = e4m3(x / scale[0]); MODE 1: q = e4m3(x / scale[channel]); MODE 2: x is e4m3 already (sums only).
+// MODE 0: q = e4m3(x / scale[0]); MODE 1: q = e4m3(x / scale[channel]); MODE 2: x is e4m3 already (sums only);
+// MODE 3: q = e4m3(x / scale[row]).
 // IEEE fp32 division, round to nearest even, saturating.  xsum[g, row] = sum of the 128 quantized values of group g
 // (every e4m3 value is a multiple of 2^-9, so the fp32 sum is exact, in any order, while it stays below 2^15).
 // Grid: x = chunks of BLOCK * 8 channels, y/z = row; a group of 128 channels is 16 adjacent lanes.
@@ -114,9 +115,9 @@ __global__ void __launch_bounds__(BLOCK) w4a8_quant_kernel(const void* __restric
       v[2 * j] = T::lo_to_float(raw[j]);
       v[2 * j + 1] = T::hi_to_float(raw[j]);
     }
-    if (MODE == 0) {
-      // one scale for all: the quotient from one reciprocal per lane (exact_div.h); an infinite input keeps the division
-      const float s = scale[0];
+    if (MODE == 0 || MODE == 3) {
+      // one scale per lane: the quotient from one reciprocal (exact_div.h); an infinite input keeps the division
+      const float s = scale[MODE == 3 ? t : 0];
       const ExactDiv div(s);
 #pragma unroll
       for (int j = 0; j < 8; ++j) v[j] = __builtin_fabsf(v[j]) == __builtin_inff() ? v[j] / s : div(v[j]);
@@ -377,7 +378,7 @@ KSQ_EXPORT int ksq_w4a8_static_quant(const void* x, const void* scale, void* q, 
                                      int mode, int dtype, void* stream) {
   const char* fn = "ksq_w4a8_static_quant";
   if (!x || !xsum || (mode != KSQ_W4A8_SUMS_ONLY && (!q || !scale))) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: null pointer", fn);
-  if (mode != KSQ_W4A8_PER_TENSOR && mode != KSQ_W4A8_PER_CHANNEL && mode != KSQ_W4A8_SUMS_ONLY)
+  if (mode != KSQ_W4A8_PER_TENSOR && mode != KSQ_W4A8_PER_CHANNEL && mode != KSQ_W4A8_SUMS_ONLY && mode != KSQ_W4A8_PER_TOKEN)
     return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: unknown mode %d", fn, mode);
   if (k == 0 || k % 128 != 0) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: k must be a positive multiple of 128", fn);
   if (mode != KSQ_W4A8_SUMS_ONLY && dtype != KSQ_F16 && dtype != KSQ_BF16)
@@ -385,7 +386,7 @@ KSQ_EXPORT int ksq_w4a8_static_quant(const void* x, const void* scale, void* q, 
   const bool sums = mode == KSQ_W4A8_SUMS_ONLY;
   if ((reinterpret_cast<uintptr_t>(x) & (sums ? 7u : 15u)) || (!sums && (reinterpret_cast<uintptr_t>(q) & 7u)) ||
       (reinterpret_cast<uintptr_t>(xsum) & 3u) || (mode == KSQ_W4A8_PER_CHANNEL && !aligned16(scale)) ||
-      (mode == KSQ_W4A8_PER_TENSOR && (reinterpret_cast<uintptr_t>(scale) & 3u)))
+      ((mode == KSQ_W4A8_PER_TENSOR || mode == KSQ_W4A8_PER_TOKEN) && (reinterpret_cast<uintptr_t>(scale) & 3u)))
     return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: misaligned pointer", fn);
   if (m == 0) return KSQ_OK;
   if (m > 0x7fffffffull || k > 0x7fffffffull) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: tensor too large", fn);
@@ -408,8 +409,10 @@ KSQ_EXPORT int ksq_w4a8_static_quant(const void* x, const void* scale, void* q, 
   } while (0)
   if (mode == KSQ_W4A8_SUMS_ONLY) KSQ_QB(F16, 2);
   else if (dtype == KSQ_F16 && mode == KSQ_W4A8_PER_TENSOR) KSQ_QB(F16, 0);
+  else if (dtype == KSQ_F16 && mode == KSQ_W4A8_PER_TOKEN) KSQ_QB(F16, 3);
   else if (dtype == KSQ_F16) KSQ_QB(F16, 1);
   else if (mode == KSQ_W4A8_PER_TENSOR) KSQ_QB(BF16, 0);
+  else if (mode == KSQ_W4A8_PER_TOKEN) KSQ_QB(BF16, 3);
   else KSQ_QB(BF16, 1);
 #undef KSQ_QB
 #undef KSQ_Q

@@ -10,7 +10,7 @@ SRC_GPTQ, SRC_AWQ, SRC_MOE_NK, SRC_INT4X2_KN = 0, 1, 2, 3
 SCALE_GN, SCALE_NG = 0, 1
 ZERO_AWQ_PACKED, ZERO_U8_GN = 0, 1
 KIND_W4A16, KIND_FP8_BLOCKWISE, KIND_MOE_W4A16 = 0, 1, 2
-W4A8_PER_TENSOR, W4A8_PER_CHANNEL, W4A8_SUMS_ONLY = 0, 1, 2
+W4A8_PER_TENSOR, W4A8_PER_CHANNEL, W4A8_SUMS_ONLY, W4A8_PER_TOKEN = 0, 1, 2, 3
 
 c_sz = ctypes.c_size_t
 c_p = ctypes.c_void_p

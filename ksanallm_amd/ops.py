@@ -388,13 +388,13 @@ def w4a8_unpack_weight(packed, K, N):
     return out
 
 
-def w4a8_static_quant(x, scale, per_channel=False):
-    """StaticQuantizeE4M3PerTensor / PerChannel: x [m,k] T, scale fp32 [1] or [k] -> (codes uint8 [m,k], group sums
-    fp32 [k/128, m])."""
+def w4a8_static_quant(x, scale, per_channel=False, per_token=False):
+    """StaticQuantizeE4M3PerTensor / PerChannel / PerToken: x [m,k] T, scale fp32 [1], [k] or [m] -> (codes uint8
+    [m,k], group sums fp32 [k/128, m])."""
     m, k = x.shape
     q = torch.empty((m, k), dtype=torch.uint8, device=x.device)
     xsum = torch.empty((k // 128, m), dtype=torch.float32, device=x.device)
-    mode = _l.W4A8_PER_CHANNEL if per_channel else _l.W4A8_PER_TENSOR
+    mode = _l.W4A8_PER_CHANNEL if per_channel else (_l.W4A8_PER_TOKEN if per_token else _l.W4A8_PER_TENSOR)
     _l.check(_lib.ksq_w4a8_static_quant(_ptr(x), _ptr(scale), _ptr(q), _ptr(xsum), m, k, mode, _dt(x), _stream()))
     return q, xsum
 

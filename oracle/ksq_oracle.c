@@ -799,12 +799,13 @@ KSQO_API void ksqo_w4a8_unpack_int4(const int8_t* w, int8_t* out, size_t K, size
   }
 }
 
-/* q[i] = e4m3(float(x[i]) / scale), scale = scale[0] or scale[i % k]: scaleMatrix<PER_TENSOR | PER_CHANNEL, true>
- * (K/others/tensorrt-llm/dev/common/cudaFp8Utils.cu:33-52); the conversion saturates to +-448 (__nv_fp8_e4m3). */
-KSQO_API void ksqo_w4a8_static_quant(const void* x, const float* scale, uint8_t* q, size_t m, size_t k, int per_channel,
+/* q[i] = e4m3(float(x[i]) / scale), scale = scale[0] (mode 0), scale[i % k] (mode 1) or scale[i / k] (mode 3):
+ * scaleMatrix<PER_TENSOR | PER_CHANNEL | PER_TOKEN, true> (K/others/tensorrt-llm/dev/common/cudaFp8Utils.cu:33-52);
+ * the conversion saturates to +-448 (__nv_fp8_e4m3). */
+KSQO_API void ksqo_w4a8_static_quant(const void* x, const float* scale, uint8_t* q, size_t m, size_t k, int mode,
                                      int dtype) {
   for (size_t i = 0; i < m * k; ++i) {
-    volatile float sc = per_channel ? scale[i % k] : scale[0];
+    volatile float sc = mode == 1 ? scale[i % k] : (mode == 3 ? scale[i / k] : scale[0]);
     volatile float r = load_t(x, i, dtype) / sc;
     q[i] = ksqo_f32_to_e4m3(fminf(fmaxf(r, -448.0f), 448.0f));
   }

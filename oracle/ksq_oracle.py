@@ -472,13 +472,13 @@ def w4a8_unpack_int4(w):
     return out
 
 
-def w4a8_static_quant(x_bits, scale, per_channel, dtype):
+def w4a8_static_quant(x_bits, scale, per_channel, dtype, per_token=False):
     x = _c(x_bits, _store_dt(dtype))
     m, k = x.shape
     s = _c(np.asarray(scale, np.float32).reshape(-1), np.float32)
-    assert s.size == (k if per_channel else 1)
+    assert s.size == (k if per_channel else (m if per_token else 1))
     q = np.empty((m, k), np.uint8)
-    lib().ksqo_w4a8_static_quant(_p(x), _p(s), _p(q), _sz(m), _sz(k), ctypes.c_int(int(per_channel)),
+    lib().ksqo_w4a8_static_quant(_p(x), _p(s), _p(q), _sz(m), _sz(k), ctypes.c_int(1 if per_channel else (3 if per_token else 0)),
                                  ctypes.c_int(dtype))
     return q
 

@@ -37,3 +37,11 @@ def test_size_queries_and_tile_selection_are_host_only():
     import pytest
     with pytest.raises(L.KsqError):
         L.select_tile(99, 1, 16, 128, 0)
+    # W4A8: packed size, and a workspace that covers every token count up to the maximum it was asked for
+    assert lib.ksq_w4a8_packed_weight_bytes(5120, 5120) == 5120 * 5120 // 2
+    assert lib.ksq_w4a8_workspace_size(32, 5120, 5120) == 0        # the streaming kernel needs none
+    need = lib.ksq_w4a8_workspace_size(4096, 256, 8192)
+    assert need > 0
+    for m in (33, 64, 100, 128, 129, 700, 4096):
+        assert lib.ksq_w4a8_workspace_size(m, 256, 8192) <= need
+    assert lib.ksq_w4a8_workspace_size(64, 256, 100) == 0          # k not a multiple of 128: no kernel, no scratch

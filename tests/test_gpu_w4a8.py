@@ -60,6 +60,17 @@ def test_static_quant_bit_exact(ops, oracle, dtype, per_channel, m, k):
     np.testing.assert_array_equal(ops.w4a8_group_sums(q).cpu().numpy().T, oracle.w4a8_group_sums(ref))
 
 
+@pytest.mark.parametrize("dtype", [H.F16, H.BF16])
+def test_static_quant_per_token_bit_exact(ops, oracle, dtype):
+    m, k = 70, 1536
+    x = make_act(31, m, k, dtype)
+    scale = (torch.rand(m, generator=H.gen(32)) * 0.2 + 0.01).float()
+    q, xsum = ops.w4a8_static_quant(x.cuda(), scale.cuda(), per_token=True)
+    ref = oracle.w4a8_static_quant(H.bits_of(x), scale.numpy(), False, dtype, per_token=True)
+    np.testing.assert_array_equal(q.cpu().numpy(), ref)
+    np.testing.assert_array_equal(xsum.cpu().numpy().T, oracle.w4a8_group_sums(ref))
+
+
 def test_static_quant_boundaries_and_specials(ops, oracle):
     """Every midpoint between neighbouring e4m3 values and its fp32 neighbours, at scale 1; saturation; infinities."""
     codes = np.arange(0, 0x7E, dtype=np.uint8)

@@ -41,6 +41,10 @@ def test_static_quant_matches_torch_cast_of_the_fp32_quotient(oracle):
             r = np.clip(xr / (s[None, :] if per_channel else s[0]), -448, 448).astype(np.float32)
             ref = torch.from_numpy(r).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
             np.testing.assert_array_equal(q, ref)
+        s = (rng.random(m) * 2 + 0.01).astype(np.float32)
+        q = oracle.w4a8_static_quant(xb, s, False, dtype, per_token=True)
+        r = np.clip(xr / s[:, None], -448, 448).astype(np.float32)
+        np.testing.assert_array_equal(q, torch.from_numpy(r).to(torch.float8_e4m3fn).view(torch.uint8).numpy())
     # saturation and specials
     xs = np.float32([[1e6, -1e6, np.inf, -np.inf, 448, -449, 0.0, -0.0] * 16])
     q = oracle.w4a8_static_quant(oracle.to_bits(xs, 1), np.float32([1.0]), False, 1)
