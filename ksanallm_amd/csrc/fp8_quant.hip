@@ -148,7 +148,7 @@ __global__ void fp8_scale_clear_kernel(float* __restrict__ scale, uint32_t chann
   if (i < channels) scale[i] = 0.f;
 }
 
-// scale[c] = max(amax(|x[c, :]|) / 448, 1 / (448 * 512)).  Every wavefront folds its maximum in with an integer
+// scale[c] = max(amax(|x[c, :]|) / 448, 1 / (448 * 512)).  Every workgroup folds its maximum in with an integer
 // atomic max on the float's bits (all candidates are positive, so the orders agree); scale[] starts at 0.
 template <typename T>
 __global__ void __launch_bounds__(256) fp8_channel_scale_kernel(const uint16_t* __restrict__ x, float* __restrict__ scale,
@@ -171,7 +171,13 @@ __global__ void __launch_bounds__(256) fp8_channel_scale_kernel(const uint16_t* 
   }
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
-  if ((threadIdx.x & 63) == 0) {
+  // one atomic per workgroup: atomics on one address are served one after the other (one per wavefront of a full grid
+  // cost more time than reading the tensor)
+  __shared__ float wave_max[4];
+  if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = amax;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    amax = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
     const float sc = fmaxf(amax / 448.0f, kMinScale);
     atomicMax(reinterpret_cast<unsigned int*>(scale + blockIdx.y), __float_as_uint(sc));
   }
@@ -184,8 +190,6 @@ __global__ void __launch_bounds__(256) fp8_channel_quant_kernel(const uint16_t* 
   const size_t base = static_cast<size_t>(blockIdx.y) * size;
   const float sc = scale[blockIdx.y];
   const ExactDiv div(sc);
-  // with a scale handed in by the caller an input may be infinite where the scale is not: that one keeps the division
-  auto quot = [&](float a) { return __builtin_fabsf(a) == __builtin_inff() ? a / sc : div(a); };
   const size_t tid = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
   const size_t stride = static_cast<size_t>(gridDim.x) * 256;
   if (vec) {
@@ -194,8 +198,20 @@ __global__ void __launch_bounds__(256) fp8_channel_quant_kernel(const uint16_t* 
       float v[8];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        v[2 * j] = quot(T::to_float(static_cast<uint16_t>(raw[j] & 0xffffu)));
-        v[2 * j + 1] = quot(T::to_float(static_cast<uint16_t>(raw[j] >> 16)));
+        v[2 * j] = T::to_float(static_cast<uint16_t>(raw[j] & 0xffffu));
+        v[2 * j + 1] = T::to_float(static_cast<uint16_t>(raw[j] >> 16));
+      }
+      // with a scale handed in by the caller an input may be infinite where the scale is not: such a lane keeps the
+      // division (a branch, not a select per element: a select would evaluate the division for every element)
+      float mx = 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) mx = fmaxf(mx, __builtin_fabsf(v[j]));
+      if (mx == __builtin_inff()) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = v[j] / sc;
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = div(v[j]);
       }
       u32x2 out{0u, 0u};
       out.x = cvt2_e4m3(v[0], v[1], out.x, false);
@@ -261,8 +277,10 @@ KSQ_EXPORT int ksq_fp8_channel_quant(const void* x, void* q, void* scale, size_t
   float* sp = static_cast<float*>(scale);
   if (!is_static) {
     fp8_scale_clear_kernel<<<static_cast<unsigned>(div_up(channels, 256)), 256, 0, st>>>(sp, static_cast<uint32_t>(channels));
-    if (dtype == KSQ_F16) fp8_channel_scale_kernel<F16><<<grid, 256, 0, st>>>(xp, sp, size, vec);
-    else fp8_channel_scale_kernel<BF16><<<grid, 256, 0, st>>>(xp, sp, size, vec);
+    // two workgroups per CU read as fast as more do and keep the atomics few
+    const dim3 sgrid(static_cast<unsigned>(bx < 512 ? bx : 512), static_cast<unsigned>(channels), 1);
+    if (dtype == KSQ_F16) fp8_channel_scale_kernel<F16><<<sgrid, 256, 0, st>>>(xp, sp, size, vec);
+    else fp8_channel_scale_kernel<BF16><<<sgrid, 256, 0, st>>>(xp, sp, size, vec);
   }
   if (dtype == KSQ_F16) fp8_channel_quant_kernel<F16><<<grid, 256, 0, st>>>(xp, static_cast<uint8_t*>(q), sp, size, vec);
   else fp8_channel_quant_kernel<BF16><<<grid, 256, 0, st>>>(xp, static_cast<uint8_t*>(q), sp, size, vec);

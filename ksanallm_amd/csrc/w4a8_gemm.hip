@@ -119,8 +119,17 @@ __global__ void __launch_bounds__(BLOCK) w4a8_quant_kernel(const void* __restric
       // one scale per lane: the quotient from one reciprocal (exact_div.h); an infinite input keeps the division
       const float s = scale[MODE == 3 ? t : 0];
       const ExactDiv div(s);
+      // a branch, not a select per element: a select would evaluate the division for every element
+      float mx = 0.f;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) v[j] = __builtin_fabsf(v[j]) == __builtin_inff() ? v[j] / s : div(v[j]);
+      for (int j = 0; j < 8; ++j) mx = fmaxf(mx, __builtin_fabsf(v[j]));
+      if (mx == __builtin_inff()) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = v[j] / s;
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = div(v[j]);
+      }
     } else {
       const f32x4 s0 = *reinterpret_cast<const f32x4*>(scale + col);
       const f32x4 s1 = *reinterpret_cast<const f32x4*>(scale + col + 4);
