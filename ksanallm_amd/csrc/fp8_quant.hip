@@ -158,14 +158,27 @@ __global__ void __launch_bounds__(256) fp8_channel_scale_kernel(const uint16_t* 
   const size_t stride = static_cast<size_t>(gridDim.x) * 256;
   float amax = 0.f;
   if (vec) {
-    for (size_t i = tid; i < size / 8; i += stride) {
-      const u32x4 raw = *reinterpret_cast<const u32x4*>(row + i * 8);
+    auto fold = [&](u32x4 raw) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         amax = fmaxf(amax, fabsf(T::to_float(static_cast<uint16_t>(raw[j] & 0xffffu))));
         amax = fmaxf(amax, fabsf(T::to_float(static_cast<uint16_t>(raw[j] >> 16))));
       }
+    };
+    const size_t n8 = size / 8;
+    size_t i = tid;
+    // four independent loads in flight per thread: one load per trip leaves the pass waiting on memory latency
+    for (; i + 3 * stride < n8; i += 4 * stride) {
+      const u32x4 r0 = *reinterpret_cast<const u32x4*>(row + i * 8);
+      const u32x4 r1 = *reinterpret_cast<const u32x4*>(row + (i + stride) * 8);
+      const u32x4 r2 = *reinterpret_cast<const u32x4*>(row + (i + 2 * stride) * 8);
+      const u32x4 r3 = *reinterpret_cast<const u32x4*>(row + (i + 3 * stride) * 8);
+      fold(r0);
+      fold(r1);
+      fold(r2);
+      fold(r3);
     }
+    for (; i < n8; i += stride) fold(*reinterpret_cast<const u32x4*>(row + i * 8));
   } else {
     for (size_t i = tid; i < size; i += stride) amax = fmaxf(amax, fabsf(T::to_float(row[i])));
   }
