@@ -322,33 +322,94 @@ __global__ void __launch_bounds__(256) moe_sum_kernel(const uint16_t* __restrict
   *reinterpret_cast<u32x4*>(out + t * d + c) = o;
 }
 
-// one wavefront per token: lane l holds experts l, l+64, ... (at most 16 each)
-template <typename LOAD>
+// ---- reductions over a whole wavefront, every lane active, result in every lane.  Four DPP row operations leave each
+// row of 16 lanes with its result, four readlanes combine the rows: a few dozen cycles, where a butterfly of LDS-crossbar
+// permutes (what __shfl_xor compiles to) costs several hundred - and the routers are nothing but chains of these.
+constexpr int kDppXor1 = 0xB1, kDppXor2 = 0x4E, kDppHalfMirror = 0x141, kDppMirror = 0x140;
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_u32(uint32_t v) {
+  return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), CTRL, 0xf, 0xf, false));
+}
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+  return __builtin_bit_cast(float, dpp_u32<CTRL>(__builtin_bit_cast(uint32_t, v)));
+}
+__device__ __forceinline__ uint32_t lane_u32(uint32_t v, int l) {
+  return static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(v), l));
+}
+__device__ __forceinline__ float lane_f32(float v, int l) {
+  return __builtin_bit_cast(float, lane_u32(__builtin_bit_cast(uint32_t, v), l));
+}
+__device__ __forceinline__ float wave_max(float v) {
+  v = fmaxf(v, dpp_f32<kDppXor1>(v));
+  v = fmaxf(v, dpp_f32<kDppXor2>(v));
+  v = fmaxf(v, dpp_f32<kDppHalfMirror>(v));
+  v = fmaxf(v, dpp_f32<kDppMirror>(v));
+  return fmaxf(fmaxf(lane_f32(v, 0), lane_f32(v, 16)), fmaxf(lane_f32(v, 32), lane_f32(v, 48)));
+}
+// the partners of every step hold equal partial sums, so all lanes of a row end with the same bits
+__device__ __forceinline__ float wave_sum(float v) {
+  v += dpp_f32<kDppXor1>(v);
+  v += dpp_f32<kDppXor2>(v);
+  v += dpp_f32<kDppHalfMirror>(v);
+  v += dpp_f32<kDppMirror>(v);
+  return (lane_f32(v, 0) + lane_f32(v, 16)) + (lane_f32(v, 32) + lane_f32(v, 48));
+}
+// A lane's candidate: the largest key wins, among equal keys the lower id; id 0xffffffff = no candidate.  pay travels
+// with the winner.
+struct Pick {
+  float key, pay;
+  uint32_t id;
+};
+constexpr uint32_t kNoPick = 0xffffffffu;
+__device__ __forceinline__ bool beats(const Pick& a, const Pick& b) {
+  return a.id != kNoPick && (b.id == kNoPick || a.key > b.key || (a.key == b.key && a.id < b.id));
+}
+template <int CTRL>
+__device__ __forceinline__ void pick_step(Pick& p) {
+  const Pick o{dpp_f32<CTRL>(p.key), dpp_f32<CTRL>(p.pay), dpp_u32<CTRL>(p.id)};
+  if (beats(o, p)) p = o;
+}
+__device__ __forceinline__ Pick wave_argmax(Pick p) {
+  pick_step<kDppXor1>(p);
+  pick_step<kDppXor2>(p);
+  pick_step<kDppHalfMirror>(p);
+  pick_step<kDppMirror>(p);
+  Pick r{lane_f32(p.key, 0), lane_f32(p.pay, 0), lane_u32(p.id, 0)};
+#pragma unroll
+  for (int row = 16; row < 64; row += 16) {
+    const Pick o{lane_f32(p.key, row), lane_f32(p.pay, row), lane_u32(p.id, row)};
+    if (beats(o, r)) r = o;
+  }
+  return r;
+}
+
+// one wavefront per token: lane l holds experts l, l+64, ... (NV each: 4 serves up to 256 experts, 16 up to 1024; a lone
+// wavefront is bound by its instruction count, and every scan below runs NV times)
+template <typename LOAD, int NV>
 __global__ void __launch_bounds__(256) topk_softmax_kernel(const void* __restrict__ gating, float* __restrict__ topk_w,
                                                            int32_t* __restrict__ topk_ids, uint32_t tokens,
                                                            uint32_t E, uint32_t top_k, int norm, float scaling) {
   const uint32_t token = blockIdx.x * 4 + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   if (token >= tokens) return;
-  float v[16];
+  float v[NV];
   float mx = -INFINITY;
 #pragma unroll
-  for (int j = 0; j < 16; ++j) {
+  for (int j = 0; j < NV; ++j) {
     const uint32_t e = j * 64 + lane;
     v[j] = e < E ? LOAD::get(gating, static_cast<size_t>(token) * E + e) : -INFINITY;
     mx = fmaxf(mx, v[j]);
   }
-#pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+  mx = wave_max(mx);
   float sum = 0.f;
 #pragma unroll
-  for (int j = 0; j < 16; ++j) {
+  for (int j = 0; j < NV; ++j) {
     const uint32_t e = j * 64 + lane;
     v[j] = e < E ? expf(v[j] - mx) : -1.0f;  // -1 never wins the arg-max below
     sum += e < E ? v[j] : 0.f;
   }
-#pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) sum += __shfl_xor(sum, off, 64);
+  sum = wave_sum(sum);
   float picked_sum = 0.f;
   float my_w = 0.f;
   int my_id = 0;
@@ -356,24 +417,20 @@ __global__ void __launch_bounds__(256) topk_softmax_kernel(const void* __restric
     float best = -2.0f;
     uint32_t best_e = 0xffffffffu;
 #pragma unroll
-    for (int j = 0; j < 16; ++j) {
+    for (int j = 0; j < NV; ++j) {
       const uint32_t e = j * 64 + lane;
       if (v[j] > best) {  // ascending e inside a lane: strict > keeps the lower id on ties
         best = v[j];
         best_e = e;
       }
     }
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) {
-      const float ob = __shfl_xor(best, off, 64);
-      const uint32_t oe = __shfl_xor(best_e, off, 64);
-      if (ob > best || (ob == best && oe < best_e)) {
-        best = ob;
-        best_e = oe;
-      }
+    {
+      const Pick w = wave_argmax(Pick{best, 0.f, best_e});
+      best = w.key;
+      best_e = w.id;
     }
 #pragma unroll
-    for (int j = 0; j < 16; ++j)
+    for (int j = 0; j < NV; ++j)
       if (static_cast<uint32_t>(j * 64 + lane) == best_e) v[j] = -1.0f;
     const float prob = best / sum;
     picked_sum += prob;
@@ -397,7 +454,7 @@ struct Load16 {
   static __device__ __forceinline__ float get(const void* p, size_t i) { return T::to_float(static_cast<const uint16_t*>(p)[i]); }
 };
 
-// Grouped routing (DeepSeek-V2/V3): one wavefront per token, lane l holds experts l, l+64, ... (at most 16 each).
+// Grouped routing (DeepSeek-V2/V3): one wavefront per token, lane l holds experts l, l+64, ... (NV each, as above).
 //   score   = softmax(gating) or sigmoid(gating), fp32
 //   choose  = score + bias (bias given) or score
 //   group g = experts [g*per_group, (g+1)*per_group): its rank value is the sum of its two largest choose values
@@ -405,7 +462,7 @@ struct Load16 {
 //   top_k rounds of wave arg-max over choose pick the experts (descending, the lower id wins ties); the routing
 //   weight of a pick is its score (without bias), divided by the sum of the picks when renormalize, times scaling.
 // Group rank values are built from the choose values staged in LDS (one row of E floats per wavefront).
-template <typename LOAD>
+template <typename LOAD, int NV>
 __global__ void __launch_bounds__(256) grouped_topk_kernel(const void* __restrict__ gating, const float* __restrict__ bias,
                                                            float* __restrict__ topk_w, int32_t* __restrict__ topk_ids,
                                                            uint32_t tokens, uint32_t E, uint32_t top_k, uint32_t groups,
@@ -419,34 +476,32 @@ __global__ void __launch_bounds__(256) grouped_topk_kernel(const void* __restric
   const uint32_t per_group = E / groups;
   float* choose_row = lds_choose + wave * E;
 
-  float score[16], choose[16];
+  float score[NV], choose[NV];
   float mx = -INFINITY;
 #pragma unroll
-  for (int j = 0; j < 16; ++j) {
+  for (int j = 0; j < NV; ++j) {
     const uint32_t e = j * 64 + lane;
     score[j] = e < E ? LOAD::get(gating, static_cast<size_t>(token) * E + e) : -INFINITY;
     mx = fmaxf(mx, score[j]);
   }
   if (sigmoid) {
 #pragma unroll
-    for (int j = 0; j < 16; ++j) score[j] = 1.0f / (1.0f + expf(-score[j]));
+    for (int j = 0; j < NV; ++j) score[j] = 1.0f / (1.0f + expf(-score[j]));
   } else {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+    mx = wave_max(mx);
     float sum = 0.f;
 #pragma unroll
-    for (int j = 0; j < 16; ++j) {
+    for (int j = 0; j < NV; ++j) {
       const uint32_t e = j * 64 + lane;
       score[j] = e < E ? expf(score[j] - mx) : 0.f;
       sum += score[j];
     }
+    sum = wave_sum(sum);
 #pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) sum += __shfl_xor(sum, off, 64);
-#pragma unroll
-    for (int j = 0; j < 16; ++j) score[j] = score[j] / sum;
+    for (int j = 0; j < NV; ++j) score[j] = score[j] / sum;
   }
 #pragma unroll
-  for (int j = 0; j < 16; ++j) {
+  for (int j = 0; j < NV; ++j) {
     const uint32_t e = j * 64 + lane;
     choose[j] = e < E ? score[j] + (bias ? bias[e] : 0.f) : -INFINITY;
     if (e < E) choose_row[e] = choose[j];
@@ -474,21 +529,12 @@ __global__ void __launch_bounds__(256) grouped_topk_kernel(const void* __restric
     float best = rank;
     uint32_t best_g = static_cast<uint32_t>(lane) < groups ? lane : 0xffffffffu;
     if ((kept >> lane) & 1) best_g = 0xffffffffu;  // taken: never wins
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) {
-      const float ob = __shfl_xor(best, off, 64);
-      const uint32_t og = __shfl_xor(best_g, off, 64);
-      const bool mine = best_g != 0xffffffffu, theirs = og != 0xffffffffu;
-      if (theirs && (!mine || ob > best || (ob == best && og < best_g))) {
-        best = ob;
-        best_g = og;
-      }
-    }
+    best_g = wave_argmax(Pick{best, 0.f, best_g}).id;
     if (best_g != 0xffffffffu) kept |= 1ull << best_g;
   }
   uint32_t taken = 0;  // bit j: expert j*64+lane is out (group not kept, past E, or already picked)
 #pragma unroll
-  for (int j = 0; j < 16; ++j) {
+  for (int j = 0; j < NV; ++j) {
     const uint32_t e = j * 64 + lane;
     if (e >= E || !((kept >> (e / per_group)) & 1)) taken |= 1u << j;
   }
@@ -499,27 +545,20 @@ __global__ void __launch_bounds__(256) grouped_topk_kernel(const void* __restric
     float best = 0.f, best_s = 0.f;
     uint32_t best_e = 0xffffffffu;
 #pragma unroll
-    for (int j = 0; j < 16; ++j) {
+    for (int j = 0; j < NV; ++j) {
       if (!((taken >> j) & 1) && (best_e == 0xffffffffu || choose[j] > best)) {  // ascending e: > keeps the lower id
         best = choose[j];
         best_s = score[j];
         best_e = j * 64 + lane;
       }
     }
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) {
-      const float ob = __shfl_xor(best, off, 64);
-      const float os = __shfl_xor(best_s, off, 64);
-      const uint32_t oe = __shfl_xor(best_e, off, 64);
-      const bool mine = best_e != 0xffffffffu, theirs = oe != 0xffffffffu;
-      if (theirs && (!mine || ob > best || (ob == best && oe < best_e))) {
-        best = ob;
-        best_s = os;
-        best_e = oe;
-      }
+    {
+      const Pick w = wave_argmax(Pick{best, best_s, best_e});
+      best_s = w.pay;
+      best_e = w.id;
     }
 #pragma unroll
-    for (int j = 0; j < 16; ++j)
+    for (int j = 0; j < NV; ++j)
       if (static_cast<uint32_t>(j * 64 + lane) == best_e) taken |= 1u << j;
     picked_sum += best_s;
     if (static_cast<uint32_t>(lane) == r) {
@@ -615,14 +654,18 @@ KSQ_EXPORT int ksq_moe_topk_softmax(const void* gating, void* topk_w, void* topk
   int32_t* ids = static_cast<int32_t*>(topk_ids);
   const uint32_t t = static_cast<uint32_t>(tokens), e = static_cast<uint32_t>(E), k = static_cast<uint32_t>(top_k);
   hipStream_t st = as_stream(stream);
-  if (dtype == KSQ_F32)
-    topk_softmax_kernel<LoadF32><<<blocks, 256, 0, st>>>(gating, w, ids, t, e, k, norm_topk_prob, routed_scaling_factor);
-  else if (dtype == KSQ_F16)
-    topk_softmax_kernel<Load16<F16>><<<blocks, 256, 0, st>>>(gating, w, ids, t, e, k, norm_topk_prob, routed_scaling_factor);
-  else if (dtype == KSQ_BF16)
-    topk_softmax_kernel<Load16<BF16>><<<blocks, 256, 0, st>>>(gating, w, ids, t, e, k, norm_topk_prob, routed_scaling_factor);
-  else
-    return fail(KSQ_ERR_UNSUPPORTED, "%s: unknown dtype %d", fn, dtype);
+#define KSQ_ROUTE(LOAD_)                                                                                             \
+  do {                                                                                                              \
+    if (E <= 256)                                                                                                   \
+      topk_softmax_kernel<LOAD_, 4><<<blocks, 256, 0, st>>>(gating, w, ids, t, e, k, norm_topk_prob, routed_scaling_factor);  \
+    else                                                                                                            \
+      topk_softmax_kernel<LOAD_, 16><<<blocks, 256, 0, st>>>(gating, w, ids, t, e, k, norm_topk_prob, routed_scaling_factor); \
+  } while (0)
+  if (dtype == KSQ_F32) KSQ_ROUTE(LoadF32);
+  else if (dtype == KSQ_F16) KSQ_ROUTE(Load16<F16>);
+  else if (dtype == KSQ_BF16) KSQ_ROUTE(Load16<BF16>);
+  else return fail(KSQ_ERR_UNSUPPORTED, "%s: unknown dtype %d", fn, dtype);
+#undef KSQ_ROUTE
   return check_launch(fn);
 }
 
@@ -655,14 +698,18 @@ KSQ_EXPORT int ksq_moe_grouped_topk(const void* gating, const void* e_bias, void
   const uint32_t g = static_cast<uint32_t>(num_expert_group), kg = static_cast<uint32_t>(topk_group);
   const int sig = scoring == KSQ_SCORE_SIGMOID;
   hipStream_t st = as_stream(stream);
-  if (dtype == KSQ_F32)
-    grouped_topk_kernel<LoadF32><<<blocks, 256, lds, st>>>(gating, b, w, ids, t, e, k, g, kg, sig, renormalize, routed_scaling_factor);
-  else if (dtype == KSQ_F16)
-    grouped_topk_kernel<Load16<F16>><<<blocks, 256, lds, st>>>(gating, b, w, ids, t, e, k, g, kg, sig, renormalize, routed_scaling_factor);
-  else if (dtype == KSQ_BF16)
-    grouped_topk_kernel<Load16<BF16>><<<blocks, 256, lds, st>>>(gating, b, w, ids, t, e, k, g, kg, sig, renormalize, routed_scaling_factor);
-  else
-    return fail(KSQ_ERR_UNSUPPORTED, "%s: unknown dtype %d", fn, dtype);
+#define KSQ_ROUTE(LOAD_)                                                                                                         \
+  do {                                                                                                                          \
+    if (E <= 256)                                                                                                               \
+      grouped_topk_kernel<LOAD_, 4><<<blocks, 256, lds, st>>>(gating, b, w, ids, t, e, k, g, kg, sig, renormalize, routed_scaling_factor);  \
+    else                                                                                                                        \
+      grouped_topk_kernel<LOAD_, 16><<<blocks, 256, lds, st>>>(gating, b, w, ids, t, e, k, g, kg, sig, renormalize, routed_scaling_factor); \
+  } while (0)
+  if (dtype == KSQ_F32) KSQ_ROUTE(LoadF32);
+  else if (dtype == KSQ_F16) KSQ_ROUTE(Load16<F16>);
+  else if (dtype == KSQ_BF16) KSQ_ROUTE(Load16<BF16>);
+  else return fail(KSQ_ERR_UNSUPPORTED, "%s: unknown dtype %d", fn, dtype);
+#undef KSQ_ROUTE
   return check_launch(fn);
 }
 

@@ -108,6 +108,7 @@ def _check_routing(w, ids, wo, io, choose_gap_ok):
     (5, 64, 6, 1, 1, "sigmoid", False, True),
     (9, 1000, 6, 1, 1, "softmax", False, True),
     (1, 256, 8, 8, 4, "sigmoid", True, True),
+    (33, 512, 6, 8, 3, "sigmoid", True, True),       # more than 256 experts with real groups: the 16-slots-per-lane form
 ])
 def test_grouped_topk(ops, oracle, T, E, topk, groups, topk_group, scoring, use_bias, renorm):
     g = H.gen(T + E)
