@@ -508,12 +508,15 @@ __global__ void __launch_bounds__(256) grouped_topk_kernel(const void* __restric
   }
   __syncthreads();
 
-  // rank value of group g = lane (groups <= 64)
-  float rank = -INFINITY;
-  if (static_cast<uint32_t>(lane) < groups) {
-    float m1 = -INFINITY, m2 = -INFINITY;
-    const float* g = choose_row + lane * per_group;
-    for (uint32_t i = 0; i < per_group; ++i) {
+  // rank value of a group (groups <= 64): the two largest choose values of group `grp` are found by LPG adjacent lanes,
+  // each scanning every LPG-th value of the group, and merged over those lanes (LPG is 8, 4, 2 or 1: the merges stay
+  // inside aligned runs of LPG lanes, and a run of lanes past the last group only ever merges with itself)
+  const uint32_t lpg = groups <= 8 ? 8u : (groups <= 16 ? 4u : (groups <= 32 ? 2u : 1u));
+  const uint32_t grp = static_cast<uint32_t>(lane) / lpg, slice = static_cast<uint32_t>(lane) % lpg;
+  float m1 = -INFINITY, m2 = -INFINITY;
+  if (grp < groups) {
+    const float* g = choose_row + grp * per_group;
+    for (uint32_t i = slice; i < per_group; i += lpg) {
       const float c = g[i];
       if (c > m1) {
         m2 = m1;
@@ -522,13 +525,21 @@ __global__ void __launch_bounds__(256) grouped_topk_kernel(const void* __restric
         m2 = c;
       }
     }
-    rank = bias ? m1 + m2 : m1;
   }
+  auto merge_top2 = [&](float o1, float o2) {
+    const float lo = fminf(m1, o1);
+    m1 = fmaxf(m1, o1);
+    m2 = fmaxf(lo, fmaxf(m2, o2));
+  };
+  if (lpg >= 2) merge_top2(dpp_f32<kDppXor1>(m1), dpp_f32<kDppXor1>(m2));
+  if (lpg >= 4) merge_top2(dpp_f32<kDppXor2>(m1), dpp_f32<kDppXor2>(m2));
+  if (lpg >= 8) merge_top2(dpp_f32<kDppHalfMirror>(m1), dpp_f32<kDppHalfMirror>(m2));
+  const float rank = grp < groups ? (bias ? m1 + m2 : m1) : -INFINITY;
   uint64_t kept = 0;
   for (uint32_t r = 0; r < topk_group; ++r) {
     float best = rank;
-    uint32_t best_g = static_cast<uint32_t>(lane) < groups ? lane : 0xffffffffu;
-    if ((kept >> lane) & 1) best_g = 0xffffffffu;  // taken: never wins
+    uint32_t best_g = (grp < groups && slice == 0) ? grp : 0xffffffffu;  // one lane per group carries its candidate
+    if (grp < groups && ((kept >> grp) & 1)) best_g = 0xffffffffu;  // taken: never wins
     best_g = wave_argmax(Pick{best, 0.f, best_g}).id;
     if (best_g != 0xffffffffu) kept |= 1ull << best_g;
   }
