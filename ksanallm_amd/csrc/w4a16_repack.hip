@@ -136,6 +136,51 @@ __global__ void __launch_bounds__(256) moe_permute_columns_kernel(const uint16_t
   reinterpret_cast<uint32_t*>(out + s * k)[c / 2] = static_cast<uint32_t>(row[p0]) | (static_cast<uint32_t>(row[p1]) << 16);
 }
 
+// The same two gathers with the source row staged in LDS: one workgroup per output row loads the row with coalesced
+// 16-byte loads, then every thread gathers eight output elements from LDS and stores them as 16 bytes.  (The kernels
+// above fetch 2-byte elements from scattered places of the row in memory: 1.7 TB/s where this form is bound by the
+// traffic.)  k % 8 == 0 and k * 2 bytes of LDS; ids == nullptr is the dense form (row r reads x[r], one perm).
+__global__ void __launch_bounds__(256) permute_row_lds_kernel(const uint16_t* __restrict__ x, const int32_t* __restrict__ perm,
+                                                              const int32_t* __restrict__ ids, uint16_t* __restrict__ out,
+                                                              uint32_t k, uint32_t top_k, uint32_t E) {
+  extern __shared__ __attribute__((aligned(16))) uint16_t row_lds[];
+  const size_t s = blockIdx.x;
+  const uint16_t* row = x + (ids ? s / top_k : s) * k;
+  const int32_t* pe = perm;
+  if (ids) {
+    uint32_t e = static_cast<uint32_t>(ids[s]);
+    e = e < E ? e : 0;
+    pe += static_cast<size_t>(e) * k;
+  }
+  for (uint32_t c = threadIdx.x * 8; c < k; c += 256 * 8)
+    *reinterpret_cast<u32x4*>(row_lds + c) = *reinterpret_cast<const u32x4*>(row + c);
+  __syncthreads();
+  for (uint32_t c = threadIdx.x * 8; c < k; c += 256 * 8) {
+    const u32x4 p0 = *reinterpret_cast<const u32x4*>(pe + c);
+    const u32x4 p1 = *reinterpret_cast<const u32x4*>(pe + c + 4);
+    uint32_t v[8];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t a = p0[j] < k ? p0[j] : k - 1, b = p1[j] < k ? p1[j] : k - 1;
+      v[j] = row_lds[a];
+      v[4 + j] = row_lds[b];
+    }
+    u32x4 o;
+    o.x = v[0] | (v[1] << 16);
+    o.y = v[2] | (v[3] << 16);
+    o.z = v[4] | (v[5] << 16);
+    o.w = v[6] | (v[7] << 16);
+    *reinterpret_cast<u32x4*>(out + s * k + c) = o;
+  }
+}
+
+// true when the LDS form serves the call: rows of whole 16-byte pieces, aligned, at most 64 KiB, and enough rows to
+// give every CU a workgroup (with few rows the direct form spreads a row over many workgroups and is faster)
+inline bool permute_in_lds(const void* x, const void* perm, const void* out, size_t rows, size_t k) {
+  return rows >= 256 && rows <= 0x7fffffffull && k % 8 == 0 && k * 2 <= 65536 && aligned16(x) && aligned16(perm) &&
+         aligned16(out);
+}
+
 // FP8 weights [E, N, K] (checkpoint, row-major) <-> 2 KiB fragments of 16 rows x 128 k, fragment (e, n/16, k/128) at
 // ((e*N/16 + n/16)*(K/128) + k/128): half h, then lane l = 16*((k%128)/32) + n%16, then the 16 bytes
 // k%32 in [16h, 16h+16) - the two 16-byte halves of the lane's operand of v_mfma_f32_16x16x128_f8f6f4.
@@ -349,6 +394,12 @@ KSQ_EXPORT int ksq_permute_columns(const void* x, const void* perm, void* out, s
   if (k == 0 || k % 2 != 0 || k > 0x7fffffffull) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: k must be positive and even", fn);
   if (x == out) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: cannot permute in place", fn);
   if (m == 0) return KSQ_OK;
+  if (permute_in_lds(x, perm, out, m, k)) {
+    permute_row_lds_kernel<<<static_cast<unsigned>(m), 256, k * 2, as_stream(stream)>>>(
+        static_cast<const uint16_t*>(x), static_cast<const int32_t*>(perm), nullptr, static_cast<uint16_t*>(out),
+        static_cast<uint32_t>(k), 1u, 1u);
+    return check_launch(fn);
+  }
   const size_t blocks = div_up(m * (k / 2), 256);
   if (blocks > 0x7fffffffull) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: tensor too large", fn);
   permute_columns_kernel<<<static_cast<unsigned>(blocks), 256, 0, as_stream(stream)>>>(
@@ -370,6 +421,12 @@ KSQ_EXPORT int ksq_moe_permute_columns(const void* x, const void* perm, const vo
     return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: top_k and E must be positive", fn);
   if (x == out) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: cannot permute in place", fn);
   if (numel == 0) return KSQ_OK;
+  if (permute_in_lds(x, perm, out, numel, k)) {
+    permute_row_lds_kernel<<<static_cast<unsigned>(numel), 256, k * 2, as_stream(stream)>>>(
+        static_cast<const uint16_t*>(x), static_cast<const int32_t*>(perm), static_cast<const int32_t*>(topk_ids),
+        static_cast<uint16_t*>(out), static_cast<uint32_t>(k), static_cast<uint32_t>(top_k), static_cast<uint32_t>(E));
+    return check_launch(fn);
+  }
   const size_t blocks = div_up(numel * (k / 2), 256);
   if (blocks > 0x7fffffffull) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: tensor too large", fn);
   moe_permute_columns_kernel<<<static_cast<unsigned>(blocks), 256, 0, as_stream(stream)>>>(

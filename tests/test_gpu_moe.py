@@ -413,7 +413,8 @@ def test_moe_full_size_properties(ops, kind, T):
 
 
 @pytest.mark.parametrize("dtype", [H.F16, H.BF16])
-@pytest.mark.parametrize("tokens,top_k,E,k", [(1, 4, 8, 128), (37, 2, 16, 384), (300, 8, 64, 2048)])
+@pytest.mark.parametrize("tokens,top_k,E,k", [(1, 4, 8, 128), (37, 2, 16, 384), (300, 8, 64, 2048),
+                                               (200, 2, 4, 36), (130, 2, 2, 40960)])   # the last two: rows the LDS form does not take
 def test_moe_permute_columns_bit_exact(ops, dtype, tokens, top_k, E, k):
     """out[s, j] = x[s // top_k, perm[ids[s], j]] for the first MoE GEMM, and with top_k = 1 (one input row per slot)
     for the second."""
@@ -428,3 +429,14 @@ def test_moe_permute_columns_bit_exact(ops, dtype, tokens, top_k, E, k):
     xs = torch.randn((tokens * top_k, k), generator=g).to(H.TORCH_DT[dtype])
     out1 = ops.moe_permute_columns(xs.cuda(), perm.cuda(), ids.cuda(), 1)
     assert torch.equal(out1.cpu(), torch.gather(xs, 1, perm[ids.long()].long()))
+
+
+@pytest.mark.parametrize("m,k", [(1, 128), (50, 7168), (300, 2048), (1000, 7168), (300, 36), (260, 40960)])
+def test_permute_columns_bit_exact(ops, m, k):
+    """out[r, j] = x[r, perm[j]]: rows staged in LDS (from 256 rows, k a multiple of 8 and at most 32768) and the direct
+    form."""
+    g = H.gen(m + k)
+    x = torch.randn((m, k), generator=g).to(torch.bfloat16)
+    perm = torch.randperm(k, generator=g).to(torch.int32)
+    out = ops.permute_columns(x.cuda(), perm.cuda())
+    assert torch.equal(out.cpu(), x[:, perm.long()])
