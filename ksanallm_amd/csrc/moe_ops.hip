@@ -259,15 +259,16 @@ void chunk_geometry(size_t numel, uint32_t* chunks, uint32_t* per) {
 // ids from which the two-launch sort is used
 constexpr size_t kParallelAlignFrom = 2048;
 
+// 8 elements per thread.  A workgroup covers 2^log2p column pieces of 256 >> log2p rows; the row comes from
+// blockIdx.y/z, the column piece from blockIdx.x, so that no index is divided (a 64-bit division is some fifty
+// instructions on this ISA, more than the rest of the kernel).
 template <typename T>
 __global__ void __launch_bounds__(256) silu_mul_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ out,
-                                                       size_t rows, uint32_t inter) {
-  // 8 elements per thread
-  const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
-  const size_t per_row = inter / 8;
-  if (i >= rows * per_row) return;
-  const size_t r = i / per_row;
-  const uint32_t c = static_cast<uint32_t>(i % per_row) * 8;
+                                                       size_t rows, uint32_t inter, uint32_t log2p) {
+  const uint32_t piece = (blockIdx.x << log2p) + (threadIdx.x & ((1u << log2p) - 1));
+  const size_t r = (static_cast<size_t>(blockIdx.z) * gridDim.y + blockIdx.y) * (256u >> log2p) + (threadIdx.x >> log2p);
+  if (piece >= inter / 8 || r >= rows) return;
+  const uint32_t c = piece * 8;
   const uint16_t* a = x + r * 2 * inter + c;
   u32x4 ra = *reinterpret_cast<const u32x4*>(a);
   u32x4 rb = *reinterpret_cast<const u32x4*>(a + inter);
@@ -732,14 +733,21 @@ KSQ_EXPORT int ksq_moe_silu_mul(const void* x, void* out, size_t rows, size_t in
     return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: inter must be a positive multiple of 8", fn);
   if (dtype != KSQ_F16 && dtype != KSQ_BF16) return fail(KSQ_ERR_UNSUPPORTED, "%s: dtype must be f16 or bf16", fn);
   if (rows == 0) return KSQ_OK;
-  const size_t blocks = div_up(rows * (inter / 8), 256);
-  if (blocks > 0x7fffffffull) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: tensor too large", fn);
+  // a workgroup's 256 threads: 2^log2p column pieces (of 8 elements) by 256 >> log2p rows
+  const size_t pieces = inter / 8;
+  uint32_t log2p = 0;
+  while (log2p < 8 && (size_t(1) << log2p) < pieces) ++log2p;
+  const size_t row_blocks = div_up(rows, size_t(256) >> log2p);
+  const size_t gy = row_blocks < 32768 ? row_blocks : 32768;
+  const size_t gz = div_up(row_blocks, gy);
+  if (gz > 65535) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: tensor too large", fn);
+  const dim3 grid(static_cast<unsigned>(div_up(pieces, size_t(1) << log2p)), static_cast<unsigned>(gy), static_cast<unsigned>(gz));
   const uint16_t* xp = static_cast<const uint16_t*>(x);
   uint16_t* op = static_cast<uint16_t*>(out);
   if (dtype == KSQ_F16)
-    silu_mul_kernel<F16><<<static_cast<unsigned>(blocks), 256, 0, as_stream(stream)>>>(xp, op, rows, static_cast<uint32_t>(inter));
+    silu_mul_kernel<F16><<<grid, 256, 0, as_stream(stream)>>>(xp, op, rows, static_cast<uint32_t>(inter), log2p);
   else
-    silu_mul_kernel<BF16><<<static_cast<unsigned>(blocks), 256, 0, as_stream(stream)>>>(xp, op, rows, static_cast<uint32_t>(inter));
+    silu_mul_kernel<BF16><<<grid, 256, 0, as_stream(stream)>>>(xp, op, rows, static_cast<uint32_t>(inter), log2p);
   return check_launch(fn);
 }
 
