@@ -47,8 +47,8 @@ MEASURED_TRAFFIC = {
     (7, "w4a8_quant"): 12690000,
     (7, "w4a8_splitk_kernel<16x32,w8>"): 14420000,
     (7, "w4a8_splitk_kernel<16x64,w4>"): 68990000,
-    (7, "w4a8_tile_kernel<128x256,w8>"): 51450000,
-    (7, "w4a8_tile_kernel<256x256,w8>"): 116860000,
+    (7, "w4a8_tile_kernel<128x256,w8>"): 61660000,
+    (7, "w4a8_tile_kernel<256x256,w8>"): 140090000,
 }
 
 

@@ -316,8 +316,8 @@ int dispatch_splitk(const W4A8Params& p, hipStream_t s) {
   return fail(KSQ_ERR_UNSUPPORTED, "no w4a8 kernel for mt=%d nt=%d waves=%d", mt, nt, waves);
 }
 
-// Prefill regime: the MFMA tile kernel of w4a8_tile.h on the grid the blockwise-FP8 planner lays out (same tile
-// shapes, same instruction; a k-step is one 128-deep group).
+// Prefill regime: the MFMA tile kernel of w4a8_tile.h on the grid plan_w4a8_tile lays out (the blockwise-FP8 tile
+// shapes; a k-step is one 128-deep group).
 template <typename TO, int WM>
 int launch_tile(const W4A8Params& q, const TilePlan& plan, float* partial, hipStream_t s) {
   constexpr int kLds = static_cast<int>(w4a8_tile_lds_bytes(WM));
@@ -435,7 +435,7 @@ KSQ_EXPORT size_t ksq_w4a8_workspace_size(size_t max_m, size_t n, size_t k) {
   size_t need = 0;
   for (size_t band_end = 128; max_m > 32; band_end += 128) {
     const size_t m = band_end < max_m ? band_end : max_m;
-    const TilePlan t = plan_fp8_tile(m, n, k);
+    const TilePlan t = plan_w4a8_tile(m, n, k);
     need = t.workspace_bytes > need ? t.workspace_bytes : need;
     if (m == max_m) break;
   }
@@ -469,7 +469,7 @@ KSQ_EXPORT int ksq_w4a8_gemm(const void* a_q, const void* xsum, const void* w_pa
   hipStream_t st = as_stream(stream);
   int rc;
   if (use_tile(m)) {
-    const TilePlan plan = plan_fp8_tile(m, n, k);
+    const TilePlan plan = plan_w4a8_tile(m, n, k);
     if (plan.splits > 1 && (!workspace || workspace_bytes < plan.workspace_bytes || !aligned16(workspace)))
       return fail(KSQ_ERR_WORKSPACE, "%s: m=%zu n=%zu k=%zu needs %zu bytes of 16-byte aligned workspace, got %zu", fn, m,
                   n, k, plan.workspace_bytes, workspace ? workspace_bytes : size_t(0));
