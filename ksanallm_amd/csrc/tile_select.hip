@@ -23,10 +23,15 @@ SplitKChoice select_splitk(size_t m, size_t n, size_t k) {
   const size_t m_blocks = div_up(m, 16 * mt);
   SplitKChoice c = select_splitk_blocks(mt, m_blocks, n, k);
   const size_t strips = n / 16;
-  if (k >= 2 * n && strips % 4 == 0 && c.nt < 4) {
+  if (strips % 4 == 0 && c.nt < 4) {
     const size_t rows = m < static_cast<size_t>(16 * mt) ? m : static_cast<size_t>(16 * mt);
-    const size_t x_bytes = rows * k * 2 * (strips / c.nt) * m_blocks;
-    if (x_bytes > k * n / 2 || k > 16384) {
+    const size_t x_bytes = rows * k * 2 * (strips / c.nt) * m_blocks;  // what all workgroups together read of x
+    // K the long side: whenever x outweighs the weights.  Otherwise from 48 MB of x re-reads: below that the second
+    // pass costs more than the traffic it saves (n = k = 5120: 16 tokens 13.8 -> 9.4 us, 32 tokens 22.1 -> 12.6 us;
+    // n = k = 4096 at 8 tokens, 17 MB of re-reads, would go 5.5 -> 7.0 us)
+    const bool long_k = k >= 2 * n && (x_bytes > k * n / 2 || k > 16384);
+    const bool heavy_x = x_bytes >= (size_t(48) << 20);
+    if (long_k || heavy_x) {
       int parts = 2;
       while (parts < 8 && strips / 4 * m_blocks * parts < 160) parts *= 2;
       while (parts > 1 && k / 128 / parts < 8) parts /= 2;
