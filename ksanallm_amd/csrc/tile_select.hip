@@ -51,7 +51,8 @@ SplitKChoice select_splitk_blocks(int mt, size_t m_blocks, size_t n, size_t k) {
   c.nt = 1;
   c.parts = 1;
   const size_t n_tiles = n / 16;
-  for (int nt = (mt == 1 ? 8 : 4); nt > 1; nt >>= 1) {
+  // (eight column tiles also with two row tiles: n = 25600, k = 5120 at 32 rows 29.0 -> 22.4 us - half the x re-reads)
+  for (int nt = 8; nt > 1; nt >>= 1) {
     if (n_tiles % nt == 0 && n_tiles / nt * m_blocks >= static_cast<size_t>(kNumCU) * 3 / 4) {
       c.nt = nt;
       break;

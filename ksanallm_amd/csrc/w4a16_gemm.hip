@@ -73,6 +73,7 @@ int dispatch_tile(SplitKParams& p, SplitKChoice c, uint32_t m_blocks, size_t gro
   KSQ_CASE(2, 4, 8)
   KSQ_CASE(2, 2, 8)
   KSQ_CASE(2, 1, 8)
+  KSQ_CASE(2, 8, 4)
   KSQ_CASE(2, 4, 4)
   KSQ_CASE(2, 2, 4)
   KSQ_CASE(2, 1, 4)

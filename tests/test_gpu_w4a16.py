@@ -45,6 +45,17 @@ def test_cfg2_awq_bf16(ops, M, N, K):
     H.check_gemm(y, H.w4a16_oracle(d), H.BF16, "cfg2 M=%d N=%d K=%d" % (M, N, K), weights_rounded=M > 32)
 
 
+# decode kernel with eight column tiles per workgroup, one and two row tiles: needs n >= 24576 to keep the grid full
+@pytest.mark.parametrize("dtype", [H.F16, H.BF16])
+@pytest.mark.parametrize("awq", [False, True])
+@pytest.mark.parametrize("M", [3, 20, 32])
+def test_decode_eight_column_tiles(ops, dtype, awq, M):
+    N, K = 24576, 256
+    d = H.make_w4a16(7000 + M, M, N, K, 128, dtype, awq=awq)
+    y = run_case(ops, d)
+    H.check_gemm(y, H.w4a16_oracle(d), dtype, "nt=8 M=%d" % M)
+
+
 # prefill regime (MFMA tile kernel): ragged M, both dtypes, with and without zero points
 @pytest.mark.parametrize("dtype", [H.F16, H.BF16])
 @pytest.mark.parametrize("awq", [False, True])
