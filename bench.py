@@ -445,11 +445,15 @@ def main():
         eager_step()
         torch.cuda.synchronize()
         graphs = [capture([c.launch for c in cases]) for _ in range(n_graphs)]
+        # and one graph that holds a whole turn of the rotation (n_graphs consecutive steps): starting a graph costs
+        # 20-30 us, as much as a step of two decode kernels takes; a serving loop replays graphs of hundreds of kernels
+        turn = capture([c.launch for c in cases] * n_graphs) if n_graphs > 1 else None
 
         def step(i):
             graphs[i % n_graphs].replay()
     else:
         step = eager_step
+        turn = None
 
     for i in range(args.warmup):
         step(i)
@@ -457,8 +461,14 @@ def main():
     t0 = time.perf_counter()
     start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     start.record()
-    for i in range(args.steps):
-        step(args.warmup + i)
+    done = 0
+    while done < args.steps:       # exactly args.steps steps: whole turns while they fit, single steps for the rest
+        if turn is not None and args.steps - done >= n_graphs:
+            turn.replay()
+            done += n_graphs
+        else:
+            step(args.warmup + done)
+            done += 1
     end.record()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
@@ -518,6 +528,7 @@ def main():
         "config": {"workload": workload, "cases": len(cases), "config_index": args.config - 1},
         "tflops": round(total_flops / step_s / 1e12, 3), "hbm_gbps": round(total_bytes / step_s / 1e9, 1),
         "wall_ms_per_step": round(wall_ms, 5), "launch": "hip graph replay" if use_graph else "python launches",
+        "steps_per_graph": (n_graphs if turn is not None and args.steps >= n_graphs else 1),
         "peaks": {"hbm_gbps": HBM_PEAK / 1e9, "mfma_tflops": {k: v / 1e12 for k, v in MFMA_PEAK.items()}},
         "roofline": roof, "per_case": per_case,
     }
