@@ -125,6 +125,10 @@ TilePlan plan_mfma_tile(size_t m, size_t n, size_t k) {
   const unsigned fill = static_cast<unsigned>(kNumCU) * 3 / 4;
   if (t.block_m == 256 && div_up(m, 256) * t.tiles_n < static_cast<unsigned>(kNumCU) / 2 && div_up(m, 128) * t.tiles_n >= fill)
     t.block_m = 128;
+  // very few 256-row tiles (at most 32) are cut so finely along K that their fp32 partial tiles outweigh what the
+  // larger tile saves: 128-row tiles need half the cut (n = k = 4096: 256 rows 34 -> 27 us, 512 rows 42 -> 33 us;
+  // n = 4096, k = 14336 at 256 rows 52 -> 45 us; with K beyond 16384 the larger tile stays 1-3 % ahead)
+  if (t.block_m == 256 && div_up(m, 256) * t.tiles_n <= 32 && k <= 16384) t.block_m = 128;
   t.tiles_m = static_cast<unsigned>(div_up(m, t.block_m));
   static const SpreadCost cost{3.0, 3.0, 2.0, 0.02};
   spread_tiles(t.tiles_m * t.tiles_n, static_cast<unsigned>(k / 128), cost, &t);
