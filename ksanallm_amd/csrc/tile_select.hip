@@ -147,6 +147,9 @@ TilePlan plan_fp8_tile(size_t m, size_t n, size_t k) {
   // 128-token tiles where 256-token ones would be half padding (the weights are then fetched once per 128 tokens);
   // with full tiles the 256-token form is faster (M = 4096: 509 against 641 us)
   t.block_m = (m <= 128 || (m < 1024 && (m - 1) % 256 < 128)) ? 128 : 256;
+  // as in plan_mfma_tile: at most 32 tiles of 256 tokens are better served by 128-token tiles and half the cut along K
+  // (n = k = 5120 at 256 tokens: 31 -> 25 us; n = k = 4096 at 512 tokens: 33 -> 27 us)
+  if (t.block_m == 256 && div_up(m, 256) * div_up(n, 256) <= 32 && k <= 16384) t.block_m = 128;
   t.tiles_m = static_cast<unsigned>(div_up(m, t.block_m));
   t.tiles_n = static_cast<unsigned>(div_up(n, 256));
   // fitted over five shapes at 64..2048 tokens; costlier cuts had left n = 25600, k = 5120 at 64..256 tokens on 100
@@ -163,6 +166,9 @@ TilePlan plan_fp8_tile(size_t m, size_t n, size_t k) {
 TilePlan plan_w4a8_tile(size_t m, size_t n, size_t k) {
   TilePlan t{};
   t.block_m = (m <= 128 || (m < 1024 && (m - 1) % 256 < 128)) ? 128 : 256;
+  // as in plan_mfma_tile: at most 32 tiles of 256 tokens are better served by 128-token tiles and half the cut along K
+  // (n = k = 5120 at 256 tokens: 31 -> 25 us; n = k = 4096 at 512 tokens: 33 -> 27 us)
+  if (t.block_m == 256 && div_up(m, 256) * div_up(n, 256) <= 32 && k <= 16384) t.block_m = 128;
   t.tiles_m = static_cast<unsigned>(div_up(m, t.block_m));
   t.tiles_n = static_cast<unsigned>(div_up(n, 256));
   static const SpreadCost cost{6.0, 4.0, 3.0, 0.03};

@@ -135,9 +135,11 @@ def test_blockwise_gemm(ops, oracle, m, n, k):
 
 # prefill regime (MFMA tile kernel, 256 x 256 or 128 x 256 tiles): ragged M and N, odd k-block counts, split-K through
 # the workspace
-@pytest.mark.parametrize("m,n,k,bm", [(65, 256, 128, 128), (300, 2320, 1152, 128), (256, 7168, 2048, 256), (1024, 512, 4096, 256),
-                                      (130, 4096, 7168, 256), (128, 7168, 2048, 128), (384, 528, 1024, 128), (100, 272, 384, 128),
-                                      (500, 768, 640, 256)])
+# (the last three: more than 32 tiles of 256 tokens, which is where the planner keeps that tile at these sizes)
+@pytest.mark.parametrize("m,n,k,bm", [(65, 256, 128, 128), (300, 2320, 1152, 128), (256, 7168, 2048, 128), (1024, 512, 4096, 128),
+                                      (130, 4096, 7168, 128), (128, 7168, 2048, 128), (384, 528, 1024, 128), (100, 272, 384, 128),
+                                      (500, 768, 640, 128), (512, 4352, 256, 256), (200, 8704, 256, 256),
+                                      (1024, 2304, 384, 256)])
 def test_blockwise_gemm_tile_kernel(ops, oracle, m, n, k, bm):
     from ksanallm_amd import lib as L
     desc = L.select_tile(L.KIND_FP8_BLOCKWISE, m, n, k, H.BF16)

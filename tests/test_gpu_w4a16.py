@@ -69,6 +69,21 @@ def test_prefill_tile_kernel(ops, dtype, awq, M, N, K):
     H.check_gemm(y, H.w4a16_oracle(d), dtype, "prefill M=%d N=%d K=%d" % (M, N, K), weights_rounded=True)
 
 
+# 256-row tiles at sizes the oracle handles: the planner keeps them where more than 32 of them exist (the last case is
+# more than one round of tiles, so that some are cut along K)
+@pytest.mark.parametrize("dtype", [H.F16, H.BF16])
+@pytest.mark.parametrize("awq", [False, True])
+@pytest.mark.parametrize("M,N,K", [(512, 4352, 256), (200, 8704, 256), (1100, 2304, 384), (1300, 12288, 1024)])
+def test_prefill_256_row_tiles(ops, dtype, awq, M, N, K):
+    from ksanallm_amd import lib as L
+    desc = L.select_tile(L.KIND_W4A16, M, N, K, dtype)
+    assert desc["kernel"] == 1 and desc["block_m"] == 256
+    d = H.make_w4a16(3400 + M + N, M, N, K, 128, dtype, awq=awq, x_std=0.5, s_lo=0.002, s_hi=0.01, z_lo=0, z_hi=15)
+    y = run_case(ops, d)
+    H.check_gemm(y, H.w4a16_oracle(d), dtype, "prefill 256-row M=%d N=%d K=%d split=%d" % (M, N, K, desc["split_k"]),
+                 weights_rounded=True)
+
+
 # few output tiles: K is split over workgroups, fp32 partials go through the workspace and a second kernel sums them
 @pytest.mark.parametrize("dtype", [H.F16, H.BF16])
 @pytest.mark.parametrize("M,N,K", [(128, 4096, 14336), (512, 4096, 14336), (64, 512, 2048), (200, 256, 1664)])

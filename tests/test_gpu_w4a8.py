@@ -120,6 +120,9 @@ def test_gemm(ops, oracle, out_dtype, m, n, k):
     (300, 1024, 1024),   # 128-token tiles with a half-empty last block
     (1024, 1024, 2048),
     (515, 13328, 512),
+    (512, 4352, 256),    # the next three: more than 32 tiles of 256 tokens, the sizes that keep the 256-token tile
+    (200, 8704, 256),
+    (1024, 2304, 384),
 ])
 @pytest.mark.parametrize("out_dtype", [H.F16, H.BF16])
 def test_gemm_tile_kernel(ops, oracle, out_dtype, m, n, k):
