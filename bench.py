@@ -36,9 +36,8 @@ MEASURED_TRAFFIC = {
     (2, "w4a16_splitk_kernel<16x16,w4>"): 31050000,
     (2, "w4a16_splitk_kernel<16x64,w4>"): 31900000,
     (2, "w4a16_splitk_kernel<32x64,w4>"): 37040000,
-    (2, "w4a16_tile_kernel<128x256,w8>"): 84610000,
-    (2, "w4a16_tile_kernel<256x256,w8>"): 216470000,
-    (3, "w4a16_tile_kernel<256x256,w8>"): 1591160000,
+    (2, "w4a16_tile_kernel<128x256,w8>"): 94830000,
+    (3, "w4a16_tile_kernel<256x256,w8>"): 1592190000,
     (4, "fp8_group_quant"): 26940000,
     (4, "fp8_splitk_kernel<16x16,w4>"): 133530000,
     (4, "fp8_splitk_kernel<16x32,w4>"): 134280000,
@@ -47,8 +46,8 @@ MEASURED_TRAFFIC = {
     (7, "w4a8_quant"): 12690000,
     (7, "w4a8_splitk_kernel<16x32,w8>"): 14420000,
     (7, "w4a8_splitk_kernel<16x64,w4>"): 68990000,
-    (7, "w4a8_tile_kernel<128x256,w8>"): 61660000,
-    (7, "w4a8_tile_kernel<256x256,w8>"): 140090000,
+    (7, "w4a8_tile_kernel<128x256,w8>"): 60220000,
+    (7, "w4a8_tile_kernel<256x256,w8>"): 197070000,
 }
 
 
