@@ -2,9 +2,11 @@
 """Benchmark of the quantized-GEMM hot path on one MI355X.
 
 One "step" is one pass over every (shape, M) case of the chosen workload with synthetic inputs already resident in
-HBM.  The default workload is the AWQ W4A16 Llama-3-8B MLP sweep (gate/up N=14336,K=4096 and down N=4096,K=14336,
-M in {1,8,32,128,512}, bf16).  Weight copies are rotated so that no launch finds its weights in the 256 MB
-Infinity Cache.
+HBM.  The default workload is the whole metric: the five benchmark configurations (GPTQ fp16 4096^2 decode, AWQ bf16
+Llama-3-8B MLP M = 1..512, GPTQ fp16 Qwen-32B-like prefill M = 2048..8192, blockwise-FP8 DeepSeek-V3 MLP M = 1..4096,
+DeepSeek-V3 int4 MoE block T = 1..4096) in one process and one JSON line; `--config N` runs one of them (6 and 7 are
+the block-fp8 MoE block and W4A8, which are not among the five).  Weight copies are rotated so that no launch finds
+its weights in the 256 MB Infinity Cache.
 
 Prints ONE JSON line.  `value` is the time-weighted fraction of the MI355X roofline over the step, in percent:
 sum over cases of max(bytes / 8 TB/s, flops / MFMA peak) divided by the measured step time.
@@ -27,28 +29,17 @@ MFMA_PEAK = {"f16": 2.5e15, "bf16": 2.5e15, "fp8": 5.0e15}   # dense FLOP/s
 CACHE_BYTES = 320 << 20                            # rotate through more than the Infinity Cache
 
 
-# HBM bytes per launch of a kernel variant, averaged over the cases that run it: rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE (KiB per dispatch), each scaled by the factor the same counter shows for a 256 MiB device copy
-# (`--calibrate-copy`): FETCH_SIZE reads half the bytes moved (x2.0), WRITE_SIZE reads them exactly (x1.0).
-# Keyed by (config, kernel variant); None where no counter run has been made for the current kernel.
-MEASURED_TRAFFIC = {
-    (1, "w4a16_splitk_kernel<16x16,w4>"): 9350000,
-    (2, "w4a16_splitk_kernel<16x16,w4>"): 31050000,
-    (2, "w4a16_splitk_kernel<16x64,w4>"): 31900000,
-    (2, "w4a16_splitk_kernel<32x64,w4>"): 37040000,
-    (2, "w4a16_tile_kernel<128x256,w8>"): 94830000,
-    (3, "w4a16_tile_kernel<256x256,w8>"): 1592190000,
-    (4, "fp8_group_quant"): 26940000,
-    (4, "fp8_splitk_kernel<16x16,w4>"): 133530000,
-    (4, "fp8_splitk_kernel<16x32,w4>"): 134280000,
-    (4, "fp8_tile_kernel<128x256,w8>"): 176820000,
-    (4, "fp8_tile_kernel<256x256,w8>"): 519390000,
-    (7, "w4a8_quant"): 12690000,
-    (7, "w4a8_splitk_kernel<16x32,w8>"): 14420000,
-    (7, "w4a8_splitk_kernel<16x64,w4>"): 68990000,
-    (7, "w4a8_tile_kernel<128x256,w8>"): 60220000,
-    (7, "w4a8_tile_kernel<256x256,w8>"): 197070000,
-}
+def measured_traffic(kernel):
+    """HBM bytes per launch of a kernel variant (fetched + written), from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+    runs whose totals are kept in profiles/traffic.json (each counter scaled by what it reads for a 256 MiB device copy,
+    `--calibrate-copy`); None when no counter run covers the variant."""
+    path = os.path.join(ROOT, "profiles", "traffic.json")
+    if not os.path.exists(path):
+        return None
+    with open(path) as f:
+        table = json.load(f)
+    row = table.get("kernels", {}).get(kernel)
+    return None if row is None else int(row["fetch_bytes"] + row["write_bytes"])
 
 
 def seeded(cfg, idx):
@@ -69,9 +60,10 @@ def awq_pack_cols(codes):
 
 
 class Case:
-    def __init__(self, name, launch, flops, nbytes, peak_key, kernel, copies=1):
+    def __init__(self, name, launch, flops, nbytes, peak_key, kernel, copies=1, kind="", m=0):
         self.name, self.launch, self.flops, self.bytes, self.peak_key, self.kernel = name, launch, flops, nbytes, peak_key, kernel
         self.copies = copies
+        self.kind, self.m = kind, m        # kind: "int4" | "fp8" | "fp8_quant" | "moe_int4" | ...; m: rows / tokens
         t_hbm = nbytes / HBM_PEAK
         t_mfma = flops / MFMA_PEAK[peak_key]
         self.bound = "hbm" if t_hbm >= t_mfma else "mfma"
@@ -82,10 +74,17 @@ def copies_needed(weight_bytes):
     return max(2, min(64, -(-CACHE_BYTES // weight_bytes) + 1))
 
 
+def kernel_label(L, kind, prefix, M, N, K, dt):
+    d = L.select_tile(kind, M, N, K, dt)
+    return "%s<%dx%d,w%d>" % (prefix + ("_splitk_kernel" if d["kernel"] == 0 else "_tile_kernel"),
+                              d["block_m"], d["block_n"], d["waves"])
+
+
 # ------------------------------------------------------------------------------------------------ workloads
 def w4a16_cases(ops, L, cfg, shapes, Ms, dtype, awq, x_std, s_lo, s_hi):
     dev = "cuda"
     tdt = torch.float16 if dtype == "f16" else torch.bfloat16
+    ldt = L.F16 if dtype == "f16" else L.BF16
     cases, keep = [], []
     for si, (tag, N, K) in enumerate(shapes):
         g = seeded(cfg, si)
@@ -101,17 +100,18 @@ def w4a16_cases(ops, L, cfg, shapes, Ms, dtype, awq, x_std, s_lo, s_hi):
         wp1 = ops.repack_weight(q.to(dev), layout, 1, K, N)
         sp1 = ops.repack_scales(scales.to(dev), L.SCALE_GN, 1, K, N, 128)
         zp1 = ops.repack_zeros(awq_pack_cols(zeros).to(dev), L.ZERO_AWQ_PACKED, K, N, 128) if awq else None
-        R = copies_needed(wp1.numel())
+        R = max(copies_needed(wp1.numel()), len(Ms))
         wps = [wp1] + [wp1.clone() for _ in range(R - 1)]
         sps = [sp1] + [sp1.clone() for _ in range(R - 1)]
         zps = [zp1] + [zp1.clone() for _ in range(R - 1)] if awq else [None] * R
         state = {"i": 0}
-        keep.append(dict(q=q, scales=scales, zeros=zeros, N=N, K=K, tag=tag, awq=awq))
+        rec = dict(kind="w4a16", q=q, scales=scales, zeros=zeros, N=N, K=K, tag=tag, awq=awq, x={}, y={})
+        keep.append(rec)
         for mi, M in enumerate(Ms):
             x = (torch.randn((M, K), generator=seeded(cfg, 100 * si + mi + 10)) * x_std).to(tdt).to(dev)
             y = torch.empty((M, N), dtype=tdt, device=dev)
-            keep[-1].setdefault("x", {})[M] = x
-            need = L.load().ksq_w4a16_workspace_size(M, N, K, 128, L.F16 if dtype == "f16" else L.BF16)
+            rec["x"][M], rec["y"][M] = x, y
+            need = L.load().ksq_w4a16_workspace_size(M, N, K, 128, ldt)
             ws = torch.empty(need, dtype=torch.uint8, device=dev) if need else None
 
             def launch(x=x, y=y, N=N, K=K, wps=wps, sps=sps, zps=zps, state=state, R=R, ws=ws):
@@ -119,11 +119,8 @@ def w4a16_cases(ops, L, cfg, shapes, Ms, dtype, awq, x_std, s_lo, s_hi):
                 ops.w4a16_gemm(x, wps[i], sps[i], zps[i], N, K, 128, out=y, workspace=ws)
 
             nbytes = K * N // 2 + G * N * 2 + (G * N // 2 if awq else 0) + 2 * M * K + 2 * M * N
-            flops = 2 * M * N * K
-            desc = L.select_tile(L.KIND_W4A16, M, N, K, L.F16 if dtype == "f16" else L.BF16)
-            kern = "%s<%dx%d,w%d>" % ("w4a16_splitk_kernel" if desc["kernel"] == 0 else "w4a16_tile_kernel",
-                                      desc["block_m"], desc["block_n"], desc["waves"])
-            cases.append(Case("%s:M=%d" % (tag, M), launch, flops, nbytes, dtype, kern, R))
+            cases.append(Case("%s:M=%d" % (tag, M), launch, 2 * M * N * K, nbytes, dtype,
+                              kernel_label(L, L.KIND_W4A16, "w4a16", M, N, K, ldt), R, "int4", M))
     return cases, keep
 
 
@@ -136,13 +133,15 @@ def fp8_cases(ops, L, cfg, shapes, Ms):
         # w/s with w/s ~ N(0, (448/4.2)^2) clipped to +-448 (amax of 16384 normals is about 4.2 sigma)
         wn = (torch.randn((N, K), generator=g) * (448.0 / 4.2)).clamp_(-448, 448)
         b = wn.to(torch.float8_e4m3fn).view(torch.uint8)
+        del wn
         b_s = torch.full(((N + 127) // 128, K // 128), 0.02 * 4.2 / 448.0, dtype=torch.float32)
-        R = copies_needed(b.numel())
+        R = max(copies_needed(b.numel()), len(Ms))
         bs_ = [ops.fp8_repack_weight(b.to(dev))]   # the load-time repack into 2 KiB MFMA fragments
         bs_ += [bs_[0].clone() for _ in range(R - 1)]
         b_sd = b_s.to(dev)
         state = {"i": 0}
-        keep.append(dict(b=b, b_s=b_s, N=N, K=K, tag=tag))
+        rec = dict(kind="fp8", b=b, b_s=b_s, N=N, K=K, tag=tag, x={}, y={}, a_q={}, a_s={})
+        keep.append(rec)
         for mi, M in enumerate(Ms):
             gx = seeded(cfg, 100 * si + mi + 10)
             x = torch.randn((M, K), generator=gx)
@@ -150,6 +149,7 @@ def fp8_cases(ops, L, cfg, shapes, Ms):
             a_q = torch.empty((M, K), dtype=torch.uint8, device=dev)
             a_s = torch.empty((K // 128, M), dtype=torch.float32, device=dev)
             y = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+            rec["x"][M], rec["y"][M], rec["a_q"][M], rec["a_s"][M] = x, y, a_q, a_s
 
             def quant(x=x, a_q=a_q, a_s=a_s, K=K):
                 ops.per_token_group_quant_fp8(x, K, 128, True, False, q=a_q, s=a_s)
@@ -163,12 +163,10 @@ def fp8_cases(ops, L, cfg, shapes, Ms):
 
             quant()
             cases.append(Case("%s:quant:M=%d" % (tag, M), quant, 0, 2 * M * K + M * K + 4 * M * K // 128, "fp8",
-                              "fp8_group_quant"))
+                              "fp8_group_quant", 1, "fp8_quant", M))
             nbytes = N * K + b_s.numel() * 4 + M * K + 4 * M * K // 128 + 2 * M * N
-            desc = L.select_tile(L.KIND_FP8_BLOCKWISE, M, N, K, L.BF16)
-            kern = "%s<%dx%d,w%d>" % ("fp8_splitk_kernel" if desc["kernel"] == 0 else "fp8_tile_kernel",
-                                      desc["block_m"], desc["block_n"], desc["waves"])
-            cases.append(Case("%s:gemm:M=%d" % (tag, M), gemm, 2 * M * N * K, nbytes, "fp8", kern, R))
+            cases.append(Case("%s:gemm:M=%d" % (tag, M), gemm, 2 * M * N * K, nbytes, "fp8",
+                              kernel_label(L, L.KIND_FP8_BLOCKWISE, "fp8", M, N, K, L.BF16), R, "fp8", M))
     return cases, keep
 
 
@@ -176,13 +174,13 @@ def w4a8_cases(ops, L, cfg, shapes, Ms):
     """W4A8: static per-tensor e4m3 quantization of bf16 activations (with the group sums the GEMM needs), then int4
     weights x e4m3 activations on the fp8 matrix instruction."""
     dev = "cuda"
-    cases, keep = [], []
+    cases = []
     for si, (tag, N, K) in enumerate(shapes):
         g = seeded(cfg, si)
         w = torch.randint(0, 256, (K, N // 2), generator=g, dtype=torch.uint8)
         scales = (torch.rand((K // 128, N), generator=g) * 0.012 + 0.003).to(torch.float16)
         wp1 = ops.w4a8_repack_weight(w.to(dev))
-        R = copies_needed(wp1.numel())
+        R = max(copies_needed(wp1.numel()), len(Ms))
         wps = [wp1] + [wp1.clone() for _ in range(R - 1)]
         sc_d = scales.to(dev)
         in_scale = torch.tensor([0.05], dtype=torch.float32, device=dev)
@@ -195,7 +193,7 @@ def w4a8_cases(ops, L, cfg, shapes, Ms):
             xsum = torch.empty((K // 128, M), dtype=torch.float32, device=dev)
             y = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
 
-            def quant(x=x, a_q=a_q, xsum=xsum, M=M, K=K):
+            def quant(x=x, a_q=a_q, xsum=xsum, M=M, K=K, in_scale=in_scale):
                 L.check(L.load().ksq_w4a8_static_quant(x.data_ptr(), in_scale.data_ptr(), a_q.data_ptr(), xsum.data_ptr(),
                                                        M, K, L.W4A8_PER_TENSOR, L.BF16,
                                                        torch.cuda.current_stream().cuda_stream))
@@ -209,25 +207,27 @@ def w4a8_cases(ops, L, cfg, shapes, Ms):
 
             quant()
             cases.append(Case("%s:quant:M=%d" % (tag, M), quant, 0, 2 * M * K + M * K + 4 * M * K // 128, "fp8",
-                              "w4a8_quant"))
+                              "w4a8_quant", 1, "w4a8_quant", M))
             nbytes = N * K // 2 + (K // 128) * N * 2 + M * K + 4 * M * K // 128 + 2 * M * N
-            if M <= 32:
-                nt = 4
-                while nt > 1 and (N % (16 * nt) or N // (16 * nt) < 128):
-                    nt //= 2
-                kern = "w4a8_splitk_kernel<%dx%d,w%d>" % (16 if M <= 16 else 32, 16 * nt, 8 if N // (16 * nt) < 256 else 4)
-            else:
-                d = L.select_tile(L.KIND_FP8_BLOCKWISE, M, N, K, L.BF16)   # the W4A8 tile kernel runs on this plan
-                kern = "w4a8_tile_kernel<%dx%d,w%d>" % (d["block_m"], d["block_n"], d["waves"])
-            cases.append(Case("%s:gemm:M=%d" % (tag, M), gemm, 2 * M * N * K, nbytes, "fp8", kern, R))
-    return cases, keep
+            cases.append(Case("%s:gemm:M=%d" % (tag, M), gemm, 2 * M * N * K, nbytes, "fp8",
+                              kernel_label(L, L.KIND_W4A8, "w4a8", M, N, K, L.BF16), R, "w4a8", M))
+    return cases, []
+
+
+def routing_variants(ids, E, touched_bytes):
+    """Expert-id sets a MoE case alternates between.  With few tokens the touched experts fit into the 256 MB Infinity
+    Cache, and replaying the same ids would time the cache, not HBM: such a case rotates through shifted copies of its
+    ids (expert e -> (e + j*E/R) mod E) so that more than the cache holds passes before a set comes round again."""
+    R = 1 if touched_bytes > CACHE_BYTES else min(8, -(-CACHE_BYTES // touched_bytes) + 1)
+    return [((ids + j * (E // R)) % E).contiguous() for j in range(R)]
 
 
 def moe_cases(ops, L, cfg, Ts, E=256, hidden=7168, inter=2048, topk=8, distinct=32):
     dev = "cuda"
     g = seeded(cfg, 0)
     tdt = torch.bfloat16
-    # `distinct` independent expert slabs tiled to E experts: 5.8 GB of device weights either way
+    # `distinct` independent expert slabs tiled to E experts (expert e holds slab e % distinct): 5.8 GB of device
+    # weights either way
     w13 = torch.randint(0, 256, (distinct, 2 * inter, hidden // 2), generator=g, dtype=torch.uint8)
     w2 = torch.randint(0, 256, (distinct, hidden, inter // 2), generator=g, dtype=torch.uint8)
     s13 = (torch.rand((distinct, 2 * inter, hidden // 128), generator=g) * 0.008 + 0.002).to(tdt)
@@ -238,22 +238,33 @@ def moe_cases(ops, L, cfg, Ts, E=256, hidden=7168, inter=2048, topk=8, distinct=
     w2p = ops.repack_weight(w2.to(dev), L.SRC_MOE_NK, distinct, inter, hidden).repeat(rep)
     s2p = ops.repack_scales(s2.to(dev), L.SCALE_NG, distinct, inter, hidden, 128).repeat(rep)
     per_expert = (2 * inter * hidden // 2 + hidden * inter // 2) + (2 * inter * hidden // 128 + hidden * inter // 128) * 2
+    rec = dict(kind="moe", w13=w13, w2=w2, s13=s13, s2=s2, distinct=distinct, E=E, hidden=hidden, inter=inter, topk=topk,
+               x={}, ids={}, tw={}, out={})
     cases = []
     for ti, T in enumerate(Ts):
         gx = seeded(cfg, 10 + ti)
-        x = torch.randn((T, hidden), generator=gx).to(tdt).to(dev)
+        x = torch.randn((T, hidden), generator=gx).to(tdt)
         logits = torch.randn((T, E), generator=gx)
         tw, ids = torch.topk(torch.softmax(logits, -1), topk, dim=-1)
         touched = int(torch.unique(ids).numel())
-        ids_d, tw_d = ids.to(torch.int32).to(dev), tw.float().contiguous().to(dev)
+        ids = ids.to(torch.int32)
+        rec["x"][T], rec["ids"][T], rec["tw"][T] = x, ids, tw.float().contiguous()
+        x_d, tw_d = x.to(dev), tw.float().contiguous().to(dev)
+        variants = [v.to(dev) for v in routing_variants(ids, E, per_expert * touched)]
+        state = {"i": -1}
+        holder = rec["out"]
 
-        def launch(x=x, ids_d=ids_d, tw_d=tw_d):
-            ops.fused_moe_w4a16(x, w13p, s13p, w2p, s2p, ids_d, tw_d, E, hidden, inter, 128)
+        def launch(x_d=x_d, variants=variants, tw_d=tw_d, state=state, holder=holder, T=T):
+            i = state["i"] = (state["i"] + 1) % len(variants)
+            out = ops.fused_moe_w4a16(x_d, w13p, s13p, w2p, s2p, variants[i], tw_d, E, hidden, inter, 128)
+            if i == 0:
+                holder[T] = out
 
         nbytes = per_expert * touched + 2 * T * hidden * 2 + 64 * T
         flops = 2 * T * topk * (2 * inter * hidden + hidden * inter)
-        cases.append(Case("moe:T=%d" % T, launch, flops, nbytes, "bf16", "moe_w4a16"))
-    return cases, []
+        cases.append(Case("moe:T=%d" % T, launch, flops, nbytes, "bf16", "moe_w4a16 block (align + 2 grouped GEMMs + sum)",
+                          len(variants), "moe_int4", T))
+    return cases, [rec]
 
 
 def moe_fp8_cases(ops, L, cfg, Ts, E=256, hidden=7168, inter=2048, topk=8, distinct=32):
@@ -280,42 +291,60 @@ def moe_fp8_cases(ops, L, cfg, Ts, E=256, hidden=7168, inter=2048, topk=8, disti
         logits = torch.randn((T, E), generator=gx)
         tw, ids = torch.topk(torch.softmax(logits, -1), topk, dim=-1)
         touched = int(torch.unique(ids).numel())
-        ids_d, tw_d = ids.to(torch.int32).to(dev), tw.float().contiguous().to(dev)
+        tw_d = tw.float().contiguous().to(dev)
+        variants = [v.to(dev) for v in routing_variants(ids.to(torch.int32), E, per_expert * touched)]
+        state = {"i": -1}
 
-        def launch(x=x, ids_d=ids_d, tw_d=tw_d):
-            ops.fused_moe_fp8_blockwise(x, w13, s13, w2, s2, ids_d, tw_d)
+        def launch(x=x, variants=variants, tw_d=tw_d, state=state):
+            i = state["i"] = (state["i"] + 1) % len(variants)
+            ops.fused_moe_fp8_blockwise(x, w13, s13, w2, s2, variants[i], tw_d)
 
         nbytes = per_expert * touched + 2 * T * hidden * 2 + 64 * T
         flops = 2 * T * topk * (2 * inter * hidden + hidden * inter)
-        cases.append(Case("moe_fp8:T=%d" % T, launch, flops, nbytes, "fp8", "moe_fp8_blockwise"))
+        cases.append(Case("moe_fp8:T=%d" % T, launch, flops, nbytes, "fp8",
+                          "moe_fp8_blockwise block (quant + align + 2 grouped GEMMs + sum)", len(variants), "moe_fp8", T))
     return cases, []
 
 
+WORKLOADS = {
+    1: "GPTQ W4A16 fp16 N=K=4096 M in {1,16}",
+    2: "AWQ W4A16 bf16 Llama-3-8B MLP gate/up(14336x4096)+down(4096x14336) M in {1,8,32,128,512}",
+    3: "GPTQ W4A16 fp16 Qwen-32B-like (25600x5120)+(5120x25600) M in {2048,4096,8192}",
+    4: "blockwise FP8 DeepSeek-V3 dense MLP (18432x7168)+(7168x18432) M in {1,16,128,1024,4096}",
+    5: "DeepSeek-V3 MoE int4 bf16 E=256 top-8 T in {1,64,512,4096}",
+    6: "DeepSeek-V3 MoE block-fp8 bf16 E=256 top-8 T in {1,64,512,4096}",
+    7: "W4A8 bf16 (5120x5120)+(25600x5120) M in {1,16,64,128,256,4096}",
+    8: "W4A16 decode on large weights: GPTQ bf16 (57344x8192), AWQ bf16 (28672x8192), GPTQ fp16 (25600x5120) M in {1,8,16}",
+}
+DTYPES = {1: "f16", 2: "bf16", 3: "f16", 4: "fp8", 5: "bf16", 6: "fp8", 7: "fp8", 8: "bf16"}
+
+
 def build(cfg, ops, L):
+    """(cases, keep) of one configuration."""
     if cfg == 1:
-        return ("GPTQ W4A16 fp16 N=K=4096 M in {1,16}",) + w4a16_cases(
-            ops, L, 1, [("q_proj", 4096, 4096)], [1, 16], "f16", False, 1.0, 0.004, 0.02) + ("f16",)
+        return w4a16_cases(ops, L, 1, [("q_proj", 4096, 4096)], [1, 16], "f16", False, 1.0, 0.004, 0.02)
     if cfg == 2:
-        return ("AWQ W4A16 bf16 Llama-3-8B MLP gate/up(14336x4096)+down(4096x14336) M in {1,8,32,128,512}",) + \
-            w4a16_cases(ops, L, 2, [("gate_up", 14336, 4096), ("down", 4096, 14336)], [1, 8, 32, 128, 512], "bf16", True,
-                        1.0, 0.003, 0.015) + ("bf16",)
+        return w4a16_cases(ops, L, 2, [("gate_up", 14336, 4096), ("down", 4096, 14336)], [1, 8, 32, 128, 512], "bf16", True,
+                           1.0, 0.003, 0.015)
     if cfg == 3:
-        return ("GPTQ W4A16 fp16 Qwen-32B-like (25600x5120)+(5120x25600) M in {2048,4096,8192}",) + w4a16_cases(
-            ops, L, 3, [("up", 25600, 5120), ("down", 5120, 25600)], [2048, 4096, 8192], "f16", False, 0.5, 0.002,
-            0.01) + ("f16",)
+        return w4a16_cases(ops, L, 3, [("up", 25600, 5120), ("down", 5120, 25600)], [2048, 4096, 8192], "f16", False, 0.5,
+                           0.002, 0.01)
     if cfg == 4:
-        return ("blockwise FP8 DeepSeek-V3 dense MLP (18432x7168)+(7168x18432) M in {1,16,128,1024,4096}",) + \
-            fp8_cases(ops, L, 4, [("up", 18432, 7168), ("down", 7168, 18432)], [1, 16, 128, 1024, 4096]) + ("fp8",)
+        return fp8_cases(ops, L, 4, [("up", 18432, 7168), ("down", 7168, 18432)], [1, 16, 128, 1024, 4096])
     if cfg == 5:
-        return ("DeepSeek-V3 MoE int4 bf16 E=256 top-8 T in {1,64,512,4096}",) + moe_cases(
-            ops, L, 5, [1, 64, 512, 4096]) + ("bf16",)
-    if cfg == 6:  # not one of the reference's five benchmark configurations: the block-fp8 expert path, same shapes as 5
-        return ("DeepSeek-V3 MoE block-fp8 bf16 E=256 top-8 T in {1,64,512,4096}",) + moe_fp8_cases(
-            ops, L, 6, [1, 64, 512, 4096]) + ("fp8",)
-    if cfg == 7:  # not one of the reference's five benchmark configurations: the W4A8 path on the shapes of the
-        # reference's own performance test (finegrained_mixed_dtype_gemm_thop_test.cu:312-321) plus decode and prefill
-        return ("W4A8 bf16 (5120x5120)+(25600x5120) M in {1,16,64,128,256,4096}",) + w4a8_cases(
-            ops, L, 7, [("sq", 5120, 5120), ("up", 25600, 5120)], [1, 16, 64, 128, 256, 4096]) + ("fp8",)
+        return moe_cases(ops, L, 5, [1, 64, 512, 4096])
+    if cfg == 6:  # not one of the five benchmark configurations: the block-fp8 expert path, same shapes as 5
+        return moe_fp8_cases(ops, L, 6, [1, 64, 512, 4096])
+    if cfg == 7:  # not one of the five benchmark configurations: the W4A8 path on the shapes of the reference's own
+        # performance test (finegrained_mixed_dtype_gemm_thop_test.cu:312-321) plus decode and prefill
+        return w4a8_cases(ops, L, 7, [("sq", 5120, 5120), ("up", 25600, 5120)], [1, 16, 64, 128, 256, 4096])
+    if cfg == 8:  # not one of the five benchmark configurations: the decode kernel where a launch moves 64 MB and more
+        a, ka = w4a16_cases(ops, L, 8, [("wide", 57344, 8192)], [1, 8, 16], "bf16", False, 1.0, 0.004, 0.02)
+        b, kb = w4a16_cases(ops, L, 8, [("awq", 28672, 8192)], [1, 8, 16], "bf16", True, 1.0, 0.003, 0.015)
+        c, kc = w4a16_cases(ops, L, 8, [("up", 25600, 5120)], [1, 8, 16], "f16", False, 1.0, 0.004, 0.02)
+        for x in c:
+            x.peak_key = "f16"
+        return a + b + c, ka + kb + kc
     raise SystemExit("unknown --config %d" % cfg)
 
 
@@ -354,53 +383,105 @@ def time_case(c, use_graph):
     return start.elapsed_time(end) / reps
 
 
-def cpu_baseline(cfg, keep, ops):
-    """The oracle's dequantize-to-fp32 + fp32 GEMM on the host cores: one pass over a bounded sample of the workload."""
-    if cfg not in (1, 2) or not keep:
-        return None
+# ------------------------------------------------------------------------------------------------ CPU baseline
+def _bits(t):
+    import numpy as np
+    return t.contiguous().cpu().view(torch.int16).numpy().view(np.uint16)
+
+
+def _err(y_gpu, ref):
+    import numpy as np
+    y = y_gpu.float().cpu().numpy()
+    d = y - ref
+    return {"rel_l2": float(np.linalg.norm(d) / max(np.linalg.norm(ref), 1e-30)), "max_abs": float(np.abs(d).max()),
+            "max_ref": float(np.abs(ref).max())}
+
+
+def cpu_baseline(keeps, budget_s):
+    """The oracle's dequantize-to-fp32 + fp32 GEMM on the host cores over a bounded sample of every configuration
+    (about budget_s seconds each), timed, and held against what the GPU left in its output buffers for the same
+    inputs: the raw figures of the parity bar (rel-L2, max-abs against the fp32 reference) appear beside the timing."""
     import numpy as np
     from oracle import ksq_oracle as orc
     orc.build()
     threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
-    prepared = []
-    for k in keep:
-        tag = orc.BF16 if k["x"][min(k["x"])].dtype == torch.bfloat16 else orc.F16
-        if k["awq"]:
-            codes = orc.awq_unpack(k["q"].numpy().view(np.uint32))
-            zeros = k["zeros"].numpy()
-        else:
-            codes = orc.gptq_unpack(k["q"].numpy().view(np.uint32))
-            zeros = None
-        sb = k["scales"].view(torch.int16).numpy().view(np.uint16)
-        xs = {M: k["x"][M].cpu().view(torch.int16).numpy().view(np.uint16) for M in sorted(k["x"])}
-        prepared.append((k, tag, codes, zeros, sb, xs))
-    # whole passes over the workload until at least 10 s of wall time have been spent (30 s cap inside a pass)
-    flops, t, passes = 0, 0.0, 0
-    while t < 10.0:
-        for k, tag, codes, zeros, sb, xs in prepared:
-            for M, xb in xs.items():
-                t0 = time.perf_counter()
-                orc.w4a16_gemm(xb, codes, sb, zeros, 128, tag)
-                t += time.perf_counter() - t0
-                flops += 2 * M * k["N"] * k["K"]
-                if t > 30.0:
-                    break
-        passes += 1
-    names = ", ".join("%s(%dx%d) M in {%s}" % (k["tag"], k["N"], k["K"], ",".join(map(str, xs)))
-                      for k, _, _, _, _, xs in prepared)
-    return {"value": round(flops / t / 1e12, 6), "unit": "TFLOP/s", "cores": threads, "kind": "port",
-            "sample": "%d pass(es) of the oracle (dequantize to fp32, fp32 GEMM, OpenMP) over %s" % (passes, names),
-            "seconds": round(t, 3)}
+    per_config, accuracy = [], []
+    tot_flops, tot_t = 0, 0.0
+    for cfg in sorted(keeps):
+        flops, t, sample = 0, 0.0, []
+        for k in keeps[cfg]:
+            if k["kind"] == "w4a16":
+                tdt = k["x"][min(k["x"])].dtype
+                tag = orc.BF16 if tdt == torch.bfloat16 else orc.F16
+                codes = orc.awq_unpack(k["q"].numpy().view(np.uint32)) if k["awq"] else orc.gptq_unpack(k["q"].numpy().view(np.uint32))
+                zeros = k["zeros"].numpy() if k["awq"] else None
+                sb = _bits(k["scales"])
+                for M in sorted(k["x"]):
+                    if t > budget_s:
+                        break
+                    rows = min(M, 256)          # prefill cases: the first 256 rows of x
+                    xb = _bits(k["x"][M][:rows])
+                    t0 = time.perf_counter()
+                    ref = orc.w4a16_gemm(xb, codes, sb, zeros, 128, tag)
+                    t += time.perf_counter() - t0
+                    flops += 2 * rows * k["N"] * k["K"]
+                    sample.append("%s:M=%d%s" % (k["tag"], M, "" if rows == M else "[rows 0..%d]" % (rows - 1)))
+                    accuracy.append(dict(case="c%d/%s:M=%d" % (cfg, k["tag"], M), rows=rows, **_err(k["y"][M][:rows], ref)))
+            elif k["kind"] == "fp8":
+                bq, b_s = k["b"].numpy(), k["b_s"].numpy()
+                for M in sorted(k["x"]):
+                    if t > budget_s or M > 128:
+                        break
+                    xb = _bits(k["x"][M])
+                    t0 = time.perf_counter()
+                    qo, so = orc.fp8_group_quant(xb, k["K"], 128, True, False, orc.BF16)
+                    ref = orc.fp8_blockwise_gemm(qo, so, bq, b_s, True)
+                    t += time.perf_counter() - t0
+                    flops += 2 * M * k["N"] * k["K"]
+                    sample.append("%s:M=%d" % (k["tag"], M))
+                    e = _err(k["y"][M], ref)
+                    e["quantizer_bits_equal"] = bool(np.array_equal(k["a_q"][M].cpu().numpy(), qo) and
+                                                     np.array_equal(k["a_s"][M].cpu().numpy(), so))
+                    accuracy.append(dict(case="c%d/%s:gemm:M=%d" % (cfg, k["tag"], M), rows=M, **e))
+            elif k["kind"] == "moe":
+                d = k["distinct"]
+                w13, w2 = k["w13"].numpy(), k["w2"].numpy()
+                s13, s2 = _bits(k["s13"]), _bits(k["s2"])
+                for T in sorted(k["x"]):
+                    if t > budget_s or T > 64:
+                        break
+                    rows = min(T, 4)            # per-expert dequantization dominates: a few tokens already touch 30 experts
+                    ids = (k["ids"][T][:rows] % d).contiguous().numpy().astype(np.int32)   # expert e holds slab e % distinct
+                    t0 = time.perf_counter()
+                    ref = orc.moe_forward(_bits(k["x"][T][:rows]), w13, s13, w2, s2, ids, k["tw"][T][:rows].numpy(), 128, orc.BF16)
+                    t += time.perf_counter() - t0
+                    flops += 2 * rows * k["topk"] * 3 * k["hidden"] * k["inter"]
+                    sample.append("moe:T=%d%s" % (T, "" if rows == T else "[tokens 0..%d]" % (rows - 1)))
+                    if T in k["out"]:
+                        accuracy.append(dict(case="c%d/moe:T=%d" % (cfg, T), rows=rows, **_err(k["out"][T][:rows], np.asarray(ref).reshape(rows, -1))))
+        if t > 0:
+            per_config.append({"config": cfg, "tflops": round(flops / t / 1e12, 6), "seconds": round(t, 3), "sample": ", ".join(sample)})
+            tot_flops += flops
+            tot_t += t
+    if tot_t == 0:
+        return None, accuracy
+    return ({"value": round(tot_flops / tot_t / 1e12, 6), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+             "sample": "the oracle (dequantize to fp32, fp32 GEMM; fp8: quantize + block-scaled GEMM; MoE: per-expert dequantization, "
+                       "both GEMMs, silu*mul, weighted sum; OpenMP) on: " +
+                       "; ".join("config %d: %s" % (p["config"], p["sample"]) for p in per_config),
+             "seconds": round(tot_t, 3), "per_config": per_config}, accuracy)
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--config", type=int, default=2, help="BASELINE.json config number 1..5 (default 2); 6 = block-fp8 MoE, same shapes as 5; 7 = W4A8")
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", default="all", help="'all' (default): the five benchmark configurations 1..5 in one "
+                    "step; or one number: 1..5, 6 = block-fp8 MoE on the shapes of 5, 7 = W4A8, 8 = W4A16 decode on large weights")
     ap.add_argument("--only", default="", help="substring filter on case names (for profiling one case)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-seconds", type=float, default=4.0, help="CPU baseline budget per configuration")
     ap.add_argument("--no-graph", action="store_true", help="launch every kernel from Python instead of replaying "
                     "captured HIP graphs (adds the host's per-launch cost to short kernels)")
     ap.add_argument("--calibrate-copy", action="store_true", help="run only a 256 MiB device-to-device copy a few "
@@ -426,27 +507,38 @@ def main():
     from ksanallm_amd import lib as L
     from ksanallm_amd import ops
 
-    workload, cases, keep, dtype = build(args.config, ops, L)
+    cfgs = [1, 2, 3, 4, 5] if args.config == "all" else [int(args.config)]
+    whole = len(cfgs) > 1
+    cases, keeps = [], {}
+    for cfg in cfgs:
+        cs, keep = build(cfg, ops, L)
+        for c in cs:
+            c.cfg = cfg
+            if whole:
+                c.name = "c%d/%s" % (cfg, c.name)
+        cases += cs
+        keeps[cfg] = keep
     if args.only:
         cases = [c for c in cases if args.only in c.name]
         if not cases:
             raise SystemExit("--only matched no case")
 
     use_graph = not args.no_graph
-    n_graphs = max(c.copies for c in cases)
+    # one captured graph per turn of the weight-copy rotation; step i replays graph i % n_graphs.  The whole metric
+    # moves gigabytes per step, so no weight survives in the Infinity Cache from one step to the next and two graphs do.
+    n_graphs = 2 if whole else max(c.copies for c in cases)
 
     def eager_step(_i=0):
         for c in cases:
             c.launch()
 
     if use_graph:
-        # one captured graph per turn of the weight-copy rotation; step i replays graph i % n_graphs
         eager_step()
         torch.cuda.synchronize()
         graphs = [capture([c.launch for c in cases]) for _ in range(n_graphs)]
         # and one graph that holds a whole turn of the rotation (n_graphs consecutive steps): starting a graph costs
         # 20-30 us, as much as a step of two decode kernels takes; a serving loop replays graphs of hundreds of kernels
-        turn = capture([c.launch for c in cases] * n_graphs) if n_graphs > 1 else None
+        turn = capture([c.launch for c in cases] * n_graphs) if (n_graphs > 1 and not whole) else None
 
         def step(i):
             graphs[i % n_graphs].replay()
@@ -489,11 +581,12 @@ def main():
     step_s = ms_per_step * 1e-3
 
     # dominant kernel = the kernel variant with the largest share of the step; its launches average over the cases
-    # that run it, which is also what a profiler's per-kernel average shows
+    # that run it, which is also what a profiler's per-kernel average shows.  A MoE block is several kernels, not one:
+    # it is left out of this choice unless nothing else runs.
     groups = {}
     for c, p in zip(cases, per_case):
         g = groups.setdefault(c.kernel, {"us": 0.0, "flops": 0, "bytes": 0, "t_hbm": 0.0, "t_mfma": 0.0, "n": 0,
-                                         "peak_key": c.peak_key, "cases": []})
+                                         "peak_key": c.peak_key, "cases": [], "block": c.kind.startswith("moe")})
         g["us"] += p["us"]
         g["flops"] += c.flops
         g["bytes"] += c.bytes
@@ -501,7 +594,8 @@ def main():
         g["t_mfma"] += c.flops / MFMA_PEAK[c.peak_key]
         g["n"] += 1
         g["cases"].append(c.name)
-    dk = max(groups, key=lambda k: groups[k]["us"])
+    single = [k for k in groups if not groups[k]["block"]] or list(groups)
+    dk = max(single, key=lambda k: groups[k]["us"])
     g = groups[dk]
     sec = g["us"] * 1e-6
     if g["t_hbm"] >= g["t_mfma"]:
@@ -512,31 +606,49 @@ def main():
         ach = g["flops"] / sec / 1e12
         roof = {"bound": "mfma", "achieved": round(ach, 3), "peak": MFMA_PEAK[g["peak_key"]] / 1e12, "unit": "TFLOP/s",
                 "frac": round(ach * 1e12 / MFMA_PEAK[g["peak_key"]], 4)}
-    traffic = MEASURED_TRAFFIC.get((args.config, dk))
-    roof["traffic"] = traffic
+    roof["traffic"] = measured_traffic(dk)
     roof["kernel"] = dk
     roof["cases"] = g["cases"]
     roof["avg_launch_us"] = round(g["us"] / g["n"], 2)
     roof["algorithmic_bytes_per_launch"] = g["bytes"] // g["n"]
     roof["algorithmic_flops_per_launch"] = g["flops"] // g["n"]
 
+    # the two throughput targets of the scope contract, from the per-case rows
+    def frac_min(pred):
+        rows = [(p["frac"], p["case"]) for c, p in zip(cases, per_case) if pred(c)]
+        return (min(rows)[0], [r[1] for r in rows]) if rows else (None, [])
+
+    dec, dec_cases = frac_min(lambda c: c.kind == "int4" and c.m <= 16)
+    big = [p["frac"] for c, p in zip(cases, per_case) if c.kind == "int4" and c.m <= 16 and c.bytes >= 64e6]
+    moe_dec, moe_dec_cases = frac_min(lambda c: c.kind == "moe_int4" and c.m <= 64)
+    pre, pre_cases = frac_min(lambda c: c.kind == "fp8" and c.m >= 2048)
+    targets = {
+        "int4_decode_hbm_frac_min": dec, "int4_decode_cases": dec_cases, "int4_decode_goal": 0.70,
+        "int4_decode_64MB_up_hbm_frac_min": min(big) if big else None,
+        "int4_moe_decode_block_hbm_frac_min": moe_dec, "int4_moe_decode_cases": moe_dec_cases,
+        "fp8_prefill_mfma_frac_min": pre, "fp8_prefill_cases": pre_cases, "fp8_prefill_goal": 0.60,
+    }
+
+    workload = "; ".join("config %d: %s" % (c, WORKLOADS[c]) for c in cfgs) if whole else WORKLOADS[cfgs[0]]
     out = {
         "metric": METRIC, "value": round(100.0 * total_bound / step_s, 3), "unit": "% of roofline",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic",
-        "config": {"workload": workload, "cases": len(cases), "config_index": args.config - 1},
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16 / bf16 / fp8-e4m3 by configuration, fp32 accumulation" if whole else DTYPES[cfgs[0]],
+        "data": "synthetic",
+        "config": {"workload": workload, "cases": len(cases), "configs": cfgs},
         "tflops": round(total_flops / step_s / 1e12, 3), "hbm_gbps": round(total_bytes / step_s / 1e9, 1),
         "wall_ms_per_step": round(wall_ms, 5), "launch": "hip graph replay" if use_graph else "python launches",
         "steps_per_graph": (n_graphs if turn is not None and args.steps >= n_graphs else 1),
         "peaks": {"hbm_gbps": HBM_PEAK / 1e9, "mfma_tflops": {k: v / 1e12 for k, v in MFMA_PEAK.items()}},
-        "roofline": roof, "per_case": per_case,
+        "roofline": roof, "targets": targets, "per_case": per_case,
     }
-    if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(args.config, keep, ops)
+    if not args.no_cpu and not args.only:
+        out["cpu_baseline"], out["accuracy_vs_fp32_reference"] = cpu_baseline(keeps, args.cpu_seconds)
     if args.details:
         for p in per_case:
-            print("%-28s %-20s %10.2f us %9.3f TFLOP/s %9.1f GB/s  %s %.1f%%" % (
-                p["case"], p["kernel"], p["us"], p["tflops"], p["gbps"], p["bound"], 100 * p["frac"]), file=sys.stderr)
+            print("%-30s %-32s %10.2f us %9.3f TFLOP/s %9.1f GB/s  %s %.1f%%" % (
+                p["case"], p["kernel"][:32], p["us"], p["tflops"], p["gbps"], p["bound"], 100 * p["frac"]), file=sys.stderr)
     print(json.dumps(out))
 
 

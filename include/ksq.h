@@ -308,7 +308,7 @@ int ksq_moe_sum(const void* in, void* out, size_t tokens, size_t topk, size_t d,
  * (K/machete/machete_wrapper.h:38-109), get_best_gemm_config (K/others/tensorrt-llm/dev/deep_gemm/jit_utils.cuh:143-222)
  * and the threshold sweep of BlockwiseMatMulLayer::Preprocess (S/layers/nvidia/blockwise_matmul_layer.cpp:71-181).
  * ------------------------------------------------------------------------------------------------------------------ */
-enum { KSQ_KIND_W4A16 = 0, KSQ_KIND_FP8_BLOCKWISE = 1, KSQ_KIND_MOE_W4A16 = 2 };
+enum { KSQ_KIND_W4A16 = 0, KSQ_KIND_FP8_BLOCKWISE = 1, KSQ_KIND_MOE_W4A16 = 2, KSQ_KIND_W4A8 = 3 };
 enum { KSQ_KERNEL_SPLITK_WAVE = 0, KSQ_KERNEL_MFMA_TILE = 1 };
 
 typedef struct ksq_tile_desc {
@@ -319,7 +319,7 @@ typedef struct ksq_tile_desc {
   int32_t waves;    /* wavefronts (64 lanes) per workgroup */
   int32_t split_k;  /* k slices reduced inside the kernel (across wavefronts and/or workgroups) */
   int32_t grid;     /* workgroups launched */
-  int32_t reserved;
+  int32_t x_chunk;  /* split-K wavefront kernel: k-tiles of activations staged through LDS at a time; 0 = through registers */
 } ksq_tile_desc;
 
 int ksq_select_tile(int kind, size_t m, size_t n, size_t k, int dtype, ksq_tile_desc* out_desc);

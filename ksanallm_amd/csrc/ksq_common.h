@@ -99,6 +99,8 @@ __device__ __forceinline__ uint32_t pack2(uint16_t lo, uint16_t hi) {
 }
 
 inline size_t div_up(size_t a, size_t b) { return (a + b - 1) / b; }
+inline size_t round_up(size_t a, size_t b) { return div_up(a, b) * b; }
+
 
 // A kernel that asks for more dynamic LDS than the default limit needs hipFuncSetAttribute once per device (the
 // attribute belongs to the function as loaded on that device; a process that drives several GPUs from several threads

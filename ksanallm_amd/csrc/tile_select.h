@@ -9,6 +9,7 @@ struct SplitKChoice {
   int nt;     // 16-column tiles per workgroup
   int waves;  // wavefronts per workgroup; wavefront w takes every waves-th k-tile
   int parts;  // workgroups along K (1: the whole of K in one workgroup); > 1 needs parts*m*n fp32 of workspace
+  int xc;     // 0: x fragments through registers; > 0: x staged through LDS in chunks of xc k-tiles (w4a16_splitk.h)
 };
 
 // m rows in one dense GEMM
@@ -35,5 +36,7 @@ bool use_fp8_tile(size_t m, size_t n, size_t k);
 TilePlan plan_fp8_tile(size_t m, size_t n, size_t k);
 // W4A8 (w4a8_tile.h): the same tile shapes with its own costs of a cut along K
 TilePlan plan_w4a8_tile(size_t m, size_t n, size_t k);
+// W4A8 streaming kernel (up to 32 tokens): column tiles per workgroup and wavefronts that split K (parts is always 1)
+SplitKChoice select_w4a8_splitk(size_t m, size_t n);
 
 }  // namespace ksq

@@ -41,6 +41,26 @@ SplitKChoice select_splitk(size_t m, size_t n, size_t k) {
       }
     }
   }
+  // x through LDS (group 128 only; the caller falls back to the register form otherwise).  Measured on MI355X:
+  // - 17..32 rows: the x fragments are twice the weights' bytes, and fetched as 64-byte pieces of 32 rows they cost
+  //   more than the weights (n = 25600, k = 5120: 27.4 -> 21.7 us; n = 14336, k = 4096: 12.8 -> 11.5 us);
+  // - up to 16 rows: pays from about 48 MB of weights (n = 57344, k = 8192: 1 row 41.9 -> 40.7 us, 16 rows
+  //   47.8 -> 46.3 us; n = 25600, k = 5120 at 16 rows 15.9 -> 15.0 us), not below (n = 14336, k = 4096 at 8 rows:
+  //   7.9 us in registers, 8.4 us through LDS), and with up to 8 rows four column tiles per wavefront beat eight
+  //   (n = 57344, k = 8192, 1 row: 40.7 against 43.1 us).
+  if (c.parts == 1 && strips % 4 == 0) {
+    if (mt == 2 && c.nt == 8) {
+      c.waves = 4;
+      c.xc = 4;
+    } else if (mt == 2 && c.nt == 4) {
+      c.waves = 8;
+      c.xc = 8;
+    } else if (mt == 1 && c.nt >= 4 && n * k / 2 >= (size_t(48) << 20)) {
+      if (m <= 8) c.nt = 4;
+      c.waves = 8;
+      c.xc = 8;
+    }
+  }
   return c;
 }
 
@@ -50,6 +70,7 @@ SplitKChoice select_splitk_blocks(int mt, size_t m_blocks, size_t n, size_t k) {
   c.waves = 4;
   c.nt = 1;
   c.parts = 1;
+  c.xc = 0;
   const size_t n_tiles = n / 16;
   // (eight column tiles also with two row tiles: n = 25600, k = 5120 at 32 rows 29.0 -> 22.4 us - half the x re-reads)
   for (int nt = 8; nt > 1; nt >>= 1) {
@@ -177,6 +198,19 @@ TilePlan plan_w4a8_tile(size_t m, size_t n, size_t k) {
   return t;
 }
 
+// W4A8 decode: a workgroup takes as many 16-column strips (up to 4) as still leave 128 workgroups, and splits K over 8
+// wavefronts instead of 4 when fewer than 256 workgroups are left.
+SplitKChoice select_w4a8_splitk(size_t m, size_t n) {
+  SplitKChoice c{};
+  c.mt = m <= 16 ? 1 : 2;
+  c.nt = 4;
+  while (c.nt > 1 && (n % (16 * c.nt) != 0 || n / (16 * c.nt) < 128)) c.nt /= 2;
+  c.waves = n / (16 * c.nt) < 256 ? 8 : 4;
+  c.parts = 1;
+  c.xc = 0;
+  return c;
+}
+
 }  // namespace ksq
 
 using namespace ksq;
@@ -233,6 +267,7 @@ KSQ_EXPORT int ksq_select_tile(int kind, size_t m, size_t n, size_t k, int dtype
       d->waves = c.waves;
       d->split_k = c.waves * c.parts;
       d->grid = static_cast<int32_t>((n / 16 / c.nt) * div_up(m, 16 * c.mt) * c.parts);
+      d->x_chunk = kind == KSQ_KIND_W4A16 ? c.xc : 0;
       return KSQ_OK;
     }
     case KSQ_KIND_FP8_BLOCKWISE: {
@@ -258,6 +293,28 @@ KSQ_EXPORT int ksq_select_tile(int kind, size_t m, size_t n, size_t k, int dtype
       d->waves = waves;
       d->split_k = waves;
       d->grid = static_cast<int32_t>(div_up(m, 16 * mt) * (n / (16 * nt)));
+      return KSQ_OK;
+    }
+    case KSQ_KIND_W4A8: {
+      if (m > 32) {
+        const TilePlan t = plan_w4a8_tile(m, n, k);
+        d->kernel = KSQ_KERNEL_MFMA_TILE;
+        d->block_m = t.block_m;
+        d->block_n = 256;
+        d->block_k = 128;
+        d->waves = 8;
+        d->split_k = static_cast<int32_t>(t.splits);
+        d->grid = static_cast<int32_t>(t.grid);
+        return KSQ_OK;
+      }
+      const SplitKChoice c = select_w4a8_splitk(m, n);
+      d->kernel = KSQ_KERNEL_SPLITK_WAVE;
+      d->block_m = 16 * c.mt;
+      d->block_n = 16 * c.nt;
+      d->block_k = 128;
+      d->waves = c.waves;
+      d->split_k = c.waves;
+      d->grid = static_cast<int32_t>(div_up(m, 16 * c.mt) * (n / (16 * c.nt)));
       return KSQ_OK;
     }
     default:

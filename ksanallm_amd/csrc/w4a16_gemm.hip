@@ -12,40 +12,46 @@
 namespace ksq {
 namespace {
 
-template <typename T, int MT, int NT, int WAVES, int GROUP, bool HAS_ZP, bool GROUPED>
-void launch_splitk(const SplitKParams& p, uint32_t m_blocks, hipStream_t s) {
+template <typename T, int MT, int NT, int WAVES, int GROUP, bool HAS_ZP, bool GROUPED, int XC = 0>
+int launch_splitk(const SplitKParams& p, uint32_t m_blocks, hipStream_t s) {
   const uint32_t parts = (GROUPED || !p.partial) ? 1u : static_cast<uint32_t>(div_up(p.K / 128, p.kt_per_part));
   dim3 grid(p.N / 16 / NT, m_blocks, parts);
   // ring depth in k-tiles and the wavefronts per SIMD the register budget is cut for
   // (32-row blocks with four column tiles: two k-tiles ahead in the dense form, 12.9 against 14.0 us at n = 14336,
   // k = 4096; the grouped form measured 4 % slower with it and keeps one)
-  constexpr int LOOK = GROUP != 128 ? 2 : (MT == 1 ? (NT == 1 ? 4 : (NT == 2 ? 3 : 2)) : ((NT <= 2 || !GROUPED) ? 2 : 1));
-  constexpr int OCC = (GROUP == 128 && MT == 1 && NT == 1) ? 4 : ((GROUP == 128 && MT == 1 && NT == 2) ? 3 : 2);
-  w4a16_splitk_kernel<T, MT, NT, WAVES, LOOK, OCC, GROUP, HAS_ZP, GROUPED><<<grid, WAVES * 64, 0, s>>>(p);
+  // (the forms that stage x through LDS keep one k-tile in flight per wavefront: twice the wavefronts instead)
+  constexpr int LOOK = XC > 0 ? 1
+                              : (GROUP != 128 ? 2 : (MT == 1 ? (NT == 1 ? 4 : (NT == 2 ? 3 : 2)) : ((NT <= 2 || !GROUPED) ? 2 : 1)));
+  constexpr int OCC = XC > 0 ? ((MT == 1 && NT == 4) ? 4 : 2)
+                             : ((GROUP == 128 && MT == 1 && NT == 1) ? 4 : ((GROUP == 128 && MT == 1 && NT == 2) ? 3 : 2));
+  typedef SplitKLds<MT, NT, WAVES, XC> Lds;
+  auto kernel = &w4a16_splitk_kernel<T, MT, NT, WAVES, LOOK, OCC, GROUP, HAS_ZP, GROUPED, XC>;
+  if (Lds::kBytes > 65536) {
+    static std::atomic<uint64_t> configured{0};
+    if (int rc = allow_dynamic_lds(configured, reinterpret_cast<const void*>(kernel), Lds::kBytes)) return rc;
+  }
+  kernel<<<grid, WAVES * 64, Lds::kBytes, s>>>(p);
+  return KSQ_OK;
 }
 
-template <typename T, int MT, int NT, int WAVES, bool GROUPED>
+template <typename T, int MT, int NT, int WAVES, bool GROUPED, int XC = 0>
 int dispatch_group_zp(const SplitKParams& p, uint32_t m_blocks, size_t group, hipStream_t s) {
   const bool zp = p.zeros != nullptr;
   if (group == 128) {
     if (zp) {
-      if constexpr (!GROUPED) launch_splitk<T, MT, NT, WAVES, 128, true, GROUPED>(p, m_blocks, s);
+      if constexpr (!GROUPED) return launch_splitk<T, MT, NT, WAVES, 128, true, GROUPED, XC>(p, m_blocks, s);
       else return fail(KSQ_ERR_UNSUPPORTED, "grouped W4A16 GEMM with zero points is not built");
-    } else {
-      launch_splitk<T, MT, NT, WAVES, 128, false, GROUPED>(p, m_blocks, s);
     }
-    return KSQ_OK;
+    return launch_splitk<T, MT, NT, WAVES, 128, false, GROUPED, XC>(p, m_blocks, s);
   }
-  if constexpr (NT <= 2 && WAVES == 4 && !GROUPED) {
+  if constexpr (NT <= 2 && WAVES == 4 && !GROUPED && XC == 0) {
     if (group == 64) {
-      if (zp) launch_splitk<T, MT, NT, 4, 64, true, false>(p, m_blocks, s);
-      else launch_splitk<T, MT, NT, 4, 64, false, false>(p, m_blocks, s);
-      return KSQ_OK;
+      return zp ? launch_splitk<T, MT, NT, 4, 64, true, false>(p, m_blocks, s)
+                : launch_splitk<T, MT, NT, 4, 64, false, false>(p, m_blocks, s);
     }
     if (group == 32) {
-      if (zp) launch_splitk<T, MT, NT, 4, 32, true, false>(p, m_blocks, s);
-      else launch_splitk<T, MT, NT, 4, 32, false, false>(p, m_blocks, s);
-      return KSQ_OK;
+      return zp ? launch_splitk<T, MT, NT, 4, 32, true, false>(p, m_blocks, s)
+                : launch_splitk<T, MT, NT, 4, 32, false, false>(p, m_blocks, s);
     }
   }
   return fail(KSQ_ERR_UNSUPPORTED, "group size %zu has no kernel for this tile", group);
@@ -56,9 +62,17 @@ int dispatch_tile(SplitKParams& p, SplitKChoice c, uint32_t m_blocks, size_t gro
   if (group != 128) {  // small groups are only built for the narrow 4-wavefront shapes
     c.nt = (p.N / 16) % 2 == 0 ? 2 : 1;
     c.waves = 4;
+    c.xc = 0;
   }
   p.nibble_mask = 0x000f000fu;
   p.magic2 = T::kMagic2;
+  if constexpr (!GROUPED) {
+    if (c.xc == 8 && c.mt == 1 && c.nt == 4 && c.waves == 8) return dispatch_group_zp<T, 1, 4, 8, false, 8>(p, m_blocks, group, s);
+    if (c.xc == 8 && c.mt == 1 && c.nt == 8 && c.waves == 8) return dispatch_group_zp<T, 1, 8, 8, false, 8>(p, m_blocks, group, s);
+    if (c.xc == 8 && c.mt == 2 && c.nt == 4 && c.waves == 8) return dispatch_group_zp<T, 2, 4, 8, false, 8>(p, m_blocks, group, s);
+    if (c.xc == 4 && c.mt == 2 && c.nt == 8 && c.waves == 4) return dispatch_group_zp<T, 2, 8, 4, false, 4>(p, m_blocks, group, s);
+  }
+  if (c.xc != 0) return fail(KSQ_ERR_UNSUPPORTED, "no split-K kernel for mt=%d nt=%d waves=%d xc=%d", c.mt, c.nt, c.waves, c.xc);
 #define KSQ_CASE(MT_, NT_, W_)                                    \
   if (c.mt == MT_ && c.nt == NT_ && c.waves == W_)                \
     return dispatch_group_zp<T, MT_, NT_, W_, GROUPED>(p, m_blocks, group, s);
@@ -79,6 +93,11 @@ int dispatch_tile(SplitKParams& p, SplitKChoice c, uint32_t m_blocks, size_t gro
   KSQ_CASE(2, 1, 4)
 #undef KSQ_CASE
   return fail(KSQ_ERR_UNSUPPORTED, "no split-K kernel for mt=%d nt=%d waves=%d", c.mt, c.nt, c.waves);
+}
+
+// Workspace of a decode launch that cuts K over `parts` workgroups: the fp32 partial sums [parts][m][n].
+size_t splitk_workspace(const SplitKChoice& c, size_t m, size_t n) {
+  return c.parts > 1 ? static_cast<size_t>(c.parts) * m * n * sizeof(float) : 0;
 }
 
 template <typename T, int WM, bool HAS_ZP>
@@ -154,11 +173,8 @@ KSQ_EXPORT size_t ksq_w4a16_workspace_size(size_t max_m, size_t n, size_t k, siz
   // decode kernel: partial sums when K is cut over workgroups
   if (group == 128) {
     for (size_t m = 1; m <= max_m && m <= 32; ++m) {
-      const SplitKChoice c = select_splitk(m, n, k);
-      if (c.parts > 1) {
-        const size_t bytes = static_cast<size_t>(c.parts) * m * n * sizeof(float);
-        need = bytes > need ? bytes : need;
-      }
+      const size_t bytes = splitk_workspace(select_splitk(m, n, k), m, n);
+      need = bytes > need ? bytes : need;
     }
   }
   // the plan is the same for all m of a band of 128 rows
@@ -173,10 +189,10 @@ KSQ_EXPORT size_t ksq_w4a16_workspace_size(size_t max_m, size_t n, size_t k, siz
   return need;
 }
 
-KSQ_EXPORT int ksq_w4a16_gemm(void* y, const void* x, const void* w_packed, const void* scales_packed,
-                              const void* zeros_packed, void* workspace, size_t workspace_bytes, size_t m, size_t n,
-                              size_t k, size_t group, int dtype, void* stream) {
-  const char* fn = "ksq_w4a16_gemm";
+namespace {
+int w4a16_gemm_impl(const char* fn, void* y, const void* x, const void* w_packed, const void* scales_packed,
+                    const void* zeros_packed, void* workspace, size_t workspace_bytes, size_t m, size_t n, size_t k,
+                    size_t group, int dtype, void* stream) {
   if (int rc = check_common(fn, y, x, w_packed, scales_packed, n, k, group, dtype)) return rc;
   if (m == 0) return KSQ_OK;
   if (m > 0x7fffffffull) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: m too large", fn);
@@ -221,7 +237,7 @@ KSQ_EXPORT int ksq_w4a16_gemm(void* y, const void* x, const void* w_packed, cons
   p.partial = nullptr;
   p.kt_per_part = static_cast<uint32_t>(k / 128);
   if (c.parts > 1 && group == 128) {
-    const size_t need = static_cast<size_t>(c.parts) * m * n * sizeof(float);
+    const size_t need = splitk_workspace(c, m, n);
     if (!workspace || workspace_bytes < need || !aligned16(workspace))
       return fail(KSQ_ERR_WORKSPACE, "%s: m=%zu n=%zu k=%zu needs %zu bytes of 16-byte aligned workspace, got %zu", fn, m, n,
                   k, need, workspace ? workspace_bytes : size_t(0));
@@ -241,6 +257,14 @@ KSQ_EXPORT int ksq_w4a16_gemm(void* y, const void* x, const void* w_packed, cons
       parts_reduce_kernel<BF16><<<blocks, 256, 0, as_stream(stream)>>>(p.partial, static_cast<uint16_t*>(y), mn, parts);
   }
   return check_launch(fn);
+}
+}  // namespace
+
+KSQ_EXPORT int ksq_w4a16_gemm(void* y, const void* x, const void* w_packed, const void* scales_packed,
+                              const void* zeros_packed, void* workspace, size_t workspace_bytes, size_t m, size_t n,
+                              size_t k, size_t group, int dtype, void* stream) {
+  return w4a16_gemm_impl("ksq_w4a16_gemm", y, x, w_packed, scales_packed, zeros_packed, workspace, workspace_bytes, m, n, k,
+                         group, dtype, stream);
 }
 
 namespace {

@@ -26,6 +26,7 @@
 #pragma once
 
 #include "ksq_common.h"
+#include "splitk_reduce.h"
 
 namespace ksq {
 
@@ -43,7 +44,11 @@ struct SplitKParams {
   const float* topk_w;
   uint32_t numel, top_k;
   // K cut over grid.z workgroups as well (dense form): part z covers k-tiles [z*kt_per_part, ...) and writes fp32
-  // partial sums [z][M][N] instead of the output; a second pass adds them up
+  // partial sums [z][M][N] instead of the output; a second pass (parts_reduce_kernel) adds them up in the order of z.
+  // (Summing them in the workgroup that finishes last, found with an arrival counter, measured slower than the second
+  // launch: partial results that cross XCDs have to go through memory with device-scope stores, an atomic and
+  // device-scope loads, three dependent round trips at the end of every workgroup - n = 4096, k = 14336, 8 rows:
+  // 15.6-17.0 us against 10.5 us.)
   float* partial;
   uint32_t kt_per_part;
   // grouped form, gate_up GEMM with silu*mul in the epilogue: the workgroup's first NT/2 column tiles are gate tiles
@@ -71,10 +76,36 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, ui
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, static_cast<int>(bytes), 0x00020000);
 }
 
-template <typename T, int MT, int NT, int WAVES, int LOOK, int OCC, int GROUP, bool HAS_ZP, bool GROUPED>
+// Geometry of the x staging through LDS (XC > 0): the workgroup walks K in chunks of XC k-tiles; the rows of x of one
+// chunk lie in LDS as [row][XC * 256 bytes + 64 bytes of padding] (the padding spreads the sixteen rows that one
+// fragment read touches over all banks), two chunks deep.  The same LDS holds the cross-wavefront reduction at the end.
+template <int MT, int NT, int WAVES, int XC, int XR = 16 * MT>
+struct SplitKLds {
+  static constexpr int kRows = XR;  // rows of x that are staged: 16 * MT, or fewer when the caller has at most that many
+  static constexpr int kRowStride = XC * 256 + 64;
+  static constexpr int kChunkBytes = kRows * kRowStride;
+  static constexpr int kRedBytes = WAVES * NT * MT * 1024;
+  static constexpr int kBytes = (XC > 0 && 2 * kChunkBytes > kRedBytes) ? 2 * kChunkBytes : kRedBytes;
+};
+
+// XC == 0: the x fragments travel through registers, in the same ring as the weights (any group size).
+// XC > 0 (group 128): x is staged through LDS a chunk of XC k-tiles at a time, each row of a chunk fetched with
+// LDS-targeted loads of 1 KiB contiguous bytes; the MFMA fragments are read back from LDS.  That takes the x loads out
+// of the ring (16 * MT registers per slot), turns them from 64-byte pieces of sixteen rows into whole cache lines, and
+// leaves rows beyond M unfetched.
+template <typename T, int MT, int NT, int WAVES, int LOOK, int OCC, int GROUP, bool HAS_ZP, bool GROUPED, int XC = 0,
+          int XR = 16 * MT>
 __global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKParams p) {
   constexpr int GPT = 128 / GROUP;  // groups per k-tile
   constexpr int SPG = GROUP / 32;   // MFMA k-steps per group
+  constexpr bool XLDS = XC > 0;
+  typedef SplitKLds<MT, NT, WAVES, XC, XR> Lds;
+  constexpr int CI = XLDS ? XC / WAVES : 1;                         // rounds per chunk
+  constexpr int ND = XLDS ? Lds::kRows * (XC / 4) / WAVES : 0;      // LDS-targeted loads per wavefront and chunk
+  constexpr int NW = NT * (1 + GPT * (HAS_ZP ? 2 : 1));             // loads of one ring slot (NT weight tiles)
+  static_assert(!XLDS || (GROUP == 128 && XC % 4 == 0 && XC % WAVES == 0 && CI % LOOK == 0 &&
+                          (Lds::kRows * (XC / 4)) % WAVES == 0 && LOOK * NW < 64),
+                "chunk geometry: whole rounds per chunk, whole ring turns per chunk, equal loads per wavefront");
   const int lane = threadIdx.x & 63;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lrow = lane & 15;
@@ -86,7 +117,8 @@ __global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKPar
   // tiles skipped between the workgroup's column tile NT/2-1 and its column tile NT/2 (0 unless fused)
   const uint32_t pair_extra = fused ? p.pair_tiles - NT / 2 : 0;
 
-  __shared__ f32x4 red[WAVES][NT * MT][64];
+  extern __shared__ __attribute__((aligned(16))) char smem[];  // SplitKLds::kBytes
+  f32x4 (*red)[NT * MT][64] = reinterpret_cast<f32x4 (*)[NT * MT][64]>(smem);
 
   // ---- rows of x this lane feeds (row operand: lane l supplies row l%16, k = 8*(l/16)..+7 of each k-step).  A lane
   // whose row lies past M (or is a pad slot) gets an offset beyond the extent of x's buffer resource: its loads fetch
@@ -224,37 +256,146 @@ __global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKPar
   };
 
   // ---- main loop.  The ring holds LOOK k-tiles, each a load group of NT weight tiles (with scales / zero points)
-  // followed by the x fragments; a group is refilled for round cur+LOOK while round cur is consumed, so LOOK-1
-  // whole groups stay in flight behind every wait.  The round count is uniform over the workgroup and a multiple
-  // of LOOK, the surplus rounds load zeros.
+  // followed, in the register form, by the x fragments; a group is refilled for round cur+LOOK while round cur is
+  // consumed, so LOOK-1 whole groups stay in flight behind every wait.  The round count is uniform over the workgroup
+  // and a multiple of LOOK (of the rounds of a chunk in the LDS form), the surplus rounds load zeros.
   const uint32_t slice_len = kt_end - kt_begin;
-  const uint32_t rounds = (slice_len + WAVES * LOOK - 1) / (WAVES * LOOK) * LOOK;
   Slot slot[LOOK][NT];
-  XBuf xb[LOOK];
+  if constexpr (!XLDS) {
+    const uint32_t rounds = (slice_len + WAVES * LOOK - 1) / (WAVES * LOOK) * LOOK;
+    XBuf xb[LOOK];
 #pragma unroll
-  for (int j = 0; j < LOOK; ++j) {
-    const KOff o = koff(j);
+    for (int j = 0; j < LOOK; ++j) {
+      const KOff o = koff(j);
 #pragma unroll
-    for (int t = 0; t < NT; ++t) load_slot(slot[j][t], t, o);
-    load_x(xb[j], o);
-    __builtin_amdgcn_sched_barrier(0);  // keep the groups in issue order, the waits below count on it
-  }
-  for (uint32_t it = 0; it < rounds; it += LOOK) {
+      for (int t = 0; t < NT; ++t) load_slot(slot[j][t], t, o);
+      load_x(xb[j], o);
+      __builtin_amdgcn_sched_barrier(0);  // keep the groups in issue order, the waits below count on it
+    }
+    for (uint32_t it = 0; it < rounds; it += LOOK) {
 #pragma unroll
-    for (int h = 0; h < LOOK; ++h) {
-      const KOff o = koff(it + h + LOOK);  // past the last round this is out of range by construction
-      f32x4 sx[GPT][MT];
-      sum_x(xb[h], sx);
+      for (int h = 0; h < LOOK; ++h) {
+        const KOff o = koff(it + h + LOOK);  // past the last round this is out of range by construction
+        f32x4 sx[GPT][MT];
+        sum_x(xb[h], sx);
 #pragma unroll
-      for (int t = 0; t < NT; ++t) {
-        compute(slot[h][t], xb[h], sx, t);
-        // the refill must be issued here, not sunk below the remaining math: the barriers pin it in place
-        __builtin_amdgcn_sched_barrier(0);
-        load_slot(slot[h][t], t, o);
+        for (int t = 0; t < NT; ++t) {
+          compute(slot[h][t], xb[h], sx, t);
+          // the refill must be issued here, not sunk below the remaining math: the barriers pin it in place
+          __builtin_amdgcn_sched_barrier(0);
+          load_slot(slot[h][t], t, o);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        load_x(xb[h], o);
         __builtin_amdgcn_sched_barrier(0);
       }
-      load_x(xb[h], o);
+    }
+  } else {
+    // Rows of the block that hold data (they come first: pad slots of an expert's block lie at its end).
+    uint32_t nrows;
+    if (GROUPED) {
+      nrows = 0;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+        nrows += static_cast<uint32_t>(__builtin_popcountll(__builtin_amdgcn_ballot_w64(lq == 0 && xrow[mt] != kNoRow)));
+      nrows = __builtin_amdgcn_readfirstlane(nrows);
+    } else {
+      const uint32_t left = p.M - blockIdx.y * (16 * MT);
+      nrows = left < static_cast<uint32_t>(Lds::kRows) ? left : static_cast<uint32_t>(Lds::kRows);
+    }
+    const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<size_t>((__attribute__((address_space(3))) char*)smem));
+    const uint32_t nchunks = (slice_len + XC - 1) / XC;
+    // Chunk c -> LDS buffer c % 2.  Wavefront w issues loads w, w + WAVES, ... of the chunk's kRows * XC/4 loads; load
+    // (r, q) moves k-tiles 4q..4q+3 of row r, 1 KiB contiguous (lane j: bytes 16j..16j+15).  Lanes past the end of the row
+    // (K/128 not a multiple of 4) re-read its start: finite values, multiplied by weights that were loaded as zero.
+    // Loads of rows that hold no data, or of k-tile groups past the range, are skipped: the counts the waits below
+    // rely on do not include these loads.
+    auto stage_chunk = [&](uint32_t c) {
+      const uint32_t kt0 = c * XC;
+#pragma unroll
+      for (int i = 0; i < ND; ++i) {
+        const uint32_t idx = wave + i * WAVES;
+        const uint32_t r = idx / (XC / 4), q = idx % (XC / 4);
+        if (r < nrows && kt0 + 4 * q < slice_len) {
+          uint32_t src_row;
+          if (GROUPED) {
+            const uint32_t v = (MT > 1 && r >= 16) ? xrow[MT - 1] : xrow[0];
+            src_row = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(v), static_cast<int>(r & 15u)));
+          } else {
+            src_row = blockIdx.y * (16 * MT) + r;
+          }
+          const uint32_t kt_abs = kt_begin + kt0 + 4 * q;
+          const char* src = static_cast<const char*>(p.x) + (static_cast<size_t>(src_row) * p.K + static_cast<size_t>(kt_abs) * 128) * 2;
+          const uint32_t left_bytes = (KT - kt_abs) * 256u;  // of the row, from this group's first byte
+          const uint32_t voff = static_cast<uint32_t>(lane) * 16u < left_bytes ? static_cast<uint32_t>(lane) * 16u : 0u;
+          const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_base + (c & 1u) * Lds::kChunkBytes + r * Lds::kRowStride + q * 1024u);
+          // (s_nop 4: scalar operands that a v_readfirstlane produced need five wait states before a vector memory
+          // instruction reads them, and the compiler inserts none inside an assembly statement.  M0 is written here
+          // without being declared: the compiler treats it as a reserved register, rejects it in a clobber list with
+          // a warning, and keeps no value of its own in it across statements - it writes M0 right in front of each
+          // instruction of its own that reads it, and this kernel has none.)
+          asm volatile("s_nop 4\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %2"
+                       :
+                       : "v"(voff), "s"(dst), "s"(src)
+                       : "memory");
+        }
+      }
+    };
+    // fragments of local k-tile `lk` of chunk c: lane (row, quarter) reads 16 bytes of each of the four k-steps
+    auto read_x = [&](XBuf& b, uint32_t c, uint32_t lk) {
+      const char* base = smem + (c & 1u) * Lds::kChunkBytes + lk * 256u + lq * 16;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int d = 0; d < 4; ++d)
+          b.xf[mt][d] = *reinterpret_cast<const u32x4*>(base + ((mt * 16 + lrow) % XR) * Lds::kRowStride + d * 64);
+    };
+    // wait until at most LOOK ring slots' loads are outstanding.  Every staging load of the next chunk was issued
+    // before the CI >= LOOK refills of this chunk, and loads retire in issue order: the chunk has landed.
+    auto wait_staged = [&]() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LOOK * NW) : "memory"); };
+
+    stage_chunk(0);
+#pragma unroll
+    for (int j = 0; j < LOOK; ++j) {
+      const KOff o = koff(j);
+#pragma unroll
+      for (int t = 0; t < NT; ++t) load_slot(slot[j][t], t, o);
       __builtin_amdgcn_sched_barrier(0);
+    }
+    wait_staged();
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");  // no LDS read may move above the barrier
+    for (uint32_t c = 0; c < nchunks; ++c) {
+      if (c + 1 < nchunks) stage_chunk(c + 1);  // into the buffer chunk c-1 used: every wavefront is past the barrier behind it
+#pragma unroll
+      for (int j = 0; j < CI; ++j) {
+        constexpr int kDummy = 0;
+        (void)kDummy;
+        const int h = j % LOOK;
+        const KOff o = koff(c * CI + j + LOOK);
+        XBuf xb;
+        read_x(xb, c, wave + j * WAVES);
+        if (wave + (c * CI + j) * WAVES >= slice_len) {
+          // a surplus round: its k-tile was not staged (whatever the LDS holds there need not be finite) and its
+          // weights and scales were loaded as zero
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int d = 0; d < 4; ++d) xb.xf[mt][d] = u32x4{0u, 0u, 0u, 0u};
+        }
+        f32x4 sx[GPT][MT];
+        sum_x(xb, sx);
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+          compute(slot[h][t], xb, sx, t);
+          __builtin_amdgcn_sched_barrier(0);
+          load_slot(slot[h][t], t, o);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+      wait_staged();
+      __builtin_amdgcn_s_barrier();  // chunk c+1 is in LDS for everyone, and everyone is done with chunk c
+      asm volatile("" ::: "memory");
     }
   }
 
@@ -295,6 +436,7 @@ __global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKPar
     return;
   }
 
+  const bool cut = !GROUPED && p.partial != nullptr;
   for (int idx = threadIdx.x; idx < NT * MT * 64; idx += WAVES * 64) {
     const int l = idx & 63;
     const int tm = idx >> 6;
@@ -319,7 +461,7 @@ __global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKPar
         valid = orow < p.M;
       }
       if (valid) {
-        if (!GROUPED && p.partial)
+        if (cut)
           p.partial[(static_cast<size_t>(blockIdx.z) * p.M + orow) * p.N + col] = v[i];
         else
           static_cast<uint16_t*>(p.y)[static_cast<size_t>(orow) * p.N + col] = T::from_float(v[i] * rw);

@@ -299,11 +299,9 @@ __global__ void __launch_bounds__(WAVES * 64) w4a8_splitk_kernel(W4A8Params p) {
 // 8.1 -> 6.1 us).
 template <typename TO>
 int dispatch_splitk(const W4A8Params& p, hipStream_t s) {
-  const int mt = p.M <= 16 ? 1 : 2;
-  int nt = 4;
-  while (nt > 1 && (p.N % (16 * nt) != 0 || p.N / (16 * nt) < 128)) nt /= 2;
+  const SplitKChoice c = select_w4a8_splitk(p.M, p.N);
+  const int mt = c.mt, nt = c.nt, waves = c.waves;
   const unsigned groups = p.N / (16 * nt);
-  const int waves = groups < 256 ? 8 : 4;
   const dim3 grid(groups, static_cast<unsigned>(div_up(p.M, 16 * mt)), 1);
 #define KSQ_CASE(MT_, NT_, W_)                                                   \
   if (mt == MT_ && nt == NT_ && waves == W_) {                                   \

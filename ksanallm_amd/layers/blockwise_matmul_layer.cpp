@@ -24,7 +24,9 @@ Status BlockwiseMatMulLayer::Init(const std::vector<std::any>& parameters, const
 size_t BlockwiseMatMulLayer::GetWorkspaceSize() {
   const size_t input_size = max_m_ * k_ * GetTypeSize(TYPE_FP8_E4M3);
   const size_t scale_size = max_m_ * DivRoundUpSz(k_, block_size_) * GetTypeSize(TYPE_FP32);
-  input_buffer_size_ = input_size + scale_size;
+  // the GEMM's scratch starts behind the quantized activations on a 256-byte boundary (the library asks for 16-byte
+  // alignment, and max_m * k/128 floats is a multiple of 16 bytes only for some max_m)
+  input_buffer_size_ = (input_size + scale_size + 255) / 256 * 256;
   gemm_workspace_size_ = ksq_fp8_blockwise_workspace_size(max_m_, n_, k_);
   workspace_size_ = input_buffer_size_ + gemm_workspace_size_;
   return workspace_size_;

@@ -14,7 +14,8 @@ Status MarlinMoeLayer::Init(const std::vector<std::any>& parameters, const Runti
   p[10] = static_cast<uint32_t>(1);   // expert_groups_topk
   p[11] = std::string("softmax");     // scoring_func
   p[12] = std::string("greedy");      // topk_method
-  p[13] = false;                      // norm_topk_prob: the norm mode alone decides
+  // norm_topk_prob: in this layer the norm mode alone decides (fused_marlin_moe takes it, marlin_moe_layer.cpp:91-95)
+  p[13] = std::any_cast<const MoeScaleNormMode>(parameters[0]) == MoeScaleNormMode::RE_NORM;
   p[14] = 1.0f;                       // routed_scaling_factor
   p[15] = false;                      // use_e_score_correction_bias
   p[8] = true;                        // the aligned-block flow is the only one here

@@ -165,7 +165,9 @@ Status MoeLayer::Forward(const std::vector<Tensor>& input_tensors, std::vector<T
   char* act_order2 = p;
 
   const int gating_dtype = input_tensors[1].dtype == TYPE_FP32 ? KSQ_F32 : KsqDtype(input_tensors[1].dtype, "MoeLayer");
-  const bool renormalize = norm_topk_prob_ || moe_scale_norm_mode_ == MoeScaleNormMode::RE_NORM;
+  // the routers take norm_topk_prob alone, as in the reference's grouped-top-k flow (moe_layer.cpp:105-109);
+  // moe_scale_norm_mode belongs to the reference's Cutlass MoE flow, which is not the one built here
+  const bool renormalize = norm_topk_prob_;
   // routing (MoeLayer::ExecuteGroupedTopk of the reference, moe_layer.cpp:380-420): the correction bias is input 5
   const void* e_bias = nullptr;
   if (use_e_score_correction_bias_) {

@@ -9,7 +9,7 @@ F16, BF16, F32 = 0, 1, 2
 SRC_GPTQ, SRC_AWQ, SRC_MOE_NK, SRC_INT4X2_KN = 0, 1, 2, 3
 SCALE_GN, SCALE_NG = 0, 1
 ZERO_AWQ_PACKED, ZERO_U8_GN = 0, 1
-KIND_W4A16, KIND_FP8_BLOCKWISE, KIND_MOE_W4A16 = 0, 1, 2
+KIND_W4A16, KIND_FP8_BLOCKWISE, KIND_MOE_W4A16, KIND_W4A8 = 0, 1, 2, 3
 W4A8_PER_TENSOR, W4A8_PER_CHANNEL, W4A8_SUMS_ONLY, W4A8_PER_TOKEN = 0, 1, 2, 3
 
 c_sz = ctypes.c_size_t
@@ -19,7 +19,7 @@ c_i = ctypes.c_int
 
 class TileDesc(ctypes.Structure):
     _fields_ = [(n, ctypes.c_int32) for n in
-                ("kernel", "block_m", "block_n", "block_k", "waves", "split_k", "grid", "reserved")]
+                ("kernel", "block_m", "block_n", "block_k", "waves", "split_k", "grid", "x_chunk")]
 
 
 # name -> (restype, argtypes); also the list the ABI test checks against the header
@@ -104,4 +104,4 @@ def check(rc):
 def select_tile(kind, m, n, k, dtype):
     d = TileDesc()
     check(load().ksq_select_tile(kind, m, n, k, dtype, ctypes.byref(d)))
-    return {n: getattr(d, n) for n, _ in TileDesc._fields_ if n != "reserved"}
+    return {n: getattr(d, n) for n, _ in TileDesc._fields_}

@@ -139,7 +139,7 @@ static int RunBlockwise(int argc, char** argv) {
   mc.quant_config.method = QUANT_BLOCK_FP8_E4M3;
   RuntimeConfig rc;
   rc.inter_data_type = T;
-  rc.max_step_token_num = (m + 3) / 4 * 4;
+  rc.max_step_token_num = argc > 8 ? std::atol(argv[8]) : (m + 3) / 4 * 4;  // optional: the layer's max_m
 
   Tensor loaded = Upload(dir + "/w.bin", TYPE_FP8_E4M3, {n, k});
   loaded.weight_scales = std::make_shared<Tensor>(Upload(dir + "/w_scale.bin", TYPE_FP32, {(n + 127) / 128, k / 128}));
@@ -223,11 +223,14 @@ static int RunW4A8(int argc, char** argv) {
   return 0;
 }
 
-static std::vector<std::any> MoeParams(size_t tokens, size_t E, size_t hidden, size_t inter, size_t topk, bool renorm,
+// renorm: 0 = NO_NORM and norm_topk_prob false, 1 = RE_NORM and norm_topk_prob true, 2 = RE_NORM with norm_topk_prob
+// false (the routers follow norm_topk_prob alone)
+static std::vector<std::any> MoeParams(size_t tokens, size_t E, size_t hidden, size_t inter, size_t topk, int renorm_arg,
                                        float scaling, DataType int_dtype = TYPE_UINT4x2, uint32_t groups = 1,
                                        uint32_t topk_group = 1, const std::string& scoring = "softmax",
                                        bool use_bias = false) {
-  return {renorm ? MoeScaleNormMode::RE_NORM : MoeScaleNormMode::NO_NORM,
+  const bool renorm = renorm_arg == 1;
+  return {renorm_arg != 0 ? MoeScaleNormMode::RE_NORM : MoeScaleNormMode::NO_NORM,
           tokens,
           int(0),
           E,
@@ -256,7 +259,7 @@ static int RunMoe(int argc, char** argv) {
   const DataType T = ParseT(argv[3]);
   const size_t tokens = std::atol(argv[4]), E = std::atol(argv[5]), hidden = std::atol(argv[6]), inter = std::atol(argv[7]),
                topk = std::atol(argv[8]);
-  const bool renorm = std::atoi(argv[9]) != 0;
+  const int renorm = std::atoi(argv[9]);
   const float scaling = static_cast<float>(std::atof(argv[10]));
   // optional grouped routing: groups topk_group scoring use_bias (bias.bin: fp32 [E])
   const uint32_t groups = argc > 11 ? std::atoi(argv[11]) : 1, topk_group = argc > 12 ? std::atoi(argv[12]) : 1;

@@ -133,6 +133,17 @@ def test_blockwise_gemm(ops, oracle, m, n, k):
     H.check_gemm(out, ref, H.BF16, "fp8 m=%d n=%d k=%d" % (m, n, k))
 
 
+# the two shapes of the DeepSeek-V3 dense MLP benchmark at its decode and small-prefill row counts, against the oracle
+@pytest.mark.parametrize("m", [1, 16, 128])
+@pytest.mark.parametrize("n,k", [(18432, 7168), (7168, 18432)])
+def test_blockwise_gemm_benchmark_shapes(ops, oracle, m, n, k):
+    x, bq, bs = make_fp8_problem(oracle, 4150 + m + n, m, n, k)
+    q, s = ops.per_token_group_quant_fp8(x.cuda(), k, 128, True)
+    out = ops.fp8_blockwise_gemm(q, s, packed(ops, bq), torch.from_numpy(bs).cuda(), torch.bfloat16)
+    ref = oracle.fp8_blockwise_gemm(q.cpu().numpy(), s.cpu().numpy(), bq, bs, True)
+    H.check_gemm(out, ref, H.BF16, "fp8 cfg4 m=%d n=%d k=%d" % (m, n, k))
+
+
 # prefill regime (MFMA tile kernel, 256 x 256 or 128 x 256 tiles): ragged M and N, odd k-block counts, split-K through
 # the workspace
 # (the last three: more than 32 tiles of 256 tokens, which is where the planner keeps that tile at these sizes)
@@ -243,12 +254,13 @@ def test_fp8_weight_repack_rejects_bad_shapes(ops):
         assert e.value.code == 1
 
 
-def test_blockwise_gemm_full_size_properties(ops, oracle):
-    """Size-independent properties of the fp8 tile kernel at a full benchmark shape (M = 4096, N = 7168, K = 18432):
+@pytest.mark.parametrize("n,k", [(7168, 18432), (18432, 7168)])
+def test_blockwise_gemm_full_size_properties(ops, oracle, n, k):
+    """Size-independent properties of the fp8 tile kernel at the full benchmark shapes (M = 4096):
     doubling the activations doubles the scales and leaves the codes alone, so every output doubles exactly; permuting
     the rows of x permutes the rows of the output bit for bit."""
-    m, n, k = 4096, 7168, 18432
-    g = H.gen(4700)
+    m = 4096
+    g = H.gen(4700 + n)
     b = torch.randint(0, 256, (n, k), generator=g, dtype=torch.uint8)
     b = torch.where((b & 0x7f) == 0x7f, b & 0xfe, b)          # no NaN codes
     bs = (torch.rand((n // 128, k // 128), generator=g) * 1e-4 + 1e-4).cuda()

@@ -71,8 +71,12 @@ def test_w4a16_layer_act_order(tmp_path, oracle, dtype, backend, m, n, k):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("dtype,m,n,k,fuse", [(H.BF16, 5, 512, 1024, 0), (H.F16, 33, 256, 512, 0), (H.BF16, 16, 512, 1024, 1)])
-def test_blockwise_layer(tmp_path, oracle, dtype, m, n, k, fuse):
+@pytest.mark.parametrize("dtype,m,n,k,fuse,max_m", [(H.BF16, 5, 512, 1024, 0, None), (H.F16, 33, 256, 512, 0, None),
+                                                    (H.BF16, 16, 512, 1024, 1, None),
+                                                    # odd max_m with K cut over workgroups: the GEMM's scratch behind
+                                                    # a_q and a_s must still start on an aligned address
+                                                    (H.BF16, 37, 256, 1664, 0, 37), (H.BF16, 35, 256, 640, 0, 41)])
+def test_blockwise_layer(tmp_path, oracle, dtype, m, n, k, fuse, max_m):
     g = H.gen(9100 + m)
     w = (torch.randn((n, k), generator=g) * 0.02).to(torch.bfloat16).float().numpy()
     bq, bs = oracle.fp8_block_quant_weight(w)
@@ -80,7 +84,7 @@ def test_blockwise_layer(tmp_path, oracle, dtype, m, n, k, fuse):
     bq.tofile(tmp_path / "w.bin")
     bs.astype(np.float32).tofile(tmp_path / "w_scale.bin")
     H.bits_of(x).tofile(tmp_path / "x.bin")
-    run_driver("blockwise", tmp_path, TNAME[dtype], m, n, k, fuse)
+    run_driver("blockwise", tmp_path, TNAME[dtype], m, n, k, fuse, *([] if max_m is None else [max_m]))
     y = read_out(tmp_path / "y.bin", dtype, (m, n))
     q, s = oracle.fp8_group_quant(H.bits_of(x), k, 128, True, bool(fuse), dtype)
     ref = oracle.fp8_blockwise_gemm(q, s, bq, bs, True)
@@ -91,6 +95,8 @@ def test_blockwise_layer(tmp_path, oracle, dtype, m, n, k, fuse):
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype,tokens,renorm,scaling,routing", [
     (H.BF16, 1, 0, 2.5, None), (H.F16, 24, 1, 1.0, None), (H.BF16, 70, 0, 1.0, None), (H.BF16, 400, 0, 1.0, None),
+    # 2: scale-norm mode RE_NORM with norm_topk_prob false - the routers follow norm_topk_prob alone (no renormalization)
+    (H.BF16, 24, 2, 1.0, None),
     # DeepSeek-V3 style routing: 4 groups of 4 experts, 2 kept, sigmoid scores with a correction bias (layer input 5)
     (H.BF16, 33, 1, 2.5, (4, 2, "sigmoid", True)), (H.F16, 5, 0, 1.0, (2, 1, "softmax", False))])
 def test_moe_layer(tmp_path, oracle, dtype, tokens, renorm, scaling, routing):
@@ -107,7 +113,7 @@ def test_moe_layer(tmp_path, oracle, dtype, tokens, renorm, scaling, routing):
         arr.tofile(tmp_path / (name + ".bin"))
     if routing is None:
         run_driver("moe", tmp_path, TNAME[dtype], tokens, E, hidden, inter, topk, renorm, scaling)
-        tw, ids = oracle.moe_topk_softmax(gating.numpy(), topk, bool(renorm), scaling, 2)
+        tw, ids = oracle.moe_topk_softmax(gating.numpy(), topk, renorm == 1, scaling, 2)
     else:
         groups, topk_group, scoring, use_bias = routing
         bias = (torch.rand(E, generator=g) * 0.2 - 0.1) if use_bias else None
@@ -116,7 +122,7 @@ def test_moe_layer(tmp_path, oracle, dtype, tokens, renorm, scaling, routing):
         run_driver("moe", tmp_path, TNAME[dtype], tokens, E, hidden, inter, topk, renorm, scaling, groups, topk_group,
                    scoring, int(use_bias))
         tw, ids = oracle.moe_grouped_topk(gating.numpy(), None if bias is None else bias.numpy(), topk, groups,
-                                          topk_group, scoring == "sigmoid", bool(renorm), scaling, 2)
+                                          topk_group, scoring == "sigmoid", renorm == 1, scaling, 2)
     y = read_out(tmp_path / "y.bin", dtype, (tokens, hidden))
     ref = oracle.moe_forward(H.bits_of(x), w13.numpy(), H.bits_of(s13), w2.numpy(), H.bits_of(s2), ids, tw, 128, dtype)
     ref = oracle.from_bits(ref, dtype)

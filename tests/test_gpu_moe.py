@@ -382,7 +382,7 @@ def _full_size_experts(ops, kind, distinct=16):
 
 
 @pytest.mark.parametrize("kind", ["int4", "fp8"])
-@pytest.mark.parametrize("T", [24, 700, 2304])      # 16-row, 32-row and tile-kernel blocks
+@pytest.mark.parametrize("T", [24, 512, 700, 2304, 4096])      # 16-row, 32-row and tile-kernel blocks; 512 and 4096 are benchmark sizes
 def test_moe_full_size_properties(ops, kind, T):
     E, hidden, inter, topk = 256, 7168, 2048, 8
     w13, s13, w2, s2 = _full_size_experts(ops, kind)

@@ -242,3 +242,76 @@ def test_prefill_full_size_properties(ops, N, K):
     perm = torch.randperm(M, generator=g).cuda()
     yp = ops.w4a16_gemm(x[perm].contiguous(), wp, sp, None, N, K, 128)
     assert torch.equal(yp, y[perm])
+
+
+# decode regime with the activations staged through LDS (17..32 rows; up to 16 rows from 48 MB of weights): K that is
+# not a whole number of 4-k-tile loads, one chunk and several, ragged row counts, both dtypes, with and without zero points
+@pytest.mark.parametrize("dtype,awq", [(H.F16, False), (H.BF16, True), (H.F16, True), (H.BF16, False)])
+@pytest.mark.parametrize("M,N,K,nt,xc", [(17, 14336, 640, 4, 8), (32, 14336, 1664, 4, 8), (25, 14336, 4096, 4, 8),
+                                         (20, 25600, 384, 8, 4), (32, 25600, 1280, 8, 4),
+                                         (1, 28672, 4096, 4, 8), (7, 57344, 2176, 4, 8), (8, 28672, 4096, 4, 8),
+                                         (9, 28672, 4096, 8, 8), (16, 57344, 2176, 8, 8)])
+def test_decode_x_through_lds(ops, dtype, awq, M, N, K, nt, xc):
+    from ksanallm_amd import lib as L
+    desc = L.select_tile(L.KIND_W4A16, M, N, K, dtype)
+    assert desc["kernel"] == 0 and desc["x_chunk"] == xc and desc["block_n"] == 16 * nt
+    d = H.make_w4a16(3900 + M + N + K, M, N, K, 128, dtype, awq=awq, z_lo=0, z_hi=15)
+    y = run_case(ops, d)
+    H.check_gemm(y, H.w4a16_oracle(d), dtype, "decode, x through LDS M=%d N=%d K=%d" % (M, N, K))
+
+
+def _carve(big, offset, t):
+    """copy tensor t into the byte buffer `big` at `offset`; returns (view of the copy, next offset rounded up to 256)"""
+    nbytes = t.numel() * t.element_size()
+    view = big[offset:offset + nbytes].view(t.dtype).view(t.shape)
+    view.copy_(t)
+    return view, (offset + nbytes + 255) // 256 * 256
+
+
+@pytest.mark.parametrize("dtype,awq", [(H.F16, False), (H.BF16, True)])
+@pytest.mark.parametrize("M,N,K", [(1, 4096, 640), (16, 4096, 640), (8, 512, 2176), (32, 1024, 1664), (5, 14336, 4096)])
+def test_decode_rounds_past_k_read_nothing(ops, dtype, awq, M, N, K):
+    """The decode kernels give the k-tiles of rounds past the end of K the byte offset 0x40000000 in the scalar offset of
+    their buffer loads and rely on the hardware's range check (offset + scalar offset against the extent of the
+    resource) to return zeros.  Here every operand lies at the start of one 1.25 GiB allocation filled with 0xFF, so
+    that base + 0x40000000 is mapped memory holding NaN patterns: a load that was not range-checked would bring NaN
+    into the sums."""
+    from ksanallm_amd import lib as L
+    assert L.select_tile(L.KIND_W4A16, M, N, K, dtype)["kernel"] == 0
+    d = H.make_w4a16(4300 + M + N + K, M, N, K, 128, dtype, awq=awq, z_lo=0, z_hi=15)
+    big = torch.full(((5 << 28),), 0xFF, dtype=torch.uint8, device="cuda")
+    off = 0
+    wp, off = _carve(big, off, ops.repack_weight(d["qweight"].cuda(), L.SRC_AWQ if awq else L.SRC_GPTQ, 1, K, N))
+    sp, off = _carve(big, off, ops.repack_scales(d["scales"].cuda(), L.SCALE_GN, 1, K, N, 128))
+    zp = None
+    if awq:
+        zp, off = _carve(big, off, ops.repack_zeros(d["qzeros"].cuda(), L.ZERO_AWQ_PACKED, K, N, 128))
+    x, off = _carve(big, off, d["x"].cuda())
+    y, off = _carve(big, off, torch.zeros((M, N), dtype=H.TORCH_DT[dtype], device="cuda"))
+    ws, off = _carve(big, off, torch.zeros(max(L.load().ksq_w4a16_workspace_size(M, N, K, 128, dtype), 256), dtype=torch.uint8, device="cuda"))
+    assert off < (1 << 28)
+    ops.w4a16_gemm(x, wp, sp, zp, N, K, 128, out=y, workspace=ws)
+    torch.cuda.synchronize()
+    assert torch.isfinite(y.float()).all()
+    H.check_gemm(y, H.w4a16_oracle(d), dtype, "sentinel offsets M=%d N=%d K=%d" % (M, N, K))
+
+
+def test_prefill_full_size_properties_8192_rows(ops):
+    """The largest prefill case of the benchmark (M = 8192, N = 25600, K = 5120): a zero row gives a zero row, doubling
+    the activations doubles the outputs, and the first 128 rows agree with the oracle."""
+    from ksanallm_amd import lib as L
+    M, N, K = 8192, 25600, 5120
+    d = H.make_w4a16(4400, 128, N, K, 128, H.F16, awq=False, x_std=0.5, s_lo=0.002, s_hi=0.01)
+    wp = ops.repack_weight(d["qweight"].cuda(), L.SRC_GPTQ, 1, K, N)
+    sp = ops.repack_scales(d["scales"].cuda(), L.SCALE_GN, 1, K, N, 128)
+    g = H.gen(4401)
+    x = (torch.randn((M, K), generator=g) * 0.5).to(torch.float16)
+    x[:128] = d["x"]
+    x[777] = 0
+    x = x.cuda()
+    y = ops.w4a16_gemm(x, wp, sp, None, N, K, 128)
+    assert torch.all(torch.isfinite(y)) and torch.all(y[777] == 0)
+    H.check_gemm(y[:128], H.w4a16_oracle(d), H.F16, "cfg3 M=8192, rows 0..127", weights_rounded=True)
+    y2 = ops.w4a16_gemm(x * 2, wp, sp, None, N, K, 128)
+    normal = y.abs() >= 2.0 ** -13
+    assert torch.equal(y2[normal], (y * 2)[normal])
