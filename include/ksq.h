@@ -134,6 +134,18 @@ int ksq_w4a16_gemm(void* y, const void* x, const void* w_packed, const void* sca
                    void* workspace, size_t workspace_bytes, size_t m, size_t n, size_t k, size_t group, int dtype,
                    void* stream);
 
+/* The same GEMM without a workspace argument, for callers that cannot allocate or hold device memory of their own at
+ * the call site: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
+ * counterpart in the reference.  The fp32 partial sums of launches that cut K go through a buffer of
+ * KSQ_W4A16_STATIC_WORKSPACE_BYTES that is part of the library's code object (each GPU the library runs on holds it
+ * until the process ends); a call whose plan needs more returns KSQ_ERR_WORKSPACE and leaves y untouched - use
+ * ksq_w4a16_gemm with a workspace then.  The call allocates nothing and frees nothing.  All calls on one GPU share the
+ * buffer: two of them that overlap in time (different streams) race on it; calls on one stream do not. */
+#define KSQ_W4A16_STATIC_WORKSPACE_BYTES (32u << 20)
+size_t ksq_w4a16_static_workspace_bytes(void);
+int ksq_w4a16_gemm_static(void* y, const void* x, const void* w_packed, const void* scales_packed,
+                          const void* zeros_packed, size_t m, size_t n, size_t k, size_t group, int dtype, void* stream);
+
 /* ------------------------------------------------------------------------------------------------------------------
  * FP8 (OCP e4m3) per-token, per-`group`-channel activation quantizer.
  *   amax = max(1e-10, max|x|); s = amax / 448; q = e4m3_rne_satfinite(x / s)   (IEEE fp32 divisions)

@@ -267,6 +267,60 @@ KSQ_EXPORT int ksq_w4a16_gemm(void* y, const void* x, const void* w_packed, cons
                          group, dtype, stream);
 }
 
+// ---- the same GEMM for callers that cannot hand over a workspace --------------------------------------------------
+// The fp32 partial sums of launches that cut K go through this array instead of a caller's buffer.  Every GPU the
+// library runs on holds its own copy from the moment the code object is loaded until the process ends.  The name below is
+// a host-side handle, not a device address: the address on the current device comes from hipGetSymbolAddress, once per
+// device, and only that pointer is ever handed to a kernel.
+static __device__ __align__(256) unsigned char scratch[KSQ_W4A16_STATIC_WORKSPACE_BYTES];
+
+namespace {
+// device address of `scratch` on the current device (nullptr after recording the error)
+void* static_scratch() {
+  static std::atomic<void*> addr[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+    set_error("ksq_w4a16_gemm_static: cannot tell the current device");
+    return nullptr;
+  }
+  void* p = addr[dev].load(std::memory_order_acquire);
+  if (p) return p;
+  const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+  if (e != hipSuccess || !p) {
+    set_error("ksq_w4a16_gemm_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+    return nullptr;
+  }
+  addr[dev].store(p, std::memory_order_release);  // every thread that races here stores the same address
+  return p;
+}
+}  // namespace
+
+KSQ_EXPORT size_t ksq_w4a16_static_workspace_bytes(void) { return KSQ_W4A16_STATIC_WORKSPACE_BYTES; }
+
+KSQ_EXPORT int ksq_w4a16_gemm_static(void* y, const void* x, const void* w_packed, const void* scales_packed,
+                                     const void* zeros_packed, size_t m, size_t n, size_t k, size_t group, int dtype,
+                                     void* stream) {
+  const char* fn = "ksq_w4a16_gemm_static";
+  // what this very call needs (the plan of its m, not the maximum over a range of m)
+  size_t need = 0;
+  if (m > 0 && n > 0 && k > 0 && k % 128 == 0 && n % 16 == 0) {
+    if (use_mfma_tile(m, n, k, group))
+      need = plan_mfma_tile(m, n, k).workspace_bytes;
+    else if (group == 128)
+      need = splitk_workspace(select_splitk(m, n, k), m, n);
+  }
+  if (need > KSQ_W4A16_STATIC_WORKSPACE_BYTES)
+    return fail(KSQ_ERR_WORKSPACE, "%s: m=%zu n=%zu k=%zu needs %zu bytes of scratch, the built-in buffer holds %zu: call "
+                "ksq_w4a16_gemm with a workspace", fn, m, n, k, need, size_t(KSQ_W4A16_STATIC_WORKSPACE_BYTES));
+  void* ws = nullptr;
+  if (need > 0) {
+    ws = static_scratch();
+    if (!ws) return KSQ_ERR_LAUNCH;
+  }
+  return w4a16_gemm_impl(fn, y, x, w_packed, scales_packed, zeros_packed, ws, need > 0 ? KSQ_W4A16_STATIC_WORKSPACE_BYTES : 0,
+                         m, n, k, group, dtype, stream);
+}
+
 namespace {
 int moe_w4a16_gemm_impl(const char* fn, bool fuse_silu, void* out, const void* x, const void* w_packed,
                         const void* scales_packed, const void* zeros_packed, const void* topk_w, const void* sorted_ids,

@@ -1,0 +1,77 @@
+"""ksq_w4a16_gemm_static: the W4A16 GEMM whose scratch is a buffer inside the library, against ksq_w4a16_gemm with a
+caller's workspace - the same kernels on the same plan, so the outputs must agree bit for bit.  Two calls in a row, the
+second on a smaller problem, both with plans that use the scratch (fp32 partial sums of launches that cut K)."""
+import pytest
+import torch
+
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+
+def _problem(ops, L, seed, M, N, K, dtype, awq):
+    d = H.make_w4a16(seed, M, N, K, 128, dtype, awq=awq, x_std=0.5, s_lo=0.002, s_hi=0.01, z_lo=0, z_hi=15)
+    wp = ops.repack_weight(d["qweight"].cuda(), L.SRC_AWQ if awq else L.SRC_GPTQ, 1, K, N)
+    sp = ops.repack_scales(d["scales"].cuda(), L.SCALE_GN, 1, K, N, 128)
+    zp = ops.repack_zeros(d["qzeros"].cuda(), L.ZERO_AWQ_PACKED, K, N, 128) if awq else None
+    return d, d["x"].cuda(), wp, sp, zp
+
+
+def _static(L, x, wp, sp, zp, N, K, dtype):
+    y = torch.full((x.shape[0], N), float("nan"), dtype=x.dtype, device=x.device)
+    L.check(L.load().ksq_w4a16_gemm_static(y.data_ptr(), x.data_ptr(), wp.data_ptr(), sp.data_ptr(),
+                                           None if zp is None else zp.data_ptr(), x.shape[0], N, K, 128, dtype,
+                                           torch.cuda.current_stream().cuda_stream))
+    return y
+
+
+@pytest.mark.parametrize("dtype,awq", [(H.BF16, True), (H.F16, False)])
+def test_static_scratch_matches_workspace_form(dtype, awq):
+    from ksanallm_amd import lib as L
+    from ksanallm_amd import ops
+    lib = L.load()
+    cap = lib.ksq_w4a16_static_workspace_bytes()
+    assert cap == 32 << 20
+    # tile kernel with K cut over workgroups, then the decode kernel with K cut over workgroups on a smaller problem,
+    # then a plan that needs no scratch at all
+    shapes = [(128, 4096, 14336), (8, 1024, 4096), (64, 512, 2048), (3, 768, 256)]
+    for i, (M, N, K) in enumerate(shapes):
+        need = lib.ksq_w4a16_workspace_size(M, N, K, 128, dtype)
+        assert need <= cap and (need > 0 or i == 3), (M, N, K, need)
+        d, x, wp, sp, zp = _problem(ops, L, 8100 + i, M, N, K, dtype, awq)
+        ref = ops.w4a16_gemm(x, wp, sp, zp, N, K, 128)
+        y = _static(L, x, wp, sp, zp, N, K, dtype)
+        torch.cuda.synchronize()
+        assert torch.equal(y.view(torch.int16), ref.view(torch.int16)), (M, N, K)
+        H.check_gemm(y, H.w4a16_oracle(d), dtype, "static scratch M=%d N=%d K=%d" % (M, N, K), weights_rounded=M > 32)
+    # the first problem once more: what the smaller calls left in the buffer must not show
+    M, N, K = shapes[0]
+    d, x, wp, sp, zp = _problem(ops, L, 8100, M, N, K, dtype, awq)
+    assert torch.equal(_static(L, x, wp, sp, zp, N, K, dtype).view(torch.int16),
+                       ops.w4a16_gemm(x, wp, sp, zp, N, K, 128).view(torch.int16))
+
+
+def test_static_scratch_rejects_plans_beyond_its_size():
+    from ksanallm_amd import lib as L
+    lib = L.load()
+    cap = lib.ksq_w4a16_static_workspace_bytes()
+    # a shape whose plan for this very m needs more than the buffer holds
+    found = None
+    for (M, N, K) in [(256, 8192, 28672), (200, 16384, 16384), (256, 14336, 8192), (256, 25600, 5120), (150, 12288, 12288)]:
+        d1 = L.select_tile(L.KIND_W4A16, M, N, K, H.BF16)
+        if d1["kernel"] == 1 and d1["split_k"] > 1 and lib.ksq_w4a16_workspace_size(M, N, K, 128, H.BF16) > cap:
+            # the workspace query is a maximum over all m up to M; the entry point looks at M alone
+            found = (M, N, K)
+            break
+    if found is None:
+        pytest.skip("no probe shape needs more scratch than the buffer holds")
+    M, N, K = found
+    x = torch.zeros((M, K), dtype=torch.bfloat16, device="cuda")
+    w = torch.zeros(K * N // 2, dtype=torch.uint8, device="cuda")
+    s = torch.zeros((K // 128) * N, dtype=torch.bfloat16, device="cuda")
+    y = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+    rc = lib.ksq_w4a16_gemm_static(y.data_ptr(), x.data_ptr(), w.data_ptr(), s.data_ptr(), None, M, N, K, 128, H.BF16,
+                                   torch.cuda.current_stream().cuda_stream)
+    if rc == 0:
+        pytest.skip("the plan for m=%d alone fits" % M)
+    assert rc == 3 and b"scratch" in lib.ksq_last_error_string()
