@@ -92,6 +92,18 @@ int ksq_w4a16_repack_act_order(const void* src_gptq, const void* perm, void* dst
 /* out[r, j] = x[r, perm[j]], x and out [m, k] T, perm int32 [k]; out must not alias x. */
 int ksq_permute_columns(const void* x, const void* perm, void* out, size_t m, size_t k, int dtype, void* stream);
 
+/* Act-order GPTQ weight of which this GPU holds a K range only (row-parallel projection under tensor parallelism,
+ * is_k_full = false: S/layers/nvidia/marlin_matmul_layer.cpp:66-96).  The rows of the range belong to arbitrary groups of
+ * the whole checkpoint, so after sorting by group the runs of equal group have arbitrary lengths; the loader pads every
+ * run to a multiple of 32 rows and the GEMM runs with group size 32 on a scale table with one row per 32 packed rows.
+ * ksq_w4a16_repack_rows: packed row j (of K_dst, a multiple of 128) takes checkpoint row rows[j] of src [K_src/8, N];
+ *   an index outside [0, K_src) marks a padding row, which takes code 8 (contributes nothing under the symmetric zero point).
+ * ksq_gather_columns: out[r, j] = x[r, idx[j]], x [m, k_in], out [m, k_out], 0 where idx[j] is outside [0, k_in).
+ * Replaces the g_idx / perm / is_k_full arguments of gptq_marlin_gemm (K/gptq_marlin/gptq_marlin.cu:568-607). */
+int ksq_w4a16_repack_rows(const void* src_gptq, const void* rows, void* dst_packed, size_t K_src, size_t K_dst, size_t N,
+                          void* stream);
+int ksq_gather_columns(const void* x, const void* idx, void* out, size_t m, size_t k_in, size_t k_out, int dtype, void* stream);
+
 /* The same for expert stacks: out[s, j] = x[s / top_k, perm[topk_ids[s], j]] for the numel = tokens * top_k slots
  * (top_k = 1: x holds one row per slot already, as in front of the second MoE GEMM); perm int32 [E, k], out [numel, k]
  * T, read by the grouped GEMM with top_k = 1.  Ids outside [0, E) take expert 0's permutation; the grouped GEMM never

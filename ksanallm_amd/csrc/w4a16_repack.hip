@@ -100,6 +100,46 @@ __global__ void __launch_bounds__(256) repack_act_order_kernel(const uint32_t* _
   dst[o] = out;
 }
 
+// The same for a K range cut out of an act-order checkpoint (a tensor-parallel rank's rows): the packed weight has
+// K_dst >= K_src rows, packed row j takes checkpoint row rows[j], and a row index outside [0, K_src) stands for a padding
+// row that must contribute nothing: it takes code 8, the symmetric zero point.
+__global__ void __launch_bounds__(256) repack_rows_kernel(const uint32_t* __restrict__ src, const int32_t* __restrict__ rows,
+                                                          uint32_t* __restrict__ dst, uint32_t K_src, Geometry g) {
+  size_t o = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  size_t total = g.K * g.N / 8;
+  if (o >= total) return;
+  size_t tile = o / 256;
+  int within = static_cast<int>(o % 256);
+  int lane = within / 4, d = within % 4;
+  size_t kt = tile % g.k_tiles;
+  size_t nt = tile / g.k_tiles;
+  size_t n = nt * 16 + (lane % 16);
+  size_t kbase = kt * 128 + d * 32 + (lane / 16) * 8;
+  uint32_t out = 0;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const uint32_t row = static_cast<uint32_t>(rows[kbase + j]);
+    uint32_t code = 8u;
+    if (row < K_src) code = (src[static_cast<size_t>(row / 8) * g.N + n] >> (4 * (row % 8))) & 15u;
+    out |= code << (4 * packed_nibble(j));
+  }
+  dst[o] = out;
+}
+
+// out[r, j] = x[r, idx[j]] for j < k_out, 0 where idx[j] lies outside [0, k_in): the activation side of the above
+__global__ void __launch_bounds__(256) gather_columns_kernel(const uint16_t* __restrict__ x, const int32_t* __restrict__ idx,
+                                                             uint16_t* __restrict__ out, size_t m, uint32_t k_in, uint32_t k_out) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;  // one thread per 2 output columns
+  const size_t per_row = k_out / 2;
+  if (i >= m * per_row) return;
+  const size_t r = i / per_row;
+  const uint32_t c = static_cast<uint32_t>(i % per_row) * 2;
+  const uint32_t p0 = static_cast<uint32_t>(idx[c]), p1 = static_cast<uint32_t>(idx[c + 1]);
+  const uint16_t* row = x + r * k_in;
+  const uint32_t lo = p0 < k_in ? row[p0] : 0u, hi = p1 < k_in ? row[p1] : 0u;
+  reinterpret_cast<uint32_t*>(out + r * k_out)[c / 2] = lo | (hi << 16);
+}
+
 // out[r, j] = x[r, perm[j]]: the activation side of act-order
 __global__ void __launch_bounds__(256) permute_columns_kernel(const uint16_t* __restrict__ x, const int32_t* __restrict__ perm,
                                                               uint16_t* __restrict__ out, size_t m, uint32_t k) {
@@ -405,6 +445,38 @@ KSQ_EXPORT int ksq_permute_columns(const void* x, const void* perm, void* out, s
   permute_columns_kernel<<<static_cast<unsigned>(blocks), 256, 0, as_stream(stream)>>>(
       static_cast<const uint16_t*>(x), static_cast<const int32_t*>(perm), static_cast<uint16_t*>(out), m,
       static_cast<uint32_t>(k));
+  return check_launch(fn);
+}
+
+KSQ_EXPORT int ksq_w4a16_repack_rows(const void* src_gptq, const void* rows, void* dst, size_t K_src, size_t K_dst, size_t N,
+                                     void* stream) {
+  const char* fn = "ksq_w4a16_repack_rows";
+  if (int rc = check_weight_args(src_gptq, dst, 1, K_dst, N, fn)) return rc;
+  if (K_src == 0 || K_src % 8 != 0 || K_src > 0x7fffffffull) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: K_src must be a positive multiple of 8", fn);
+  if (!rows || (reinterpret_cast<uintptr_t>(rows) & 3u)) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: rows must be a 4-byte aligned pointer", fn);
+  Geometry g{1, K_dst, N, K_dst / 128, N / 16};
+  unsigned blocks = static_cast<unsigned>(div_up(K_dst * N / 8, 256));
+  repack_rows_kernel<<<blocks, 256, 0, as_stream(stream)>>>(static_cast<const uint32_t*>(src_gptq), static_cast<const int32_t*>(rows),
+                                                             static_cast<uint32_t*>(dst), static_cast<uint32_t>(K_src), g);
+  return check_launch(fn);
+}
+
+KSQ_EXPORT int ksq_gather_columns(const void* x, const void* idx, void* out, size_t m, size_t k_in, size_t k_out, int dtype,
+                                  void* stream) {
+  const char* fn = "ksq_gather_columns";
+  if (!x || !idx || !out) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: null pointer", fn);
+  if ((reinterpret_cast<uintptr_t>(x) & 1u) || (reinterpret_cast<uintptr_t>(out) & 3u) || (reinterpret_cast<uintptr_t>(idx) & 3u))
+    return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: x must be 2-byte, out and idx 4-byte aligned", fn);
+  if (dtype != KSQ_F16 && dtype != KSQ_BF16) return fail(KSQ_ERR_UNSUPPORTED, "%s: dtype must be f16 or bf16", fn);
+  if (k_in == 0 || k_out == 0 || k_out % 2 != 0 || k_in > 0x7fffffffull || k_out > 0x7fffffffull)
+    return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: k_in must be positive, k_out positive and even", fn);
+  if (x == out) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: cannot gather in place", fn);
+  if (m == 0) return KSQ_OK;
+  const size_t blocks = div_up(m * (k_out / 2), 256);
+  if (blocks > 0x7fffffffull) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: tensor too large", fn);
+  gather_columns_kernel<<<static_cast<unsigned>(blocks), 256, 0, as_stream(stream)>>>(
+      static_cast<const uint16_t*>(x), static_cast<const int32_t*>(idx), static_cast<uint16_t*>(out), m,
+      static_cast<uint32_t>(k_in), static_cast<uint32_t>(k_out));
   return check_launch(fn);
 }
 

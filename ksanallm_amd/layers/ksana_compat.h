@@ -8,12 +8,16 @@
 //   Tensor                  src/ksana_llm/utils/tensor.h (shape/dtype/GetPtr and the quantization side tensors)
 //   Context, Stream         src/ksana_llm/utils/context.h, utils/nvidia/cuda_utils.h
 //   RuntimeConfig           src/ksana_llm/utils/config/schedule_config_parser.h:316
-//   ModelConfig, QuantMode, LinearComputeBackend, MoeComputeBackend   src/ksana_llm/utils/config/model_config.h:36-120
+//   ModelConfig, QuantConfig, MoeConfig, MlaConfig, QuantMode, LinearComputeBackend, MoeComputeBackend
+//                           src/ksana_llm/utils/config/model_config.h:36-212 (the members the factories read)
+//   WeightStatus            src/ksana_llm/weight_status.h:16-19
+//   BaseWeight              src/ksana_llm/models/base/base_weight.h:14-22 (GetModelWeights only)
 //   Singleton               src/ksana_llm/utils/singleton.h
 #pragma once
 
 #ifdef KSQ_IN_KSANA_TREE
 #  include "ksana_llm/models/common_moe/moe_config.h"
+#  include "ksana_llm/models/base/base_weight.h"
 #  include "ksana_llm/utils/context.h"
 #  include "ksana_llm/utils/singleton.h"
 #  include "ksana_llm/utils/status.h"
@@ -29,6 +33,7 @@
 #  include <sstream>
 #  include <stdexcept>
 #  include <string>
+#  include <unordered_map>
 #  include <vector>
 
 namespace ksana_llm {
@@ -183,18 +188,6 @@ class Stream {
   hipStream_t stream_;
 };
 
-class Context {
- public:
-  explicit Context(int tensor_parallel_size = 1, hipStream_t compute_stream = nullptr)
-      : tp_(tensor_parallel_size), compute_streams_(static_cast<size_t>(tensor_parallel_size), Stream(compute_stream)) {}
-  int GetTensorParallelSize() const { return tp_; }
-  std::vector<Stream>& GetComputeStreams() { return compute_streams_; }
-
- private:
-  int tp_;
-  std::vector<Stream> compute_streams_;
-};
-
 struct BaseLayerParameters {};
 
 enum QuantMode {
@@ -216,6 +209,35 @@ enum LinearComputeBackend {
   MACHETE_LINEAR_BACKEND
 };
 enum MoeComputeBackend { DEFAULT_MOE_BACKEND, CUTLASS_MOE_BACKEND, MARLIN_MOE_BACKEND, TRITON_MOE_BACKEND };
+enum class W4AFP8_MOE_BACKEND { Default, GroupTriton, TensorTriton };
+
+// What the loader records about one weight (src/ksana_llm/weight_status.h:16-19): W4A8 weights carry their n and k here.
+struct WeightStatus {
+  QuantMode quant_mode = QuantMode::QUANT_NONE;
+  std::unordered_map<std::string, size_t> layout;
+};
+
+class Context {
+ public:
+  explicit Context(int tensor_parallel_size = 1, hipStream_t compute_stream = nullptr)
+      : tp_(tensor_parallel_size), compute_streams_(static_cast<size_t>(tensor_parallel_size), Stream(compute_stream)) {}
+  int GetTensorParallelSize() const { return tp_; }
+  std::vector<Stream>& GetComputeStreams() { return compute_streams_; }
+  void SetWeightStatus(const std::string& key, const WeightStatus& status) { weight_status_map_[key] = status; }
+  WeightStatus& GetWeightStatus(const std::string& key) { return weight_status_map_[key]; }  // default entry if absent
+
+ private:
+  int tp_;
+  std::vector<Stream> compute_streams_;
+  std::unordered_map<std::string, WeightStatus> weight_status_map_;
+};
+
+// The part of the model-weight interface the factories use (src/ksana_llm/models/base/base_weight.h:14-22).
+class BaseWeight {
+ public:
+  virtual ~BaseWeight() {}
+  virtual Tensor GetModelWeights(const std::string& weight_name) = 0;
+};
 enum class MoeScaleNormMode { NO_NORM = 0, RE_NORM = 1 };
 
 struct QuantConfig {
@@ -225,14 +247,47 @@ struct QuantConfig {
   bool desc_act = false;
   std::vector<size_t> weight_block_size{128, 128};
   LinearComputeBackend backend = CUTLASS_LINEAR_BACKEND;
+  bool is_fp8_blockwise = false;
+  std::vector<std::string> pattern_layers;
+  std::vector<std::string> ignored_layers;
+};
+
+struct MoeConfig {
+  size_t num_experts = 1;
+  size_t experts_topk = 1;
+  size_t moe_inter_size = 0;
+  size_t shared_expert_inter_size = 0;
+  uint32_t num_expert_group = 1;
+  uint32_t expert_groups_topk = 1;
+  std::string scoring_func = "softmax";
+  std::string topk_method = "greedy";
+  bool norm_topk_prob = false;
+  bool use_e_score_correction_bias = false;
+  float routed_scaling_factor = 1.0f;
+  bool use_vllm_moe = false;
+  bool apply_weight = false;
+};
+
+struct MlaConfig {
+  uint32_t q_lora_rank = 0;
+  uint32_t kv_lora_rank = 0;
+  uint32_t qk_nope_head_dim = 0;
+  uint32_t qk_rope_head_dim = 0;
+  uint32_t v_head_dim = 0;
 };
 
 struct ModelConfig {
   std::string type;
   bool is_quant = false;
   QuantConfig quant_config;
+  std::vector<QuantConfig> sub_quant_configs;
   size_t hidden_units = 0;
   size_t inter_size = 0;
+  size_t head_num = 0;
+  size_t num_key_value_heads = 0;
+  size_t size_per_head = 0;
+  MoeConfig moe_config;
+  MlaConfig mla_config;
 };
 
 struct ParallelismBasicConfig {
@@ -250,6 +305,7 @@ struct RuntimeConfig {
   size_t max_batch_size = 256;
   size_t max_step_token_num = 4096;
   bool enable_full_shared_expert = false;
+  W4AFP8_MOE_BACKEND w4afp8_moe_backend = W4AFP8_MOE_BACKEND::Default;
 };
 
 template <typename T>

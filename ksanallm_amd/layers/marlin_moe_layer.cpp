@@ -5,10 +5,17 @@ namespace ksana_llm {
 Status MarlinMoeLayer::Init(const std::vector<std::any>& parameters, const RuntimeConfig& runtime_config,
                             std::shared_ptr<Context> context, int rank) {
   if (parameters.size() < 20) return Status(RET_INVALID_ARGUMENT, "MarlinMoeLayer: expects 20 init parameters");
-  // the same values in MoeLayer's order: the layer index is the one this interface does not carry
-  std::vector<std::any> p(parameters.begin(), parameters.begin() + 2);
-  p.push_back(static_cast<int>(0));
-  p.insert(p.end(), parameters.begin() + 2, parameters.begin() + 20);
+  // the same values in MoeLayer's order.  The reference's Init reads 20 values without a layer index
+  // (marlin_moe_layer.cpp:17-36), while its factory's vector carries the layer index as third value
+  // (moe_layer_factory.cpp:150-151): both orders are accepted, told apart by the type of the third value.
+  std::vector<std::any> p;
+  if (parameters.size() >= 21 && parameters[2].type() == typeid(int)) {
+    p.assign(parameters.begin(), parameters.begin() + 21);
+  } else {
+    p.assign(parameters.begin(), parameters.begin() + 2);
+    p.push_back(static_cast<int>(0));
+    p.insert(p.end(), parameters.begin() + 2, parameters.begin() + 20);
+  }
   // fused_marlin_moe routes with a plain softmax top-k whatever the routing fields say, and never scales the weights
   p[9] = static_cast<uint32_t>(1);    // num_expert_group
   p[10] = static_cast<uint32_t>(1);   // expert_groups_topk
@@ -19,7 +26,7 @@ Status MarlinMoeLayer::Init(const std::vector<std::any>& parameters, const Runti
   p[14] = 1.0f;                       // routed_scaling_factor
   p[15] = false;                      // use_e_score_correction_bias
   p[8] = true;                        // the aligned-block flow is the only one here
-  if (std::any_cast<DataType>(parameters[16]) != TYPE_INVALID)
+  if (std::any_cast<DataType>(p[17]) != TYPE_INVALID)
     return Status(RET_INVALID_ARGUMENT, "MarlinMoeLayer: fp8 expert weights do not belong to this layer");
   p[18] = TYPE_UINT4x2;               // int_weight_dtype: 4-bit codes, two per byte
   if (runtime_config.inter_data_type != TYPE_FP16)

@@ -5,18 +5,86 @@
 
 namespace ksana_llm {
 
+namespace {
+
+// Act-order weight of which this rank holds a K range: `groups` are the checkpoint-wide group numbers of its K rows,
+// `scales` [G_total, N] the scales of all groups.  Sorted by group, the runs of equal group have arbitrary lengths: each
+// run is padded to a multiple of 32 rows (padding rows: index -1, code 8, no contribution) and the whole to a multiple of
+// 128, and the scale table gets one row per 32 packed rows, so that the group-32 kernels apply the scales by position.
+Tensor PackActOrderSlice(const Tensor& qweight, const Tensor& scales, const std::vector<int32_t>& groups, size_t K, size_t N,
+                         int rank, hipStream_t stream) {
+  const char* who = "PackGroupQuantWeight";
+  const size_t G_total = scales.shape[0];
+  std::vector<int32_t> order(K);
+  for (size_t i = 0; i < K; ++i) order[i] = static_cast<int32_t>(i);
+  std::stable_sort(order.begin(), order.end(), [&](int32_t a, int32_t b) { return groups[a] < groups[b]; });
+  std::vector<int32_t> rows, sorted, block_group;
+  rows.reserve(K + K / 4);
+  for (size_t i = 0; i < K;) {
+    const int32_t g = groups[order[i]];
+    if (g < 0 || static_cast<size_t>(g) >= G_total) KLLM_THROW("PackGroupQuantWeight: g_idx names a group the scales do not hold");
+    size_t j = i;
+    while (j < K && groups[order[j]] == g) rows.push_back(order[j++]);
+    while (rows.size() % 32 != 0) rows.push_back(-1);
+    sorted.resize(rows.size(), g);
+    block_group.resize(rows.size() / 32, g);
+    i = j;
+  }
+  while (rows.size() % 128 != 0) {
+    rows.push_back(-1);
+    sorted.push_back(sorted.back());
+    if (rows.size() % 32 == 0) block_group.push_back(block_group.back());
+  }
+  const size_t Kp = rows.size();
+  Tensor packed(MemoryLocation::LOCATION_DEVICE, TYPE_I4_GROUP, {Kp, N / 2}, rank);
+  packed.perm = std::make_shared<Tensor>(MemoryLocation::LOCATION_DEVICE, TYPE_INT32, std::vector<size_t>{Kp}, rank);
+  packed.g_idx = std::make_shared<Tensor>(MemoryLocation::LOCATION_DEVICE, TYPE_INT32, std::vector<size_t>{Kp}, rank);
+  if (hipMemcpy(packed.perm->GetPtr<void>(), rows.data(), Kp * sizeof(int32_t), hipMemcpyHostToDevice) != hipSuccess ||
+      hipMemcpy(packed.g_idx->GetPtr<void>(), sorted.data(), Kp * sizeof(int32_t), hipMemcpyHostToDevice) != hipSuccess) {
+    KLLM_THROW("PackGroupQuantWeight: cannot upload perm");
+  }
+  KsqCheck(ksq_w4a16_repack_rows(qweight.GetPtr<void>(), packed.perm->GetPtr<void>(), packed.GetPtr<void>(), K, Kp, N, stream), who);
+  // scale row of every 32 packed rows, then the packed scale layout for group size 32
+  const size_t row_bytes = N * GetTypeSize(scales.dtype);
+  Tensor expanded(MemoryLocation::LOCATION_DEVICE, scales.dtype, {Kp / 32, N}, rank);
+  for (size_t b = 0; b < Kp / 32; ++b) {
+    if (hipMemcpyAsync(expanded.GetPtr<char>() + b * row_bytes, scales.GetPtr<char>() + static_cast<size_t>(block_group[b]) * row_bytes,
+                       row_bytes, hipMemcpyDeviceToDevice, stream) != hipSuccess) {
+      KLLM_THROW("PackGroupQuantWeight: cannot gather the scale rows");
+    }
+  }
+  packed.scales = std::make_shared<Tensor>(MemoryLocation::LOCATION_DEVICE, scales.dtype, std::vector<size_t>{Kp / 32, N}, rank);
+  KsqCheck(ksq_w4a16_repack_scales(expanded.GetPtr<void>(), KSQ_SCALE_GN, packed.scales->GetPtr<void>(), 1, Kp, N, 32,
+                                   KsqDtype(scales.dtype, who), stream), who);
+  if (hipStreamSynchronize(stream) != hipSuccess) KLLM_THROW("PackGroupQuantWeight: stream error");  // `expanded` dies here
+  return packed;
+}
+
+}  // namespace
+
 Tensor PackGroupQuantWeight(const Tensor& qweight, const Tensor& scales, const Tensor* qzeros, QuantMode method,
-                            size_t group_size, int rank, hipStream_t stream, const Tensor* g_idx) {
+                            size_t group_size, int rank, hipStream_t stream, const Tensor* g_idx, bool k_full) {
   const char* who = "PackGroupQuantWeight";
   if (method != QUANT_GPTQ && method != QUANT_AWQ) KLLM_THROW("PackGroupQuantWeight: method must be GPTQ or AWQ");
   if (qweight.shape.size() != 2 || scales.shape.size() != 2) KLLM_THROW("PackGroupQuantWeight: 2-D tensors expected");
   const bool awq = method == QUANT_AWQ;
   const size_t K = awq ? qweight.shape[0] : qweight.shape[0] * 8;
   const size_t N = awq ? qweight.shape[1] * 8 : qweight.shape[1];
-  if (scales.shape[0] * group_size != K || scales.shape[1] != N) KLLM_THROW("PackGroupQuantWeight: scales shape mismatch");
+  const bool k_slice = g_idx != nullptr && !k_full;  // the scales then cover the whole checkpoint's groups
+  if ((!k_slice && scales.shape[0] * group_size != K) || scales.shape[1] != N) KLLM_THROW("PackGroupQuantWeight: scales shape mismatch");
   if (awq && !qzeros) KLLM_THROW("PackGroupQuantWeight: AWQ needs qzeros");
   const int dtype = KsqDtype(scales.dtype, who);
 
+  if (k_slice) {
+    if (awq) KLLM_THROW("PackGroupQuantWeight: g_idx (act-order) belongs to GPTQ checkpoints");
+    if (g_idx->GetElementNumber() != K) KLLM_THROW("PackGroupQuantWeight: g_idx must have K entries");
+    std::vector<int32_t> groups(K);
+    if (hipStreamSynchronize(stream) != hipSuccess ||
+        hipMemcpy(groups.data(), g_idx->GetPtr<void>(), K * sizeof(int32_t), hipMemcpyDeviceToHost) != hipSuccess) {
+      KLLM_THROW("PackGroupQuantWeight: cannot read g_idx");
+    }
+    return PackActOrderSlice(qweight, scales, groups, K, N, rank, stream);
+  }
   Tensor packed(MemoryLocation::LOCATION_DEVICE, TYPE_I4_GROUP, {K, N / 2}, rank);
   if (g_idx) {
     if (awq) KLLM_THROW("PackGroupQuantWeight: g_idx (act-order) belongs to GPTQ checkpoints");
@@ -62,7 +130,7 @@ Tensor PackGptqExpertWeight(const Tensor& qweight, const Tensor& scales, size_t 
     KLLM_THROW("PackGptqExpertWeight: scales shape mismatch");
   }
   const int dtype = KsqDtype(scales.dtype, who);
-  Tensor packed(MemoryLocation::LOCATION_DEVICE, TYPE_I4_GROUP, {E, K, N / 2}, rank);
+  Tensor packed(MemoryLocation::LOCATION_DEVICE, TYPE_INT32, {E, K / 16, 2 * N}, rank);
   if (g_idx) {
     // act-order: every expert has its own group index; its rows are sorted by group (stable), as MarlinSortGIdx and the
     // perm form of gptq_marlin_repack do per expert, and the layer gathers the activation columns through `perm`
@@ -110,7 +178,7 @@ Tensor PackMoeExpertWeight(const Tensor& experts, const Tensor& scales, size_t g
     KLLM_THROW("PackMoeExpertWeight: scales shape mismatch");
   }
   const int dtype = KsqDtype(scales.dtype, who);
-  Tensor packed(MemoryLocation::LOCATION_DEVICE, TYPE_UINT4x2, experts.shape, rank);
+  Tensor packed(MemoryLocation::LOCATION_DEVICE, TYPE_UINT8, experts.shape, rank);
   KsqCheck(ksq_w4a16_repack(experts.GetPtr<void>(), KSQ_SRC_MOE_NK, packed.GetPtr<void>(), E, K, N, stream), who);
   packed.scales = std::make_shared<Tensor>(MemoryLocation::LOCATION_DEVICE, scales.dtype, scales.shape, rank);
   KsqCheck(ksq_w4a16_repack_scales(scales.GetPtr<void>(), KSQ_SCALE_NG, packed.scales->GetPtr<void>(), E, K, N, group_size, dtype, stream), who);

@@ -17,15 +17,23 @@ namespace ksana_llm {
 // packed in the order perm = stable argsort(g_idx) (MarlinSortGIdx, src/ksana_llm/models/quant/marlin_utils.cpp:106-122;
 // computed on the host, which synchronizes `stream`) and `perm` and the sorted `g_idx` are bound to the result.
 // Returns a TYPE_I4_GROUP tensor of logical shape {K, N/2} with `scales` (and `zeros`) bound.
+// k_full = false (with g_idx): the tensors are a tensor-parallel rank's K range of an act-order checkpoint
+// (row-parallel projection): qweight holds the rank's K rows, g_idx their checkpoint-wide group numbers and scales the
+// scales of ALL groups, [G_total, N].  The rows are sorted by group, every run of equal group padded to a multiple of
+// 32 rows; the result has shape {K', N/2}, K' >= K a multiple of 128, `scales` [K'/32, N] (one row per 32 packed rows:
+// the layer runs it with group size 32), `perm` [K'] (-1 for padding rows) and the sorted `g_idx`.
 Tensor PackGroupQuantWeight(const Tensor& qweight, const Tensor& scales, const Tensor* qzeros, QuantMode method,
-                            size_t group_size, int rank, hipStream_t stream, const Tensor* g_idx = nullptr);
+                            size_t group_size, int rank, hipStream_t stream, const Tensor* g_idx = nullptr,
+                            bool k_full = true);
 
 // experts: [E, N, K/2] uint8, low nibble = even k.  scales: [E, N, K/group] in T.
-// Returns a TYPE_UINT4x2 tensor of logical shape {E, N, K/2} with `scales` bound.
+// Returns a TYPE_UINT8 tensor of logical shape {E, N, K/2} (dtype and shape of the reference's moe-int4 stacks, which
+// MoeLayerFactory::AutoCreateMoeLayer reads) with `scales` bound.
 Tensor PackMoeExpertWeight(const Tensor& experts, const Tensor& scales, size_t group_size, int rank, hipStream_t stream);
 
 // GPTQ expert stack as the Marlin MoE loader holds it before its own repack: qweight [E, K/8, N] int32, scales
-// [E, K/group, N] in T (symmetric).  Returns a TYPE_I4_GROUP tensor of logical shape {E, K, N/2} with `scales` bound:
+// [E, K/group, N] in T (symmetric).  Returns a TYPE_INT32 tensor of logical shape {E, K/16, 2*N} (the shape the
+// reference's Marlin repack gives, which AutoCreateMoeLayer derives the hidden size from) with `scales` bound, holding
 // the same packed tiles PackMoeExpertWeight produces, for MarlinMoeLayer.  With g_idx (int32 [E, K], the checkpoint's
 // act-order group index of every expert) each expert's rows are sorted by group and `perm` / the sorted `g_idx`
 // ([E, K] each) are bound, as the reference binds them for fused_marlin_moe (S/layers/nvidia/marlin_moe_layer.cpp:71-81).

@@ -1,5 +1,7 @@
 #include "w4a16_matmul_layer.h"
 
+#include <algorithm>
+
 namespace ksana_llm {
 
 Status W4A16MatMulLayer::Init(const std::vector<std::any>& parameters, const RuntimeConfig& runtime_config,
@@ -20,10 +22,6 @@ Status W4A16MatMulLayer::Init(const std::vector<std::any>& parameters, const Run
   weight_data_type_ = std::any_cast<const DataType>(parameters[parameter_index++]);
   is_k_full_ = is_gptq_desc_ ? is_k_full_ : true;
   if (is_gptq_desc_ && is_awq_) return Status(RET_INVALID_ARGUMENT, std::string(Name()) + ": desc_act belongs to GPTQ, not AWQ");
-  if (is_gptq_desc_ && !is_k_full_) {
-    // a K range cut out of an act-order weight does not hold whole quantization groups
-    return Status(RET_INVALID_ARGUMENT, std::string(Name()) + ": desc_act (act-order) weights split along K are not supported");
-  }
   return Status();
 }
 
@@ -35,7 +33,15 @@ size_t W4A16MatMulLayer::GetWorkspaceSize() {
   gemm_workspace_size_ = ksq_w4a16_workspace_size(max_m_, max_n_, max_k_, groupsize_, KsqDtype(inter_data_type_, Name()));
   gemm_workspace_size_ = (gemm_workspace_size_ + 255) & ~static_cast<size_t>(255);
   // act-order: the activations with their columns permuted, behind the GEMM's scratch
-  permuted_input_size_ = is_gptq_desc_ ? max_m_ * max_k_ * GetTypeSize(inter_data_type_) : 0;
+  // (a K range of an act-order weight is packed with every run of equal group padded to 32 rows: up to 31 more rows
+  // for each of the checkpoint's groups - k * ranks / groupsize of them - that has rows in the range)
+  size_t permuted_k = max_k_;
+  if (is_gptq_desc_ && !is_k_full_) {
+    const size_t ranks = static_cast<size_t>(std::max(1, context_->GetTensorParallelSize()));
+    const size_t groups = std::min(max_k_, max_k_ * ranks / std::max<size_t>(1, groupsize_));
+    permuted_k = (max_k_ + 31 * groups + 127) / 128 * 128;
+  }
+  permuted_input_size_ = is_gptq_desc_ ? max_m_ * permuted_k * GetTypeSize(inter_data_type_) : 0;
   workspace_size_ = gemm_workspace_size_ + permuted_input_size_;
   return workspace_size_;
 }
@@ -83,6 +89,25 @@ Status W4A16MatMulLayer::Forward(const std::vector<Tensor>& input_tensors, std::
       KLLM_THROW(std::string(Name()) + ": workspace buffer missing or smaller than GetWorkspaceSize()");
     }
     void* permuted = ws + gemm_workspace_size_;
+    if (!is_k_full_) {
+      // a K range of the checkpoint, packed with padded runs of equal group (PackGroupQuantWeight, k_full = false):
+      // K' packed rows, one scale row per 32 of them
+      const size_t kp = weight_tensor.shape.empty() ? 0 : weight_tensor.shape[0];
+      if (kp < k || kp % 128 != 0 || weight_tensor.perm->GetElementNumber() != kp ||
+          weight_tensor.scales->shape.empty() || weight_tensor.scales->shape[0] * 32 != kp) {
+        KLLM_THROW(std::string(Name()) + ": act-order weight cut along K must come from PackGroupQuantWeight with k_full = false");
+      }
+      if (ws_bytes < gemm_workspace_size_ + m * kp * GetTypeSize(inter_data_type_)) {
+        KLLM_THROW(std::string(Name()) + ": workspace buffer smaller than the padded activations need");
+      }
+      KsqCheck(ksq_gather_columns(x, weight_tensor.perm->GetPtr<void>(), permuted, m, k, kp, dtype, stream), Name());
+      KsqCheck(ksq_w4a16_gemm(output_tensors[0].GetPtr<void>(), permuted, p_qweight, p_scales, nullptr, ws, gemm_workspace_size_,
+                              m, n, kp, 32, dtype, stream),
+               Name());
+      output_tensors[0].shape = {m, n};
+      output_tensors[0].dtype = input_tensors[0].dtype;
+      return Status();
+    }
     KsqCheck(ksq_permute_columns(x, weight_tensor.perm->GetPtr<void>(), permuted, m, k, dtype, stream), Name());
     x = permuted;
     ws_bytes = gemm_workspace_size_;

@@ -51,6 +51,8 @@ SIGNATURES = {
                                          c_i, c_p]),
     "ksq_w4a16_repack_act_order": (c_i, [c_p, c_p, c_p, c_sz, c_sz, c_p]),
     "ksq_permute_columns": (c_i, [c_p, c_p, c_p, c_sz, c_sz, c_i, c_p]),
+    "ksq_w4a16_repack_rows": (c_i, [c_p, c_p, c_p, c_sz, c_sz, c_sz, c_p]),
+    "ksq_gather_columns": (c_i, [c_p, c_p, c_p, c_sz, c_sz, c_sz, c_i, c_p]),
     "ksq_moe_permute_columns": (c_i, [c_p, c_p, c_p, c_p, c_sz, c_sz, c_sz, c_sz, c_i, c_p]),
     "ksq_fp8_repack_weight": (c_i, [c_p, c_p, c_sz, c_sz, c_sz, c_p]),
     "ksq_fp8_unpack_weight": (c_i, [c_p, c_p, c_sz, c_sz, c_sz, c_p]),

@@ -1,4 +1,5 @@
-// Driver for the C++ layer classes: builds a layer through its factory exactly as model code would, feeds it the raw
+// Driver for the C++ layer classes: builds every layer the way model code does - MatMulLayerFactory::AutoCreateLayer /
+// MoeLayerFactory::AutoCreateMoeLayer from a weight name, the loaded weight and a model configuration - feeds it the raw
 // tensors found in a directory and writes the output next to them.  tests/test_gpu_layers.py creates the inputs,
 // runs this program and compares the output with the CPU oracle.
 //
@@ -17,6 +18,7 @@
 #include <cstring>
 #include <fstream>
 #include <iostream>
+#include <map>
 
 #include "blockwise_matmul_layer.h"
 #include "layer_factory.h"
@@ -69,6 +71,16 @@ static void Download(const Tensor& t, const std::string& path) {
   f.write(host.data(), static_cast<std::streamsize>(host.size()));
 }
 
+// the model weights the factories look up by name
+class TestWeights : public BaseWeight {
+ public:
+  Tensor GetModelWeights(const std::string& weight_name) override {
+    auto it = weights.find(weight_name);
+    return it == weights.end() ? Tensor() : it->second;
+  }
+  std::map<std::string, Tensor> weights;
+};
+
 static DataType ParseT(const char* s) { return std::strcmp(s, "bf16") == 0 ? TYPE_BF16 : TYPE_FP16; }
 
 static void Drive(std::shared_ptr<BaseLayer> layer, const ModelConfig& mc, const RuntimeConfig& rc,
@@ -106,16 +118,31 @@ static int RunW4A16(int argc, char** argv) {
   rc.max_step_token_num = m;
 
   Tensor qweight = awq ? Upload(dir + "/qweight.bin", TYPE_INT32, {k, n / 8}) : Upload(dir + "/qweight.bin", TYPE_INT32, {k / 8, n});
-  Tensor scales = Upload(dir + "/scales.bin", T, {k / group, n});
+  // argv[11] = 1: the tensors are one rank's K range of an act-order checkpoint twice as deep (scales.bin then holds the
+  // scales of all 2k/group groups, g_idx.bin the checkpoint-wide group numbers of the range's rows)
+  const bool k_range = argc > 11 && std::atoi(argv[11]) != 0;
+  Tensor scales = Upload(dir + "/scales.bin", T, {(k_range ? 2 * k : k) / group, n});
   Tensor qzeros;
   if (awq) qzeros = Upload(dir + "/qzeros.bin", TYPE_INT32, {k / group, n / 8});
   Tensor g_idx;
   if (desc_act) g_idx = Upload(dir + "/g_idx.bin", TYPE_INT32, {k});
   Tensor weight = PackGroupQuantWeight(qweight, scales, awq ? &qzeros : nullptr, mc.quant_config.method, group, 0, stream,
-                                       desc_act ? &g_idx : nullptr);
+                                       desc_act ? &g_idx : nullptr, !k_range);
 
+  // a column-parallel projection of a model with hidden size k and inter size n (mlp.gate_proj: all of K on this
+  // rank), or - k_slice - the row-parallel mlp.down_proj of a model with inter size k and hidden size n, whose K is a
+  // rank's slice of the checkpoint's
+  const bool k_slice = k_range;
+  if (k_slice) context = std::make_shared<Context>(2, stream);  // two tensor-parallel ranks, this is rank 0
+  mc.hidden_units = k_slice ? n : k;
+  mc.inter_size = k_slice ? 2 * k : n;
+  const std::string name = k_slice ? "model.layers.0.mlp.down_proj.weight" : "model.layers.0.mlp.gate_proj.weight";
+  auto weights = std::make_shared<TestWeights>();
+  weights->weights[name] = weight;
   MatMulLayerFactory factory(mc, rc, 0, context);
-  auto layer = factory.CreateLayer(TYPE_I4_GROUP, T, T, factory.GroupMatMulParams(n, k, true), mc.quant_config.method, backend);
+  if (k_slice) rc.parallel_basic_config.tensor_parallel_size = 2;
+  MatMulLayerFactory tp_factory(mc, rc, 0, context);
+  auto layer = (k_slice ? tp_factory : factory).AutoCreateLayer(weights, name, TYPE_I4_GROUP, T, T, backend, {});
   Tensor x = Upload(dir + "/x.bin", T, {m, k});
   std::vector<Tensor> outputs{Tensor(MemoryLocation::LOCATION_DEVICE, T, {m, n}, 0)};
   Drive(layer, mc, rc, {x, weight}, outputs);
@@ -144,9 +171,12 @@ static int RunBlockwise(int argc, char** argv) {
   Tensor loaded = Upload(dir + "/w.bin", TYPE_FP8_E4M3, {n, k});
   loaded.weight_scales = std::make_shared<Tensor>(Upload(dir + "/w_scale.bin", TYPE_FP32, {(n + 127) / 128, k / 128}));
   Tensor weight = PackFp8Weight(loaded, 0, stream);
-  std::vector<std::any> params{rc.max_step_token_num, n, k, size_t(128), weight};
+  const std::string name = "model.layers.0.mlp.up_proj.weight";
+  auto weights = std::make_shared<TestWeights>();
+  weights->weights[name] = weight;
+  mc.quant_config.weight_block_size = {128, 128};
   MatMulLayerFactory factory(mc, rc, 0, context);
-  auto layer = factory.CreateLayer(TYPE_FP8_E4M3, T, T, params, QUANT_BLOCK_FP8_E4M3, DEFAULT_LINEAR_BACKEND);
+  auto layer = factory.AutoCreateLayer(weights, name, TYPE_FP8_E4M3, T, T, DEFAULT_LINEAR_BACKEND, {false});  // skip_quant
   Tensor x = Upload(dir + "/x.bin", T, {m, fuse ? 2 * k : k});
   std::vector<Tensor> outputs{Tensor(MemoryLocation::LOCATION_DEVICE, T, {m, n}, 0)};
   Drive(layer, mc, rc, {x, weight}, outputs);
@@ -173,9 +203,13 @@ static int RunFp8Tensor(int argc, char** argv) {
   loaded.weight_scales = std::make_shared<Tensor>(Upload(dir + "/w_scale.bin", TYPE_FP32, {1}));
   if (is_static) loaded.input_scales = std::make_shared<Tensor>(Upload(dir + "/in_scale.bin", TYPE_FP32, {1}));
   Tensor weight = PackFp8Weight(loaded, 0, stream);
-  std::vector<std::any> params{rc.max_step_token_num, k};
+  const std::string name = "model.layers.0.mlp.up_proj.weight";
+  auto weights = std::make_shared<TestWeights>();
+  weights->weights[name] = weight;
+  mc.is_quant = true;
+  mc.quant_config.method = QUANT_FP8_E4M3;
   MatMulLayerFactory factory(mc, rc, 0, context);
-  auto layer = factory.CreateLayer(TYPE_FP8_E4M3, T, T, params, QUANT_FP8_E4M3, DEFAULT_LINEAR_BACKEND);
+  auto layer = factory.AutoCreateLayer(weights, name, TYPE_FP8_E4M3, T, T, DEFAULT_LINEAR_BACKEND, {});
   Tensor x = Upload(dir + "/x.bin", T, {m, k});
   std::vector<Tensor> outputs{Tensor(MemoryLocation::LOCATION_DEVICE, T, {m, n}, 0)};
   Drive(layer, mc, rc, {x, weight}, outputs);
@@ -205,16 +239,16 @@ static int RunW4A8(int argc, char** argv) {
   if (per_channel) loaded.pre_quant_scales = std::make_shared<Tensor>(Upload(dir + "/pqs.bin", TYPE_FP32, {k}));
   loaded.alpha = alpha;
   Tensor weight = PackW4A8Weight(loaded, 0, stream);
-  FinegrainedMixedDtypeGemmLayerParameters param;
-  param.m = rc.max_step_token_num;
-  param.n = n;
-  param.k = k;
-  param.group_size = 128;
-  param.has_zero = false;
-  param.activation_type = TYPE_FP8_E4M3;
-  param.output_type = T;
+  // the loader's record of a W4A8 weight: the mode, and the logical n and k the packed tensor no longer shows
+  const std::string name = "model.layers.0.mlp.up_proj.weight";
+  WeightStatus status;
+  status.quant_mode = QUANT_W4A8_AWQ;
+  status.layout = {{"n", n}, {"k", k}};
+  context->SetWeightStatus(name, status);
+  auto weights = std::make_shared<TestWeights>();
+  weights->weights[name] = weight;
   MatMulLayerFactory factory(mc, rc, 0, context);
-  auto layer = factory.CreateLayer(TYPE_I4_GROUP, T, T, {param}, QUANT_W4A8_AWQ, CUTLASS_LINEAR_BACKEND);
+  auto layer = factory.AutoCreateLayer(weights, name, TYPE_I4_GROUP, T, T, CUTLASS_LINEAR_BACKEND, {});
   Tensor x = Upload(dir + "/x.bin", T, {m, k});
   std::vector<Tensor> outputs{Tensor(MemoryLocation::LOCATION_DEVICE, T, {m, n}, 0)};
   Drive(layer, mc, rc, {x, weight}, outputs);
@@ -223,34 +257,35 @@ static int RunW4A8(int argc, char** argv) {
   return 0;
 }
 
-// renorm: 0 = NO_NORM and norm_topk_prob false, 1 = RE_NORM and norm_topk_prob true, 2 = RE_NORM with norm_topk_prob
-// false (the routers follow norm_topk_prob alone)
-static std::vector<std::any> MoeParams(size_t tokens, size_t E, size_t hidden, size_t inter, size_t topk, int renorm_arg,
-                                       float scaling, DataType int_dtype = TYPE_UINT4x2, uint32_t groups = 1,
-                                       uint32_t topk_group = 1, const std::string& scoring = "softmax",
-                                       bool use_bias = false) {
-  const bool renorm = renorm_arg == 1;
-  return {renorm_arg != 0 ? MoeScaleNormMode::RE_NORM : MoeScaleNormMode::NO_NORM,
-          tokens,
-          int(0),
-          E,
-          hidden,
-          inter,
-          topk,
-          size_t(1),
-          true,
-          groups,
-          topk_group,
-          scoring,
-          std::string("greedy"),
-          renorm,
-          scaling,
-          use_bias,
-          false,
-          TYPE_INVALID,
-          int_dtype,
-          int(128),
-          false};
+// Model and runtime configuration of a MoE model with E experts.  renorm: 0 = NO_NORM and norm_topk_prob false,
+// 1 = RE_NORM and norm_topk_prob true, 2 = RE_NORM with norm_topk_prob false (the routers follow norm_topk_prob alone).
+static MoeScaleNormMode MoeModel(ModelConfig& mc, RuntimeConfig& rc, size_t tokens, size_t E, size_t hidden, size_t inter,
+                                 size_t topk, int renorm_arg, float scaling, uint32_t groups = 1, uint32_t topk_group = 1,
+                                 const std::string& scoring = "softmax", bool use_bias = false) {
+  rc.max_step_token_num = tokens;
+  mc.hidden_units = hidden;
+  mc.moe_config.num_experts = E;
+  mc.moe_config.experts_topk = topk;
+  mc.moe_config.moe_inter_size = inter;
+  mc.moe_config.use_vllm_moe = true;
+  mc.moe_config.num_expert_group = groups;
+  mc.moe_config.expert_groups_topk = topk_group;
+  mc.moe_config.scoring_func = scoring;
+  mc.moe_config.norm_topk_prob = renorm_arg == 1;
+  mc.moe_config.routed_scaling_factor = scaling;
+  mc.moe_config.use_e_score_correction_bias = use_bias;
+  return renorm_arg != 0 ? MoeScaleNormMode::RE_NORM : MoeScaleNormMode::NO_NORM;
+}
+
+static std::shared_ptr<BaseLayer> AutoMoe(const ModelConfig& mc, const RuntimeConfig& rc, std::shared_ptr<Context> context,
+                                          const Tensor& w13, const Tensor& w2, DataType T, MoeScaleNormMode mode) {
+  auto weights = std::make_shared<TestWeights>();
+  weights->weights["model.layers.3.mlp.experts.up_gate_proj.weight"] = w13;
+  weights->weights["model.layers.3.mlp.experts.down_proj.weight"] = w2;
+  MoeLayerFactory factory(mc, rc, 0, context);
+  return factory.AutoCreateMoeLayer(weights, {"model.layers.3.mlp.experts.up_gate_proj.weight",
+                                              "model.layers.3.mlp.experts.down_proj.weight"},
+                                    w13.dtype, T, T, 3, {mode});
 }
 
 static int RunMoe(int argc, char** argv) {
@@ -277,11 +312,12 @@ static int RunMoe(int argc, char** argv) {
   Tensor w2 = PackMoeExpertWeight(Upload(dir + "/w2.bin", TYPE_UINT8, {E, hidden, inter / 2}),
                                   Upload(dir + "/s2.bin", T, {E, hidden, inter / 128}), 128, 0, stream);
   HIP_OK(hipStreamSynchronize(stream));
-  MoeLayerFactory factory(mc, rc, 0, context);
-  auto layer = factory.CreateLayer(TYPE_UINT8, T, T,
-                                   MoeParams(tokens, E, hidden, inter, topk, renorm, scaling, TYPE_UINT4x2, groups,
-                                             topk_group, scoring, use_bias),
-                                   MOE_QUANT_GPTQ, TRITON_MOE_BACKEND);
+  mc.is_quant = true;
+  mc.quant_config.method = QUANT_GPTQ;
+  mc.quant_config.bits = 4;
+  mc.quant_config.group_size = 128;
+  const MoeScaleNormMode mode = MoeModel(mc, rc, tokens, E, hidden, inter, topk, renorm, scaling, groups, topk_group, scoring, use_bias);
+  auto layer = AutoMoe(mc, rc, context, w13, w2, T, mode);
   Tensor x = Upload(dir + "/x.bin", T, {tokens, hidden});
   Tensor gating = Upload(dir + "/gating.bin", TYPE_FP32, {tokens, E});
   std::vector<Tensor> outputs{Tensor(MemoryLocation::LOCATION_DEVICE, T, {tokens, hidden}, 0)};
@@ -325,13 +361,15 @@ static int RunMarlinMoe(int argc, char** argv) {
                                    Upload(dir + "/s2.bin", T, {E, inter / 128, hidden}), 128, 0, stream,
                                    act_order ? &g2 : nullptr);
   HIP_OK(hipStreamSynchronize(stream));
-  // the reference's 20 positional values (marlin_moe_layer.cpp:16-36); the routing fields are ignored by this layer
-  std::vector<std::any> params{renorm ? MoeScaleNormMode::RE_NORM : MoeScaleNormMode::NO_NORM,
-                               tokens, E, hidden, inter, topk, size_t(1), false, uint32_t(1), uint32_t(1),
-                               std::string("softmax"), std::string("greedy"), false, 1.0f, false, false,
-                               TYPE_INVALID, TYPE_I4_GROUP, int(128), false};
-  MoeLayerFactory factory(mc, rc, 0, context);
-  auto layer = factory.CreateLayer(TYPE_I4_GROUP, T, T, params, MOE_QUANT_GPTQ, MARLIN_MOE_BACKEND);
+  // GPTQ experts of a model that does not take the aligned-block flow (use_vllm_moe false): the Marlin MoE layer
+  mc.is_quant = true;
+  mc.quant_config.method = QUANT_GPTQ;
+  mc.quant_config.bits = 4;
+  mc.quant_config.group_size = 128;
+  const MoeScaleNormMode mode = MoeModel(mc, rc, tokens, E, hidden, inter, topk, renorm ? 1 : 0, 1.0f);
+  mc.moe_config.use_vllm_moe = false;
+  mc.moe_config.norm_topk_prob = false;  // this layer's router follows the scale-norm mode
+  auto layer = AutoMoe(mc, rc, context, w13, w2, T, mode);
   Tensor x = Upload(dir + "/x.bin", T, {tokens, hidden});
   Tensor gating = Upload(dir + "/gating.bin", T, {tokens, E});
   std::vector<Tensor> outputs{Tensor(MemoryLocation::LOCATION_DEVICE, T, {tokens, hidden}, 0)};
@@ -377,10 +415,11 @@ static int RunMoeFp8(int argc, char** argv) {
   w2_loaded.weight_scales = std::make_shared<Tensor>(Upload(dir + "/s2.bin", TYPE_FP32, {E, (hidden + 127) / 128, inter / 128}));
   Tensor w13 = PackFp8Weight(w13_loaded, 0, stream);
   Tensor w2 = PackFp8Weight(w2_loaded, 0, stream);
-  auto params = MoeParams(tokens, E, hidden, inter, topk, renorm, scaling, TYPE_INVALID);
-  params[17] = TYPE_BLOCK_FP8_E4M3;
-  MoeLayerFactory factory(mc, rc, 0, context);
-  auto layer = factory.CreateLayer(TYPE_FP8_E4M3, T, T, params, MOE_QUANT_BLOCK_FP8_E4M3, TRITON_MOE_BACKEND);
+  mc.is_quant = true;
+  mc.quant_config.method = QUANT_BLOCK_FP8_E4M3;
+  mc.quant_config.is_fp8_blockwise = true;
+  const MoeScaleNormMode mode = MoeModel(mc, rc, tokens, E, hidden, inter, topk, renorm ? 1 : 0, scaling);
+  auto layer = AutoMoe(mc, rc, context, w13, w2, T, mode);
   Tensor x = Upload(dir + "/x.bin", T, {tokens, hidden});
   Tensor gating = Upload(dir + "/gating.bin", TYPE_FP32, {tokens, E});
   std::vector<Tensor> outputs{Tensor(MemoryLocation::LOCATION_DEVICE, T, {tokens, hidden}, 0)};
@@ -430,7 +469,9 @@ static int RunErrors() {
     expect(layer.GetWorkspaceSize() >= plain.GetWorkspaceSize() + 16 * 256 * 2, "desc_act workspace holds permuted x");
     p[5] = true;
     p[6] = false;
-    expect(!sliced.Init(p, rc, context, 0).OK(), "desc_act with a K slice is rejected");
+    expect(sliced.Init(p, rc, context, 0).OK(), "desc_act with a K slice init");
+    // every group of the checkpoint may have rows in the slice, each run padded to 32 rows: 256 + 31 * 2 rows -> 384
+    expect(sliced.GetWorkspaceSize() >= plain.GetWorkspaceSize() + 16 * 384 * 2, "K-slice workspace holds the padded x");
     p[6] = true;
     p[4] = true;
     expect(!awq.Init(p, rc, context, 0).OK(), "desc_act with AWQ is rejected");
@@ -522,7 +563,10 @@ static int RunErrors() {
   // moe: fp8 experts / impossible expert groups rejected, int4 and grouped routing accepted
   {
     MoeLayer a, b, c;
-    auto p = MoeParams(64, 8, 256, 256, 2, false, 1.0f);
+    // (a raw parameter vector on purpose: these are checks of what Init itself refuses)
+    std::vector<std::any> p{MoeScaleNormMode::NO_NORM, size_t(64), int(0), size_t(8), size_t(256), size_t(256), size_t(2),
+                            size_t(1), true, uint32_t(1), uint32_t(1), std::string("softmax"), std::string("greedy"), false,
+                            1.0f, false, false, TYPE_INVALID, TYPE_UINT4x2, int(128), false};
     expect(a.Init(p, rc, context, 0).OK(), "moe int4 init");
     expect(a.GetWorkspaceSize() > 0, "moe workspace size");
     auto q = p;
@@ -550,6 +594,56 @@ static int RunErrors() {
     expect(!f.Init(r, rc, context, 0).OK(), "unknown scoring function is rejected");
     expect(ksq_moe_block_m(8 * 2, 8) == 16 && ksq_moe_block_m(64 * 2, 8) == 32 && ksq_moe_block_m(4096 * 8, 256) == 128,
            "block_m thresholds");
+  }
+  // the Auto factories: what they derive and what they refuse
+  {
+    ModelConfig m2;
+    m2.is_quant = true;
+    m2.quant_config.method = QUANT_GPTQ;
+    m2.hidden_units = 4096;
+    m2.inter_size = 14336;
+    m2.head_num = 32;
+    m2.num_key_value_heads = 8;
+    m2.size_per_head = 128;
+    RuntimeConfig r2 = rc;
+    r2.parallel_basic_config.tensor_parallel_size = 2;
+    r2.parallel_basic_config.attn_tensor_parallel_size = 2;
+    MatMulLayerFactory f2(m2, r2, 0, context);
+    size_t k = 0, n = 0;
+    bool k_full = false;
+    expect(f2.ProjectionShape("model.layers.7.mlp.down_proj.weight", &k, &n, &k_full) && k == 7168 && n == 4096 && !k_full,
+           "down_proj: K is the rank's slice");
+    expect(f2.ProjectionShape("model.layers.7.mlp.gate_proj.weight", &k, &n, &k_full) && k == 4096 && n == 7168 && k_full,
+           "gate_proj: N is the rank's slice");
+    expect(f2.ProjectionShape("model.layers.7.self_attn.query_key_value.weight", &k, &n, &k_full) && k == 4096 &&
+               n == 128 * (32 + 16) / 2 && k_full, "fused qkv");
+    expect(f2.ProjectionShape("model.layers.7.self_attn.o_proj.weight", &k, &n, &k_full) && k == 2048 && n == 4096 && !k_full,
+           "o_proj");
+    expect(!f2.ProjectionShape("lm_head.weight", &k, &n, &k_full), "a name that is no projection");
+    auto weights = std::make_shared<TestWeights>();
+    static char placeholder[16];  // shapes and dtypes are all the factories read: no device memory behind these
+    weights->weights["lm_head.weight"] = Tensor(MemoryLocation::LOCATION_DEVICE, TYPE_FP16, {16, 16}, 0, placeholder);
+    expect(throws([&] { f2.AutoCreateLayer(weights, "lm_head.weight", TYPE_FP16, TYPE_FP16, TYPE_FP16, CUTLASS_LINEAR_BACKEND, {}); }),
+           "an unquantized weight has no layer here");
+    ModelConfig m3;
+    m3.is_quant = true;
+    m3.quant_config.method = QUANT_GPTQ;
+    m3.hidden_units = 256;
+    m3.moe_config.num_experts = 8;
+    m3.moe_config.experts_topk = 2;
+    m3.moe_config.moe_inter_size = 128;
+    m3.moe_config.use_vllm_moe = true;
+    MoeLayerFactory f3(m3, rc, 0, context);
+    weights->weights["up"] = Tensor(MemoryLocation::LOCATION_DEVICE, TYPE_UINT8, {8, 256, 128}, 0, placeholder);
+    weights->weights["down"] = Tensor(MemoryLocation::LOCATION_DEVICE, TYPE_UINT8, {8, 256, 64}, 0, placeholder);
+    weights->weights["down7"] = Tensor(MemoryLocation::LOCATION_DEVICE, TYPE_UINT8, {7, 256, 64}, 0, placeholder);
+    weights->weights["down_h"] = Tensor(MemoryLocation::LOCATION_DEVICE, TYPE_UINT8, {8, 512, 64}, 0, placeholder);
+    expect(f3.AutoCreateMoeLayer(weights, {"up", "down"}, TYPE_UINT8, TYPE_BF16, TYPE_BF16, 0, {MoeScaleNormMode::NO_NORM}) != nullptr,
+           "int4 experts through the auto factory");
+    expect(throws([&] { f3.AutoCreateMoeLayer(weights, {"up", "down7"}, TYPE_UINT8, TYPE_BF16, TYPE_BF16, 0, {MoeScaleNormMode::NO_NORM}); }),
+           "expert counts that differ are refused");
+    expect(throws([&] { f3.AutoCreateMoeLayer(weights, {"up", "down_h"}, TYPE_UINT8, TYPE_BF16, TYPE_BF16, 0, {MoeScaleNormMode::NO_NORM}); }),
+           "hidden sizes that differ are refused");
   }
   std::printf(failures ? "layer errors: %d FAILED\n" : "layer errors: OK\n", failures);
   return failures ? 1 : 0;

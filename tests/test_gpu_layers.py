@@ -71,6 +71,27 @@ def test_w4a16_layer_act_order(tmp_path, oracle, dtype, backend, m, n, k):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("dtype,backend,m,n,k", [(H.F16, "marlin", 3, 512, 1024), (H.BF16, "marlin", 40, 256, 1536)])
+def test_w4a16_layer_act_order_k_range(tmp_path, oracle, dtype, backend, m, n, k):
+    """is_k_full = false: this rank holds rows [0, k) of an act-order checkpoint with 2k rows (mlp.down_proj under two
+    tensor-parallel ranks).  Its rows belong to arbitrary groups of the whole checkpoint; the oracle is the definition
+    y = x . ((code - 8) * scale[g_idx[row]]) over the rank's rows."""
+    g = H.gen(9070 + k)
+    full = H.make_w4a16(9071 + m, m, n, 2 * k, 128, dtype, False)         # the whole checkpoint: codes, scales of all groups
+    g_idx_full = (torch.randperm(2 * k, generator=g) // 128).to(torch.int32)
+    codes, g_idx = full["codes"][:k], g_idx_full[:k].contiguous()
+    x = full["x"][:, :k].contiguous()
+    torch.from_numpy(oracle.gptq_pack(codes).view(np.int32)).numpy().tofile(tmp_path / "qweight.bin")
+    H.bits_of(full["scales"]).tofile(tmp_path / "scales.bin")
+    H.bits_of(x).tofile(tmp_path / "x.bin")
+    g_idx.numpy().tofile(tmp_path / "g_idx.bin")
+    run_driver("w4a16", tmp_path, "gptq", TNAME[dtype], backend, m, n, k, 128, 1, 1)
+    y = read_out(tmp_path / "y.bin", dtype, (m, n))
+    ref = oracle.gptq_act_order_gemm(H.bits_of(x), codes, H.bits_of(full["scales"]), g_idx.numpy(), dtype)
+    H.check_gemm(y, ref, dtype, "%s act-order K-range layer" % backend)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("dtype,m,n,k,fuse,max_m", [(H.BF16, 5, 512, 1024, 0, None), (H.F16, 33, 256, 512, 0, None),
                                                     (H.BF16, 16, 512, 1024, 1, None),
                                                     # odd max_m with K cut over workgroups: the GEMM's scratch behind

@@ -120,3 +120,32 @@ def test_full_size_roundtrip_checksum(ops):
         b = t.view(torch.uint8).reshape(-1)
         return torch.bincount((b & 15).int(), minlength=16) + torch.bincount((b >> 4).int(), minlength=16)
     assert torch.equal(nibble_hist(packed), nibble_hist(q))
+
+
+def test_repack_rows_and_gather_columns(ops, oracle):
+    """Padded act-order packing: packed row j takes checkpoint row rows[j], index -1 is a padding row with code 8; the
+    activation side gathers the same columns and reads 0 for the padding."""
+    from ksanallm_amd import lib as L
+    K_src, K_dst, N, m = 256, 384, 64, 5
+    g = H.gen(77)
+    codes = torch.randint(0, 16, (K_src, N), generator=g, dtype=torch.uint8).numpy()
+    rows = torch.full((K_dst,), -1, dtype=torch.int32)
+    pick = torch.randperm(K_dst, generator=g)[:K_src].sort().values
+    rows[pick] = torch.randperm(K_src, generator=g).to(torch.int32)
+    q = torch.from_numpy(oracle.gptq_pack(codes).view(np.int32)).cuda()
+    dst = torch.empty(K_dst * N // 2, dtype=torch.uint8, device="cuda")
+    rows_d = rows.cuda()
+    L.check(L.load().ksq_w4a16_repack_rows(q.data_ptr(), rows_d.data_ptr(), dst.data_ptr(), K_src, K_dst, N,
+                                           torch.cuda.current_stream().cuda_stream))
+    want = np.full((K_dst, N), 8, dtype=np.uint8)
+    want[rows.numpy() >= 0] = codes[rows.numpy()[rows.numpy() >= 0]]
+    ref = ops.repack_weight(torch.from_numpy(oracle.gptq_pack(want).view(np.int32)).cuda(), L.SRC_GPTQ, 1, K_dst, N)
+    assert torch.equal(dst, ref)
+    x = torch.randn((m, K_src), generator=g).to(torch.bfloat16)
+    out = torch.empty((m, K_dst), dtype=torch.bfloat16, device="cuda")
+    x_d = x.cuda()
+    L.check(L.load().ksq_gather_columns(x_d.data_ptr(), rows_d.data_ptr(), out.data_ptr(), m, K_src, K_dst, L.BF16,
+                                        torch.cuda.current_stream().cuda_stream))
+    expect = torch.zeros((m, K_dst), dtype=torch.bfloat16)
+    expect[:, rows >= 0] = x[:, rows[rows >= 0].long()]
+    assert torch.equal(out.cpu(), expect)
