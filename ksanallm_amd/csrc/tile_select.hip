@@ -88,7 +88,7 @@ SplitKChoice select_splitk_blocks(int mt, size_t m_blocks, size_t n, size_t k) {
 bool use_mfma_tile(size_t m, size_t n, size_t k, size_t group) {
   (void)k;
   (void)n;
-  return m > 32 && group == 128;
+  return m > 32 && (group == 128 || group == 64 || group == 32);
 }
 
 // 256-row tiles halve the weight traffic per output row, 128-row tiles waste less when m sits just above a multiple

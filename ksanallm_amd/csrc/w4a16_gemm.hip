@@ -100,14 +100,22 @@ size_t splitk_workspace(const SplitKChoice& c, size_t m, size_t n) {
   return c.parts > 1 ? static_cast<size_t>(c.parts) * m * n * sizeof(float) : 0;
 }
 
-template <typename T, int WM, bool HAS_ZP>
-int launch_tile_zp(const TileParams& p, unsigned grid, hipStream_t s) {
+template <typename T, int WM, bool HAS_ZP, int GROUP>
+int launch_tile_group(const TileParams& p, unsigned grid, hipStream_t s) {
   constexpr int kLds = 4 * WM * 2 * 1024;  // NS stages of WM*2 fragments
   // more dynamic LDS than a kernel may use without asking: once per device
   static std::atomic<uint64_t> configured{0};
-  if (int rc = allow_dynamic_lds(configured, reinterpret_cast<const void*>(&w4a16_tile_kernel<T, WM, HAS_ZP>), kLds)) return rc;
-  w4a16_tile_kernel<T, WM, HAS_ZP><<<grid, 512, kLds, s>>>(p);
+  auto kernel = &w4a16_tile_kernel<T, WM, HAS_ZP, false, GROUP>;
+  if (int rc = allow_dynamic_lds(configured, reinterpret_cast<const void*>(kernel), kLds)) return rc;
+  kernel<<<grid, 512, kLds, s>>>(p);
   return KSQ_OK;
+}
+
+template <typename T, int WM, bool HAS_ZP>
+int launch_tile_zp(const TileParams& p, unsigned grid, size_t group, hipStream_t s) {
+  if (group == 64) return launch_tile_group<T, WM, HAS_ZP, 64>(p, grid, s);
+  if (group == 32) return launch_tile_group<T, WM, HAS_ZP, 32>(p, grid, s);
+  return launch_tile_group<T, WM, HAS_ZP, 128>(p, grid, s);
 }
 
 // grouped (MoE) form: one 128-row block of the aligned permutation per row tile, no split-K
@@ -122,7 +130,7 @@ int launch_tile_grouped(const TileParams& p, hipStream_t s) {
 }
 
 template <typename T>
-int dispatch_mfma_tile(TileParams p, const TilePlan& plan, hipStream_t s) {
+int dispatch_mfma_tile(TileParams p, const TilePlan& plan, size_t group, hipStream_t s) {
   p.tiles_m = plan.tiles_m;
   p.tiles_n = plan.tiles_n;
   p.main_items = plan.main_items;
@@ -130,9 +138,9 @@ int dispatch_mfma_tile(TileParams p, const TilePlan& plan, hipStream_t s) {
   p.kt_per_split = plan.kt_per_split;
   int rc;
   if (plan.block_m == 128)
-    rc = p.zeros ? launch_tile_zp<T, 8, true>(p, plan.grid, s) : launch_tile_zp<T, 8, false>(p, plan.grid, s);
+    rc = p.zeros ? launch_tile_zp<T, 8, true>(p, plan.grid, group, s) : launch_tile_zp<T, 8, false>(p, plan.grid, group, s);
   else
-    rc = p.zeros ? launch_tile_zp<T, 16, true>(p, plan.grid, s) : launch_tile_zp<T, 16, false>(p, plan.grid, s);
+    rc = p.zeros ? launch_tile_zp<T, 16, true>(p, plan.grid, group, s) : launch_tile_zp<T, 16, false>(p, plan.grid, group, s);
   if (rc) return rc;
   if (plan.splits > 1) {
     const unsigned cut = plan.tiles_m * plan.tiles_n - plan.main_items;
@@ -226,8 +234,8 @@ int w4a16_gemm_impl(const char* fn, void* y, const void* x, const void* w_packed
       tp.partial = static_cast<float*>(workspace);
     }
     if (256 * k * 2 > 0xffffffffull) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: k too large", fn);
-    int rc = dtype == KSQ_F16 ? dispatch_mfma_tile<F16>(tp, plan, as_stream(stream))
-                              : dispatch_mfma_tile<BF16>(tp, plan, as_stream(stream));
+    int rc = dtype == KSQ_F16 ? dispatch_mfma_tile<F16>(tp, plan, group, as_stream(stream))
+                              : dispatch_mfma_tile<BF16>(tp, plan, group, as_stream(stream));
     if (rc) return rc;
     return check_launch(fn);
   }

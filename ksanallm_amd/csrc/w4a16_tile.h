@@ -129,11 +129,12 @@ struct Dequant<BF16, HAS_ZP> {
   }
 };
 
-// One column tile's packed weights, scale and zero point for one k-tile of 128.
+// One column tile's packed weights for one k-tile of 128, with the scale and zero point of each of its GPT groups.
+template <int GPT>
 struct WSlot {
   u32x4 wq;
-  uint32_t sc;
-  uint32_t zp;
+  uint32_t sc[GPT];
+  uint32_t zp[GPT];
 };
 
 // 8 wavefronts side by side along N; each computes WM x 2 tiles of 16x16.  BM = 16*WM, BN = 256.
@@ -141,8 +142,12 @@ struct WSlot {
 // sorted_ids (slot id s reads x row s / top_k, pad slots carry s >= numel), its weights are those of expert
 // expert_ids[tile_m], its results are scattered to out[s, :] (times topk_w[s] when given).  Blocks past num_post_pad
 // leave at once.  There is no split-K in this form.
-template <typename T, int WM, bool HAS_ZP, bool GROUPED = false>
+// GROUP: rows of a quantization group, 128, 64 or 32 (GPT = 128 / GROUP groups per k-tile).
+template <typename T, int WM, bool HAS_ZP, bool GROUPED = false, int GROUP = 128>
 __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
+  static_assert(GROUP == 128 || GROUP == 64 || GROUP == 32, "group size");
+  constexpr int GPT = 128 / GROUP;
+  typedef ksq::WSlot<GPT> WSlot;
   constexpr int WAVES = 8;
   constexpr int WN = 2;
   constexpr int BM = WM * 16;
@@ -152,7 +157,7 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
   constexpr int FRAGS = WM * (BK / 32);  // 1 KiB fragments per stage
   constexpr int STAGE_BYTES = FRAGS * 1024;
   constexpr int AP = FRAGS / WAVES;      // fragments this wavefront fetches per stage
-  constexpr int WL = HAS_ZP ? 3 : 2;     // loads per weight slot
+  constexpr int WL = 1 + GPT * (HAS_ZP ? 2 : 1);  // loads per weight slot: the tile, and a scale (and zero point) per group
   constexpr int L = WL + AP;             // vector memory loads per wavefront per stage
   constexpr int WAIT_N = (NS - 2) * L;   // loads issued after the stage that is about to be consumed
   static_assert(FRAGS % WAVES == 0 && AP % 2 == 0, "fragments must split evenly, in k pairs, over the wavefronts");
@@ -230,8 +235,8 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
   for (int t = 0; t < WN; ++t) {
     const size_t nt = static_cast<size_t>(expert) * n_tiles + ((nt0 + t < n_tiles) ? nt0 + t : n_tiles - 1);
     w_base[t] = static_cast<const char*>(p.w) + (nt * KT + kt_begin) * 1024;
-    s_base[t] = static_cast<const char*>(p.scales) + (nt * KT + kt_begin) * 32;
-    z_base[t] = HAS_ZP ? static_cast<const char*>(p.zeros) + (nt * KT + kt_begin) * 16 : nullptr;
+    s_base[t] = static_cast<const char*>(p.scales) + (nt * KT + kt_begin) * (GPT * 32);
+    z_base[t] = HAS_ZP ? static_cast<const char*>(p.zeros) + (nt * KT + kt_begin) * (GPT * 16) : nullptr;
   }
   const uint32_t w_voff = lane * 16, s_voff = lrow * 2, z_voff = lrow;
 
@@ -253,11 +258,11 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
     kt = kt < kt_count ? kt : kt_count - 1;
     const char* w0 = w_base[0] + static_cast<size_t>(kt) * 1024;
     const char* w1 = w_base[1] + static_cast<size_t>(kt) * 1024;
-    const char* s0 = s_base[0] + static_cast<size_t>(kt) * 32;
-    const char* s1 = s_base[1] + static_cast<size_t>(kt) * 32;
+    const char* s0 = s_base[0] + static_cast<size_t>(kt) * (GPT * 32);
+    const char* s1 = s_base[1] + static_cast<size_t>(kt) * (GPT * 32);
     if (HAS_ZP) {
-      const char* z0 = z_base[0] + static_cast<size_t>(kt) * 16;
-      const char* z1 = z_base[1] + static_cast<size_t>(kt) * 16;
+      const char* z0 = z_base[0] + static_cast<size_t>(kt) * (GPT * 16);
+      const char* z1 = z_base[1] + static_cast<size_t>(kt) * (GPT * 16);
       asm volatile(
           "s_nop 4\n\t"
           "global_load_dwordx4 %0, %6, %9\n\t"
@@ -266,9 +271,26 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
           "global_load_dwordx4 %3, %6, %12\n\t"
           "global_load_ushort %4, %7, %13\n\t"
           "global_load_ubyte %5, %8, %14"
-          : "=&v"(dst[0].wq), "=&v"(dst[0].sc), "=&v"(dst[0].zp), "=&v"(dst[1].wq), "=&v"(dst[1].sc), "=&v"(dst[1].zp)
+          : "=&v"(dst[0].wq), "=&v"(dst[0].sc[0]), "=&v"(dst[0].zp[0]), "=&v"(dst[1].wq), "=&v"(dst[1].sc[0]), "=&v"(dst[1].zp[0])
           : "v"(w_voff), "v"(s_voff), "v"(z_voff), "s"(w0), "s"(s0), "s"(z0), "s"(w1), "s"(s1), "s"(z1)
           : "memory");
+      // the further groups of the k-tile (group sizes 64 and 32): the same loads 32 / 16 bytes further each
+#pragma unroll
+      for (int gi = 1; gi < GPT; ++gi) {
+        const char* s0g = s0 + gi * 32;
+        const char* s1g = s1 + gi * 32;
+        const char* z0g = z0 + gi * 16;
+        const char* z1g = z1 + gi * 16;
+        asm volatile(
+            "s_nop 4\n\t"
+            "global_load_ushort %0, %4, %6\n\t"
+            "global_load_ubyte %1, %5, %7\n\t"
+            "global_load_ushort %2, %4, %8\n\t"
+            "global_load_ubyte %3, %5, %9"
+            : "=&v"(dst[0].sc[gi]), "=&v"(dst[0].zp[gi]), "=&v"(dst[1].sc[gi]), "=&v"(dst[1].zp[gi])
+            : "v"(s_voff), "v"(z_voff), "s"(s0g), "s"(z0g), "s"(s1g), "s"(z1g)
+            : "memory");
+      }
     } else {
       asm volatile(
           "s_nop 4\n\t"
@@ -276,11 +298,26 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
           "global_load_ushort %1, %5, %7\n\t"
           "global_load_dwordx4 %2, %4, %8\n\t"
           "global_load_ushort %3, %5, %9"
-          : "=&v"(dst[0].wq), "=&v"(dst[0].sc), "=&v"(dst[1].wq), "=&v"(dst[1].sc)
+          : "=&v"(dst[0].wq), "=&v"(dst[0].sc[0]), "=&v"(dst[1].wq), "=&v"(dst[1].sc[0])
           : "v"(w_voff), "v"(s_voff), "s"(w0), "s"(s0), "s"(w1), "s"(s1)
           : "memory");
-      dst[0].zp = 8u;
-      dst[1].zp = 8u;
+#pragma unroll
+      for (int gi = 1; gi < GPT; ++gi) {
+        const char* s0g = s0 + gi * 32;
+        const char* s1g = s1 + gi * 32;
+        asm volatile(
+            "s_nop 4\n\t"
+            "global_load_ushort %0, %2, %3\n\t"
+            "global_load_ushort %1, %2, %4"
+            : "=&v"(dst[0].sc[gi]), "=&v"(dst[1].sc[gi])
+            : "v"(s_voff), "s"(s0g), "s"(s1g)
+            : "memory");
+      }
+#pragma unroll
+      for (int gi = 0; gi < GPT; ++gi) {
+        dst[0].zp[gi] = 8u;
+        dst[1].zp[gi] = 8u;
+      }
     }
   };
   // x stage `stage` -> LDS slot stage % NS.  The instruction offset of an LDS-targeted load is added to the LDS address
@@ -315,10 +352,15 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
   // wait until at most `n` loads are outstanding; the weight slots named become valid with this wait and are tied to it
   auto wait_tie = [&](auto n, WSlot (&fresh)[WN]) {
     asm volatile("s_waitcnt vmcnt(%6)"
-                 : "+v"(fresh[0].wq), "+v"(fresh[0].sc), "+v"(fresh[0].zp), "+v"(fresh[1].wq), "+v"(fresh[1].sc),
-                   "+v"(fresh[1].zp)
+                 : "+v"(fresh[0].wq), "+v"(fresh[0].sc[0]), "+v"(fresh[0].zp[0]), "+v"(fresh[1].wq), "+v"(fresh[1].sc[0]),
+                   "+v"(fresh[1].zp[0])
                  : "n"(decltype(n)::value)
                  : "memory");
+    // (the further groups' registers became valid with the same wait: an empty statement, which stays behind the wait
+    // like every volatile statement, ties them to it)
+#pragma unroll
+    for (int gi = 1; gi < GPT; ++gi)
+      asm volatile("" : "+v"(fresh[0].sc[gi]), "+v"(fresh[0].zp[gi]), "+v"(fresh[1].sc[gi]), "+v"(fresh[1].zp[gi])::"memory");
   };
   auto wait_only = [&](auto n) { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(decltype(n)::value) : "memory"); };
 
@@ -344,9 +386,9 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
       typename T::frag(&bnext)[WN] = bfrag[P ^ 1];
       const char* cur = frag_ptr(slot, ks);
       const char* nxt = ks == 0 ? frag_ptr(slot, 1) : frag_ptr((slot + 1) % NS, 0);
-      if (dn == 0) {
+      if (dn % (4 / GPT) == 0) {  // the next step opens a new quantization group
   #pragma unroll
-        for (int t = 0; t < WN; ++t) dq[t].set(wn[t].sc, wn[t].zp);
+        for (int t = 0; t < WN; ++t) dq[t].set(wn[t].sc[dn / (4 / GPT)], wn[t].zp[dn / (4 / GPT)]);
       }
   #pragma unroll
       for (int i = 0; i < WMV; ++i) {
@@ -381,7 +423,7 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
     __builtin_amdgcn_s_barrier();
   #pragma unroll
     for (int t = 0; t < WN; ++t) {
-      dq[t].set(ring[0][t].sc, ring[0][t].zp);
+      dq[t].set(ring[0][t].sc[0], ring[0][t].zp[0]);
       bfrag[0][t] = dq[t](ring[0][t].wq[0]);
     }
   #pragma unroll

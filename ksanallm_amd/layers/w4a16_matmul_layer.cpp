@@ -40,6 +40,12 @@ size_t W4A16MatMulLayer::GetWorkspaceSize() {
     const size_t ranks = static_cast<size_t>(std::max(1, context_->GetTensorParallelSize()));
     const size_t groups = std::min(max_k_, max_k_ * ranks / std::max<size_t>(1, groupsize_));
     permuted_k = (max_k_ + 31 * groups + 127) / 128 * 128;
+    // the GEMM then runs over the padded rows with group size 32: its scratch for any padded depth up to the bound
+    const int dtype = KsqDtype(inter_data_type_, Name());
+    for (size_t kk = (max_k_ + 127) / 128 * 128; kk <= permuted_k; kk += 128) {
+      const size_t need = (ksq_w4a16_workspace_size(max_m_, max_n_, kk, 32, dtype) + 255) & ~static_cast<size_t>(255);
+      gemm_workspace_size_ = std::max(gemm_workspace_size_, need);
+    }
   }
   permuted_input_size_ = is_gptq_desc_ ? max_m_ * permuted_k * GetTypeSize(inter_data_type_) : 0;
   workspace_size_ = gemm_workspace_size_ + permuted_input_size_;

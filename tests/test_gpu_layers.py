@@ -88,7 +88,7 @@ def test_w4a16_layer_act_order_k_range(tmp_path, oracle, dtype, backend, m, n, k
     run_driver("w4a16", tmp_path, "gptq", TNAME[dtype], backend, m, n, k, 128, 1, 1)
     y = read_out(tmp_path / "y.bin", dtype, (m, n))
     ref = oracle.gptq_act_order_gemm(H.bits_of(x), codes, H.bits_of(full["scales"]), g_idx.numpy(), dtype)
-    H.check_gemm(y, ref, dtype, "%s act-order K-range layer" % backend)
+    H.check_gemm(y, ref, dtype, "%s act-order K-range layer" % backend, weights_rounded=m > 32)
 
 
 @pytest.mark.gpu

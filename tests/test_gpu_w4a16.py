@@ -69,6 +69,18 @@ def test_prefill_tile_kernel(ops, dtype, awq, M, N, K):
     H.check_gemm(y, H.w4a16_oracle(d), dtype, "prefill M=%d N=%d K=%d" % (M, N, K), weights_rounded=True)
 
 
+# the same kernel with quantization groups of 64 and 32 rows (two or four scales and zero points per k-tile)
+@pytest.mark.parametrize("dtype", [H.F16, H.BF16])
+@pytest.mark.parametrize("awq", [False, True])
+@pytest.mark.parametrize("group", [64, 32])
+@pytest.mark.parametrize("M,N,K", [(33, 256, 256), (130, 512, 1024), (300, 768, 512), (1100, 512, 896), (512, 4352, 256),
+                                   (200, 256, 1664)])
+def test_prefill_tile_kernel_small_groups(ops, dtype, awq, group, M, N, K):
+    d = H.make_w4a16(3050 + M + N + group, M, N, K, group, dtype, awq=awq, x_std=0.5, s_lo=0.002, s_hi=0.01, z_lo=0, z_hi=15)
+    y = run_case(ops, d)
+    H.check_gemm(y, H.w4a16_oracle(d), dtype, "prefill group %d M=%d N=%d K=%d" % (group, M, N, K), weights_rounded=True)
+
+
 # 256-row tiles at sizes the oracle handles: the planner keeps them where more than 32 of them exist (the last case is
 # more than one round of tiles, so that some are cut along K)
 @pytest.mark.parametrize("dtype", [H.F16, H.BF16])
@@ -134,7 +146,7 @@ def test_cfg3_gptq_fp16_prefill(ops, N, K):
 def test_small_shapes_all_groups(ops, dtype, group, awq, M):
     d = H.make_w4a16(77 + M + group, M, 48, 384, group, dtype, awq=awq, z_lo=0, z_hi=15)
     y = run_case(ops, d)
-    H.check_gemm(y, H.w4a16_oracle(d), dtype, "small", weights_rounded=(M > 32 and group == 128))
+    H.check_gemm(y, H.w4a16_oracle(d), dtype, "small", weights_rounded=M > 32)
 
 
 def test_extreme_codes_and_zero_points(ops):
