@@ -94,6 +94,25 @@ __device__ __forceinline__ typename T::frag dequant_magic(uint32_t w) {
   return as_frag<T>(v);
 }
 
+// silu(g) * u in fp32, the one definition every kernel that applies the activation uses: exp through the hardware's
+// base-2 exponential (one multiply in front, no library expansion), 1 + e, an IEEE division and a multiply, with
+// contraction switched off.  Two kernels that must agree bit for bit (the MoE GEMM with the activation in its epilogue
+// and the stand-alone activation kernel) then execute the same five roundings; with expf, and with the result flowing
+// straight into a conversion, the compiler was free to fuse differently from one call site to the next, which showed as
+// one last-place difference in half a million outputs.  Accurate to about 2e-6 relative for |g| < 20, far inside one unit of fp16 / bf16.
+__device__ __forceinline__ float silu_mul_f32(float g, float u) {
+#pragma clang fp contract(off)
+  const float t = g * -1.44269504088896340736f;
+  const float e = __builtin_amdgcn_exp2f(t);
+  const float d = 1.0f + e;
+  const float q = g / d;
+  float y = q * u;
+  // the product exists as an fp32 value of its own: without this the compiler may fold the multiply into the caller's
+  // conversion to fp16 (one mixed-precision instruction that rounds once), which differs from rounding twice at ties
+  asm("" : "+v"(y));
+  return y;
+}
+
 __device__ __forceinline__ uint32_t pack2(uint16_t lo, uint16_t hi) {
   return static_cast<uint32_t>(lo) | (static_cast<uint32_t>(hi) << 16);
 }

@@ -277,8 +277,8 @@ __global__ void __launch_bounds__(256) silu_mul_kernel(const uint16_t* __restric
   for (int j = 0; j < 4; ++j) {
     float a0 = T::to_float(static_cast<uint16_t>(ra[j] & 0xffffu)), a1 = T::to_float(static_cast<uint16_t>(ra[j] >> 16));
     float b0 = T::to_float(static_cast<uint16_t>(rb[j] & 0xffffu)), b1 = T::to_float(static_cast<uint16_t>(rb[j] >> 16));
-    float y0 = a0 / (1.0f + expf(-a0)) * b0;
-    float y1 = a1 / (1.0f + expf(-a1)) * b1;
+    float y0 = silu_mul_f32(a0, b0);
+    float y1 = silu_mul_f32(a1, b1);
     o[j] = pack2(T::from_float(y0), T::from_float(y1));
   }
   *reinterpret_cast<u32x4*>(out + r * inter + c) = o;

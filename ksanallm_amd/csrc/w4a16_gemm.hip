@@ -66,12 +66,10 @@ int dispatch_tile(SplitKParams& p, SplitKChoice c, uint32_t m_blocks, size_t gro
   }
   p.nibble_mask = 0x000f000fu;
   p.magic2 = T::kMagic2;
-  if constexpr (!GROUPED) {
-    if (c.xc == 8 && c.mt == 1 && c.nt == 4 && c.waves == 8) return dispatch_group_zp<T, 1, 4, 8, false, 8>(p, m_blocks, group, s);
-    if (c.xc == 8 && c.mt == 1 && c.nt == 8 && c.waves == 8) return dispatch_group_zp<T, 1, 8, 8, false, 8>(p, m_blocks, group, s);
-    if (c.xc == 8 && c.mt == 2 && c.nt == 4 && c.waves == 8) return dispatch_group_zp<T, 2, 4, 8, false, 8>(p, m_blocks, group, s);
-    if (c.xc == 4 && c.mt == 2 && c.nt == 8 && c.waves == 4) return dispatch_group_zp<T, 2, 8, 4, false, 4>(p, m_blocks, group, s);
-  }
+  if (c.xc == 8 && c.mt == 1 && c.nt == 4 && c.waves == 8) return dispatch_group_zp<T, 1, 4, 8, GROUPED, 8>(p, m_blocks, group, s);
+  if (c.xc == 8 && c.mt == 1 && c.nt == 8 && c.waves == 8) return dispatch_group_zp<T, 1, 8, 8, GROUPED, 8>(p, m_blocks, group, s);
+  if (c.xc == 8 && c.mt == 2 && c.nt == 4 && c.waves == 8) return dispatch_group_zp<T, 2, 4, 8, GROUPED, 8>(p, m_blocks, group, s);
+  if (c.xc == 4 && c.mt == 2 && c.nt == 8 && c.waves == 4) return dispatch_group_zp<T, 2, 8, 4, GROUPED, 4>(p, m_blocks, group, s);
   if (c.xc != 0) return fail(KSQ_ERR_UNSUPPORTED, "no split-K kernel for mt=%d nt=%d waves=%d xc=%d", c.mt, c.nt, c.waves, c.xc);
 #define KSQ_CASE(MT_, NT_, W_)                                    \
   if (c.mt == MT_ && c.nt == NT_ && c.waves == W_)                \
@@ -119,13 +117,13 @@ int launch_tile_zp(const TileParams& p, unsigned grid, size_t group, hipStream_t
 }
 
 // grouped (MoE) form: one 128-row block of the aligned permutation per row tile, no split-K
-template <typename T>
+template <typename T, int WM>
 int launch_tile_grouped(const TileParams& p, hipStream_t s) {
-  constexpr int kLds = 4 * 8 * 2 * 1024;
+  constexpr int kLds = 4 * WM * 2 * 1024;
   // more dynamic LDS than a kernel may use without asking: once per device
   static std::atomic<uint64_t> configured{0};
-  if (int rc = allow_dynamic_lds(configured, reinterpret_cast<const void*>(&w4a16_tile_kernel<T, 8, false, true>), kLds)) return rc;
-  w4a16_tile_kernel<T, 8, false, true><<<p.tiles_m * p.tiles_n, 512, kLds, s>>>(p);
+  if (int rc = allow_dynamic_lds(configured, reinterpret_cast<const void*>(&w4a16_tile_kernel<T, WM, false, true>), kLds)) return rc;
+  w4a16_tile_kernel<T, WM, false, true><<<p.tiles_m * p.tiles_n, 512, kLds, s>>>(p);
   return KSQ_OK;
 }
 
@@ -337,18 +335,18 @@ int moe_w4a16_gemm_impl(const char* fn, bool fuse_silu, void* out, const void* x
   if (int rc = check_common(fn, out, x, w_packed, scales_packed, n, k, group, dtype)) return rc;
   if (fuse_silu) {
     if (n % 32 != 0) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: n = 2 * inter must be a multiple of 32", fn);
-    if (block_m == 128)
-      return fail(KSQ_ERR_UNSUPPORTED, "%s: 128-row blocks run the plain GEMM and ksq_silu_mul", fn);
+    if (block_m >= 128)
+      return fail(KSQ_ERR_UNSUPPORTED, "%s: 128- and 256-row blocks run the plain GEMM and ksq_silu_mul", fn);
   }
   if (!sorted_ids || !expert_ids || !num_post_pad) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: null index buffer", fn);
   if (zeros_packed) return fail(KSQ_ERR_UNSUPPORTED, "%s: zero points are not supported for expert weights", fn);
   if (group != 128) return fail(KSQ_ERR_UNSUPPORTED, "%s: expert weights need group size 128", fn);
   if (top_k == 0 || E == 0) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: top_k and E must be positive", fn);
-  if (block_m != 16 && block_m != 32 && block_m != 128)
-    return fail(KSQ_ERR_UNSUPPORTED, "%s: block_m %zu not in {16,32,128}", fn, block_m);
+  if (block_m != 16 && block_m != 32 && block_m != 128 && block_m != 256)
+    return fail(KSQ_ERR_UNSUPPORTED, "%s: block_m %zu not in {16,32,128,256}", fn, block_m);
   if (numel == 0) return KSQ_OK;
   const size_t cap_blocks = (numel + E * (block_m - 1)) / block_m;  // upper bound on aligned blocks
-  if (block_m == 128) {  // prefill regime: MFMA tile kernel, rows gathered / scattered through the permutation
+  if (block_m >= 128) {  // prefill regime: MFMA tile kernel, rows gathered / scattered through the permutation
     if (numel > 0x7fffffffull || (numel / top_k + 1) * k * 2 > 0xffffffffull)
       return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: x too large", fn);
     TileParams tp{};
@@ -356,7 +354,7 @@ int moe_w4a16_gemm_impl(const char* fn, bool fuse_silu, void* out, const void* x
     tp.x = x;
     tp.w = w_packed;
     tp.scales = scales_packed;
-    tp.M = static_cast<uint32_t>(cap_blocks * 128);
+    tp.M = static_cast<uint32_t>(cap_blocks * block_m);
     tp.N = static_cast<uint32_t>(n);
     tp.K = static_cast<uint32_t>(k);
     tp.tiles_m = static_cast<uint32_t>(cap_blocks);
@@ -370,7 +368,11 @@ int moe_w4a16_gemm_impl(const char* fn, bool fuse_silu, void* out, const void* x
     tp.topk_w = static_cast<const float*>(topk_w);
     tp.numel = static_cast<uint32_t>(numel);
     tp.top_k = static_cast<uint32_t>(top_k);
-    int rc = dtype == KSQ_F16 ? launch_tile_grouped<F16>(tp, as_stream(stream)) : launch_tile_grouped<BF16>(tp, as_stream(stream));
+    int rc;
+    if (block_m == 256)
+      rc = dtype == KSQ_F16 ? launch_tile_grouped<F16, 16>(tp, as_stream(stream)) : launch_tile_grouped<BF16, 16>(tp, as_stream(stream));
+    else
+      rc = dtype == KSQ_F16 ? launch_tile_grouped<F16, 8>(tp, as_stream(stream)) : launch_tile_grouped<BF16, 8>(tp, as_stream(stream));
     if (rc) return rc;
     return check_launch(fn);
   }
@@ -399,6 +401,21 @@ int moe_w4a16_gemm_impl(const char* fn, bool fuse_silu, void* out, const void* x
   if (fuse_silu) {
     if (c.nt < 2) c.nt = 2;  // a workgroup holds gate and up tiles in pairs
     p.pair_tiles = static_cast<uint32_t>(n / 32);
+  }
+  // activations through LDS (w4a16_splitk.h) as in the dense form: 2-3 % at E = 256, hidden 7168, inter 2048 from a
+  // few tokens per expert on (64 tokens 813 -> 788 us, 512 tokens 1353 -> 1316 us for the whole block), not for a
+  // handful of blocks (1 token: 50.1 -> 52.6 us)
+  if ((n / 16) % 4 == 0 && numel >= 32) {
+    if (c.mt == 2 && c.nt == 8) {
+      c.waves = 4;
+      c.xc = 4;
+    } else if (c.mt == 2 && c.nt == 4) {
+      c.waves = 8;
+      c.xc = 8;
+    } else if (c.mt == 1 && c.nt >= 4) {
+      c.waves = 8;
+      c.xc = 8;
+    }
   }
   int rc = dtype == KSQ_F16 ? dispatch_tile<F16, true>(p, c, static_cast<uint32_t>(cap_blocks), group, as_stream(stream))
                             : dispatch_tile<BF16, true>(p, c, static_cast<uint32_t>(cap_blocks), group, as_stream(stream));

@@ -428,7 +428,7 @@ __global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKPar
         const uint32_t sid = static_cast<uint32_t>(p.sorted_ids[blockIdx.y * (16 * MT) + r]);
         if (sid < p.numel) {
           const float gv = T::to_float(T::from_float(g[i])), uv = T::to_float(T::from_float(u[i]));
-          const float y = gv / (1.0f + expf(-gv)) * uv;
+          const float y = silu_mul_f32(gv, uv);
           static_cast<uint16_t*>(p.y)[static_cast<size_t>(sid) * out_n + col] = T::from_float(y);
         }
       }

@@ -457,10 +457,21 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
       }
     }
   };
-  if (live_tiles <= WM / 2)
+  if (GROUPED && WM == 16) {
+    // 256-slot expert blocks: the row tiles that hold slots, in steps of four (the depth of the fragment prefetch)
+    if (live_tiles <= 4)
+      run(std::integral_constant<int, 4>{});
+    else if (live_tiles <= 8)
+      run(std::integral_constant<int, 8>{});
+    else if (live_tiles <= 12)
+      run(std::integral_constant<int, (WM == 16 ? 12 : WM)>{});
+    else
+      run(std::integral_constant<int, WM>{});
+  } else if (live_tiles <= WM / 2) {
     run(std::integral_constant<int, WM / 2>{});
-  else
+  } else {
     run(std::integral_constant<int, WM>{});
+  }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // drain the clamped prefetches before the LDS is released
 
   // ---- store: lane holds row m = l%16 of the 16x16 tile and columns 4*(l/16) .. +3

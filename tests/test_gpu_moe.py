@@ -237,7 +237,7 @@ def pack_moe(ops, d):
 
 
 @pytest.mark.parametrize("dtype", [H.F16, H.BF16])
-@pytest.mark.parametrize("T,bm", [(1, 16), (5, 16), (64, 16), (64, 32), (64, 128), (300, 128), (512, 128)])
+@pytest.mark.parametrize("T,bm", [(1, 16), (5, 16), (64, 16), (64, 32), (64, 128), (300, 128), (512, 128), (300, 256), (700, 256)])
 def test_grouped_gemm_stages(ops, oracle, dtype, T, bm):
     d = make_moe(oracle, 5000 + T, 16, 256, 128, T, 4, 128, dtype)
     w13p, s13p, w2p, s2p = pack_moe(ops, d)
