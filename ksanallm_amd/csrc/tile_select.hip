@@ -235,8 +235,9 @@ KSQ_EXPORT size_t ksq_moe_block_m(size_t numel, size_t E) {
   if (E == 0) return 16;
   const size_t per_expert = numel / E;
   // 256-row blocks (the tile kernel multiplies the row tiles that hold rows, in steps of four) dequantize an expert's
-  // weights once where two 128-row blocks do it twice: 4 % at 256 rows per expert (8.71 -> 8.36 ms), level at 128
-  if (per_expert >= 192) return 256;
+  // weights once where two 128-row blocks do it twice.  E = 256, hidden 7168, inter 2048, top-8, whole call, 128- against
+  // 256-row blocks: 3.56 / 3.58 ms at 112 rows per expert, 4.57 / 4.21 at 128, 5.91 / 5.06 at 192, 7.90 / 7.05 at 256
+  if (per_expert >= 120) return 256;
   if (per_expert >= 40) return 128;
   return per_expert < 16 ? 16 : 32;
 }

@@ -39,10 +39,25 @@ __host__ __device__ __forceinline__ uint32_t xcd_range(uint32_t b, uint32_t tota
   return xcd * per + (xcd < rem ? xcd : rem) + local;  // XCDs 0..rem-1 own per+1 items
 }
 
+// The grouped (MoE) launches size their grid for the largest number of row blocks an alignment can produce, and the
+// blocks past the aligned length - up to half of the grid, all at the end of each band of the linear order - leave at
+// once.  A contiguous range per XCD would hand some XCDs nothing but such blocks; here every run of 256 consecutive
+// workgroups covers 256 consecutive items, 32 consecutive ones (4 row blocks x 8 column tiles) per XCD, so the blocks
+// that compute are spread over all XCDs at every moment of the launch.
+__host__ __device__ __forceinline__ uint32_t xcd_interleave(uint32_t b, uint32_t total) {
+  if (b >= total / 256 * 256) return b;
+  return (b & ~255u) + (b % 8) * 32 + (b % 256) / 8;
+}
+
 __host__ __device__ __forceinline__ TileWork tile_work(uint32_t b, uint32_t tiles_m, uint32_t tiles_n, uint32_t main_items,
-                                              uint32_t splits) {
+                                              uint32_t splits, bool grouped = false) {
   TileWork w;
-  if (main_items == 0) {
+  if (grouped) {
+    tile_order(xcd_interleave(b, tiles_m * tiles_n), tiles_m, tiles_n, &w.tile_m, &w.tile_n);
+    w.part = 0;
+    w.slot = 0;
+    w.direct = true;
+  } else if (main_items == 0) {
     const uint32_t cols = tiles_n * splits;
     uint32_t col;
     tile_order(xcd_range(b, tiles_m * cols), tiles_m, cols, &w.tile_m, &col);

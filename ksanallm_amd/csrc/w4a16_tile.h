@@ -172,7 +172,7 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
 
   // ---- work id (tile_work.h): output tile and the part of K this workgroup computes
   // (the divisions inside run on the vector unit: readfirstlane brings the wave-uniform results back to scalars)
-  const TileWork work = tile_work(blockIdx.x, p.tiles_m, p.tiles_n, p.main_items, p.splits);
+  const TileWork work = tile_work(blockIdx.x, p.tiles_m, p.tiles_n, p.main_items, p.splits, GROUPED);
   const uint32_t tile_m = __builtin_amdgcn_readfirstlane(work.tile_m), tile_n = __builtin_amdgcn_readfirstlane(work.tile_n);
   const uint32_t part = __builtin_amdgcn_readfirstlane(work.part), slot = __builtin_amdgcn_readfirstlane(work.slot);
   const bool direct = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(work.direct)) != 0;

@@ -37,8 +37,38 @@ static int check(uint32_t tiles_m, uint32_t tiles_n, uint32_t main_items, uint32
   return 0;
 }
 
+// grouped launches: every tile once, all direct; any 256 consecutive workgroups that lie inside the interleaved part
+// take 256 consecutive items, the 32 of one XCD (b % 8) consecutive among them
+static int check_grouped(uint32_t tiles_m, uint32_t tiles_n) {
+  const uint32_t tiles = tiles_m * tiles_n;
+  std::vector<int> whole(tiles, 0);
+  for (uint32_t b = 0; b < tiles; ++b) {
+    const TileWork w = tile_work(b, tiles_m, tiles_n, 0, 1, true);
+    if (w.tile_m >= tiles_m || w.tile_n >= tiles_n || !w.direct || w.part != 0) return 1;
+    if (whole[w.tile_m * tiles_n + w.tile_n]++) return 2;
+    const uint32_t lin = xcd_interleave(b, tiles);
+    if (lin >= tiles) return 3;
+    if (b < tiles / 256 * 256) {
+      if (lin / 256 != b / 256) return 4;
+      if ((lin % 256) / 32 != b % 8) return 5;
+    } else if (lin != b) {
+      return 6;
+    }
+  }
+  return 0;
+}
+
 int main() {
   int cases = 0;
+  for (uint32_t tm : {1u, 3u, 16u, 33u, 510u, 766u})
+    for (uint32_t tn : {1u, 7u, 16u, 28u}) {
+      const int rc = check_grouped(tm, tn);
+      ++cases;
+      if (rc) {
+        std::printf("FAIL grouped rc=%d tiles_m=%u tiles_n=%u\n", rc, tm, tn);
+        return 1;
+      }
+    }
   const uint32_t ms[] = {1, 2, 3, 5, 16, 33};
   const uint32_t ns[] = {1, 7, 8, 9, 20, 53, 100};
   for (uint32_t tm : ms)
