@@ -48,6 +48,7 @@ struct F16 {
     return __builtin_bit_cast(uint16_t, static_cast<_Float16>(f));
   }
   static constexpr uint32_t kOne2 = 0x3c003c00u;  // (1.0, 1.0)
+  static constexpr uint32_t kNegSym2 = 0xe408e408u;  // (-1032, -1032): minus (magic + 8), the offset of a code without zero point
   // low / high 16 bits of a dword as float
   static __device__ __forceinline__ float lo_to_float(uint32_t w) { return to_float(static_cast<uint16_t>(w)); }
   static __device__ __forceinline__ float hi_to_float(uint32_t w) { return to_float(static_cast<uint16_t>(w >> 16)); }
@@ -73,6 +74,7 @@ struct BF16 {
     return static_cast<uint16_t>(x >> 16);
   }
   static constexpr uint32_t kOne2 = 0x3f803f80u;
+  static constexpr uint32_t kNegSym2 = 0xc308c308u;  // (-136, -136)
   static __device__ __forceinline__ float lo_to_float(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
   static __device__ __forceinline__ float hi_to_float(uint32_t w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
 };

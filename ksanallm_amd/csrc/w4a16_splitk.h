@@ -11,7 +11,8 @@
 // magic+code with seven bit operations, x is the row operand and the weights the column operand of
 // v_mfma_f32_16x16x32, so a lane's four results share one output column, hence one scale and one zero point:
 //     acc += s * (sum_k x*(magic+code) - (magic+zp) * sum_k x)
-// with sum_k x from one more MFMA against an all-ones operand, shared by the NT tiles.
+// with sum_k x from one more MFMA against an all-ones operand, shared by the NT tiles.  Without zero points that MFMA
+// multiplies by -(magic + 8) itself and the weight MFMAs accumulate on top of its result: acc += s * r.
 //
 // What bounds the kernel is HBM latency x bandwidth, so the loads of a wavefront form one ring in issue order
 // (vmcnt retires loads in order: a second, shallower ring would drain the first each time it is waited for).  The
@@ -219,7 +220,11 @@ __global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKPar
       for (int d = 0; d < 4; ++d) b.xf[mt][d] = __builtin_amdgcn_raw_buffer_load_b128(xr, x_off[mt], o.x + d * 64, 0);
   };
 
-  const typename T::frag ones = as_frag<T>(u32x4{T::kOne2, T::kOne2, T::kOne2, T::kOne2});
+  // The operand of the sum-of-x MFMA: ones with zero points (the sum is then multiplied by each column's own offset);
+  // without them the offset is the same -(magic + 8) for every column, so the MFMA multiplies by it directly and its
+  // result is what the weight MFMAs of the group start from: r = -(magic + 8) * sum(x) + sum((magic + code) * x).
+  constexpr uint32_t kSumOperand = HAS_ZP ? T::kOne2 : T::kNegSym2;
+  const typename T::frag ones = as_frag<T>(u32x4{kSumOperand, kSumOperand, kSumOperand, kSumOperand});
   uint32_t magic2 = p.magic2;
   asm volatile("" : "+v"(magic2));  // no instruction: keeps the value in a VGPR so the three-operand form applies
   const uint32_t nmask = p.nibble_mask;
@@ -245,12 +250,13 @@ __global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKPar
       for (int d = 0; d < SPG; ++d) wf[d] = dequant_magic_fast<T>(s.wq[gi * SPG + d], nmask, magic2);
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
-        f32x4 r{0.f, 0.f, 0.f, 0.f};
+        f32x4 r = HAS_ZP ? f32x4{0.f, 0.f, 0.f, 0.f} : sx[gi][mt];
 #pragma unroll
         for (int d = 0; d < SPG; ++d) r = T::mfma(as_frag<T>(b.xf[mt][gi * SPG + d]), wf[d], r);
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-          acc[t][mt][i] = __builtin_fmaf(sc, __builtin_fmaf(ncz, sx[gi][mt][i], r[i]), acc[t][mt][i]);
+          acc[t][mt][i] = HAS_ZP ? __builtin_fmaf(sc, __builtin_fmaf(ncz, sx[gi][mt][i], r[i]), acc[t][mt][i])
+                                 : __builtin_fmaf(sc, r[i], acc[t][mt][i]);
       }
     }
   };
