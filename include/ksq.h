@@ -268,8 +268,7 @@ int ksq_moe_w4a16_gemm(void* out, const void* x, const void* w_packed, const voi
 /* The first MoE GEMM with the activation in its epilogue: w_packed holds [gate | up] rows (n = 2 * inter), and for every
  * valid sorted slot id s   out[s, c] = T(silu(T(g)) * T(u)),  g = x[s / top_k, :] . W[e, c, :],  u = x[s / top_k, :] . W[e, inter + c, :],
  * out [numel, inter] T: bit for bit what ksq_moe_w4a16_gemm into a [numel, 2 * inter] buffer followed by ksq_silu_mul
- * gives, in one launch and without that buffer.  block_m 16 or 32 (the decode regime, where a launch is a sizeable part
- * of the layer's time); 128 returns KSQ_ERR_UNSUPPORTED: run the two calls.
+ * gives, in one launch and without that buffer.  block_m 16, 32, 128 or 256, as for ksq_moe_w4a16_gemm.
  * Replaces the pair InvokeMoeWna16Gemm + InvokeSiluAndMul of InvokeFusedMoe
  * (S/kernels/nvidia/moe_kernel_wrapper.cpp:616-640). */
 int ksq_moe_w4a16_gate_up_silu(void* out, const void* x, const void* w_packed, const void* scales_packed,

@@ -335,8 +335,6 @@ int moe_w4a16_gemm_impl(const char* fn, bool fuse_silu, void* out, const void* x
   if (int rc = check_common(fn, out, x, w_packed, scales_packed, n, k, group, dtype)) return rc;
   if (fuse_silu) {
     if (n % 32 != 0) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: n = 2 * inter must be a multiple of 32", fn);
-    if (block_m >= 128)
-      return fail(KSQ_ERR_UNSUPPORTED, "%s: 128- and 256-row blocks run the plain GEMM and ksq_silu_mul", fn);
   }
   if (!sorted_ids || !expert_ids || !num_post_pad) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: null index buffer", fn);
   if (zeros_packed) return fail(KSQ_ERR_UNSUPPORTED, "%s: zero points are not supported for expert weights", fn);
@@ -358,7 +356,8 @@ int moe_w4a16_gemm_impl(const char* fn, bool fuse_silu, void* out, const void* x
     tp.N = static_cast<uint32_t>(n);
     tp.K = static_cast<uint32_t>(k);
     tp.tiles_m = static_cast<uint32_t>(cap_blocks);
-    tp.tiles_n = static_cast<uint32_t>(div_up(n, 256));
+    tp.tiles_n = static_cast<uint32_t>(div_up(n, 256));  // paired: 128 gate + 128 up columns per workgroup, the same count
+    tp.pair_tiles = fuse_silu ? static_cast<uint32_t>(n / 32) : 0;
     tp.main_items = 0;
     tp.splits = 1;
     tp.kt_per_split = static_cast<uint32_t>(k / 128);

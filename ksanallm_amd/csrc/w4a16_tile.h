@@ -46,6 +46,10 @@ struct TileParams {
   const int32_t* num_post_pad;
   const float* topk_w;  // optional: multiplied into the output row of slot id s
   uint32_t numel, top_k;
+  // grouped form, gate_up weights with silu(gate) * up in the epilogue: a wavefront's second column tile is the up tile
+  // pair_tiles (= N / 32) column tiles behind its gate tile, a workgroup covers 128 gate columns and the output has
+  // N / 2 columns.  0: plain GEMM.
+  uint32_t pair_tiles;
 };
 
 // dequantize one packed dword (8 codes) to 8 T values with (code - zp) * s applied
@@ -222,13 +226,16 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
 
   // ---- weights: this wavefront's two column tiles (clamped inside N; results of clamped tiles are not stored)
   const uint32_t n_tiles = p.N / 16;
-  const uint32_t nt0 = n0 / 16 + wave * WN;
+  const bool paired = GROUPED && p.pair_tiles != 0;
+  const uint32_t nt0 = paired ? tile_n * WAVES + wave : n0 / 16 + wave * WN;
   const char* w_base[WN];
   const char* s_base[WN];
   const char* z_base[WN];
 #pragma unroll
   for (int t = 0; t < WN; ++t) {
-    const size_t nt = static_cast<size_t>(expert) * n_tiles + ((nt0 + t < n_tiles) ? nt0 + t : n_tiles - 1);
+    uint32_t col_tile = (nt0 + t < n_tiles) ? nt0 + t : n_tiles - 1;
+    if (paired) col_tile = (nt0 < p.pair_tiles ? nt0 : p.pair_tiles - 1) + t * p.pair_tiles;
+    const size_t nt = static_cast<size_t>(expert) * n_tiles + col_tile;
     w_base[t] = static_cast<const char*>(p.w) + (nt * KT + kt_begin) * 1024;
     s_base[t] = static_cast<const char*>(p.scales) + (nt * KT + kt_begin) * (GPT * 32);
     z_base[t] = HAS_ZP ? static_cast<const char*>(p.zeros) + (nt * KT + kt_begin) * (GPT * 16) : nullptr;
@@ -483,7 +490,23 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
     } else {
       live = row < p.M;
     }
-    if (live) {
+    if (GROUPED && paired) {
+      // T(silu(T(gate)) * T(up)): both sums rounded to T as the plain GEMM would store them, so that the result has the
+      // bits of the two-launch form
+      if (live && nt0 < p.pair_tiles) {
+        u32x2 o;
+        uint16_t h[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float gv = T::to_float(T::from_float(acc[0][i][j])), uv = T::to_float(T::from_float(acc[1][i][j]));
+          h[j] = T::from_float(silu_mul_f32(gv, uv));
+        }
+        o.x = pack2(h[0], h[1]);
+        o.y = pack2(h[2], h[3]);
+        const size_t col = static_cast<size_t>(nt0) * 16 + 4 * lq;
+        *reinterpret_cast<u32x2*>(static_cast<uint16_t*>(p.y) + static_cast<size_t>(row) * (p.N / 2) + col) = o;
+      }
+    } else if (live) {
 #pragma unroll
       for (int t = 0; t < WN; ++t) {
         if (nt0 + t < n_tiles) {

@@ -190,7 +190,9 @@ def test_silu_mul_and_sum(ops, oracle, dtype):
 
 @pytest.mark.parametrize("dtype", [H.F16, H.BF16])
 @pytest.mark.parametrize("T,E,topk,hidden,inter,bm", [(1, 8, 2, 256, 128, 16), (5, 16, 4, 512, 256, 16), (70, 8, 2, 384, 80 * 16, 32),
-                                                      (33, 256, 8, 7168, 2048, 16), (300, 16, 4, 256, 16, 32)])
+                                                      (33, 256, 8, 7168, 2048, 16), (300, 16, 4, 256, 16, 32),
+                                                      (300, 6, 3, 256, 80 * 16, 128), (700, 4, 2, 384, 1024, 256),
+                                                      (130, 2, 1, 256, 16, 256), (520, 8, 2, 512, 2048, 128)])
 def test_gate_up_with_silu_in_the_epilogue_equals_the_two_launches(ops, dtype, T, E, topk, hidden, inter, bm):
     """ksq_moe_w4a16_gate_up_silu against ksq_moe_w4a16_gemm + ksq_silu_mul on the same inputs: the same bits."""
     from ksanallm_amd import lib as L
@@ -208,8 +210,8 @@ def test_gate_up_with_silu_in_the_epilogue_equals_the_two_launches(ops, dtype, T
     one = ops.moe_w4a16_gate_up_silu(x, wp, sp, s, e, npp, numel, topk, E, 2 * inter, hidden, 128, bm)
     torch.cuda.synchronize()
     assert torch.equal(one.view(torch.int16), two.view(torch.int16))
-    with pytest.raises(L.KsqError) as err:
-        ops.moe_w4a16_gate_up_silu(x, wp, sp, s, e, npp, numel, topk, E, 2 * inter, hidden, 128, 128)
+    with pytest.raises(L.KsqError) as err:   # a block size that no kernel has
+        ops.moe_w4a16_gate_up_silu(x, wp, sp, s, e, npp, numel, topk, E, 2 * inter, hidden, 128, 64)
     assert err.value.code == 2
 
 
