@@ -206,23 +206,8 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
   // 16*(j%4); it fetches piece (j%4) ^ (j/16) of row j/4, so that MFMA lane (row r, k piece q) finds its operand at
   // 64*r + 16*(q ^ (r/4)): the sixteen lanes that read together (same q) then hit sixteen different bank groups.
   const char* x_tile = static_cast<const char*>(p.x) + (static_cast<size_t>(GROUPED ? 0 : m0) * p.K + kt_begin * 128) * 2;
-  uint32_t a_voff[AP / 2];
-#pragma unroll
-  for (int j = 0; j < AP / 2; ++j) {
-    const uint32_t rb = wave * (AP / 2) + j;
-    uint32_t row = rb * 16 + (lane >> 2);
-    if (GROUPED) {
-      uint32_t sid = static_cast<uint32_t>(p.sorted_ids[m0 + row]);
-      sid = sid < p.numel ? sid : p.numel - 1;  // pad slots read some valid row; their results are dropped
-      row = sid / p.top_k;
-    } else {
-      row = (m0 + row < p.M) ? row : (p.M - 1 - m0);  // rows past M repeat the last row; their results are dropped
-    }
-    a_voff[j] = (row * p.K + 8 * ((lane & 3) ^ (lane >> 4))) * 2;
-  }
   const uint32_t a_rd = 64 * lrow + 16 * (lq ^ (lrow >> 2));  // this lane's operand inside a fragment
   const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<size_t>((__attribute__((address_space(3))) char*)lds));
-  const uint32_t a_lds_wave = lds_base + wave * AP * 1024;
 
   // ---- weights: this wavefront's two column tiles (clamped inside N; results of clamped tiles are not stored)
   const uint32_t n_tiles = p.N / 16;
@@ -322,35 +307,6 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
       }
     }
   };
-  // x stage `stage` -> LDS slot stage % NS.  The instruction offset of an LDS-targeted load is added to the LDS address
-  // as well as to the global one: the second fragment's 64-byte global offset is taken back out of its LDS base.
-  auto load_a = [&](uint32_t stage) {
-    const uint32_t st = stage < stages ? stage : stages - 1;
-    const char* src = x_tile + static_cast<size_t>(st) * (BK * 2);
-    const uint32_t d0 = __builtin_amdgcn_readfirstlane(a_lds_wave + (stage % NS) * STAGE_BYTES);
-    const uint32_t d1 = d0 + 1024 - 64;
-    if (AP == 2) {
-      asm volatile(
-          "s_nop 4\n\t"
-          "s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %3\n\t"
-          "s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %3 offset:64"
-          :
-          : "v"(a_voff[0]), "s"(d0), "s"(d1), "s"(src)
-          : "memory");
-    } else {
-      static_assert(AP == 2 || AP == 4, "two or four fragments per wavefront and stage");
-      const uint32_t d2 = d0 + 2048, d3 = d1 + 2048;
-      asm volatile(
-          "s_nop 4\n\t"
-          "s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %6\n\t"
-          "s_mov_b32 m0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %6 offset:64\n\t"
-          "s_mov_b32 m0, %4\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %6\n\t"
-          "s_mov_b32 m0, %5\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %6 offset:64"
-          :
-          : "v"(a_voff[0]), "v"(a_voff[AP / 2 - 1]), "s"(d0), "s"(d1), "s"(d2), "s"(d3), "s"(src)
-          : "memory");
-    }
-  };
   // wait until at most `n` loads are outstanding; the weight slots named become valid with this wait and are tied to it
   auto wait_tie = [&](auto n, WSlot (&fresh)[WN]) {
     asm volatile("s_waitcnt vmcnt(%6)"
@@ -372,6 +328,53 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
   // blocks and lose the interleaving of LDS reads, conversions and MFMAs (measured: 20 % slower, not faster).
   auto run = [&](auto wmv_c) {
     constexpr int WMV = decltype(wmv_c)::value;
+    // Fragments this wavefront stages per x stage.  A 256-slot expert block of which at most the lower eight row tiles
+    // hold slots stages those only (two fragments per wavefront instead of four); the reads below never reach further.
+    constexpr int APV = (GROUPED && WM == 16 && WMV <= 8) ? 2 : AP;
+    uint32_t a_voff[APV / 2];
+#pragma unroll
+    for (int j = 0; j < APV / 2; ++j) {
+      const uint32_t rb = wave * (APV / 2) + j;
+      uint32_t row = rb * 16 + (lane >> 2);
+      if (GROUPED) {
+        uint32_t sid = static_cast<uint32_t>(p.sorted_ids[m0 + row]);
+        sid = sid < p.numel ? sid : p.numel - 1;  // pad slots read some valid row; their results are dropped
+        row = sid / p.top_k;
+      } else {
+        row = (m0 + row < p.M) ? row : (p.M - 1 - m0);  // rows past M repeat the last row; their results are dropped
+      }
+      a_voff[j] = (row * p.K + 8 * ((lane & 3) ^ (lane >> 4))) * 2;
+    }
+    const uint32_t a_lds_wave = lds_base + wave * APV * 1024;
+    // x stage `stage` -> LDS slot stage % NS.  The instruction offset of an LDS-targeted load is added to the LDS address
+    // as well as to the global one: the second fragment's 64-byte global offset is taken back out of its LDS base.
+    auto load_a = [&](uint32_t stage) {
+      const uint32_t st = stage < stages ? stage : stages - 1;
+      const char* src = x_tile + static_cast<size_t>(st) * (BK * 2);
+      const uint32_t d0 = __builtin_amdgcn_readfirstlane(a_lds_wave + (stage % NS) * STAGE_BYTES);
+      const uint32_t d1 = d0 + 1024 - 64;
+      if constexpr (APV == 2) {
+        asm volatile(
+            "s_nop 4\n\t"
+            "s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %3\n\t"
+            "s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %3 offset:64"
+            :
+            : "v"(a_voff[0]), "s"(d0), "s"(d1), "s"(src)
+            : "memory");
+      } else {
+        static_assert(APV == 2 || APV == 4, "two or four fragments per wavefront and stage");
+        const uint32_t d2 = d0 + 2048, d3 = d1 + 2048;
+        asm volatile(
+            "s_nop 4\n\t"
+            "s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %6\n\t"
+            "s_mov_b32 m0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %6 offset:64\n\t"
+            "s_mov_b32 m0, %4\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %6\n\t"
+            "s_mov_b32 m0, %5\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %6 offset:64"
+            :
+            : "v"(a_voff[0]), "v"(a_voff[APV / 2 - 1]), "s"(d0), "s"(d1), "s"(d2), "s"(d3), "s"(src)
+            : "memory");
+      }
+    };
     // ---- compute pipeline, in steps of 32 k (two per stage).  A fragments are read DEPTH ahead of the MFMAs that use
     // them, across step and stage boundaries; the weight fragments of step g+1 are dequantized while step g multiplies.
     constexpr int DEPTH = 4;
@@ -412,10 +415,10 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
     // stage c): wait for x stage c+1, barrier, then issue [weights of k-tile c/2+2 when c is even][x stage c+3] - the LDS
     // slot of stage c+3 is the one stage c-1 used, and every wavefront is past that.  Weights of k-tile kt are issued at
     // sync 2kt-4, complete at sync 2kt-2 and are first dequantized during the last step of k-tile kt-1.
-    // Loads outstanding after x stage c+1 at sync c: those of sync c-1, i.e. AP, plus 2*WL when c-1 is even.
-    using WaitEven = std::integral_constant<int, AP>;
-    using WaitOdd = std::integral_constant<int, AP + WN * WL>;
-    using WaitFirst = std::integral_constant<int, 2 * AP + WN * WL>;
+    // Loads outstanding after x stage c+1 at sync c: those of sync c-1, i.e. APV, plus 2*WL when c-1 is even.
+    using WaitEven = std::integral_constant<int, APV>;
+    using WaitOdd = std::integral_constant<int, APV + WN * WL>;
+    using WaitFirst = std::integral_constant<int, 2 * APV + WN * WL>;
     load_w(ring[0], 0);  // sync -4
     load_a(0);           // sync -3
     load_w(ring[1], 1);  // sync -2
