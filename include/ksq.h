@@ -202,7 +202,7 @@ int ksq_fp8_tensor_gemm(const void* a_q, const void* a_scale, const void* b, con
                         size_t n, size_t k, int out_dtype, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------------------------------------------------
- * W4A8: int4 weights (group 128, fp16 scales, no zero points) against statically quantized e4m3 activations,
+ * W4A8: int4 weights (group 128 or 64, fp16 scales, no zero points) against statically quantized e4m3 activations,
  *   out[m,n] = T(alpha * sum_g scale[g,n] * sum_{k in g} a_q[m,k] * w[k,n]),  w in -8..7, fp32 accumulation.
  * The path of FinegrainedMixedDtypeGemmLayer (S/layers/nvidia/finegrained_mixed_dtype_gemm_layer.cpp:15-183) over
  * FinegrainedMixedDtypeGemmWrapper (K/gemm/finegrained_mixed_dtype_gemm/finegrained_mixed_dtype_gemm_wrapper.cpp).
@@ -219,12 +219,13 @@ int ksq_fp8_tensor_gemm(const void* a_q, const void* a_scale, const void* b, con
  *   takes x that is e4m3 already and writes xsum only (q and scale unused).
  *   Replaces StaticQuantizeE4M3PerTensor / PerToken / PerChannel (wrapper.cpp:128-153 -> scaleMatrix,
  *   K/others/tensorrt-llm/dev/common/cudaFp8Utils.cu:38-52).
- * ksq_w4a8_gemm: a_q [m,k] e4m3 row-major, xsum [k/128,m], w_packed from ksq_w4a8_repack_weight, scales fp16
- *   [k/128, n] as the reference holds them (weight_scale / weight_scale_2), alpha = input_scale * weight_scale_2.
+ * ksq_w4a8_gemm: a_q [m,k] e4m3 row-major, xsum [k/group,m], w_packed from ksq_w4a8_repack_weight, scales fp16
+ *   [k/group, n] as the reference holds them (weight_scale / weight_scale_2), alpha = input_scale * weight_scale_2.
  *   Replaces FinegrainedMixedDtypeGemmWrapper::Forward (wrapper.cpp:68-100); no tactic argument: the kernel is
  *   chosen from the shape.
  * ------------------------------------------------------------------------------------------------------------------ */
-enum { KSQ_W4A8_PER_TENSOR = 0, KSQ_W4A8_PER_CHANNEL = 1, KSQ_W4A8_SUMS_ONLY = 2, KSQ_W4A8_PER_TOKEN = 3 };
+enum { KSQ_W4A8_PER_TENSOR = 0, KSQ_W4A8_PER_CHANNEL = 1, KSQ_W4A8_SUMS_ONLY = 2, KSQ_W4A8_PER_TOKEN = 3,
+       KSQ_W4A8_SUMS_PER_64 = 16 /* or-ed into the mode: xsum [k/64, m], one sum per 64 channels (GEMM group size 64) */ };
 size_t ksq_w4a8_packed_weight_bytes(size_t n, size_t k);
 int ksq_w4a8_repack_weight(const void* src, void* dst_packed, size_t n, size_t k, void* stream);
 int ksq_w4a8_unpack_weight(const void* packed, void* dst, size_t n, size_t k, void* stream);

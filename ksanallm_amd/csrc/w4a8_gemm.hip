@@ -94,7 +94,8 @@ __device__ __forceinline__ float sum8_e4m3(u32x2 q) {
 // IEEE fp32 division, round to nearest even, saturating.  xsum[g, row] = sum of the 128 quantized values of group g
 // (every e4m3 value is a multiple of 2^-9, so the fp32 sum is exact, in any order, while it stays below 2^15).
 // Grid: x = chunks of BLOCK * 8 channels, y/z = row; a group of 128 channels is 16 adjacent lanes.
-template <typename T, int MODE, int BLOCK>
+// SG: channels per sum, 128 or 64 (16 or 8 adjacent lanes).
+template <typename T, int MODE, int BLOCK, int SG = 128>
 __global__ void __launch_bounds__(BLOCK) w4a8_quant_kernel(const void* __restrict__ xin, const float* __restrict__ scale,
                                                          uint8_t* __restrict__ q, float* __restrict__ xsum, uint32_t m,
                                                          uint32_t k) {
@@ -146,18 +147,18 @@ __global__ void __launch_bounds__(BLOCK) w4a8_quant_kernel(const void* __restric
   }
   float sum = sum8_e4m3(out);
 #pragma unroll
-  for (int off = 1; off < 16; off <<= 1) sum += __shfl_xor(sum, off, 16);
+  for (int off = 1; off < SG / 8; off <<= 1) sum += __shfl_xor(sum, off, 16);
   if (!live) return;
   if (MODE != 2) *reinterpret_cast<u32x2*>(q + e0) = out;
-  if ((threadIdx.x & 15) == 0) xsum[static_cast<size_t>(col / 128) * m + t] = sum;
+  if ((threadIdx.x & (SG / 8 - 1)) == 0) xsum[static_cast<size_t>(col / SG) * m + t] = sum;
 }
 
 // ------------------------------------------------------------------------------------------------ GEMM
 struct W4A8Params {
   const uint8_t* a;      // [M, K] e4m3
-  const float* xsum;     // [K/128, M]
+  const float* xsum;     // [K/group, M]
   const uint8_t* w;      // packed fragments
-  const uint16_t* sc;    // fp16 [K/128, N]
+  const uint16_t* sc;    // fp16 [K/group, N]
   void* out;             // [M, N]
   uint32_t M, N, K;
   float alpha512;        // alpha * 2^9
@@ -182,8 +183,12 @@ __device__ __forceinline__ i32x8 expand_u4(i32x4 p) {
 // wavefront w takes the k-blocks w, w+WAVES, ... with LOOK of them loaded ahead into registers.  Blocks past the end
 // are clamped to the last one and given zero scales, so that control flow stays uniform.  Partials are summed through
 // LDS in wavefront order.
-template <typename TO, int MT, int NT, int WAVES, int LOOK>
+// GROUP = 64: the instruction still spans 128 k; it is issued twice per k-block, once with the activation bytes of the
+// upper 64 k (lanes 32..63 of the operand) cleared and once with those of the lower 64 k cleared, each with its own
+// addend and its own scales - exact, at twice the MFMAs, which a kernel that waits for HBM does not notice.
+template <typename TO, int MT, int NT, int WAVES, int LOOK, int GROUP = 128>
 __global__ void __launch_bounds__(WAVES * 64) w4a8_splitk_kernel(W4A8Params p) {
+  constexpr int GH = 128 / GROUP;  // scale groups per k-block
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lrow = lane & 15;
@@ -214,9 +219,9 @@ __global__ void __launch_bounds__(WAVES * 64) w4a8_splitk_kernel(W4A8Params p) {
 
   struct Stage {
     i32x4 w[NT];
-    u32x2 sc[NT];
+    u32x2 sc[NT][GH];
     i32x4 a0[MT], a1[MT];
-    float xs[MT];
+    float xs[MT][GH];
   };
   Stage ring[LOOK];
   auto load_stage = [&](Stage& s, uint32_t kb) {
@@ -226,29 +231,42 @@ __global__ void __launch_bounds__(WAVES * 64) w4a8_splitk_kernel(W4A8Params p) {
     for (int nt = 0; nt < NT; ++nt) {
       const uint8_t* wp = wptr + (static_cast<size_t>(nt) * KB + kb) * 1024;
       s.w[nt] = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(wp));
-      const u32x2 sc = *reinterpret_cast<const u32x2*>(scptr + static_cast<size_t>(kb) * p.N + nt * 16);
-      s.sc[nt] = live ? sc : u32x2{0u, 0u};
+#pragma unroll
+      for (int h = 0; h < GH; ++h) {
+        const u32x2 sc = *reinterpret_cast<const u32x2*>(scptr + (static_cast<size_t>(kb) * GH + h) * p.N + nt * 16);
+        s.sc[nt][h] = live ? sc : u32x2{0u, 0u};
+      }
     }
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       const i32x4* ap = reinterpret_cast<const i32x4*>(aptr[mt] + static_cast<size_t>(kb) * 128);
       s.a0[mt] = ap[0];
       s.a1[mt] = ap[1];
-      s.xs[mt] = xsptr[mt][static_cast<size_t>(kb) * p.M];
+#pragma unroll
+      for (int h = 0; h < GH; ++h) s.xs[mt][h] = xsptr[mt][(static_cast<size_t>(kb) * GH + h) * p.M];
     }
   };
   auto compute_stage = [&](const Stage& s) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       const i32x8 a{s.a0[mt].x, s.a0[mt].y, s.a0[mt].z, s.a0[mt].w, s.a1[mt].x, s.a1[mt].y, s.a1[mt].z, s.a1[mt].w};
-      const float c = s.xs[mt] * -0.015625f;  // -8 * 2^-9 * xsum
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt) {
-        const f32x4 r = mfma_fp8_128(expand_u4(s.w[nt]), a, f32x4{c, c, c, c});
-        acc[nt][mt][0] = __builtin_fmaf(r[0], F16::lo_to_float(s.sc[nt].x), acc[nt][mt][0]);
-        acc[nt][mt][1] = __builtin_fmaf(r[1], F16::hi_to_float(s.sc[nt].x), acc[nt][mt][1]);
-        acc[nt][mt][2] = __builtin_fmaf(r[2], F16::lo_to_float(s.sc[nt].y), acc[nt][mt][2]);
-        acc[nt][mt][3] = __builtin_fmaf(r[3], F16::hi_to_float(s.sc[nt].y), acc[nt][mt][3]);
+      for (int h = 0; h < GH; ++h) {
+        i32x8 ah = a;
+        if (GH == 2) {  // this lane's 32 k lie in half lq / 2 of the k-block
+          const int keep = (lq >> 1) == h ? -1 : 0;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) ah[e] = a[e] & keep;
+        }
+        const float c = s.xs[mt][h] * -0.015625f;  // -8 * 2^-9 * xsum
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+          const f32x4 r = mfma_fp8_128(expand_u4(s.w[nt]), ah, f32x4{c, c, c, c});
+          acc[nt][mt][0] = __builtin_fmaf(r[0], F16::lo_to_float(s.sc[nt][h].x), acc[nt][mt][0]);
+          acc[nt][mt][1] = __builtin_fmaf(r[1], F16::hi_to_float(s.sc[nt][h].x), acc[nt][mt][1]);
+          acc[nt][mt][2] = __builtin_fmaf(r[2], F16::lo_to_float(s.sc[nt][h].y), acc[nt][mt][2]);
+          acc[nt][mt][3] = __builtin_fmaf(r[3], F16::hi_to_float(s.sc[nt][h].y), acc[nt][mt][3]);
+        }
       }
     }
   };
@@ -297,7 +315,7 @@ __global__ void __launch_bounds__(WAVES * 64) w4a8_splitk_kernel(W4A8Params p) {
 // more resident wavefronts, and those hide the latency better than a ring does (a ring 2, 3 or 4 deep measured 6-15 %
 // slower each step).  Grids below one workgroup per CU split K over eight wavefronts instead of four (n = 5120:
 // 8.1 -> 6.1 us).
-template <typename TO>
+template <typename TO, int GROUP = 128>
 int dispatch_splitk(const W4A8Params& p, hipStream_t s) {
   const SplitKChoice c = select_w4a8_splitk(p.M, p.N);
   const int mt = c.mt, nt = c.nt, waves = c.waves;
@@ -305,7 +323,7 @@ int dispatch_splitk(const W4A8Params& p, hipStream_t s) {
   const dim3 grid(groups, static_cast<unsigned>(div_up(p.M, 16 * mt)), 1);
 #define KSQ_CASE(MT_, NT_, W_)                                                   \
   if (mt == MT_ && nt == NT_ && waves == W_) {                                   \
-    w4a8_splitk_kernel<TO, MT_, NT_, W_, 1><<<grid, W_ * 64, 0, s>>>(p);         \
+    w4a8_splitk_kernel<TO, MT_, NT_, W_, 1, GROUP><<<grid, W_ * 64, 0, s>>>(p);  \
     return KSQ_OK;                                                               \
   }
   KSQ_CASE(1, 1, 4) KSQ_CASE(1, 2, 4) KSQ_CASE(1, 4, 4) KSQ_CASE(2, 1, 4) KSQ_CASE(2, 2, 4) KSQ_CASE(2, 4, 4)
@@ -316,11 +334,11 @@ int dispatch_splitk(const W4A8Params& p, hipStream_t s) {
 
 // Prefill regime: the MFMA tile kernel of w4a8_tile.h on the grid plan_w4a8_tile lays out (the blockwise-FP8 tile
 // shapes; a k-step is one 128-deep group).
-template <typename TO, int WM>
+template <typename TO, int WM, int GROUP = 128>
 int launch_tile(const W4A8Params& q, const TilePlan& plan, float* partial, hipStream_t s) {
   constexpr int kLds = static_cast<int>(w4a8_tile_lds_bytes(WM));
   static std::atomic<uint64_t> configured{0};
-  if (int rc = allow_dynamic_lds(configured, reinterpret_cast<const void*>(&w4a8_tile_kernel<TO, WM>), kLds)) return rc;
+  if (int rc = allow_dynamic_lds(configured, reinterpret_cast<const void*>(&w4a8_tile_kernel<TO, WM, GROUP>), kLds)) return rc;
   W4A8TileParams p{};
   p.a = q.a;
   p.xsum = q.xsum;
@@ -337,7 +355,7 @@ int launch_tile(const W4A8Params& q, const TilePlan& plan, float* partial, hipSt
   p.splits = plan.splits;
   p.kb_per_split = plan.kt_per_split;
   p.alpha512 = q.alpha512;
-  w4a8_tile_kernel<TO, WM><<<plan.grid, 512, kLds, s>>>(p);
+  w4a8_tile_kernel<TO, WM, GROUP><<<plan.grid, 512, kLds, s>>>(p);
   if (plan.splits > 1) {
     const unsigned cut = plan.tiles_m * plan.tiles_n - plan.main_items;
     splitk_reduce_kernel<TO, 32 * WM><<<cut * (4 * WM), 256, 0, s>>>(partial, static_cast<uint16_t*>(p.out), p.M, p.N,
@@ -384,6 +402,8 @@ KSQ_EXPORT int ksq_w4a8_unpack_weight(const void* packed, void* dst, size_t n, s
 KSQ_EXPORT int ksq_w4a8_static_quant(const void* x, const void* scale, void* q, void* xsum, size_t m, size_t k,
                                      int mode, int dtype, void* stream) {
   const char* fn = "ksq_w4a8_static_quant";
+  const bool per64 = (mode & KSQ_W4A8_SUMS_PER_64) != 0;  // group sums per 64 channels: what the GEMM with group 64 reads
+  mode &= ~KSQ_W4A8_SUMS_PER_64;
   if (!x || !xsum || (mode != KSQ_W4A8_SUMS_ONLY && (!q || !scale))) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: null pointer", fn);
   if (mode != KSQ_W4A8_PER_TENSOR && mode != KSQ_W4A8_PER_CHANNEL && mode != KSQ_W4A8_SUMS_ONLY && mode != KSQ_W4A8_PER_TOKEN)
     return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: unknown mode %d", fn, mode);
@@ -406,8 +426,12 @@ KSQ_EXPORT int ksq_w4a8_static_quant(const void* x, const void* scale, void* q, 
   const uint32_t mm = static_cast<uint32_t>(m), kk = static_cast<uint32_t>(k);
   // the largest block whose chunks tile a row without idle lanes (k is a multiple of 128 = 16 lanes)
   const int block = k % 2048 == 0 ? 256 : (k % 1024 == 0 ? 128 : (k % 512 == 0 || k < 2048 ? 64 : 256));
-#define KSQ_Q(TT, MODE_, B_)                                                                                      \
-  w4a8_quant_kernel<TT, MODE_, B_><<<dim3(static_cast<unsigned>(div_up(k, B_ * 8)), gy, gz), B_, 0, st>>>(x, sp, qp, xs, mm, kk)
+#define KSQ_Q(TT, MODE_, B_)                                                                                              \
+  do {                                                                                                                    \
+    const dim3 qgrid(static_cast<unsigned>(div_up(k, B_ * 8)), gy, gz);                                                   \
+    if (per64) w4a8_quant_kernel<TT, MODE_, B_, 64><<<qgrid, B_, 0, st>>>(x, sp, qp, xs, mm, kk);                         \
+    else w4a8_quant_kernel<TT, MODE_, B_, 128><<<qgrid, B_, 0, st>>>(x, sp, qp, xs, mm, kk);                              \
+  } while (0)
 #define KSQ_QB(TT, MODE_)                        \
   do {                                           \
     if (block == 256) KSQ_Q(TT, MODE_, 256);     \
@@ -445,7 +469,7 @@ KSQ_EXPORT int ksq_w4a8_gemm(const void* a_q, const void* xsum, const void* w_pa
                              size_t workspace_bytes, void* stream) {
   const char* fn = "ksq_w4a8_gemm";
   if (!a_q || !xsum || !w_packed || !scales || !out) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: null pointer", fn);
-  if (group != 128) return fail(KSQ_ERR_UNSUPPORTED, "%s: group size %zu (only 128)", fn, group);
+  if (group != 128 && group != 64) return fail(KSQ_ERR_UNSUPPORTED, "%s: group size %zu (128 or 64)", fn, group);
   if (n == 0 || k == 0 || n % 16 != 0 || k % 128 != 0)
     return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: n must be a positive multiple of 16 and k of 128 (n=%zu k=%zu)", fn, n, k);
   if (out_dtype != KSQ_F16 && out_dtype != KSQ_BF16) return fail(KSQ_ERR_UNSUPPORTED, "%s: out dtype must be f16 or bf16", fn);
@@ -466,7 +490,23 @@ KSQ_EXPORT int ksq_w4a8_gemm(const void* a_q, const void* xsum, const void* w_pa
   p.alpha512 = alpha * 512.0f;
   hipStream_t st = as_stream(stream);
   int rc;
-  if (use_tile(m)) {
+  if (group == 64) {
+    // two scale groups per k-block: the streaming kernel, or 128-token tiles over all of K (no workspace)
+    if (use_tile(m)) {
+      if (256 * k > 0xffffffffull || 16 * (k / 128) * 1024 > 0xffffffffull) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: k too large", fn);
+      TilePlan plan{};
+      plan.block_m = 128;
+      plan.tiles_m = static_cast<unsigned>(div_up(m, 128));
+      plan.tiles_n = static_cast<unsigned>(div_up(n, 256));
+      plan.main_items = 0;
+      plan.splits = 1;
+      plan.kt_per_split = static_cast<unsigned>(k / 128);
+      plan.grid = plan.tiles_m * plan.tiles_n;
+      rc = out_dtype == KSQ_F16 ? launch_tile<F16, 4, 64>(p, plan, nullptr, st) : launch_tile<BF16, 4, 64>(p, plan, nullptr, st);
+    } else {
+      rc = out_dtype == KSQ_F16 ? dispatch_splitk<F16, 64>(p, st) : dispatch_splitk<BF16, 64>(p, st);
+    }
+  } else if (use_tile(m)) {
     const TilePlan plan = plan_w4a8_tile(m, n, k);
     if (plan.splits > 1 && (!workspace || workspace_bytes < plan.workspace_bytes || !aligned16(workspace)))
       return fail(KSQ_ERR_WORKSPACE, "%s: m=%zu n=%zu k=%zu needs %zu bytes of 16-byte aligned workspace, got %zu", fn, m,

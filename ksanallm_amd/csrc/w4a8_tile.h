@@ -54,9 +54,15 @@ __device__ __forceinline__ i32x8 w4a8_expand(i32x4 p) {
 }
 
 // WM = 8: 256-token tiles.  WM = 4: 128-token tiles.
-template <typename TO, int WM>
+// GROUP = 64 (128-token tiles only): a k-block holds two scale groups.  Its two rows of group sums and of weight scales
+// ride the same loads as the one row of GROUP = 128 (the lanes that repeat data there fetch the second row here), and
+// every MFMA is issued twice, once with the weight bytes of the upper 64 k cleared and once with the lower ones
+// cleared (this lane's 32 k lie in half lane / 32), each with its own addend and scales.
+template <typename TO, int WM, int GROUP = 128>
 __global__ void __launch_bounds__(512, 1) w4a8_tile_kernel(W4A8TileParams p) {
   static_assert(WM == 8 || WM == 4, "256- or 128-token tiles");
+  static_assert(GROUP == 128 || (GROUP == 64 && WM == 4), "group 64 runs on 128-token tiles");
+  constexpr int GH = 128 / GROUP;
   constexpr int WAVES_N = 4;
   constexpr int WN = 4;  // 16x16 tiles per wavefront: 16*WM tokens x 64 weight columns
   constexpr int BM = 2 * WM * 16, BN = 256;
@@ -124,22 +130,29 @@ __global__ void __launch_bounds__(512, 1) w4a8_tile_kernel(W4A8TileParams p) {
   // the last four).  Otherwise wavefronts 0..BM/64-1 copy 64 each, 4 bytes per lane, every lane clamped on its own.
   const bool s_vec = (p.M & 3) == 0;
   uint32_t s_row = s_vec ? m0 + 4 * lane : m0 + (wave & 3) * 64 + lane;
-  if (s_vec && 4 * lane >= BM) s_row = m0;
-  if (!s_vec && (wave & 3) * 64 >= BM) s_row = m0;
+  uint32_t s_half = 0;  // GROUP = 64: the lanes / wavefronts past the tile's tokens fetch the second row of sums
+  if (s_vec && 4 * lane >= BM) {
+    s_row = GH == 2 ? m0 + 4 * lane - BM : m0;
+    s_half = GH == 2 ? 1 : 0;
+  }
+  if (!s_vec && (wave & 3) * 64 >= BM) {
+    s_row = GH == 2 ? m0 + (wave & 3) * 64 + lane - BM : m0;
+    s_half = GH == 2 ? 1 : 0;
+  }
   {
     const uint32_t s_last = s_vec ? p.M - 4 : p.M - 1;
     s_row = s_row < s_last ? s_row : s_last;
   }
-  const uint32_t s_voff = s_row * 4;
-  const char* xs_base = reinterpret_cast<const char*>(p.xsum) + static_cast<size_t>(kb_begin) * p.M * 4;
+  const uint32_t s_voff = (s_half * p.M + s_row) * 4;
+  const char* xs_base = reinterpret_cast<const char*>(p.xsum) + static_cast<size_t>(kb_begin) * GH * p.M * 4;
   const uint32_t s_lds = lds_base + XS_BASE + (s_vec ? 0 : (wave & 3) * 256);
-  const bool has_xs_load = s_vec ? wave == 0 : wave < BM / 64;
+  const bool has_xs_load = s_vec ? wave == 0 : wave < (GH == 2 ? 4 : BM / 64);
   // ---- weight scales of a k-block: 256 fp16 = 512 bytes, lanes 0..31 of wavefront 4 take 16 bytes (8 columns) each;
   // lanes 32..63 repeat them (their copy lands in the unused half of the slot)
   uint32_t ws_col = n0 + 8 * (lane & 31);
   ws_col = ws_col + 8 <= p.N ? ws_col : p.N - 8;
-  const uint32_t ws_voff = (ws_col - n0) * 2;
-  const char* ws_base = reinterpret_cast<const char*>(p.sc) + (static_cast<size_t>(kb_begin) * p.N + n0) * 2;
+  const uint32_t ws_voff = (ws_col - n0) * 2 + ((GH == 2 && lane >= 32) ? p.N * 2 : 0);  // lanes 32..63: the second row
+  const char* ws_base = reinterpret_cast<const char*>(p.sc) + (static_cast<size_t>(kb_begin) * GH * p.N + n0) * 2;
   const uint32_t ws_lds = lds_base + WS_BASE;
   const uint32_t n_wave = n0 + wn * 64;
 
@@ -149,7 +162,7 @@ __global__ void __launch_bounds__(512, 1) w4a8_tile_kernel(W4A8TileParams p) {
   auto load_scales = [&](uint32_t kb) {
     const uint32_t k = kb < kb_count ? kb : kb_count - 1;
     if (has_xs_load) {
-      const char* ap = xs_base + static_cast<size_t>(k) * p.M * 4;
+      const char* ap = xs_base + static_cast<size_t>(k) * GH * p.M * 4;
       const uint32_t d = __builtin_amdgcn_readfirstlane(s_lds + (kb % NS) * 1024);
       if (s_vec)
         asm volatile("s_nop 4\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %2" ::"v"(s_voff), "s"(d), "s"(ap)
@@ -159,7 +172,7 @@ __global__ void __launch_bounds__(512, 1) w4a8_tile_kernel(W4A8TileParams p) {
                      : "memory");
     }
     if (wave == 4) {
-      const char* wp = ws_base + static_cast<size_t>(k) * p.N * 2;
+      const char* wp = ws_base + static_cast<size_t>(k) * GH * p.N * 2;
       const uint32_t d = __builtin_amdgcn_readfirstlane(ws_lds + (kb % NS) * 1024);
       asm volatile("s_nop 4\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %2" ::"v"(ws_voff), "s"(d), "s"(wp)
                    : "memory");
@@ -250,6 +263,56 @@ __global__ void __launch_bounds__(512, 1) w4a8_tile_kernel(W4A8TileParams p) {
   // one k-block: WM*WN MFMAs; the scale FMAs of MFMA j are placed after MFMA j+2 so that they run in its shadow, and
   // the loads of k-block `next` are issued after the first MFMA.
   auto compute = [&](uint32_t slot, uint32_t next) {
+    if constexpr (GH == 2) {
+      // group 64: sums of half h at [h][BM] floats, scales of half h at [h][256] fp16 of the stage's slots
+      float cs[2][WM];
+      float sc[2][WN][4];
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+#pragma unroll
+        for (int i = 0; i < WM; ++i) cs[h][i] = xs_lds[slot * 256 + h * BM + i * 16] * -0.015625f;
+#pragma unroll
+        for (int t = 0; t < WN; ++t) {
+          const u32x2 v = *reinterpret_cast<const u32x2*>(wsc_lds + slot * 1024 + h * 512 + t * 32);
+          sc[h][t][0] = F16::lo_to_float(v.x);
+          sc[h][t][1] = F16::hi_to_float(v.x);
+          sc[h][t][2] = F16::lo_to_float(v.y);
+          sc[h][t][3] = F16::hi_to_float(v.y);
+        }
+      }
+      const char* act = lds + slot * STAGE_BYTES + (wm * WM) * FRAG;
+      const char* wgt = lds + slot * STAGE_BYTES + W_BASE + (wn * WN) * WFRAG + 16 * lane;
+      i32x8 wf[2][WN];
+      const int keep_lo = lane < 32 ? -1 : 0;
+#pragma unroll
+      for (int t = 0; t < WN; ++t) {
+        const i32x8 w = w4a8_expand(*reinterpret_cast<const i32x4*>(wgt + t * WFRAG));
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          wf[0][t][e] = w[e] & keep_lo;
+          wf[1][t][e] = w[e] & ~keep_lo;
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < WM; ++i) {
+        const i32x8 af = read_frag(act + i * FRAG);
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const f32x4 cv{cs[h][i], cs[h][i], cs[h][i], cs[h][i]};
+#pragma unroll
+          for (int t = 0; t < WN; ++t) {
+            const f32x4 r = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[h][t], af, cv, 0, 0, 0, 0, 0, 0);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[t][i][e] = __builtin_fmaf(r[e], sc[h][t][e], acc[t][i][e]);
+          }
+        }
+        if (i == 0) {
+          load_scales(next);
+          load_operands(next);
+        }
+      }
+      return;
+    }
     float cs[WM];
 #pragma unroll
     for (int i = 0; i < WM; ++i) cs[i] = xs_lds[slot * 256 + i * 16] * -0.015625f;  // -8 * 2^-9 * xsum

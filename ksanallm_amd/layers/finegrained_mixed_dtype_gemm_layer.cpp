@@ -9,9 +9,9 @@ Status FinegrainedMixedDtypeGemmLayer::Init(const std::vector<std::any>& paramet
   STATUS_CHECK_FAILURE(BaseLayer::Init(parameters, runtime_config, context, rank));
   if (parameters.empty()) return Status(RET_INVALID_ARGUMENT, "FinegrainedMixedDtypeGemmLayer: expects its parameter struct");
   params_ = std::any_cast<const FinegrainedMixedDtypeGemmLayerParameters>(parameters.front());
-  if (params_.group_size != 128) {
+  if (params_.group_size != 128 && params_.group_size != 64) {
     return Status(RET_INVALID_ARGUMENT, "FinegrainedMixedDtypeGemmLayer: group size " + std::to_string(params_.group_size) +
-                                            " has no kernel (128 only)");
+                                            " has no kernel (128 or 64)");
   }
   if (params_.has_zero) return Status(RET_INVALID_ARGUMENT, "FinegrainedMixedDtypeGemmLayer: zero points have no kernel");
   if (params_.activation_type != TYPE_FP8_E4M3) {
@@ -29,7 +29,7 @@ Status FinegrainedMixedDtypeGemmLayer::Init(const std::vector<std::any>& paramet
 size_t FinegrainedMixedDtypeGemmLayer::GetWorkspaceSize() {
   kernel_workspace_size_ = AlignTo256(ksq_w4a8_workspace_size(params_.m, params_.n, params_.k));
   quantized_size_ = AlignTo256(params_.m * params_.k * sizeof(char));
-  sums_size_ = AlignTo256(params_.m * (params_.k / 128) * sizeof(float));
+  sums_size_ = AlignTo256(params_.m * (params_.k / params_.group_size) * sizeof(float));
   return kernel_workspace_size_ + quantized_size_ + sums_size_;
 }
 
@@ -67,13 +67,14 @@ Status FinegrainedMixedDtypeGemmLayer::Forward(const std::vector<Tensor>& input_
   char* kernel_workspace = workspace_buffer_->GetPtr<char>();
   char* quantized_input = kernel_workspace + kernel_workspace_size_;
   char* group_sums = quantized_input + quantized_size_;
+  const int sums = params_.group_size == 64 ? KSQ_W4A8_SUMS_PER_64 : 0;  // one activation sum per scale group
   if (weight.pre_quant_scales) {
     KsqCheck(ksq_w4a8_static_quant(input_tensors[0].GetPtr<void>(), weight.pre_quant_scales->GetPtr<void>(), quantized_input,
-                                   group_sums, m, k, KSQ_W4A8_PER_CHANNEL, dtype, stream),
+                                   group_sums, m, k, KSQ_W4A8_PER_CHANNEL | sums, dtype, stream),
              "FinegrainedMixedDtypeGemmLayer");
   } else {
     KsqCheck(ksq_w4a8_static_quant(input_tensors[0].GetPtr<void>(), weight.input_scales->GetPtr<void>(), quantized_input,
-                                   group_sums, m, k, KSQ_W4A8_PER_TENSOR, dtype, stream),
+                                   group_sums, m, k, KSQ_W4A8_PER_TENSOR | sums, dtype, stream),
              "FinegrainedMixedDtypeGemmLayer");
   }
   KsqCheck(ksq_w4a8_gemm(quantized_input, group_sums, weight.GetPtr<void>(), weight.weight_scales->GetPtr<void>(),

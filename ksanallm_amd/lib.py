@@ -11,6 +11,7 @@ SCALE_GN, SCALE_NG = 0, 1
 ZERO_AWQ_PACKED, ZERO_U8_GN = 0, 1
 KIND_W4A16, KIND_FP8_BLOCKWISE, KIND_MOE_W4A16, KIND_W4A8 = 0, 1, 2, 3
 W4A8_PER_TENSOR, W4A8_PER_CHANNEL, W4A8_SUMS_ONLY, W4A8_PER_TOKEN = 0, 1, 2, 3
+W4A8_SUMS_PER_64 = 16
 
 c_sz = ctypes.c_size_t
 c_p = ctypes.c_void_p

@@ -390,27 +390,30 @@ def w4a8_unpack_weight(packed, K, N):
     return out
 
 
-def w4a8_static_quant(x, scale, per_channel=False, per_token=False):
+def w4a8_static_quant(x, scale, per_channel=False, per_token=False, group=128):
     """StaticQuantizeE4M3PerTensor / PerChannel / PerToken: x [m,k] T, scale fp32 [1], [k] or [m] -> (codes uint8
-    [m,k], group sums fp32 [k/128, m])."""
+    [m,k], group sums fp32 [k/group, m]); group 128 or 64."""
     m, k = x.shape
     q = torch.empty((m, k), dtype=torch.uint8, device=x.device)
-    xsum = torch.empty((k // 128, m), dtype=torch.float32, device=x.device)
+    xsum = torch.empty((k // group, m), dtype=torch.float32, device=x.device)
     mode = _l.W4A8_PER_CHANNEL if per_channel else (_l.W4A8_PER_TOKEN if per_token else _l.W4A8_PER_TENSOR)
+    if group == 64:
+        mode |= _l.W4A8_SUMS_PER_64
     _l.check(_lib.ksq_w4a8_static_quant(_ptr(x), _ptr(scale), _ptr(q), _ptr(xsum), m, k, mode, _dt(x), _stream()))
     return q, xsum
 
 
-def w4a8_group_sums(a_q):
-    """Group sums of activations that are e4m3 already (uint8 [m,k]) -> fp32 [k/128, m]."""
+def w4a8_group_sums(a_q, group=128):
+    """Group sums of activations that are e4m3 already (uint8 [m,k]) -> fp32 [k/group, m]; group 128 or 64."""
     m, k = a_q.shape
-    xsum = torch.empty((k // 128, m), dtype=torch.float32, device=a_q.device)
-    _l.check(_lib.ksq_w4a8_static_quant(_ptr(a_q), None, None, _ptr(xsum), m, k, _l.W4A8_SUMS_ONLY, F16, _stream()))
+    xsum = torch.empty((k // group, m), dtype=torch.float32, device=a_q.device)
+    mode = _l.W4A8_SUMS_ONLY | (_l.W4A8_SUMS_PER_64 if group == 64 else 0)
+    _l.check(_lib.ksq_w4a8_static_quant(_ptr(a_q), None, None, _ptr(xsum), m, k, mode, F16, _stream()))
     return xsum
 
 
-def w4a8_gemm(a_q, xsum, w_packed, scales, alpha, n, out_dtype=torch.bfloat16, out=None, workspace=None):
-    """FinegrainedMixedDtypeGemmWrapper::Forward: a_q [m,k] e4m3 bytes, scales fp16 [k/128, n]."""
+def w4a8_gemm(a_q, xsum, w_packed, scales, alpha, n, out_dtype=torch.bfloat16, out=None, workspace=None, group=128):
+    """FinegrainedMixedDtypeGemmWrapper::Forward: a_q [m,k] e4m3 bytes, xsum [k/group, m], scales fp16 [k/group, n]."""
     m, k = a_q.shape
     if out is None:
         out = torch.empty((m, n), dtype=out_dtype, device=a_q.device)
@@ -419,5 +422,5 @@ def w4a8_gemm(a_q, xsum, w_packed, scales, alpha, n, out_dtype=torch.bfloat16, o
         workspace = torch.empty(max(need, 1), dtype=torch.uint8, device=a_q.device)
     assert scales.dtype == torch.float16
     _l.check(_lib.ksq_w4a8_gemm(_ptr(a_q), _ptr(xsum), _ptr(w_packed), _ptr(scales), float(alpha), _ptr(out), m, n, k,
-                                128, _dt(out), _ptr(workspace), workspace.numel(), _stream()))
+                                group, _dt(out), _ptr(workspace), workspace.numel(), _stream()))
     return out

@@ -812,13 +812,16 @@ KSQO_API void ksqo_w4a8_static_quant(const void* x, const float* scale, uint8_t*
 }
 
 /* xsum[m, g] = sum of the 128 decoded e4m3 values of group g (in double, rounded once). */
-KSQO_API void ksqo_w4a8_group_sums(const uint8_t* q, float* xsum, size_t m, size_t k) {
+KSQO_API void ksqo_w4a8_group_sums_g(const uint8_t* q, float* xsum, size_t m, size_t k, size_t group) {
   for (size_t i = 0; i < m; ++i)
-    for (size_t g = 0; g < k / 128; ++g) {
+    for (size_t g = 0; g < k / group; ++g) {
       double acc = 0.0;
-      for (size_t j = 0; j < 128; ++j) acc += (double)ksqo_e4m3_to_f32(q[i * k + g * 128 + j]);
-      xsum[i * (k / 128) + g] = (float)acc;
+      for (size_t j = 0; j < group; ++j) acc += (double)ksqo_e4m3_to_f32(q[i * k + g * group + j]);
+      xsum[i * (k / group) + g] = (float)acc;
     }
+}
+KSQO_API void ksqo_w4a8_group_sums(const uint8_t* q, float* xsum, size_t m, size_t k) {
+  ksqo_w4a8_group_sums_g(q, xsum, m, k, 128);
 }
 
 /* out[m,n] = alpha * sum_k a[m,k] * (w[k,n] * scale[k/group, n]): the reference test's formula

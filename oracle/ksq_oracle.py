@@ -483,11 +483,11 @@ def w4a8_static_quant(x_bits, scale, per_channel, dtype, per_token=False):
     return q
 
 
-def w4a8_group_sums(q):
+def w4a8_group_sums(q, group=128):
     q = _c(q, np.uint8)
     m, k = q.shape
-    out = np.empty((m, k // 128), np.float32)
-    lib().ksqo_w4a8_group_sums(_p(q), _p(out), _sz(m), _sz(k))
+    out = np.empty((m, k // group), np.float32)
+    lib().ksqo_w4a8_group_sums_g(_p(q), _p(out), _sz(m), _sz(k), _sz(group))
     return out
 
 

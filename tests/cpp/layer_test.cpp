@@ -218,7 +218,8 @@ static int RunFp8Tensor(int argc, char** argv) {
   return 0;
 }
 
-// w4a8 <dir> <f16|bf16> <m> <n> <k> <per_channel> <alpha>
+// w4a8 <dir> <f16|bf16> <m> <n> <k> <per_channel> <alpha> [group]
+// (group 64 is built from the parameter struct: the factory's weight-name path, like the reference's, knows 128 only)
 static int RunW4A8(int argc, char** argv) {
   if (argc < 9) return 2;
   const std::string dir = argv[2];
@@ -226,6 +227,7 @@ static int RunW4A8(int argc, char** argv) {
   const size_t m = std::atol(argv[4]), n = std::atol(argv[5]), k = std::atol(argv[6]);
   const bool per_channel = std::atoi(argv[7]) != 0;
   const float alpha = static_cast<float>(std::atof(argv[8]));
+  const size_t group = argc > 9 ? std::atol(argv[9]) : 128;
   hipStream_t stream;
   HIP_OK(hipStreamCreate(&stream));
   auto context = std::make_shared<Context>(1, stream);
@@ -234,7 +236,7 @@ static int RunW4A8(int argc, char** argv) {
   rc.inter_data_type = T;
   rc.max_step_token_num = m;
   Tensor loaded = Upload(dir + "/w.bin", TYPE_INT8, {k, n / 2});
-  loaded.weight_scales = std::make_shared<Tensor>(Upload(dir + "/w_scale.bin", TYPE_FP16, {k / 128, n}));
+  loaded.weight_scales = std::make_shared<Tensor>(Upload(dir + "/w_scale.bin", TYPE_FP16, {k / group, n}));
   loaded.input_scales = std::make_shared<Tensor>(Upload(dir + "/in_scale.bin", TYPE_FP32, {1}));
   if (per_channel) loaded.pre_quant_scales = std::make_shared<Tensor>(Upload(dir + "/pqs.bin", TYPE_FP32, {k}));
   loaded.alpha = alpha;
@@ -248,7 +250,20 @@ static int RunW4A8(int argc, char** argv) {
   auto weights = std::make_shared<TestWeights>();
   weights->weights[name] = weight;
   MatMulLayerFactory factory(mc, rc, 0, context);
-  auto layer = factory.AutoCreateLayer(weights, name, TYPE_I4_GROUP, T, T, CUTLASS_LINEAR_BACKEND, {});
+  std::shared_ptr<BaseLayer> layer;
+  if (group == 128) {
+    layer = factory.AutoCreateLayer(weights, name, TYPE_I4_GROUP, T, T, CUTLASS_LINEAR_BACKEND, {});
+  } else {
+    FinegrainedMixedDtypeGemmLayerParameters param;
+    param.m = m;
+    param.n = n;
+    param.k = k;
+    param.group_size = group;
+    param.has_zero = false;
+    param.activation_type = TYPE_FP8_E4M3;
+    param.output_type = T;
+    layer = factory.CreateLayer(TYPE_I4_GROUP, T, T, {param}, QUANT_W4A8_AWQ, CUTLASS_LINEAR_BACKEND);
+  }
   Tensor x = Upload(dir + "/x.bin", T, {m, k});
   std::vector<Tensor> outputs{Tensor(MemoryLocation::LOCATION_DEVICE, T, {m, n}, 0)};
   Drive(layer, mc, rc, {x, weight}, outputs);
@@ -535,7 +550,14 @@ static int RunErrors() {
       FinegrainedMixedDtypeGemmLayer l;
       expect(!l.Init({p}, rc, context, 0).OK(), what);
     };
-    bad([](auto& p) { p.group_size = 64; }, "w4a8 rejects group size 64");
+    bad([](auto& p) { p.group_size = 32; }, "w4a8 rejects group size 32");
+    {
+      FinegrainedMixedDtypeGemmLayerParameters p64 = good;
+      p64.group_size = 64;
+      FinegrainedMixedDtypeGemmLayer l64;
+      expect(l64.Init({p64}, rc, context, 0).OK(), "w4a8 init with group size 64");
+      expect(l64.GetWorkspaceSize() >= 64 * 512 + 64 * 8 * 4, "w4a8 workspace with group size 64 holds twice the group sums");
+    }
     bad([](auto& p) { p.has_zero = true; }, "w4a8 rejects zero points");
     bad([](auto& p) { p.activation_type = TYPE_FP16; }, "w4a8 rejects a 16-bit activation type");
     bad([](auto& p) { p.k = 200; }, "w4a8 rejects k = 200");

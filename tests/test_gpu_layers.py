@@ -294,3 +294,24 @@ def test_w4a8_layer(tmp_path, oracle, dtype, m, n, k, per_channel):
     xq = oracle.w4a8_static_quant(H.bits_of(x), pqs if per_channel else in_scale, bool(per_channel), dtype)
     ref = oracle.w4a8_gemm(xq, w.view(np.int8), H.bits_of(ws), alpha)
     H.check_gemm(y, ref, dtype, "w4a8 layer")
+
+
+@pytest.mark.parametrize("m", [5, 200])
+def test_w4a8_layer_group_64(tmp_path, oracle, m):
+    """The layer with scale groups of 64 (the parameter struct's other group size)."""
+    n, k, dtype = 512, 1024, H.BF16
+    g = H.gen(9750 + m)
+    w = torch.randint(0, 256, (k, n // 2), generator=g, dtype=torch.uint8).numpy()
+    ws = (torch.rand((k // 64, n), generator=g) * 0.02 + 0.002).to(torch.float16)
+    x = torch.randn((m, k), generator=g).to(H.TORCH_DT[dtype])
+    in_scale = np.array([0.03], np.float32)
+    alpha = float(np.float32(0.03 * 0.8))
+    w.tofile(tmp_path / "w.bin")
+    H.bits_of(ws).tofile(tmp_path / "w_scale.bin")
+    in_scale.tofile(tmp_path / "in_scale.bin")
+    H.bits_of(x).tofile(tmp_path / "x.bin")
+    run_driver("w4a8", tmp_path, TNAME[dtype], m, n, k, 0, repr(alpha), 64)
+    y = read_out(tmp_path / "y.bin", dtype, (m, n))
+    xq = oracle.w4a8_static_quant(H.bits_of(x), in_scale, False, dtype)
+    ref = oracle.w4a8_gemm(xq, w.view(np.int8), H.bits_of(ws), alpha, group=64)
+    H.check_gemm(y, ref, dtype, "w4a8 layer, group 64")

@@ -231,13 +231,39 @@ def test_gemm_meets_the_reference_tests_own_tolerance(ops, oracle):
     assert float((out.float() - ref).abs().max()) <= atol
 
 
+@pytest.mark.parametrize("m,n,k", [(1, 2048, 1024), (16, 48, 640), (17, 8192, 512), (32, 16, 128),     # streaming kernel
+                                   (33, 48, 128), (130, 2064, 1024), (257, 512, 640), (300, 1024, 1024),  # 128-token tiles
+                                   (1024, 2304, 384)])
+@pytest.mark.parametrize("out_dtype", [H.F16, H.BF16])
+def test_gemm_group_64(ops, oracle, out_dtype, m, n, k):
+    """Scale groups of 64: sums per 64 channels bit-exact, the GEMM (both kernels) against the oracle; and with scales
+    equal in both halves of every 128 channels the result has the bits of the group-128 launch."""
+    g = H.gen(m + n + k)
+    w = torch.randint(0, 256, (k, n // 2), generator=g, dtype=torch.uint8)
+    s64 = (torch.rand((k // 64, n), generator=g) * 0.02 + 0.002).to(torch.float16)
+    x = make_act(m * 7 + k, m, k, H.BF16)
+    in_scale = torch.tensor([0.05], dtype=torch.float32)
+    xq, xsum = ops.w4a8_static_quant(x.cuda(), in_scale.cuda(), False, group=64)
+    np.testing.assert_array_equal(xsum.cpu().numpy().T, oracle.w4a8_group_sums(xq.cpu().numpy(), 64))
+    np.testing.assert_array_equal(ops.w4a8_group_sums(xq, 64).cpu().numpy(), xsum.cpu().numpy())
+    wp = ops.w4a8_repack_weight(w.cuda())
+    out = ops.w4a8_gemm(xq, xsum, wp, s64.cuda(), 0.03, n, H.TORCH_DT[out_dtype], group=64)
+    ref = oracle.w4a8_gemm(xq.cpu().numpy(), w.numpy().view(np.int8), H.bits_of(s64), 0.03, group=64)
+    H.check_gemm(out, ref, out_dtype, "w4a8 g64 m=%d n=%d k=%d" % (m, n, k))
+    s128 = s64[0::2].contiguous()
+    same = s128.repeat_interleave(2, 0).contiguous()
+    a = ops.w4a8_gemm(xq, xsum, wp, same.cuda(), 0.03, n, H.TORCH_DT[out_dtype], group=64)
+    b = ops.w4a8_gemm(xq, ops.w4a8_group_sums(xq), wp, s128.cuda(), 0.03, n, H.TORCH_DT[out_dtype])
+    H.check_gemm(a, b.float().cpu().numpy(), out_dtype, "w4a8 g64 against g128")
+
+
 def test_gemm_rejects_what_it_does_not_do(ops):
     from ksanallm_amd import lib as L
     lib = L.load()
     z = torch.zeros(4096, dtype=torch.uint8, device="cuda")
     p = z.data_ptr()
-    # group 64
-    assert lib.ksq_w4a8_gemm(p, p, p, p, 1.0, p, 1, 16, 128, 64, L.BF16, None, 0, None) == 2
+    # group 32
+    assert lib.ksq_w4a8_gemm(p, p, p, p, 1.0, p, 1, 16, 128, 32, L.BF16, None, 0, None) == 2
     # n not a multiple of 16, k not of 128
     assert lib.ksq_w4a8_gemm(p, p, p, p, 1.0, p, 1, 24, 128, 128, L.BF16, None, 0, None) == 1
     assert lib.ksq_w4a8_gemm(p, p, p, p, 1.0, p, 1, 16, 100, 128, L.BF16, None, 0, None) == 1

@@ -62,6 +62,29 @@ def test_group_sums_against_numpy(oracle):
     assert np.all(ref == got.astype(np.float64))
 
 
+def test_group_sums_and_gemm_with_group_64(oracle):
+    """Group size 64: sums against numpy float64, and the GEMM against the reference test's formula with the scales
+    repeated 64 times; scales that are equal in both halves of every 128 give the group-128 result."""
+    rng = np.random.default_rng(14)
+    m, n, k = 6, 32, 384
+    a = rng.integers(0, 256, (m, k), dtype=np.uint8)
+    a[(a & 0x7F) == 0x7F] = 0x28
+    got = oracle.w4a8_group_sums(a, 64)
+    ref = oracle.e4m3_to_f32(a).astype(np.float64).reshape(m, k // 64, 64).sum(-1)
+    np.testing.assert_array_equal(got, ref.astype(np.float32))
+    w = rng.integers(0, 256, (k, n // 2), dtype=np.uint8).view(np.int8)
+    s64 = (rng.random((k // 64, n)) * 0.02 + 0.001).astype(np.float16)
+    out = oracle.w4a8_gemm(a, w, s64.view(np.uint16), 0.5, group=64)
+    wt = torch.from_numpy(oracle.w4a8_unpack_int4(w)).double()
+    sc = torch.from_numpy(s64.astype(np.float64)).repeat_interleave(64, 0)
+    act = torch.from_numpy(a).view(torch.float8_e4m3fn).double() * 0.5
+    np.testing.assert_allclose(out, (act @ (wt * sc)).numpy(), rtol=2e-7, atol=1e-12)
+    s128 = s64[0::2].copy()
+    same = np.repeat(s128, 2, axis=0)
+    np.testing.assert_array_equal(oracle.w4a8_gemm(a, w, same.view(np.uint16), 0.5, group=64),
+                                  oracle.w4a8_gemm(a, w, s128.view(np.uint16), 0.5, group=128))
+
+
 def test_gemm_is_the_reference_tests_formula(oracle):
     """finegrained_mixed_dtype_gemm_thop_test.cu:186-206 in torch float64: unpack, times the repeated scales, matmul
     with the alpha-scaled activations."""
