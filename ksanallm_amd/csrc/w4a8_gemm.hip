@@ -1,4 +1,4 @@
-// W4A8 (int4 weights, group-128 fp16 scales, statically quantized e4m3 activations) GEMM:
+// W4A8 (int4 weights, fp16 scales per group of 128 or 64, statically quantized e4m3 activations) GEMM:
 //   out[m,n] = alpha * sum_g scale[g,n] * sum_{k in g} a_q[m,k] * w[k,n],      w in -8..7
 //
 // The fp8 matrix instruction does the products.  An int4 code needs no table to become an e4m3 byte: the byte 0x0u
@@ -6,8 +6,9 @@
 // field 1 continues it with (8 + m) * 2^-9), so a packed dword expands into two operand dwords with one shift and two
 // ANDs.  The offset goes into the instruction's addend: with xsum[m,g] = sum_{k in g} a_q[m,k],
 //   sum_k a_q * (u - 8) * 2^-9 = mfma(u_bytes, a_q, C = -xsum / 64).
-// One v_mfma_f32_16x16x128_f8f6f4 spans exactly one scale group; its four results per lane are four consecutive
-// output columns of one token and take their four scales in fp32.  The factor 2^9 is folded into alpha.
+// One v_mfma_f32_16x16x128_f8f6f4 spans exactly one scale group of 128 (two of 64: then it is issued once per half,
+// the other half's operand bytes cleared); its four results per lane are four consecutive output columns of one token
+// and take their four scales in fp32.  The factor 2^9 is folded into alpha.
 //
 // Packed weight layout: a fragment of 16 weight columns x 128 k is 1 KiB, 16 bytes per lane in lane order; lane l
 // (column l % 16, quarter q = l / 16) holds dwords P0..P3, nibble 2j of Pi = u(k = 32q + 8i + j), nibble 2j+1 of
