@@ -296,6 +296,7 @@ def test_w4a8_layer(tmp_path, oracle, dtype, m, n, k, per_channel):
     H.check_gemm(y, ref, dtype, "w4a8 layer")
 
 
+@pytest.mark.gpu
 @pytest.mark.parametrize("m", [5, 200])
 def test_w4a8_layer_group_64(tmp_path, oracle, m):
     """The layer with scale groups of 64 (the parameter struct's other group size)."""
