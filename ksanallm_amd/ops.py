@@ -37,8 +37,17 @@ def _ptr(t):
 
 
 # ----------------------------------------------------------------------------------------------- load-time repack
+def _need_bytes(t, nbytes, what):
+    """The C-ABI takes bare pointers: a tensor that is smaller than the layout it is declared to hold would be read
+    past its end on the device, so the wrappers check the size here."""
+    have = t.numel() * t.element_size()
+    if have < nbytes:
+        raise ValueError("%s: tensor holds %d bytes, the declared layout needs %d" % (what, have, nbytes))
+
+
 def repack_weight(src, layout, E, K, N):
     """Checkpoint int4 weight -> CDNA4 tile layout (uint8 tensor of E*K*N/2 bytes)."""
+    _need_bytes(src, E * K * N // 2, "repack_weight")
     dst = torch.empty(_lib.ksq_w4a16_packed_weight_bytes(E, K, N), dtype=torch.uint8, device=src.device)
     _l.check(_lib.ksq_w4a16_repack(_ptr(src), layout, _ptr(dst), E, K, N, _stream()))
     return dst
@@ -59,6 +68,7 @@ def unpack_weight(packed, layout, E, K, N):
 
 
 def repack_scales(src, layout, E, K, N, group):
+    _need_bytes(src, E * (K // group) * N * src.element_size(), "repack_scales")
     dst = torch.empty(E * (K // group) * N, dtype=src.dtype, device=src.device)
     _l.check(_lib.ksq_w4a16_repack_scales(_ptr(src), layout, _ptr(dst), E, K, N, group, _dt(src), _stream()))
     return dst
@@ -73,6 +83,7 @@ def unpack_scales(packed, layout, E, K, N, group):
 
 
 def repack_zeros(src, layout, K, N, group):
+    _need_bytes(src, (K // group) * N // (2 if layout == _l.ZERO_AWQ_PACKED else 1), "repack_zeros")
     dst = torch.empty((K // group) * N, dtype=torch.uint8, device=src.device)
     _l.check(_lib.ksq_w4a16_repack_zeros(_ptr(src), layout, _ptr(dst), K, N, group, _stream()))
     return dst
@@ -111,6 +122,11 @@ def _w4a16_workspace(device, m, n, k, group, dt):
 def w4a16_gemm(x, w_packed, scales_packed, zeros_packed, n, k, group, out=None, workspace=None):
     """InvokeFpAIntBGroupCudaGemm / InvokeFpAIntBGroupCutlassGemm / InvokeMarlinGemm / InvokeMacheteGemm."""
     m = x.shape[0]
+    _need_bytes(x, m * k * 2, "w4a16_gemm: x")
+    _need_bytes(w_packed, k * n // 2, "w4a16_gemm: packed weight")
+    _need_bytes(scales_packed, (k // group) * n * 2, "w4a16_gemm: scales")
+    if zeros_packed is not None:
+        _need_bytes(zeros_packed, (k // group) * n, "w4a16_gemm: zero points")
     if out is None:
         out = torch.empty((m, n), dtype=x.dtype, device=x.device)
     if workspace is None:
@@ -172,6 +188,9 @@ def moe_align_block_size(topk_ids, num_experts, block_m):
 def moe_w4a16_gemm(x, w_packed, scales_packed, topk_w, sorted_ids, expert_ids, num_post_pad, numel, top_k, E, n, k,
                    group, block_m, out=None):
     """InvokeMoeWna16Gemm / InvokeFusedMoeGptqAwqKernel: out [numel, n]."""
+    _need_bytes(x, ((numel + top_k - 1) // top_k) * k * 2, "moe_w4a16_gemm: x")
+    _need_bytes(w_packed, E * k * n // 2, "moe_w4a16_gemm: packed weight")
+    _need_bytes(scales_packed, E * (k // group) * n * 2, "moe_w4a16_gemm: scales")
     if out is None:
         out = torch.empty((numel, n), dtype=x.dtype, device=x.device)
     _l.check(_lib.ksq_moe_w4a16_gemm(_ptr(out), _ptr(x), _ptr(w_packed), _ptr(scales_packed), None, _ptr(topk_w),
@@ -182,8 +201,11 @@ def moe_w4a16_gemm(x, w_packed, scales_packed, topk_w, sorted_ids, expert_ids, n
 
 def moe_w4a16_gate_up_silu(x, w_packed, scales_packed, sorted_ids, expert_ids, num_post_pad, numel, top_k, E, n, k, group,
                            block_m, out=None):
-    """The first MoE GEMM with silu*mul in its epilogue (block_m 16 or 32): out [numel, n/2], bit for bit what
+    """The first MoE GEMM with silu*mul in its epilogue (any block size of moe_w4a16_gemm): out [numel, n/2], bit for bit what
     moe_w4a16_gemm followed by silu_and_mul gives."""
+    _need_bytes(x, ((numel + top_k - 1) // top_k) * k * 2, "moe_w4a16_gate_up_silu: x")
+    _need_bytes(w_packed, E * k * n // 2, "moe_w4a16_gate_up_silu: packed weight")
+    _need_bytes(scales_packed, E * (k // group) * n * 2, "moe_w4a16_gate_up_silu: scales")
     if out is None:
         out = torch.empty((numel, n // 2), dtype=x.dtype, device=x.device)
     _l.check(_lib.ksq_moe_w4a16_gate_up_silu(_ptr(out), _ptr(x), _ptr(w_packed), _ptr(scales_packed), None,
