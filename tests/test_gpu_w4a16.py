@@ -182,9 +182,12 @@ def test_bad_arguments(ops):
     with pytest.raises(L.KsqError) as e:
         ops.w4a16_gemm(x, w, w, None, 16, 100, 128)
     assert e.value.code == 1 and "k % 128" in str(e.value)
+    x128 = torch.zeros((1, 128), dtype=torch.float16, device="cuda")
     with pytest.raises(L.KsqError) as e:
-        ops.w4a16_gemm(x, w, w, None, 16, 128, 100)
+        ops.w4a16_gemm(x128, w, w, None, 16, 128, 100)
     assert e.value.code == 2
+    with pytest.raises(ValueError):  # the wrapper itself refuses a tensor smaller than the layout it is declared to hold
+        ops.w4a16_gemm(x, w, w, None, 16, 128, 128)
 
 
 # GPTQ act-order (desc_act): rows sorted by g_idx at repack time, activations permuted in front of the GEMM
