@@ -155,6 +155,9 @@ def fp8_blockwise_gemm(a_q, a_s, b, b_s, out_dtype=torch.bfloat16, out=None, wor
     fp8_repack_weight, b_s [n/128,k/128]."""
     m, k = a_q.shape
     n = b.shape[0]
+    _need_bytes(a_s, (k // 128) * m * 4, "fp8_blockwise_gemm: activation scales")
+    _need_bytes(b, n * k, "fp8_blockwise_gemm: weight")
+    _need_bytes(b_s, ((n + 127) // 128) * (k // 128) * 4, "fp8_blockwise_gemm: weight scales")
     if out is None:
         out = torch.empty((m, n), dtype=out_dtype, device=a_q.device)
     if workspace is None:
@@ -437,6 +440,9 @@ def w4a8_group_sums(a_q, group=128):
 def w4a8_gemm(a_q, xsum, w_packed, scales, alpha, n, out_dtype=torch.bfloat16, out=None, workspace=None, group=128):
     """FinegrainedMixedDtypeGemmWrapper::Forward: a_q [m,k] e4m3 bytes, xsum [k/group, m], scales fp16 [k/group, n]."""
     m, k = a_q.shape
+    _need_bytes(xsum, (k // group) * m * 4, "w4a8_gemm: group sums")
+    _need_bytes(w_packed, n * k // 2, "w4a8_gemm: packed weight")
+    _need_bytes(scales, (k // group) * n * 2, "w4a8_gemm: scales")
     if out is None:
         out = torch.empty((m, n), dtype=out_dtype, device=a_q.device)
     if workspace is None:
