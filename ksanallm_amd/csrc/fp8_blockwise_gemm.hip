@@ -155,6 +155,20 @@ __global__ void __launch_bounds__(WAVES * 64) fp8_splitk_kernel(Fp8Params p) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) red[wave][nt][mt][lane] = acc[nt][mt];
   __syncthreads();
+  // Grouped form: the slot ids and routing weights of this lane's rows, fetched before the first store.  Read next to
+  // each store they would wait for the stores in front of them (the compiler cannot know that the output does not
+  // overlap the index arrays), one memory round trip after the other.
+  static_assert(MT <= 2, "the epilogue selects between two row tiles");
+  uint32_t esid0 = 0, esid1 = 0;
+  float erw0 = 1.0f, erw1 = 1.0f;
+  if (GROUPED) {
+    esid0 = static_cast<uint32_t>(p.sorted_ids[m0 + (lane & 15)]);
+    if (MT > 1) esid1 = static_cast<uint32_t>(p.sorted_ids[m0 + 16 + (lane & 15)]);
+    if (p.topk_w) {
+      if (esid0 < p.numel) erw0 = p.topk_w[esid0];
+      if (MT > 1 && esid1 < p.numel) erw1 = p.topk_w[esid1];
+    }
+  }
   for (int idx = threadIdx.x; idx < NT * MT * 64; idx += WAVES * 64) {
     const int l = idx & 63, mt = (idx >> 6) % MT, nt = (idx >> 6) / MT;
     f32x4 v = red[0][nt][mt][l];
@@ -163,10 +177,10 @@ __global__ void __launch_bounds__(WAVES * 64) fp8_splitk_kernel(Fp8Params p) {
     uint32_t row = m0 + mt * 16 + (l & 15);
     bool live = row < p.M;
     if (GROUPED) {
-      const uint32_t sid = static_cast<uint32_t>(p.sorted_ids[row]);
+      const uint32_t sid = mt ? esid1 : esid0;
       live = sid < p.numel;
       row = sid;
-      if (live && p.topk_w) v *= p.topk_w[sid];
+      v *= mt ? erw1 : erw0;
     }
     if (live) {
       u32x2 o;

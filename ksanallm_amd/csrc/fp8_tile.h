@@ -351,16 +351,26 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // drain the clamped prefetches before the LDS is released
 
   // ---- store: lane holds token m = l%16 of the tile and weight rows (output columns) 4*(l/16) .. +3
+  // Grouped form: the slot ids and routing weights of this lane's rows, fetched before the first store.  Read next to
+  // each store they would wait for the stores in front of them (the compiler cannot know that the output does not
+  // overlap the index arrays), one memory round trip after the other.
+  uint32_t sids[WM];
+  float rws[WM];
+  if (GROUPED) {
+#pragma unroll
+    for (int i = 0; i < WM; ++i) sids[i] = static_cast<uint32_t>(p.sorted_ids[m0 + wm * (WM * 16) + i * 16 + lrow]);
+#pragma unroll
+    for (int i = 0; i < WM; ++i) rws[i] = (sids[i] < p.numel && p.topk_w) ? p.topk_w[sids[i]] : 1.0f;
+  }
 #pragma unroll
   for (int i = 0; i < WM; ++i) {
     uint32_t row = m0 + wm * (WM * 16) + i * 16 + lrow;
     bool live = row < p.M;
     float rw = 1.0f;
     if (GROUPED) {
-      const uint32_t sid = static_cast<uint32_t>(p.sorted_ids[row]);
-      live = sid < p.numel;
-      row = sid;
-      if (live && p.topk_w) rw = p.topk_w[sid];
+      live = sids[i] < p.numel;
+      row = sids[i];
+      rw = rws[i];
     }
     if (live) {
 #pragma unroll

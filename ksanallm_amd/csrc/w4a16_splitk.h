@@ -412,6 +412,25 @@ __global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKPar
     for (int mt = 0; mt < MT; ++mt) red[wave][t * MT + mt][lane] = acc[t][mt];
   __syncthreads();
 
+  // Grouped form: the slot ids (and routing weights) of the rows this thread stores, fetched before the first store.
+  // Read next to each store they would wait for the stores in front of them - the compiler cannot know that the output
+  // does not overlap the index arrays - one memory round trip after the other.
+  static_assert(MT <= 2, "the epilogue selects between two row tiles");
+  u32x4 esid[MT];
+  f32x4 erw[MT];
+  if (GROUPED) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        esid[mt][i] = static_cast<uint32_t>(p.sorted_ids[blockIdx.y * (16 * MT) + mt * 16 + 4 * lq + i]);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        erw[mt][i] = (!fused && esid[mt][i] < p.numel && p.topk_w) ? p.topk_w[esid[mt][i]] : 1.0f;
+  }
+
   if (GROUPED && NT > 1 && fused) {
     // gate_up with silu*mul: both sums are rounded to T as the unfused GEMM would store them, then
     // silu(g) * u in fp32 and one more rounding, the arithmetic of silu_mul_kernel
@@ -428,10 +447,10 @@ __global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKPar
         u += red[w][(t + HALF) * MT + mt][l];
       }
       const uint32_t col = (nt0 + t) * 16 + (l & 15);
+      const u32x4 msid = (MT > 1 && mt) ? esid[MT - 1] : esid[0];  // (a select: no register is indexed)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const uint32_t r = mt * 16 + 4 * (l >> 4) + i;
-        const uint32_t sid = static_cast<uint32_t>(p.sorted_ids[blockIdx.y * (16 * MT) + r]);
+        const uint32_t sid = msid[i];
         if (sid < p.numel) {
           const float gv = T::to_float(T::from_float(g[i])), uv = T::to_float(T::from_float(u[i]));
           const float y = silu_mul_f32(gv, uv);
@@ -451,6 +470,12 @@ __global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKPar
 #pragma unroll
     for (int w = 1; w < WAVES; ++w) v += red[w][tm][l];
     const uint32_t col = (nt0 + t) * 16 + (l & 15);
+    u32x4 msid = {};
+    f32x4 mrw = {};
+    if (GROUPED) {  // (selects: no register is indexed)
+      msid = (MT > 1 && mt) ? esid[MT - 1] : esid[0];
+      mrw = (MT > 1 && mt) ? erw[MT - 1] : erw[0];
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const uint32_t r = mt * 16 + 4 * (l >> 4) + i;
@@ -458,10 +483,10 @@ __global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKPar
       bool valid;
       float rw = 1.0f;
       if (GROUPED) {
-        uint32_t sid = static_cast<uint32_t>(p.sorted_ids[blockIdx.y * (16 * MT) + r]);
+        const uint32_t sid = msid[i];
         valid = sid < p.numel;
         orow = sid;
-        if (valid && p.topk_w) rw = p.topk_w[sid];
+        rw = mrw[i];
       } else {
         orow = blockIdx.y * (16 * MT) + r;
         valid = orow < p.M;
