@@ -472,6 +472,45 @@ def cpu_baseline(keeps, budget_s):
              "seconds": round(tot_t, 3), "per_config": per_config}, accuracy)
 
 
+def library_gemm(steps, warmup):
+    """Plain GEMMs of the vendor library at the prefill shapes (context for the roofline fractions, not a product path)."""
+    def timed(f):
+        for _ in range(warmup):
+            f()
+        beg, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        beg.record()
+        for _ in range(steps):
+            f()
+        end.record()
+        torch.cuda.synchronize()
+        return beg.elapsed_time(end) / steps * 1e3
+    rows = []
+    for dt, name in ((torch.float16, "fp16"), (torch.bfloat16, "bf16")):
+        for n, k in ((25600, 5120), (5120, 25600)):
+            for m in (2048, 4096, 8192):
+                x = torch.randn(m, k, device="cuda", dtype=dt) * 0.5
+                w = torch.randn(n, k, device="cuda", dtype=dt) * 0.01
+                us = timed(lambda: torch.matmul(x, w.t()))
+                tf = 2.0 * m * n * k / us / 1e6
+                rows.append({"m": m, "n": n, "k": k, "dtype": name, "us": round(us, 1), "tflops": round(tf, 1),
+                             "frac": round(tf * 1e12 / MFMA_PEAK["f16"], 3)})
+    for n, k in ((18432, 7168), (7168, 18432)):
+        for m in (1024, 4096):
+            x = torch.randn(m, k, device="cuda").to(torch.float8_e4m3fn)
+            w = torch.randn(n, k, device="cuda").to(torch.float8_e4m3fn)
+            for scaling, sa, sb in (("per tensor", torch.ones((), device="cuda"), torch.ones((), device="cuda")),
+                                    ("per row", torch.ones(m, 1, device="cuda"), torch.ones(1, n, device="cuda"))):
+                us = timed(lambda: torch._scaled_mm(x, w.t(), scale_a=sa, scale_b=sb, out_dtype=torch.bfloat16))
+                tf = 2.0 * m * n * k / us / 1e6
+                rows.append({"m": m, "n": n, "k": k, "dtype": "e4m3, scales " + scaling, "us": round(us, 1),
+                             "tflops": round(tf, 1), "frac": round(tf * 1e12 / MFMA_PEAK["fp8"], 3)})
+    for r in rows:
+        print("%5d x %5d x %5d  %-22s %9.1f us %8.1f TFLOP/s  %5.1f %% of peak" %
+              (r["m"], r["n"], r["k"], r["dtype"], r["us"], r["tflops"], 100 * r["frac"]), file=sys.stderr)
+    print(json.dumps({"library_gemm": rows}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -487,6 +526,9 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true", help="run only a 256 MiB device-to-device copy a few "
                     "times (the known-size kernel hardware traffic counters are scaled by) and exit")
     ap.add_argument("--details", action="store_true", help="also print a per-case table to stderr")
+    ap.add_argument("--library-gemm", action="store_true", help="run only the vendor library's plain GEMMs (torch.matmul "
+                    "fp16 / bf16, torch._scaled_mm e4m3; no dequantization, no block scales) at the prefill shapes of "
+                    "configurations 3 and 4 and exit: what a dense GEMM reaches on this part, beside the MFMA peak")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU's throughput; --gpus %d is not supported (this path has no "
@@ -502,6 +544,10 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         print(json.dumps({"copy_bytes_read": n, "copy_bytes_written": n, "launches": 5}))
+        return
+
+    if args.library_gemm:
+        library_gemm(args.steps, args.warmup)
         return
 
     from ksanallm_amd import lib as L
