@@ -202,10 +202,10 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
     if (s_vec) {
       if (wave == 0)
         asm volatile("s_nop 4\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %2" ::"v"(s_voff), "s"(d), "s"(ap)
-                     : "memory");
+                     : "memory", "m0");
     } else if (wave < BM / 64) {
       asm volatile("s_nop 4\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, %2" ::"v"(s_voff), "s"(d), "s"(ap)
-                   : "memory");
+                   : "memory", "m0");
     }
   };
   // operands of k-block `kb` -> LDS slot kb % 2.  The instruction offset of an LDS-targeted load is added to the LDS
@@ -226,7 +226,7 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
           :
           : "v"(d_voff[0]), "v"(d_voff[1]), "v"(d_voff_hi[0]), "v"(d_voff_hi[1]), "s"(f0), "s"(f0h), "s"(f1), "s"(f1h),
             "s"(src)
-          : "memory");
+          : "memory", "m0");
       return;
     }
     const uint32_t f2 = f1 + FRAG, f2h = f1h + FRAG;
@@ -245,7 +245,7 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
         : "v"(d_voff[0]), "v"(d_voff[1]), "v"(d_voff[2]), "v"(d_voff[3]), "v"(d_voff_hi[0]), "v"(d_voff_hi[1]),
           "v"(d_voff_hi[2]), "v"(d_voff_hi[3]), "s"(f0), "s"(f0h), "s"(f1), "s"(f1h), "s"(f2), "s"(f2h), "s"(f3),
           "s"(f3h), "s"(src)
-        : "memory");
+        : "memory", "m0");
   };
   // Everything this wavefront issued has landed, except the loads of the youngest stage when three stages are in use
   // (vmcnt retires in issue order; a wavefront issues the same loads every stage: 8 weight loads, or 2*AFW activation

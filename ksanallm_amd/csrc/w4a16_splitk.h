@@ -343,7 +343,7 @@ __global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKPar
           asm volatile("s_nop 4\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %2"
                        :
                        : "v"(voff), "s"(dst), "s"(src)
-                       : "memory");
+                       : "memory", "m0");
         }
       }
     };

@@ -360,7 +360,7 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
             "s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %3 offset:64"
             :
             : "v"(a_voff[0]), "s"(d0), "s"(d1), "s"(src)
-            : "memory");
+            : "memory", "m0");
       } else {
         static_assert(APV == 2 || APV == 4, "two or four fragments per wavefront and stage");
         const uint32_t d2 = d0 + 2048, d3 = d1 + 2048;
@@ -372,7 +372,7 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
             "s_mov_b32 m0, %5\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %6 offset:64"
             :
             : "v"(a_voff[0]), "v"(a_voff[APV / 2 - 1]), "s"(d0), "s"(d1), "s"(d2), "s"(d3), "s"(src)
-            : "memory");
+            : "memory", "m0");
       }
     };
     // ---- compute pipeline, in steps of 32 k (two per stage).  A fragments are read DEPTH ahead of the MFMAs that use

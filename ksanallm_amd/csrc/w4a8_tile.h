@@ -166,16 +166,16 @@ __global__ void __launch_bounds__(512, 1) w4a8_tile_kernel(W4A8TileParams p) {
       const uint32_t d = __builtin_amdgcn_readfirstlane(s_lds + (kb % NS) * 1024);
       if (s_vec)
         asm volatile("s_nop 4\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %2" ::"v"(s_voff), "s"(d), "s"(ap)
-                     : "memory");
+                     : "memory", "m0");
       else
         asm volatile("s_nop 4\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, %2" ::"v"(s_voff), "s"(d), "s"(ap)
-                     : "memory");
+                     : "memory", "m0");
     }
     if (wave == 4) {
       const char* wp = ws_base + static_cast<size_t>(k) * GH * p.N * 2;
       const uint32_t d = __builtin_amdgcn_readfirstlane(ws_lds + (kb % NS) * 1024);
       asm volatile("s_nop 4\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %2" ::"v"(ws_voff), "s"(d), "s"(wp)
-                   : "memory");
+                   : "memory", "m0");
     }
   };
   // operands of k-block `kb` -> LDS slot kb % NS.  The instruction offset of an LDS-targeted load is added to the LDS
@@ -194,7 +194,7 @@ __global__ void __launch_bounds__(512, 1) w4a8_tile_kernel(W4A8TileParams p) {
           "s_mov_b32 m0, %7\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %3, %8"
           :
           : "v"(d_voff[0]), "v"(d_voff[1]), "v"(d_voff[2]), "v"(d_voff[3]), "s"(f0), "s"(f1), "s"(f2), "s"(f3), "s"(src)
-          : "memory");
+          : "memory", "m0");
       return;
     }
     const uint32_t f0h = f0 + 1024 - 64;
@@ -208,7 +208,7 @@ __global__ void __launch_bounds__(512, 1) w4a8_tile_kernel(W4A8TileParams p) {
           "s_mov_b32 m0, %5\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %6 offset:64"
           :
           : "v"(d_voff[0]), "v"(d_voff[1]), "s"(f0), "s"(f0h), "s"(f1), "s"(f1h), "s"(src)
-          : "memory");
+          : "memory", "m0");
       return;
     }
     const uint32_t f2 = f1 + FRAG, f2h = f1h + FRAG;
@@ -226,7 +226,7 @@ __global__ void __launch_bounds__(512, 1) w4a8_tile_kernel(W4A8TileParams p) {
         :
         : "v"(d_voff[0]), "v"(d_voff[1]), "v"(d_voff[2]), "v"(d_voff[3]), "s"(f0), "s"(f0h), "s"(f1), "s"(f1h), "s"(f2),
           "s"(f2h), "s"(f3), "s"(f3h), "s"(src)
-        : "memory");
+        : "memory", "m0");
   };
   // Everything this wavefront issued has landed except the loads of the youngest stage (vmcnt retires in issue order;
   // a wavefront issues the same loads every stage: 4 weight loads with or without the weight-scale load, or 2*AFW
