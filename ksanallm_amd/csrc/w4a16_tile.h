@@ -5,12 +5,15 @@
 //     for whole 1 KiB MFMA fragments (16 rows x 32 k, four lanes per row so that every load touches 64 contiguous
 //     bytes per row, pieces swizzled so that the read-back is free of bank conflicts), into a ring of NS stages of
 //     64 k each.  The fragment is read back with one ds_read_b128 per lane, DEPTH fragments ahead of the MFMAs that
-//     use it.  Two to three stages are in flight while one is consumed; the one barrier per stage sits in the middle of the stage, so the fragment reads never
-//     drain at a stage boundary.
+//     use it.  Two to three stages are in flight while one is consumed; the one barrier per stage sits in the middle
+//     of the stage, so the fragment reads never drain at a stage boundary.
 //   - packed int4 weights never touch LDS: the 8 wavefronts split the 256 columns (2 column tiles of 16 each), so
 //     every weight fragment belongs to exactly one wavefront and no weight is dequantized twice.  A wavefront loads
 //     its 1 KiB tiles straight from global memory (16 bytes per lane) three stages ahead and dequantizes them in
 //     registers to T with (code - zp) * s applied.
+//   - the loads of a stage are not issued in one run behind the barrier - eight wavefronts would queue at the memory
+//     pipeline at once, each stalled until its loads are accepted - but one group at a time between the MFMAs of the
+//     steps: x fragments during the second step of every stage, weights during the first step of every other one.
 //   - all vector memory loads of the main loop are issued from inline assembly in a fixed order, the same number
 //     every stage (addresses are clamped past the end), so that one `s_waitcnt vmcnt(N)` per stage with a constant N
 //     releases exactly the stage that is needed: vmcnt retires in issue order.  The registers a wait makes valid are
@@ -240,72 +243,55 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
   // before the statement starts, and should the compiler have produced one of them with a VALU instruction
   // (v_readfirstlane), the five wait states a vector memory instruction needs after that have passed.  The compiler
   // inserts such wait states for its own instructions, not inside assembly.
-  auto load_w = [&](WSlot (&dst)[WN], uint32_t kt) {
-    static_assert(WN == 2, "the load group below names two column tiles");
+  // the loads of one column tile for k-tile kt: the packed tile, and a scale (and zero point) per group
+  auto load_w_part = [&](WSlot (&dst)[WN], uint32_t kt, auto tc) {
+    constexpr int t = decltype(tc)::value;
     kt = kt < kt_count ? kt : kt_count - 1;
-    const char* w0 = w_base[0] + static_cast<size_t>(kt) * 1024;
-    const char* w1 = w_base[1] + static_cast<size_t>(kt) * 1024;
-    const char* s0 = s_base[0] + static_cast<size_t>(kt) * (GPT * 32);
-    const char* s1 = s_base[1] + static_cast<size_t>(kt) * (GPT * 32);
+    const char* w0 = w_base[t] + static_cast<size_t>(kt) * 1024;
+    const char* s0 = s_base[t] + static_cast<size_t>(kt) * (GPT * 32);
     if (HAS_ZP) {
-      const char* z0 = z_base[0] + static_cast<size_t>(kt) * (GPT * 16);
-      const char* z1 = z_base[1] + static_cast<size_t>(kt) * (GPT * 16);
+      const char* z0 = z_base[t] + static_cast<size_t>(kt) * (GPT * 16);
       asm volatile(
           "s_nop 4\n\t"
-          "global_load_dwordx4 %0, %6, %9\n\t"
-          "global_load_ushort %1, %7, %10\n\t"
-          "global_load_ubyte %2, %8, %11\n\t"
-          "global_load_dwordx4 %3, %6, %12\n\t"
-          "global_load_ushort %4, %7, %13\n\t"
-          "global_load_ubyte %5, %8, %14"
-          : "=&v"(dst[0].wq), "=&v"(dst[0].sc[0]), "=&v"(dst[0].zp[0]), "=&v"(dst[1].wq), "=&v"(dst[1].sc[0]), "=&v"(dst[1].zp[0])
-          : "v"(w_voff), "v"(s_voff), "v"(z_voff), "s"(w0), "s"(s0), "s"(z0), "s"(w1), "s"(s1), "s"(z1)
+          "global_load_dwordx4 %0, %3, %6\n\t"
+          "global_load_ushort %1, %4, %7\n\t"
+          "global_load_ubyte %2, %5, %8"
+          : "=&v"(dst[t].wq), "=&v"(dst[t].sc[0]), "=&v"(dst[t].zp[0])
+          : "v"(w_voff), "v"(s_voff), "v"(z_voff), "s"(w0), "s"(s0), "s"(z0)
           : "memory");
-      // the further groups of the k-tile (group sizes 64 and 32): the same loads 32 / 16 bytes further each
 #pragma unroll
       for (int gi = 1; gi < GPT; ++gi) {
         const char* s0g = s0 + gi * 32;
-        const char* s1g = s1 + gi * 32;
         const char* z0g = z0 + gi * 16;
-        const char* z1g = z1 + gi * 16;
         asm volatile(
             "s_nop 4\n\t"
-            "global_load_ushort %0, %4, %6\n\t"
-            "global_load_ubyte %1, %5, %7\n\t"
-            "global_load_ushort %2, %4, %8\n\t"
-            "global_load_ubyte %3, %5, %9"
-            : "=&v"(dst[0].sc[gi]), "=&v"(dst[0].zp[gi]), "=&v"(dst[1].sc[gi]), "=&v"(dst[1].zp[gi])
-            : "v"(s_voff), "v"(z_voff), "s"(s0g), "s"(z0g), "s"(s1g), "s"(z1g)
+            "global_load_ushort %0, %2, %4\n\t"
+            "global_load_ubyte %1, %3, %5"
+            : "=&v"(dst[t].sc[gi]), "=&v"(dst[t].zp[gi])
+            : "v"(s_voff), "v"(z_voff), "s"(s0g), "s"(z0g)
             : "memory");
       }
     } else {
       asm volatile(
           "s_nop 4\n\t"
-          "global_load_dwordx4 %0, %4, %6\n\t"
-          "global_load_ushort %1, %5, %7\n\t"
-          "global_load_dwordx4 %2, %4, %8\n\t"
-          "global_load_ushort %3, %5, %9"
-          : "=&v"(dst[0].wq), "=&v"(dst[0].sc[0]), "=&v"(dst[1].wq), "=&v"(dst[1].sc[0])
-          : "v"(w_voff), "v"(s_voff), "s"(w0), "s"(s0), "s"(w1), "s"(s1)
+          "global_load_dwordx4 %0, %2, %4\n\t"
+          "global_load_ushort %1, %3, %5"
+          : "=&v"(dst[t].wq), "=&v"(dst[t].sc[0])
+          : "v"(w_voff), "v"(s_voff), "s"(w0), "s"(s0)
           : "memory");
 #pragma unroll
       for (int gi = 1; gi < GPT; ++gi) {
         const char* s0g = s0 + gi * 32;
-        const char* s1g = s1 + gi * 32;
-        asm volatile(
-            "s_nop 4\n\t"
-            "global_load_ushort %0, %2, %3\n\t"
-            "global_load_ushort %1, %2, %4"
-            : "=&v"(dst[0].sc[gi]), "=&v"(dst[1].sc[gi])
-            : "v"(s_voff), "s"(s0g), "s"(s1g)
-            : "memory");
+        asm volatile("s_nop 4\n\tglobal_load_ushort %0, %1, %2" : "=&v"(dst[t].sc[gi]) : "v"(s_voff), "s"(s0g) : "memory");
       }
 #pragma unroll
-      for (int gi = 0; gi < GPT; ++gi) {
-        dst[0].zp[gi] = 8u;
-        dst[1].zp[gi] = 8u;
-      }
+      for (int gi = 0; gi < GPT; ++gi) dst[t].zp[gi] = 8u;
     }
+  };
+  auto load_w = [&](WSlot (&dst)[WN], uint32_t kt) {
+    static_assert(WN == 2, "two column tiles per wavefront");
+    load_w_part(dst, kt, std::integral_constant<int, 0>{});
+    load_w_part(dst, kt, std::integral_constant<int, 1>{});
   };
   // wait until at most `n` loads are outstanding; the weight slots named become valid with this wait and are tied to it
   auto wait_tie = [&](auto n, WSlot (&fresh)[WN]) {
@@ -346,34 +332,29 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
       a_voff[j] = (row * p.K + 8 * ((lane & 3) ^ (lane >> 4))) * 2;
     }
     const uint32_t a_lds_wave = lds_base + wave * APV * 1024;
-    // x stage `stage` -> LDS slot stage % NS.  The instruction offset of an LDS-targeted load is added to the LDS address
-    // as well as to the global one: the second fragment's 64-byte global offset is taken back out of its LDS base.
-    auto load_a = [&](uint32_t stage) {
+    // x stage `stage` -> LDS slot stage % NS, fragment pair `part` of this wavefront's APV / 2 pairs.  The instruction
+    // offset of an LDS-targeted load is added to the LDS address as well as to the global one: the second fragment's
+    // 64-byte global offset is taken back out of its LDS base.
+    auto load_a_part = [&](uint32_t stage, auto pc) {
+      constexpr int part = decltype(pc)::value;
+      if constexpr (part >= APV / 2) return;
       const uint32_t st = stage < stages ? stage : stages - 1;
       const char* src = x_tile + static_cast<size_t>(st) * (BK * 2);
-      const uint32_t d0 = __builtin_amdgcn_readfirstlane(a_lds_wave + (stage % NS) * STAGE_BYTES);
+      const uint32_t d0 = __builtin_amdgcn_readfirstlane(a_lds_wave + (stage % NS) * STAGE_BYTES) + part * 2048;
       const uint32_t d1 = d0 + 1024 - 64;
-      if constexpr (APV == 2) {
-        asm volatile(
-            "s_nop 4\n\t"
-            "s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %3\n\t"
-            "s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %3 offset:64"
-            :
-            : "v"(a_voff[0]), "s"(d0), "s"(d1), "s"(src)
-            : "memory", "m0");
-      } else {
-        static_assert(APV == 2 || APV == 4, "two or four fragments per wavefront and stage");
-        const uint32_t d2 = d0 + 2048, d3 = d1 + 2048;
-        asm volatile(
-            "s_nop 4\n\t"
-            "s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %6\n\t"
-            "s_mov_b32 m0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %6 offset:64\n\t"
-            "s_mov_b32 m0, %4\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %6\n\t"
-            "s_mov_b32 m0, %5\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %6 offset:64"
-            :
-            : "v"(a_voff[0]), "v"(a_voff[APV / 2 - 1]), "s"(d0), "s"(d1), "s"(d2), "s"(d3), "s"(src)
-            : "memory", "m0");
-      }
+      const uint32_t av = a_voff[part < APV / 2 ? part : 0];
+      asm volatile(
+          "s_nop 4\n\t"
+          "s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %3\n\t"
+          "s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %3 offset:64"
+          :
+          : "v"(av), "s"(d0), "s"(d1), "s"(src)
+          : "memory", "m0");
+    };
+    auto load_a = [&](uint32_t stage) {
+      static_assert(APV == 2 || APV == 4, "one or two fragment pairs per wavefront and stage");
+      load_a_part(stage, std::integral_constant<int, 0>{});
+      load_a_part(stage, std::integral_constant<int, 1>{});
     };
     // ---- compute pipeline, in steps of 32 k (two per stage).  A fragments are read DEPTH ahead of the MFMAs that use
     // them, across step and stage boundaries; the weight fragments of step g+1 are dequantized while step g multiplies.
@@ -385,7 +366,7 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
 
     auto frag_ptr = [&](uint32_t slot, int ks) { return lds + slot * STAGE_BYTES + ks * 1024 + a_rd; };
     // `wn`/`dn`: weight slot and dword (32-k block of its k-tile) the NEXT step uses
-    auto step = [&](auto parity, uint32_t slot, int ks, WSlot (&wn)[WN], int dn) {
+    auto step = [&](auto parity, uint32_t slot, int ks, WSlot (&wn)[WN], int dn, auto&& issue) {
       constexpr int P = decltype(parity)::value;
       typename T::frag(&bcur)[WN] = bfrag[P];
       typename T::frag(&bnext)[WN] = bfrag[P ^ 1];
@@ -405,6 +386,7 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
         for (int t = 0; t < WN; ++t) acc[t][i] = T::mfma(bcur[t], as_frag<T>(a), acc[t][i]);
         if (i == 1) bnext[0] = dq[0](wn[0].wq[dn]);
         if (i == WMV / 2 + 1) bnext[1] = dq[1](wn[1].wq[dn]);
+        issue(std::integral_constant<int, 0>{}, i);
         __builtin_amdgcn_sched_barrier(0x6);  // VALU / SALU may move; LDS reads and MFMAs keep this order
       }
     };
@@ -412,18 +394,19 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
     using Odd = std::integral_constant<int, 1>;
 
     // ---- schedule.  One synchronisation point per stage, in its middle ("sync c" sits between the two steps of
-    // stage c): wait for x stage c+1, barrier, then issue [weights of k-tile c/2+2 when c is even][x stage c+3] - the LDS
-    // slot of stage c+3 is the one stage c-1 used, and every wavefront is past that.  Weights of k-tile kt are issued at
-    // sync 2kt-4, complete at sync 2kt-2 and are first dequantized during the last step of k-tile kt-1.
-    // Loads outstanding after x stage c+1 at sync c: those of sync c-1, i.e. APV, plus 2*WL when c-1 is even.
+    // stage c): wait for x stage c+1, barrier.  x stage c+3 is issued during the second step of stage c - its LDS slot is
+    // the one stage c-1 used, and every wavefront is past that -, the weights of k-tile (c+3)/2 during the first step of
+    // the odd stages c: issued in stage 2kt-3, they are waited for at sync 2kt-2 and first dequantized during the last
+    // step of k-tile kt-1.  Issue order around sync c: ... x(c+1) [w((c+2)/2), c even] x(c+2) [w((c+3)/2), c odd] | sync c:
+    // after x stage c+1 (and, c even, the weights behind it) come APV loads when c is even, APV + 2*WL when c is odd.
     using WaitEven = std::integral_constant<int, APV>;
     using WaitOdd = std::integral_constant<int, APV + WN * WL>;
     using WaitFirst = std::integral_constant<int, 2 * APV + WN * WL>;
-    load_w(ring[0], 0);  // sync -4
-    load_a(0);           // sync -3
-    load_w(ring[1], 1);  // sync -2
+    load_w(ring[0], 0);
+    load_a(0);
+    load_w(ring[1], 1);
     load_a(1);
-    load_a(2);           // sync -1
+    load_a(2);
     wait_tie(WaitFirst{}, ring[0]);  // x stage 0 and k-tile 0 are in
     __builtin_amdgcn_s_barrier();
   #pragma unroll
@@ -441,23 +424,46 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
         const uint32_t slot = s % NS;
         constexpr int kDummy = 0;
         (void)kDummy;
+        auto none = [](auto, int) {};
+        // The loads are spread over the row tiles of the steps (one group per row tile) instead of issued in one run
+        // behind the barrier, where all eight wavefronts queue at the memory pipeline at once: the weights of k-tile
+        // s/2+2 during the first step of the odd stages (registers: no barrier to wait for), x stage s+3 during the
+        // second step of every stage (its LDS slot is free once every wavefront is past the barrier).
+        auto spread_w = [&](auto, int i) {
+          if (i == 0) load_w_part(ring[(u / 2 + 2) % 3], s / 2 + 2, std::integral_constant<int, 0>{});
+          if (i == 2) load_w_part(ring[(u / 2 + 2) % 3], s / 2 + 2, std::integral_constant<int, 1>{});
+        };
+        auto spread_a = [&](auto, int i) {
+          if (i == 0) load_a_part(s + 3, std::integral_constant<int, 0>{});
+          if (i == 2) load_a_part(s + 3, std::integral_constant<int, 1>{});
+        };
         // first step of the stage: k block 2*(u%2) of k-tile u/2; the next step uses block 2*(u%2)+1 of the same tile
-        if (s < stages) step(Even{}, slot, 0, ring[(u / 2) % 3], 2 * (u % 2) + 1);
+        if (u % 2 == 0) {
+          if (s < stages) step(Even{}, slot, 0, ring[(u / 2) % 3], 2 * (u % 2) + 1, none);
+        } else {
+          if (s < stages) {
+            step(Even{}, slot, 0, ring[(u / 2) % 3], 2 * (u % 2) + 1, spread_w);
+          } else {
+            spread_w(0, 0);
+            spread_w(0, 2);
+          }
+        }
         // sync s
         if (u % 2 == 0) {
-          wait_tie(WaitEven{}, ring[(u / 2 + 1) % 3]);  // k-tile s/2+1, issued at sync s-2
+          wait_tie(WaitEven{}, ring[(u / 2 + 1) % 3]);  // k-tile s/2+1, issued during stage s-1
         } else {
           wait_only(WaitOdd{});
         }
         __builtin_amdgcn_s_barrier();
-        if (u % 2 == 0) load_w(ring[(u / 2 + 2) % 3], s / 2 + 2);
-        load_a(s + 3);
         // second step: the next step is block 2 of this k-tile (u even) or block 0 of the next k-tile (u odd)
         if (s < stages) {
           if (u % 2 == 0)
-            step(Odd{}, slot, 1, ring[(u / 2) % 3], 2);
+            step(Odd{}, slot, 1, ring[(u / 2) % 3], 2, spread_a);
           else
-            step(Odd{}, slot, 1, ring[(u / 2 + 1) % 3], 0);
+            step(Odd{}, slot, 1, ring[(u / 2 + 1) % 3], 0, spread_a);
+        } else {
+          spread_a(0, 0);
+          spread_a(0, 2);
         }
       }
     }
