@@ -359,7 +359,9 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
     // ---- compute pipeline, in steps of 32 k (two per stage).  A fragments are read DEPTH ahead of the MFMAs that use
     // them, across step and stage boundaries; the weight fragments of step g+1 are dequantized while step g multiplies.
     constexpr int DEPTH = 4;
-    static_assert(WMV % DEPTH == 0, "the A prefetch ring must divide the row tiles");
+    // the prefetch ring runs on through the steps: a step of WMV reads leaves it turned by WMV % DEPTH places, so the
+    // second step of a stage starts there and the first one (two steps later) at place 0 again
+    static_assert((2 * WMV) % DEPTH == 0 && WMV >= DEPTH, "two steps must turn the A prefetch ring a whole number of times");
     u32x4 abuf[DEPTH];
     typename T::frag bfrag[2][WN];  // weight fragments of the current step [g % 2] and the next one
     Dequant<T, HAS_ZP> dq[WN];
@@ -378,9 +380,10 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
       }
   #pragma unroll
       for (int i = 0; i < WMV; ++i) {
-        const u32x4 a = abuf[i % DEPTH];
+        constexpr int TURN = P * (WMV % DEPTH);
+        const u32x4 a = abuf[(i + TURN) % DEPTH];
         const int ni = i + DEPTH;
-        abuf[i % DEPTH] = ni < WMV ? *reinterpret_cast<const u32x4*>(cur + ni * 2048)
+        abuf[(i + TURN) % DEPTH] = ni < WMV ? *reinterpret_cast<const u32x4*>(cur + ni * 2048)
                                    : *reinterpret_cast<const u32x4*>(nxt + (ni - WMV) * 2048);
   #pragma unroll
         for (int t = 0; t < WN; ++t) acc[t][i] = T::mfma(bcur[t], as_frag<T>(a), acc[t][i]);
@@ -469,11 +472,14 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
     }
   };
   if (GROUPED && WM == 16) {
-    // 256-slot expert blocks: the row tiles that hold slots, in steps of four (the depth of the fragment prefetch)
+    // 256-slot expert blocks: the row tiles that hold slots, in steps of four, and ten (129..160 slots: what an expert
+    // with 128 slots on average holds when it holds more than 128)
     if (live_tiles <= 4)
       run(std::integral_constant<int, 4>{});
     else if (live_tiles <= 8)
       run(std::integral_constant<int, 8>{});
+    else if (live_tiles <= 10)
+      run(std::integral_constant<int, (WM == 16 ? 10 : WM)>{});
     else if (live_tiles <= 12)
       run(std::integral_constant<int, (WM == 16 ? 12 : WM)>{});
     else
