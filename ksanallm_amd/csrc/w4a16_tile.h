@@ -359,17 +359,18 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
     // ---- compute pipeline, in steps of 32 k (two per stage).  A fragments are read DEPTH ahead of the MFMAs that use
     // them, across step and stage boundaries; the weight fragments of step g+1 are dequantized while step g multiplies.
     constexpr int DEPTH = 4;
-    // the prefetch ring runs on through the steps: a step of WMV reads leaves it turned by WMV % DEPTH places, so the
-    // second step of a stage starts there and the first one (two steps later) at place 0 again
-    static_assert((2 * WMV) % DEPTH == 0 && WMV >= DEPTH, "two steps must turn the A prefetch ring a whole number of times");
+    // the prefetch ring runs on through the steps: a step of WMV reads leaves it turned by WMV % DEPTH places, and the
+    // twelve steps of one turn of the main loop by a whole number of turns
+    static_assert((12 * WMV) % DEPTH == 0 && WMV >= DEPTH, "the main loop must turn the A prefetch ring a whole number of times");
     u32x4 abuf[DEPTH];
     typename T::frag bfrag[2][WN];  // weight fragments of the current step [g % 2] and the next one
     Dequant<T, HAS_ZP> dq[WN];
 
     auto frag_ptr = [&](uint32_t slot, int ks) { return lds + slot * STAGE_BYTES + ks * 1024 + a_rd; };
     // `wn`/`dn`: weight slot and dword (32-k block of its k-tile) the NEXT step uses
-    auto step = [&](auto parity, uint32_t slot, int ks, WSlot (&wn)[WN], int dn, auto&& issue) {
+    auto step = [&](auto parity, auto turn, uint32_t slot, int ks, WSlot (&wn)[WN], int dn, auto&& issue) {
       constexpr int P = decltype(parity)::value;
+      constexpr int TURN = decltype(turn)::value;  // where the prefetch ring stands when this step starts
       typename T::frag(&bcur)[WN] = bfrag[P];
       typename T::frag(&bnext)[WN] = bfrag[P ^ 1];
       const char* cur = frag_ptr(slot, ks);
@@ -380,7 +381,6 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
       }
   #pragma unroll
       for (int i = 0; i < WMV; ++i) {
-        constexpr int TURN = P * (WMV % DEPTH);
         const u32x4 a = abuf[(i + TURN) % DEPTH];
         const int ni = i + DEPTH;
         abuf[(i + TURN) % DEPTH] = ni < WMV ? *reinterpret_cast<const u32x4*>(cur + ni * 2048)
@@ -420,68 +420,83 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
   #pragma unroll
     for (int j = 0; j < DEPTH; ++j) abuf[j] = *reinterpret_cast<const u32x4*>(frag_ptr(0, 0) + j * 2048);
 
-    for (uint32_t base = 0; base < stages; base += 6) {
-  #pragma unroll
-      for (int u = 0; u < 6; ++u) {
-        const uint32_t s = base + u;
-        const uint32_t slot = s % NS;
-        constexpr int kDummy = 0;
-        (void)kDummy;
-        auto none = [](auto, int) {};
-        // The loads are spread over the row tiles of the steps (one group per row tile) instead of issued in one run
-        // behind the barrier, where all eight wavefronts queue at the memory pipeline at once: the weights of k-tile
-        // s/2+2 during the first step of the odd stages (registers: no barrier to wait for), x stage s+3 during the
-        // second step of every stage (its LDS slot is free once every wavefront is past the barrier).
-        auto spread_w = [&](auto, int i) {
-          if (i == 0) load_w_part(ring[(u / 2 + 2) % 3], s / 2 + 2, std::integral_constant<int, 0>{});
-          if (i == 2) load_w_part(ring[(u / 2 + 2) % 3], s / 2 + 2, std::integral_constant<int, 1>{});
-        };
-        auto spread_a = [&](auto, int i) {
-          if (i == 0) load_a_part(s + 3, std::integral_constant<int, 0>{});
-          if (i == 2) load_a_part(s + 3, std::integral_constant<int, 1>{});
-        };
-        // first step of the stage: k block 2*(u%2) of k-tile u/2; the next step uses block 2*(u%2)+1 of the same tile
-        if (u % 2 == 0) {
-          if (s < stages) step(Even{}, slot, 0, ring[(u / 2) % 3], 2 * (u % 2) + 1, none);
-        } else {
-          if (s < stages) {
-            step(Even{}, slot, 0, ring[(u / 2) % 3], 2 * (u % 2) + 1, spread_w);
-          } else {
-            spread_w(0, 0);
-            spread_w(0, 2);
-          }
-        }
-        // sync s
-        if (u % 2 == 0) {
-          wait_tie(WaitEven{}, ring[(u / 2 + 1) % 3]);  // k-tile s/2+1, issued during stage s-1
-        } else {
-          wait_only(WaitOdd{});
-        }
-        __builtin_amdgcn_s_barrier();
-        // second step: the next step is block 2 of this k-tile (u even) or block 0 of the next k-tile (u odd)
+    // stage base + u of the six stages (three k-tiles) one turn of the main loop covers
+    auto stage = [&](auto uc, uint32_t base) {
+      constexpr int u = decltype(uc)::value;
+      using Turn0 = std::integral_constant<int, (2 * u * WMV) % DEPTH>;
+      using Turn1 = std::integral_constant<int, ((2 * u + 1) * WMV) % DEPTH>;
+      const uint32_t s = base + u;
+      const uint32_t slot = s % NS;
+      auto none = [](auto, int) {};
+      // The loads are spread over the row tiles of the steps (one group per row tile) instead of issued in one run
+      // behind the barrier, where all eight wavefronts queue at the memory pipeline at once: the weights of k-tile
+      // s/2+2 during the first step of the odd stages (registers: no barrier to wait for), x stage s+3 during the
+      // second step of every stage (its LDS slot is free once every wavefront is past the barrier).
+      auto spread_w = [&](auto, int i) {
+        if (i == 0) load_w_part(ring[(u / 2 + 2) % 3], s / 2 + 2, std::integral_constant<int, 0>{});
+        if (i == 2) load_w_part(ring[(u / 2 + 2) % 3], s / 2 + 2, std::integral_constant<int, 1>{});
+      };
+      auto spread_a = [&](auto, int i) {
+        if (i == 0) load_a_part(s + 3, std::integral_constant<int, 0>{});
+        if (i == 2) load_a_part(s + 3, std::integral_constant<int, 1>{});
+      };
+      // first step of the stage: k block 2*(u%2) of k-tile u/2; the next step uses block 2*(u%2)+1 of the same tile
+      if constexpr (u % 2 == 0) {
+        if (s < stages) step(Even{}, Turn0{}, slot, 0, ring[(u / 2) % 3], 2 * (u % 2) + 1, none);
+      } else {
         if (s < stages) {
-          if (u % 2 == 0)
-            step(Odd{}, slot, 1, ring[(u / 2) % 3], 2, spread_a);
-          else
-            step(Odd{}, slot, 1, ring[(u / 2 + 1) % 3], 0, spread_a);
+          step(Even{}, Turn0{}, slot, 0, ring[(u / 2) % 3], 2 * (u % 2) + 1, spread_w);
         } else {
-          spread_a(0, 0);
-          spread_a(0, 2);
+          spread_w(0, 0);
+          spread_w(0, 2);
         }
       }
+      // sync s
+      if constexpr (u % 2 == 0) {
+        wait_tie(WaitEven{}, ring[(u / 2 + 1) % 3]);  // k-tile s/2+1, issued during stage s-1
+      } else {
+        wait_only(WaitOdd{});
+      }
+      __builtin_amdgcn_s_barrier();
+      // second step: the next step is block 2 of this k-tile (u even) or block 0 of the next k-tile (u odd)
+      if (s < stages) {
+        if constexpr (u % 2 == 0)
+          step(Odd{}, Turn1{}, slot, 1, ring[(u / 2) % 3], 2, spread_a);
+        else
+          step(Odd{}, Turn1{}, slot, 1, ring[(u / 2 + 1) % 3], 0, spread_a);
+      } else {
+        spread_a(0, 0);
+        spread_a(0, 2);
+      }
+    };
+    for (uint32_t base = 0; base < stages; base += 6) {
+      stage(std::integral_constant<int, 0>{}, base);
+      stage(std::integral_constant<int, 1>{}, base);
+      stage(std::integral_constant<int, 2>{}, base);
+      stage(std::integral_constant<int, 3>{}, base);
+      stage(std::integral_constant<int, 4>{}, base);
+      stage(std::integral_constant<int, 5>{}, base);
     }
   };
   if (GROUPED && WM == 16) {
-    // 256-slot expert blocks: the row tiles that hold slots, in steps of four, and ten (129..160 slots: what an expert
-    // with 128 slots on average holds when it holds more than 128)
+    // 256-slot expert blocks: an instance of the main loop over the row tiles that hold slots - every count from six
+    // to ten (an expert with 128 slots on average holds 97..160), and 4, 12, 14, 16
     if (live_tiles <= 4)
       run(std::integral_constant<int, 4>{});
+    else if (live_tiles <= 6)
+      run(std::integral_constant<int, (WM == 16 ? 6 : WM)>{});
+    else if (live_tiles <= 7)
+      run(std::integral_constant<int, (WM == 16 ? 7 : WM)>{});
     else if (live_tiles <= 8)
       run(std::integral_constant<int, 8>{});
+    else if (live_tiles <= 9)
+      run(std::integral_constant<int, (WM == 16 ? 9 : WM)>{});
     else if (live_tiles <= 10)
       run(std::integral_constant<int, (WM == 16 ? 10 : WM)>{});
     else if (live_tiles <= 12)
       run(std::integral_constant<int, (WM == 16 ? 12 : WM)>{});
+    else if (live_tiles <= 14)
+      run(std::integral_constant<int, (WM == 16 ? 14 : WM)>{});
     else
       run(std::integral_constant<int, WM>{});
   } else if (live_tiles <= WM / 2) {
