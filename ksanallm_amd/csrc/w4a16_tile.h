@@ -131,6 +131,19 @@ struct Dequant<BF16, HAS_ZP> {
   }
 };
 
+// f(integral_constant<N>) for the smallest N in LO..HI with count <= N (N = HI when there is none)
+template <int LO, int HI, typename F>
+__device__ __forceinline__ void for_tile_count(uint32_t count, F&& f) {
+  if constexpr (LO >= HI) {
+    f(std::integral_constant<int, HI>{});
+  } else {
+    if (count <= static_cast<uint32_t>(LO))
+      f(std::integral_constant<int, LO>{});
+    else
+      for_tile_count<LO + 1, HI>(count, f);
+  }
+}
+
 // One column tile's packed weights for one k-tile of 128, with the scale and zero point of each of its GPT groups.
 template <int GPT>
 struct WSlot {
@@ -478,27 +491,12 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
       stage(std::integral_constant<int, 5>{}, base);
     }
   };
-  if (GROUPED && WM == 16) {
-    // 256-slot expert blocks: an instance of the main loop over the row tiles that hold slots - every count from six
-    // to ten (an expert with 128 slots on average holds 97..160), and 4, 12, 14, 16
-    if (live_tiles <= 4)
-      run(std::integral_constant<int, 4>{});
-    else if (live_tiles <= 6)
-      run(std::integral_constant<int, (WM == 16 ? 6 : WM)>{});
-    else if (live_tiles <= 7)
-      run(std::integral_constant<int, (WM == 16 ? 7 : WM)>{});
-    else if (live_tiles <= 8)
-      run(std::integral_constant<int, 8>{});
-    else if (live_tiles <= 9)
-      run(std::integral_constant<int, (WM == 16 ? 9 : WM)>{});
-    else if (live_tiles <= 10)
-      run(std::integral_constant<int, (WM == 16 ? 10 : WM)>{});
-    else if (live_tiles <= 12)
-      run(std::integral_constant<int, (WM == 16 ? 12 : WM)>{});
-    else if (live_tiles <= 14)
-      run(std::integral_constant<int, (WM == 16 ? 14 : WM)>{});
-    else
-      run(std::integral_constant<int, WM>{});
+  if (GROUPED) {
+    // expert blocks: an instance of the main loop for every number of row tiles that hold slots, from four (the depth
+    // of the fragment prefetch) to all of them.  What a padded row tile costs is not so much time in the loop as power
+    // - its MFMAs multiply real rows -, and the clock: at 128 slots per expert on average, instances over 9 and 10
+    // row tiles next to those over 8 and 12 took a tenth off the whole call.
+    for_tile_count<4, WM>(live_tiles, run);
   } else if (live_tiles <= WM / 2) {
     run(std::integral_constant<int, WM / 2>{});
   } else {
