@@ -229,16 +229,15 @@ KSQ_EXPORT size_t ksq_moe_fp8_block_m(size_t numel, size_t E) {
 
 // Rows per expert block for numel routed (token, slot) pairs over E experts.  Replaces the M thresholds of
 // InvokeFusedMoe (16 / 32 / 64 rows by token count): below about 40 rows per expert the weights are streamed once per
-// 16- or 32-row block (HBM-bound); above, 128-row blocks feed the MFMA tile kernel (E = 256, hidden 7168, inter 2048,
-// top-8: 2.52 against 2.70 ms at 32 rows per expert, 3.37 against 3.00 ms at 48).
+// 16- or 32-row block (HBM-bound); above, the MFMA tile kernel takes 256-row blocks, of which it multiplies the row
+// tiles that hold rows (an instance of its main loop per count), so that an expert's weights are dequantized once
+// however many of the 256 rows it fills.  E = 256, hidden 7168, inter 2048, top-8, whole call with 32- / 128- /
+// 256-row blocks: 1.97 / 2.34 / 2.37 ms at 32 rows per expert, 2.41 / 2.40 / 2.39 at 40, 2.58 / 2.46 / 2.45 at 48,
+// 3.21 / 2.60 / 2.55 at 64, 4.39 / 3.06 / 3.02 at 96, 4.96 / 3.44 / 3.30 at 112, 5.60 / 4.40 / 3.57 at 128.
 KSQ_EXPORT size_t ksq_moe_block_m(size_t numel, size_t E) {
   if (E == 0) return 16;
   const size_t per_expert = numel / E;
-  // 256-row blocks (the tile kernel multiplies the row tiles that hold rows, in steps of four) dequantize an expert's
-  // weights once where two 128-row blocks do it twice.  E = 256, hidden 7168, inter 2048, top-8, whole call, 128- against
-  // 256-row blocks: 3.56 / 3.58 ms at 112 rows per expert, 4.57 / 4.21 at 128, 5.91 / 5.06 at 192, 7.90 / 7.05 at 256
-  if (per_expert >= 120) return 256;
-  if (per_expert >= 40) return 128;
+  if (per_expert >= 40) return 256;
   return per_expert < 16 ? 16 : 32;
 }
 

@@ -614,7 +614,7 @@ static int RunErrors() {
     r = p;
     r[11] = std::string("tanh");
     expect(!f.Init(r, rc, context, 0).OK(), "unknown scoring function is rejected");
-    expect(ksq_moe_block_m(8 * 2, 8) == 16 && ksq_moe_block_m(64 * 2, 8) == 32 && ksq_moe_block_m(2048 * 8, 256) == 128 && ksq_moe_block_m(4096 * 8, 256) == 256,
+    expect(ksq_moe_block_m(8 * 2, 8) == 16 && ksq_moe_block_m(64 * 2, 8) == 32 && ksq_moe_block_m(1024 * 8, 256) == 32 && ksq_moe_block_m(2048 * 8, 256) == 256 && ksq_moe_block_m(4096 * 8, 256) == 256,
            "block_m thresholds");
   }
   // the Auto factories: what they derive and what they refuse

@@ -258,6 +258,25 @@ def test_grouped_gemm_stages(ops, oracle, dtype, T, bm):
     H.check_gemm(c3, ref3, dtype, "moe gemm2", weights_rounded=bm == 128)
 
 
+@pytest.mark.parametrize("dtype", [H.F16, H.BF16])
+@pytest.mark.parametrize("bm", [128, 256])
+def test_grouped_tile_kernel_every_count_of_live_row_tiles(ops, oracle, dtype, bm):
+    """The tile kernel has an instance of its main loop per number of row tiles that hold rows: experts with
+    16c - 5 rows for c = 4..16, and one with 3 rows, meet every instance of the 256-row form (and, cut into 128-row
+    blocks, of the 128-row form)."""
+    rows = [16 * c - 5 for c in range(4, 17)] + [3]
+    E, T = len(rows), sum(rows)
+    d = make_moe(oracle, 5900 + bm, E, 256, 128, T, 1, 128, dtype)
+    ids = torch.cat([torch.full((r,), e, dtype=torch.int32) for e, r in enumerate(rows)])
+    ids = ids[torch.randperm(T, generator=H.gen(77))].reshape(T, 1).contiguous()
+    w13p, s13p, _, _ = pack_moe(ops, d)
+    s, e, npp = ops.moe_align_block_size(ids.cuda(), E, bm)
+    c1 = ops.moe_w4a16_gemm(d["x"].cuda(), w13p, s13p, None, s, e, npp, T, 1, E, 2 * d["inter"], d["hidden"], 128, bm)
+    ref1 = oracle.moe_w4a16_gemm(H.bits_of(d["x"]), d["w13"].numpy(), H.bits_of(d["s13"]), ids.numpy(), d["tw"].numpy(), 1,
+                                 128, False, dtype)
+    H.check_gemm(c1, ref1, dtype, "grouped tile kernel, %d-row blocks" % bm, weights_rounded=True)
+
+
 @pytest.mark.parametrize("T", [1, 64, 2048])
 def test_moe_block_deepseek_shape(ops, oracle, T):
     """256 experts, hidden 7168, inter 2048, top-8; weights for all experts are generated but only touched ones
