@@ -283,15 +283,16 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
     return i32x8{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
   };
 
-  // one k-block: 32 MFMAs; the scale FMAs of MFMA j are placed after MFMA j+2 so that they run in its shadow, and the
-  // loads of k-block `next` (scales, then operands into the LDS slot the previous stage used) are issued after the
-  // first MFMA.
-  auto compute = [&](uint32_t slot, uint32_t kb, uint32_t next) {
-    float sc[WM];
+  // one k-block: WMV * 4 MFMAs (WMV = this wavefront's row tiles that hold tokens); the scale FMAs of MFMA j are placed
+  // after MFMA j+2 so that they run in its shadow, and the loads of k-block `next` (scales, then operands into the LDS
+  // slot the previous stage used) are issued after the first MFMA.
+  auto compute = [&](auto wmv_c, uint32_t slot, uint32_t kb, uint32_t next) {
+    constexpr int WMV = decltype(wmv_c)::value;
+    float sc[WMV];
     {
       const float bs = bs_lds[kb];
 #pragma unroll
-      for (int i = 0; i < WM; ++i) sc[i] = as_lds[slot * 256 + i * 16] * bs;
+      for (int i = 0; i < WMV; ++i) sc[i] = as_lds[slot * 256 + i * 16] * bs;
     }
     const char* act = lds + slot * STAGE_BYTES + (wm * WM) * FRAG;
     const char* wgt = lds + slot * STAGE_BYTES + (W_FRAG0 + wn * WN) * FRAG;
@@ -305,10 +306,10 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
     f32x4 tmp[3];
     const f32x4 zero{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int j = 0; j < WM * WN + 2; ++j) {
+    for (int j = 0; j < WMV * WN + 2; ++j) {
       const int i = j / WN, t = j % WN;
-      if (j < WM * WN) {
-        if (t == 0 && i + 1 < WM) af[(i + 1) & 1] = read_frag(act + (i + 1) * FRAG);
+      if (j < WMV * WN) {
+        if (t == 0 && i + 1 < WMV) af[(i + 1) & 1] = read_frag(act + (i + 1) * FRAG);
         tmp[j % 3] = mfma_fp8_k128(wf[t], af[i & 1], zero);
       }
       __builtin_amdgcn_sched_barrier(0x4);
@@ -338,15 +339,23 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
   wait_stage();
   __syncthreads();  // also publishes the weight-scale table written with ordinary stores above
 
-  for (uint32_t c = 0; c < kb_count; ++c) {
-    if (idle) {
+  // The main loop exists once per number of this wavefront's row tiles that hold tokens: a padded row tile costs its
+  // MFMAs' time on this SIMD and their power whether or not its results are stored.
+  if (idle) {
+    for (uint32_t c = 0; c < kb_count; ++c) {
       load_scales(c + NS - 1);
       load_operands(c + NS - 1);
-    } else {
-      compute(c % NS, c, c + NS - 1);
+      wait_stage();  // operands and scales of c+1
+      __builtin_amdgcn_s_barrier();
     }
-    wait_stage();  // operands and scales of c+1
-    __builtin_amdgcn_s_barrier();
+  } else {
+    for_tile_count<1, WM>(live_tiles - wm * WM, [&](auto wmv_c) {
+      for (uint32_t c = 0; c < kb_count; ++c) {
+        compute(wmv_c, c % NS, c, c + NS - 1);
+        wait_stage();  // operands and scales of c+1
+        __builtin_amdgcn_s_barrier();
+      }
+    });
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // drain the clamped prefetches before the LDS is released
 

@@ -7,6 +7,7 @@
 #include <atomic>
 #include <cstdarg>
 #include <cstdio>
+#include <type_traits>
 
 #include "ksq.h"
 
@@ -136,6 +137,19 @@ inline int allow_dynamic_lds(std::atomic<uint64_t>& done, const void* kernel, in
   if (e != hipSuccess) return fail(KSQ_ERR_LAUNCH, "hipFuncSetAttribute(LDS %d): %s", bytes, hipGetErrorString(e));
   done.fetch_or(bit, std::memory_order_release);
   return 0;
+}
+
+// f(integral_constant<N>) for the smallest N in LO..HI with count <= N (N = HI when there is none)
+template <int LO, int HI, typename F>
+__device__ __forceinline__ void for_tile_count(uint32_t count, F&& f) {
+  if constexpr (LO >= HI) {
+    f(std::integral_constant<int, HI>{});
+  } else {
+    if (count <= static_cast<uint32_t>(LO))
+      f(std::integral_constant<int, LO>{});
+    else
+      for_tile_count<LO + 1, HI>(count, f);
+  }
 }
 
 }  // namespace ksq

@@ -216,15 +216,18 @@ SplitKChoice select_w4a8_splitk(size_t m, size_t n) {
 using namespace ksq;
 
 // The same for block-fp8 experts (ksq_moe_fp8_blockwise_gemm): 16- and 32-row blocks stream through the split-K
-// kernel; from about 28 rows per expert the MFMA tile kernel is faster even with most of a 128-row block padding
-// (E = 256, hidden 7168, inter 2048, top-8: 2.63 against 3.24 ms at 32 rows per expert, 3.07 against 5.56 ms at 64),
-// and 256-row blocks take over where they fill (level at 256 rows per expert, 6 % ahead at 384).
+// kernel; from 16 rows per expert the MFMA tile kernel is faster even with most of a 128-row block padding (each of its
+// wavefronts multiplies the row tiles that hold rows), and 256-row blocks take over from 128 rows per expert, where an
+// expert would otherwise need a second block and its weights a second pass.  E = 256, hidden 7168, inter 2048, top-8,
+// whole call with 16- / 32- / 128- / 256-row blocks: 1.50 / 1.49 / 1.61 / - ms at 2 rows per expert, 1.85 / 1.84 /
+// 1.95 / - at 8, 2.08 / 1.94 / 1.97 / - at 12, 2.60 / 2.06 / 2.01 / 2.46 at 16, - / 3.21 / 2.16 / 2.46 at 32,
+// - / 5.51 / 2.37 / 2.66 at 64, - / 9.89 / 3.36 / 3.33 at 128, - / - / 4.23 / 3.84 at 192, - / - / 5.46 / 5.07 at 256.
 KSQ_EXPORT size_t ksq_moe_fp8_block_m(size_t numel, size_t E) {
   if (E == 0) return 16;
   const size_t per_expert = numel / E;
-  if (per_expert >= 256) return 256;
-  if (per_expert >= 28) return 128;
-  return per_expert < 8 ? 16 : 32;
+  if (per_expert >= 128) return 256;
+  if (per_expert >= 16) return 128;
+  return per_expert < 2 ? 16 : 32;
 }
 
 // Rows per expert block for numel routed (token, slot) pairs over E experts.  Replaces the M thresholds of

@@ -131,19 +131,6 @@ struct Dequant<BF16, HAS_ZP> {
   }
 };
 
-// f(integral_constant<N>) for the smallest N in LO..HI with count <= N (N = HI when there is none)
-template <int LO, int HI, typename F>
-__device__ __forceinline__ void for_tile_count(uint32_t count, F&& f) {
-  if constexpr (LO >= HI) {
-    f(std::integral_constant<int, HI>{});
-  } else {
-    if (count <= static_cast<uint32_t>(LO))
-      f(std::integral_constant<int, LO>{});
-    else
-      for_tile_count<LO + 1, HI>(count, f);
-  }
-}
-
 // One column tile's packed weights for one k-tile of 128, with the scale and zero point of each of its GPT groups.
 template <int GPT>
 struct WSlot {
