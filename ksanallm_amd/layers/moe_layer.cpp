@@ -237,8 +237,8 @@ Status MoeLayer::Forward(const std::vector<Tensor>& input_tensors, std::vector<T
       gemm1_in = act_order1;
       gemm1_topk = 1;
     }
-    // the activation runs in the first GEMM's epilogue, except with 128-row blocks, where the two launches measured
-    // faster (64 rows per expert: 1.75 against 1.87 ms; level from 128 rows per expert, where 256-row blocks are used)
+    // the activation runs in the first GEMM's epilogue, except with 128-row blocks (a size ksq_moe_block_m no longer
+    // picks but a caller may ask for), where the two launches measured faster (64 rows per expert: 1.75 against 1.87 ms)
     if (block_m != 128 && (2 * inter) % 32 == 0) {
       KsqCheck(ksq_moe_w4a16_gate_up_silu(cache2, gemm1_in, w1, w1_scale, nullptr, sorted_ids, expert_ids, num_post_pad,
                                           numel, gemm1_topk, E, 2 * inter, hidden_size, group_size_, block_m, dtype, stream),

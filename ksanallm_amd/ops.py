@@ -274,8 +274,8 @@ def fused_moe_w4a16(x, w13_packed, s13_packed, w2_packed, s2_packed, topk_ids, t
         block_m = _lib.ksq_moe_block_m(numel, E)
     sorted_ids, expert_ids, npp = moe_align_block_size(topk_ids, E, block_m)
     tw = topk_w.reshape(-1).to(torch.float32).contiguous()
-    # the activation runs in the first GEMM's epilogue, except with 128-row blocks, where the two launches measured
-    # faster (64 rows per expert: 1.75 against 1.87 ms; level from 128 rows per expert, where 256-row blocks are used)
+    # the activation runs in the first GEMM's epilogue, except with 128-row blocks (a size ksq_moe_block_m no longer
+    # picks but a caller may ask for), where the two launches measured faster (64 rows per expert: 1.75 against 1.87 ms)
     if block_m != 128 and (2 * inter) % 32 == 0:
         c2 = moe_w4a16_gate_up_silu(x, w13_packed, s13_packed, sorted_ids, expert_ids, npp, numel, topk, E, 2 * inter,
                                     hidden, group, block_m)

@@ -599,7 +599,7 @@ static int RunErrors() {
     expect(!b2.Init(q, rc, context, 0).OK(), "int4 weights with fp8 activations are rejected");
     q[18] = TYPE_INVALID;
     expect(b3.Init(q, rc, context, 0).OK(), "block-fp8 experts init");
-    expect(b3.GetWorkspaceSize() > 0 && b3.BlockM(4096) == 256 && b3.BlockM(64) == 32, "block-fp8 workspace and block size");
+    expect(b3.GetWorkspaceSize() > 0 && b3.BlockM(4096) == 256 && b3.BlockM(64) == 128 && b3.BlockM(32) == 32, "block-fp8 workspace and block size");
     auto r = p;
     r[9] = uint32_t(4);   // 4 groups of 2 experts, 2 kept: top-2 fits
     r[10] = uint32_t(2);
