@@ -336,10 +336,9 @@ __global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKPar
           const uint32_t voff = static_cast<uint32_t>(lane) * 16u < left_bytes ? static_cast<uint32_t>(lane) * 16u : 0u;
           const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_base + (c & 1u) * Lds::kChunkBytes + r * Lds::kRowStride + q * 1024u);
           // (s_nop 4: scalar operands that a v_readfirstlane produced need five wait states before a vector memory
-          // instruction reads them, and the compiler inserts none inside an assembly statement.  M0 is written here
-          // without being declared: the compiler treats it as a reserved register, rejects it in a clobber list with
-          // a warning, and keeps no value of its own in it across statements - it writes M0 right in front of each
-          // instruction of its own that reads it, and this kernel has none.)
+          // instruction reads them, and the compiler inserts none inside an assembly statement.  M0 is named as
+          // clobbered; the compiler treats it as a reserved register and keeps no value of its own in it across
+          // statements - it writes M0 right in front of each instruction of its own that reads it.)
           asm volatile("s_nop 4\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %2"
                        :
                        : "v"(voff), "s"(dst), "s"(src)
