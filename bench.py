@@ -81,6 +81,9 @@ def kernel_label(L, kind, prefix, M, N, K, dt):
 
 
 # ------------------------------------------------------------------------------------------------ workloads
+CONSTANT_DATA = False   # --constant-data: every weight code, scale and activation the same value (configs 1-4)
+
+
 def w4a16_cases(ops, L, cfg, shapes, Ms, dtype, awq, x_std, s_lo, s_hi):
     dev = "cuda"
     tdt = torch.float16 if dtype == "f16" else torch.bfloat16
@@ -97,6 +100,9 @@ def w4a16_cases(ops, L, cfg, shapes, Ms, dtype, awq, x_std, s_lo, s_hi):
             layout = L.SRC_GPTQ
         scales = (torch.rand((G, N), generator=g) * (s_hi - s_lo) + s_lo).to(tdt)
         zeros = torch.randint(6, 10, (G, N), generator=g, dtype=torch.uint8) if awq else None
+        if CONSTANT_DATA:   # the same instructions on operands that never toggle: what the data costs in clock
+            q = torch.full_like(q, 0x11111111 * 9 - 2**32)   # every code 9
+            scales = torch.full_like(scales, (s_lo + s_hi) / 2)
         wp1 = ops.repack_weight(q.to(dev), layout, 1, K, N)
         sp1 = ops.repack_scales(scales.to(dev), L.SCALE_GN, 1, K, N, 128)
         zp1 = ops.repack_zeros(awq_pack_cols(zeros).to(dev), L.ZERO_AWQ_PACKED, K, N, 128) if awq else None
@@ -109,6 +115,8 @@ def w4a16_cases(ops, L, cfg, shapes, Ms, dtype, awq, x_std, s_lo, s_hi):
         keep.append(rec)
         for mi, M in enumerate(Ms):
             x = (torch.randn((M, K), generator=seeded(cfg, 100 * si + mi + 10)) * x_std).to(tdt).to(dev)
+            if CONSTANT_DATA:
+                x = torch.full_like(x, x_std)
             y = torch.empty((M, N), dtype=tdt, device=dev)
             rec["x"][M], rec["y"][M] = x, y
             need = L.load().ksq_w4a16_workspace_size(M, N, K, 128, ldt)
@@ -132,6 +140,8 @@ def fp8_cases(ops, L, cfg, shapes, Ms):
         # e4m3 codes of bf16 N(0,0.02^2) weights under a per-128x128 amax/448 scale: drawn directly as the codes of
         # w/s with w/s ~ N(0, (448/4.2)^2) clipped to +-448 (amax of 16384 normals is about 4.2 sigma)
         wn = (torch.randn((N, K), generator=g) * (448.0 / 4.2)).clamp_(-448, 448)
+        if CONSTANT_DATA:
+            wn.fill_(112.0)
         b = wn.to(torch.float8_e4m3fn).view(torch.uint8)
         del wn
         b_s = torch.full(((N + 127) // 128, K // 128), 0.02 * 4.2 / 448.0, dtype=torch.float32)
@@ -146,6 +156,8 @@ def fp8_cases(ops, L, cfg, shapes, Ms):
             gx = seeded(cfg, 100 * si + mi + 10)
             x = torch.randn((M, K), generator=gx)
             x = torch.where(torch.rand((M, K), generator=gx) < 0.01, x * 20, x).to(torch.bfloat16).to(dev)
+            if CONSTANT_DATA:
+                x = torch.full_like(x, 1.0)
             a_q = torch.empty((M, K), dtype=torch.uint8, device=dev)
             a_s = torch.empty((K // 128, M), dtype=torch.float32, device=dev)
             y = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
@@ -189,6 +201,8 @@ def w4a8_cases(ops, L, cfg, shapes, Ms):
             gx = seeded(cfg, 100 * si + mi + 10)
             x = torch.randn((M, K), generator=gx)
             x = torch.where(torch.rand((M, K), generator=gx) < 0.01, x * 20, x).to(torch.bfloat16).to(dev)
+            if CONSTANT_DATA:
+                x = torch.full_like(x, 1.0)
             a_q = torch.empty((M, K), dtype=torch.uint8, device=dev)
             xsum = torch.empty((K // 128, M), dtype=torch.float32, device=dev)
             y = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
@@ -491,6 +505,8 @@ def library_gemm(steps, warmup):
             for m in (2048, 4096, 8192):
                 x = torch.randn(m, k, device="cuda", dtype=dt) * 0.5
                 w = torch.randn(n, k, device="cuda", dtype=dt) * 0.01
+                if CONSTANT_DATA:
+                    x, w = torch.full_like(x, 0.5), torch.full_like(w, 0.005)
                 us = timed(lambda: torch.matmul(x, w.t()))
                 tf = 2.0 * m * n * k / us / 1e6
                 rows.append({"m": m, "n": n, "k": k, "dtype": name, "us": round(us, 1), "tflops": round(tf, 1),
@@ -499,6 +515,9 @@ def library_gemm(steps, warmup):
         for m in (1024, 4096):
             x = torch.randn(m, k, device="cuda").to(torch.float8_e4m3fn)
             w = torch.randn(n, k, device="cuda").to(torch.float8_e4m3fn)
+            if CONSTANT_DATA:
+                x = torch.full((m, k), 0.5, device="cuda").to(torch.float8_e4m3fn)
+                w = torch.full((n, k), 0.5, device="cuda").to(torch.float8_e4m3fn)
             for scaling, sa, sb in (("per tensor", torch.ones((), device="cuda"), torch.ones((), device="cuda")),
                                     ("per row", torch.ones(m, 1, device="cuda"), torch.ones(1, n, device="cuda"))):
                 us = timed(lambda: torch._scaled_mm(x, w.t(), scale_a=sa, scale_b=sb, out_dtype=torch.bfloat16))
@@ -526,6 +545,9 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true", help="run only a 256 MiB device-to-device copy a few "
                     "times (the known-size kernel hardware traffic counters are scaled by) and exit")
     ap.add_argument("--details", action="store_true", help="also print a per-case table to stderr")
+    ap.add_argument("--constant-data", action="store_true", help="dense W4A16 and block-fp8 cases: every weight code, every scale and every "
+                    "activation holds one value (a valid GEMM on operands that never toggle), to show how much of the "
+                    "kernel's time is the clock the data allows; not a benchmark figure")
     ap.add_argument("--library-gemm", action="store_true", help="run only the vendor library's plain GEMMs (torch.matmul "
                     "fp16 / bf16, torch._scaled_mm e4m3; no dequantization, no block scales) at the prefill shapes of "
                     "configurations 3 and 4 and exit: what a dense GEMM reaches on this part, beside the MFMA peak")
@@ -546,6 +568,8 @@ def main():
         print(json.dumps({"copy_bytes_read": n, "copy_bytes_written": n, "launches": 5}))
         return
 
+    global CONSTANT_DATA
+    CONSTANT_DATA = args.constant_data
     if args.library_gemm:
         library_gemm(args.steps, args.warmup)
         return
@@ -681,7 +705,7 @@ def main():
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16 / bf16 / fp8-e4m3 by configuration, fp32 accumulation" if whole else DTYPES[cfgs[0]],
-        "data": "synthetic",
+        "data": "synthetic, one constant value per operand (--constant-data)" if CONSTANT_DATA else "synthetic",
         "config": {"workload": workload, "cases": len(cases), "configs": cfgs},
         "tflops": round(total_flops / step_s / 1e12, 3), "hbm_gbps": round(total_bytes / step_s / 1e9, 1),
         "wall_ms_per_step": round(wall_ms, 5), "launch": "hip graph replay" if use_graph else "python launches",

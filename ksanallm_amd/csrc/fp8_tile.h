@@ -251,6 +251,9 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
   // (vmcnt retires in issue order; a wavefront issues the same loads every stage: 8 weight loads, or 2*AFW activation
   // loads with or without the one scale load in front of them).
   const bool has_scale_load = s_vec ? wave == 0 : wave < BM / 64;
+  // This wavefront's fragment reads of the stage have returned: behind the barrier other wavefronts refill the slot they
+  // came from, and a bare s_barrier waits for nothing by itself.
+  auto reads_done = [&]() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); };
   auto wait_stage = [&]() {
     if (NS == 2) {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -346,6 +349,7 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
       load_scales(c + NS - 1);
       load_operands(c + NS - 1);
       wait_stage();  // operands and scales of c+1
+      reads_done();
       __builtin_amdgcn_s_barrier();
     }
   } else {
@@ -353,6 +357,7 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
       for (uint32_t c = 0; c < kb_count; ++c) {
         compute(wmv_c, c % NS, c, c + NS - 1);
         wait_stage();  // operands and scales of c+1
+        reads_done();
         __builtin_amdgcn_s_barrier();
       }
     });

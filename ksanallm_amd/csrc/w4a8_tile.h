@@ -231,6 +231,9 @@ __global__ void __launch_bounds__(512, 1) w4a8_tile_kernel(W4A8TileParams p) {
   // Everything this wavefront issued has landed except the loads of the youngest stage (vmcnt retires in issue order;
   // a wavefront issues the same loads every stage: 4 weight loads with or without the weight-scale load, or 2*AFW
   // activation loads with or without the group-sum load).
+  // This wavefront's fragment reads of the stage have returned: behind the barrier other wavefronts refill the slot they
+  // came from, and a bare s_barrier waits for nothing by itself.
+  auto reads_done = [&]() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); };
   auto wait_stage = [&]() {
     if (!stage_act) {
       if (wave == 4)
@@ -379,6 +382,7 @@ __global__ void __launch_bounds__(512, 1) w4a8_tile_kernel(W4A8TileParams p) {
       compute(c % NS, c + NS - 1);
     }
     wait_stage();  // operands and scales of c+1
+    reads_done();
     __builtin_amdgcn_s_barrier();
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // drain the clamped prefetches before the LDS is released
