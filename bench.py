@@ -10,6 +10,10 @@ its weights in the 256 MB Infinity Cache.
 
 Prints ONE JSON line.  `value` is the time-weighted fraction of the MI355X roofline over the step, in percent:
 sum over cases of max(bytes / 8 TB/s, flops / MFMA peak) divided by the measured step time.
+
+Two side measurements, neither a benchmark figure: `--library-gemm` times the vendor library's plain GEMMs at the
+prefill shapes, and `--constant-data` gives every operand of the dense cases one value (the same kernels and cycle
+counts at the clock that operands which never toggle allow).
 """
 import argparse
 import json
