@@ -354,6 +354,31 @@ def test_grouped_fp8_gemm_stage(ops, oracle, T, E, topk, n, k, bm, colmajor, wit
     H.check_gemm(out, ref, H.BF16, "grouped fp8 T=%d n=%d k=%d" % (T, n, k))
 
 
+@pytest.mark.parametrize("bm", [128, 256])
+def test_grouped_fp8_tile_kernel_every_count_of_live_row_tiles(ops, oracle, bm):
+    """Every wavefront of the fp8 tile kernel has an instance of its main loop per number of its row tiles that hold
+    tokens: experts with 16c - 5 slots for c = 1..16 meet every count of the lower and of the upper wavefronts of a
+    256-slot block (cut into 128-slot blocks: of that form)."""
+    rows = [16 * c - 5 for c in range(1, 17)]
+    E, T, n, k = len(rows), sum(rows), 256, 384
+    g = H.gen(7700 + bm)
+    bq, bs = _fp8_experts(oracle, 7710, E, n, k)
+    x = torch.randn((T, k), generator=g).to(torch.bfloat16)
+    ids = torch.cat([torch.full((r,), e, dtype=torch.int32) for e, r in enumerate(rows)])
+    ids = ids[torch.randperm(T, generator=g)].reshape(T, 1).contiguous()
+    q, s = ops.per_token_group_quant_fp8(x.cuda(), k, 128, False)
+    sorted_ids, expert_ids, npp = ops.moe_align_block_size(ids.cuda(), E, bm)
+    out = ops.moe_fp8_blockwise_gemm(q, s, False, ops.fp8_repack_weight(torch.from_numpy(bq).cuda()), torch.from_numpy(bs).cuda(),
+                                     None, sorted_ids, expert_ids, npp, T, 1, bm, torch.bfloat16)
+    qh, sh = q.cpu().numpy(), s.cpu().numpy()
+    ref = np.zeros((T, n), np.float32)
+    flat = ids.reshape(-1).numpy()
+    for e in range(E):
+        slots = np.nonzero(flat == e)[0]
+        ref[slots] = oracle.fp8_blockwise_gemm(qh[slots], np.ascontiguousarray(sh[slots]), bq[e], bs[e], False)
+    H.check_gemm(out, ref, H.BF16, "grouped fp8 tile kernel, %d-slot blocks" % bm)
+
+
 @pytest.mark.parametrize("dtype", [H.F16, H.BF16])
 @pytest.mark.parametrize("T,E,topk,hidden,inter", [(1, 8, 2, 256, 128), (48, 16, 4, 512, 256), (200, 8, 2, 384, 640),
                                                    (1200, 8, 2, 512, 256)])   # the last: 300 slots per expert, 256-slot blocks
