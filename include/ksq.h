@@ -256,8 +256,9 @@ int ksq_moe_align(const void* topk_ids, size_t numel, size_t E, size_t block_m, 
  *   out[s, :] = x[s / top_k, :] . dequant(W[expert of s's block]) * (topk_w ? topk_w[s] : 1)
  * x [rows, k] T, out [numel, n] T, W/scales packed per expert as by ksq_w4a16_repack(E = experts),
  * zeros_packed NULL for symmetric (code-8).  top_k = 1 reads x rows by slot (second MoE GEMM).
- * block_m is the block size the permutation was aligned with: 16 or 32 run the streaming (decode) kernel, 128 the MFMA
- * tile kernel; ksq_moe_block_m() gives the choice for a problem size.
+ * block_m is the block size the permutation was aligned with: 16 or 32 run the streaming (decode) kernel, 128 or 256
+ * the MFMA tile kernel (which multiplies only the 16-row tiles of a block that hold rows); ksq_moe_block_m() gives the
+ * choice for a problem size.
  * Replaces InvokeMoeWna16Gemm (K/moe/moe_wna16/moe_wna16.cu:263-288) and the Triton
  * InvokeFusedMoeGptqAwqKernel (S/kernels/nvidia/triton_wrapper.h:68-75). */
 size_t ksq_moe_block_m(size_t numel, size_t E);
