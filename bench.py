@@ -85,7 +85,7 @@ def kernel_label(L, kind, prefix, M, N, K, dt):
 
 
 # ------------------------------------------------------------------------------------------------ workloads
-CONSTANT_DATA = False   # --constant-data: every weight code, scale and activation the same value (configs 1-4)
+CONSTANT_DATA = ""   # --constant-data: "all", "weights" or "activations" hold one value each (configs 1-4)
 
 
 def w4a16_cases(ops, L, cfg, shapes, Ms, dtype, awq, x_std, s_lo, s_hi):
@@ -104,7 +104,7 @@ def w4a16_cases(ops, L, cfg, shapes, Ms, dtype, awq, x_std, s_lo, s_hi):
             layout = L.SRC_GPTQ
         scales = (torch.rand((G, N), generator=g) * (s_hi - s_lo) + s_lo).to(tdt)
         zeros = torch.randint(6, 10, (G, N), generator=g, dtype=torch.uint8) if awq else None
-        if CONSTANT_DATA:   # the same instructions on operands that never toggle: what the data costs in clock
+        if CONSTANT_DATA in ("all", "weights"):   # the same instructions on operands that never toggle
             q = torch.full_like(q, 0x11111111 * 9 - 2**32)   # every code 9
             scales = torch.full_like(scales, (s_lo + s_hi) / 2)
         wp1 = ops.repack_weight(q.to(dev), layout, 1, K, N)
@@ -119,7 +119,7 @@ def w4a16_cases(ops, L, cfg, shapes, Ms, dtype, awq, x_std, s_lo, s_hi):
         keep.append(rec)
         for mi, M in enumerate(Ms):
             x = (torch.randn((M, K), generator=seeded(cfg, 100 * si + mi + 10)) * x_std).to(tdt).to(dev)
-            if CONSTANT_DATA:
+            if CONSTANT_DATA in ("all", "activations"):
                 x = torch.full_like(x, x_std)
             y = torch.empty((M, N), dtype=tdt, device=dev)
             rec["x"][M], rec["y"][M] = x, y
@@ -144,7 +144,7 @@ def fp8_cases(ops, L, cfg, shapes, Ms):
         # e4m3 codes of bf16 N(0,0.02^2) weights under a per-128x128 amax/448 scale: drawn directly as the codes of
         # w/s with w/s ~ N(0, (448/4.2)^2) clipped to +-448 (amax of 16384 normals is about 4.2 sigma)
         wn = (torch.randn((N, K), generator=g) * (448.0 / 4.2)).clamp_(-448, 448)
-        if CONSTANT_DATA:
+        if CONSTANT_DATA in ("all", "weights"):
             wn.fill_(112.0)
         b = wn.to(torch.float8_e4m3fn).view(torch.uint8)
         del wn
@@ -160,7 +160,7 @@ def fp8_cases(ops, L, cfg, shapes, Ms):
             gx = seeded(cfg, 100 * si + mi + 10)
             x = torch.randn((M, K), generator=gx)
             x = torch.where(torch.rand((M, K), generator=gx) < 0.01, x * 20, x).to(torch.bfloat16).to(dev)
-            if CONSTANT_DATA:
+            if CONSTANT_DATA in ("all", "activations"):
                 x = torch.full_like(x, 1.0)
             a_q = torch.empty((M, K), dtype=torch.uint8, device=dev)
             a_s = torch.empty((K // 128, M), dtype=torch.float32, device=dev)
@@ -205,7 +205,7 @@ def w4a8_cases(ops, L, cfg, shapes, Ms):
             gx = seeded(cfg, 100 * si + mi + 10)
             x = torch.randn((M, K), generator=gx)
             x = torch.where(torch.rand((M, K), generator=gx) < 0.01, x * 20, x).to(torch.bfloat16).to(dev)
-            if CONSTANT_DATA:
+            if CONSTANT_DATA in ("all", "activations"):
                 x = torch.full_like(x, 1.0)
             a_q = torch.empty((M, K), dtype=torch.uint8, device=dev)
             xsum = torch.empty((K // 128, M), dtype=torch.float32, device=dev)
@@ -549,8 +549,9 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true", help="run only a 256 MiB device-to-device copy a few "
                     "times (the known-size kernel hardware traffic counters are scaled by) and exit")
     ap.add_argument("--details", action="store_true", help="also print a per-case table to stderr")
-    ap.add_argument("--constant-data", action="store_true", help="dense W4A16 and block-fp8 cases: every weight code, every scale and every "
-                    "activation holds one value (a valid GEMM on operands that never toggle), to show how much of the "
+    ap.add_argument("--constant-data", nargs="?", const="all", default="", choices=["all", "weights", "activations"],
+                    help="dense W4A16 and block-fp8 cases: every weight code and scale, every activation, or both (the "
+                    "default) hold one value (a valid GEMM on operands that never toggle), to show how much of the "
                     "kernel's time is the clock the data allows; not a benchmark figure")
     ap.add_argument("--library-gemm", action="store_true", help="run only the vendor library's plain GEMMs (torch.matmul "
                     "fp16 / bf16, torch._scaled_mm e4m3; no dequantization, no block scales) at the prefill shapes of "
@@ -709,7 +710,7 @@ def main():
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16 / bf16 / fp8-e4m3 by configuration, fp32 accumulation" if whole else DTYPES[cfgs[0]],
-        "data": "synthetic, one constant value per operand (--constant-data)" if CONSTANT_DATA else "synthetic",
+        "data": "synthetic, constant %s (--constant-data)" % CONSTANT_DATA if CONSTANT_DATA else "synthetic",
         "config": {"workload": workload, "cases": len(cases), "configs": cfgs},
         "tflops": round(total_flops / step_s / 1e12, 3), "hbm_gbps": round(total_bytes / step_s / 1e9, 1),
         "wall_ms_per_step": round(wall_ms, 5), "launch": "hip graph replay" if use_graph else "python launches",
