@@ -144,6 +144,26 @@ def test_blockwise_gemm_benchmark_shapes(ops, oracle, m, n, k):
     H.check_gemm(out, ref, H.BF16, "fp8 cfg4 m=%d n=%d k=%d" % (m, n, k))
 
 
+# the same two shapes at the benchmark's prefill row counts: the GPU multiplies all rows, the oracle the first 128 of
+# them (rows are independent in the quantizer and in the GEMM), from the very codes and scales the GPU produced
+@pytest.mark.parametrize("m", [1024, 4096])
+@pytest.mark.parametrize("n,k", [(18432, 7168), (7168, 18432)])
+def test_blockwise_gemm_benchmark_shapes_prefill_rows(ops, oracle, m, n, k):
+    rows = 128
+    x, bq, bs = make_fp8_problem(oracle, 4170 + m + n, m, n, k)
+    q, s = ops.per_token_group_quant_fp8(x.cuda(), k, 128, True)
+    qo, so = oracle.fp8_group_quant(H.bits_of(x[:rows]), k, 128, True, False, H.BF16)
+    np.testing.assert_array_equal(q[:rows].cpu().numpy(), qo)
+    np.testing.assert_array_equal(s[:, :rows].cpu().numpy().view(np.uint32), so.view(np.uint32))
+    out = ops.fp8_blockwise_gemm(q, s, packed(ops, bq), torch.from_numpy(bs).cuda(), torch.bfloat16)
+    ref = oracle.fp8_blockwise_gemm(qo, so, bq, bs, True)
+    H.check_gemm(out[:rows], ref, H.BF16, "fp8 cfg4 m=%d n=%d k=%d, rows 0..%d" % (m, n, k, rows - 1))
+    # and the last rows, which the last row tile and (at n = 7168) the cut tiles of the tail hold
+    qo, so = oracle.fp8_group_quant(H.bits_of(x[m - 32:]), k, 128, True, False, H.BF16)
+    ref = oracle.fp8_blockwise_gemm(qo, so, bq, bs, True)
+    H.check_gemm(out[m - 32:], ref, H.BF16, "fp8 cfg4 m=%d n=%d k=%d, last 32 rows" % (m, n, k))
+
+
 # prefill regime (MFMA tile kernel, 256 x 256 or 128 x 256 tiles): ragged M and N, odd k-block counts, split-K through
 # the workspace
 # (the last three: more than 32 tiles of 256 tokens, which is where the planner keeps that tile at these sizes)

@@ -307,6 +307,34 @@ def test_moe_block_deepseek_shape(ops, oracle, T):
                  rel_l2_max=5e-3 * (2 ** 0.5 if rounded else 1.0))
 
 
+@pytest.mark.parametrize("T", [512, 4096])
+def test_moe_block_benchmark_token_counts(ops, oracle, T):
+    """The benchmark's two larger token counts at its own shapes (256 experts, hidden 7168, inter 2048, top-8): the GPU
+    runs the whole block, the oracle the first 8 and the last 4 tokens of it (a token's output depends on its own
+    row, experts and routing weights only)."""
+    E, hidden, inter, topk = 256, 7168, 2048, 8
+    base = make_moe(oracle, 5200 + T, 8, hidden, inter, T, topk, 128, H.BF16)
+    rep = E // 8
+    d = dict(base)
+    d["E"] = E
+    for k in ("w13", "w2", "s13", "s2"):
+        d[k] = base[k].repeat((rep, 1, 1))
+    logits = torch.randn((T, E), generator=H.gen(78 + T))
+    tw, ids = torch.topk(torch.softmax(logits, -1), topk, dim=-1)
+    d["ids"], d["tw"] = ids.to(torch.int32), tw.float().contiguous()
+    w13p, s13p, w2p, s2p = pack_moe(ops, d)
+    out = ops.fused_moe_w4a16(d["x"].cuda(), w13p, s13p, w2p, s2p, d["ids"].cuda(), d["tw"].cuda(), E, hidden, inter,
+                              128)
+    from ksanallm_amd import lib as L
+    rounded = L.load().ksq_moe_block_m(T * topk, E) >= 128
+    for sel in (slice(0, 8), slice(T - 4, T)):
+        ref = oracle.moe_forward(H.bits_of(d["x"][sel]), d["w13"].numpy(), H.bits_of(d["s13"]), d["w2"].numpy(),
+                                 H.bits_of(d["s2"]), d["ids"][sel].contiguous().numpy(), d["tw"][sel].contiguous().numpy(),
+                                 128, H.BF16)
+        H.check_gemm(out[sel], oracle.from_bits(ref, H.BF16), H.BF16, "moe block T=%d tokens %s" % (T, sel),
+                     weights_rounded=rounded, rel_l2_max=5e-3 * (2 ** 0.5 if rounded else 1.0))
+
+
 # ---- block-quantized fp8 experts -------------------------------------------------------------------------------------
 
 def _fp8_experts(oracle, seed, E, n, k):

@@ -330,3 +330,19 @@ def test_prefill_full_size_properties_8192_rows(ops):
     y2 = ops.w4a16_gemm(x * 2, wp, sp, None, N, K, 128)
     normal = y.abs() >= 2.0 ** -13
     assert torch.equal(y2[normal], (y * 2)[normal])
+
+
+# the other prefill cases of the benchmark: the first 128 and the last 32 rows against the oracle
+@pytest.mark.parametrize("M,N,K", [(4096, 25600, 5120), (4096, 5120, 25600), (8192, 5120, 25600), (2048, 5120, 25600)])
+def test_cfg3_prefill_row_counts_first_and_last_rows(ops, M, N, K):
+    from ksanallm_amd import lib as L
+    d = H.make_w4a16(4500 + M + N, 160, N, K, 128, H.F16, awq=False, x_std=0.5, s_lo=0.002, s_hi=0.01)
+    wp = ops.repack_weight(d["qweight"].cuda(), L.SRC_GPTQ, 1, K, N)
+    sp = ops.repack_scales(d["scales"].cuda(), L.SCALE_GN, 1, K, N, 128)
+    x = (torch.randn((M, K), generator=H.gen(4501)) * 0.5).to(torch.float16)
+    x[:128] = d["x"][:128]
+    x[M - 32:] = d["x"][128:]
+    y = ops.w4a16_gemm(x.cuda(), wp, sp, None, N, K, 128)
+    ref = H.w4a16_oracle(d)
+    H.check_gemm(y[:128], ref[:128], H.F16, "cfg3 M=%d N=%d, rows 0..127" % (M, N), weights_rounded=True)
+    H.check_gemm(y[M - 32:], ref[128:], H.F16, "cfg3 M=%d N=%d, last 32 rows" % (M, N), weights_rounded=True)
