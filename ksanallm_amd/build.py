@@ -20,7 +20,55 @@ FLAGS = [
     # the assembly statements that write M0 say so in their clobber lists; the compiler answers that M0 is a reserved
     # register (it never keeps a value of its own there across a statement), once per instantiation
     "-Wno-inline-asm",
+    # one remark block per kernel with its registers, spills, scratch and LDS: read by check_resources below
+    "-Rpass-analysis=kernel-resource-usage",
 ]
+
+# The tile and streaming kernels issue their loads from inline assembly and count them by hand (`s_waitcnt vmcnt(N)`
+# with a constant N); a register that an assembly load has been issued into must stay where it is until the wait that
+# makes it valid.  A spill breaks that silently (the spilled copy is taken before the data has arrived), and scratch
+# memory of any kind adds vector memory operations that the hand-kept counts do not know.  So the build refuses a
+# kernel of these families that spills, uses scratch memory, or asks for more static LDS than a CU has.
+GUARDED_KERNELS = ("_tile_kernel", "_splitk_kernel")
+LDS_LIMIT = 160 * 1024
+
+
+def parse_resource_remarks(text):
+    """{kernel symbol: {"vgprs", "agprs", "sgprs", "scratch", "sgpr_spill", "vgpr_spill", "lds"}} from the compiler's
+    kernel-resource-usage remarks."""
+    import re
+    keys = {"TotalSGPRs": "sgprs", "VGPRs": "vgprs", "AGPRs": "agprs", "ScratchSize [bytes/lane]": "scratch",
+            "SGPRs Spill": "sgpr_spill", "VGPRs Spill": "vgpr_spill", "LDS Size [bytes/block]": "lds"}
+    out, cur = {}, None
+    for line in text.splitlines():
+        m = re.search(r"remark:\s+(.*?)\s*\[-Rpass-analysis=kernel-resource-usage\]", line)
+        if not m:
+            continue
+        body = m.group(1)
+        if body.startswith("Function Name:"):
+            cur = out.setdefault(body.split(":", 1)[1].strip(), {})
+        elif cur is not None and ":" in body:
+            k, v = body.rsplit(":", 1)
+            if k.strip() in keys and v.strip().lstrip("-").isdigit():
+                cur[keys[k.strip()]] = int(v)
+    return out
+
+
+def check_resources(text, src=""):
+    """Raises if a guarded kernel spills, uses scratch memory or exceeds the LDS; returns the parsed table."""
+    table = parse_resource_remarks(text)
+    bad = []
+    for name, r in table.items():
+        if not any(g in name for g in GUARDED_KERNELS):
+            continue
+        # (scalar registers spill into lanes of a vector register, not into memory: slower, not unsafe)
+        if r.get("scratch", 0) or r.get("vgpr_spill", 0) or r.get("lds", 0) > LDS_LIMIT:
+            bad.append("%s: scratch %d B/lane, VGPR spills %d, SGPR spills %d, LDS %d B" % (
+                name, r.get("scratch", 0), r.get("vgpr_spill", 0), r.get("sgpr_spill", 0), r.get("lds", 0)))
+    if bad:
+        raise RuntimeError("kernels with hand-counted load pipelines must not spill or use scratch memory (%s):\n  %s"
+                           % (src, "\n  ".join(bad)))
+    return table
 
 
 def sources():
@@ -34,7 +82,11 @@ def _compile(src):
     err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
     if r.returncode != 0:
         raise RuntimeError("hipcc failed for %s:\n%s" % (src, err))
-    return obj, err
+    check_resources(r.stderr, src)
+    # the remarks (and the source lines the compiler quotes under them) are for the check, not for the reader
+    if "warning:" not in err and "error:" not in err:
+        return obj, ""
+    return obj, "\n".join(l for l in err.splitlines() if "-Rpass-analysis=kernel-resource-usage" not in l)
 
 
 def build(verbose=False, jobs=None):

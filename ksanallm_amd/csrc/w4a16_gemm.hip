@@ -20,8 +20,11 @@ int launch_splitk(const SplitKParams& p, uint32_t m_blocks, hipStream_t s) {
   // (32-row blocks with four column tiles: two k-tiles ahead in the dense form, 12.9 against 14.0 us at n = 14336,
   // k = 4096; the grouped form measured 4 % slower with it and keeps one)
   // (the forms that stage x through LDS keep one k-tile in flight per wavefront: twice the wavefronts instead)
+  // (two row tiles, eight column tiles and zero points in the register form: a ring of two does not fit the registers)
   constexpr int LOOK = XC > 0 ? 1
-                              : (GROUP != 128 ? 2 : (MT == 1 ? (NT == 1 ? 4 : (NT == 2 ? 3 : 2)) : ((NT <= 2 || !GROUPED) ? 2 : 1)));
+                              : (GROUP != 128 ? 2
+                                              : (MT == 1 ? (NT == 1 ? 4 : (NT == 2 ? 3 : 2))
+                                                         : ((NT <= 2 || (!GROUPED && !(NT == 8 && HAS_ZP))) ? 2 : 1)));
   constexpr int OCC = XC > 0 ? ((MT == 1 && NT == 4) ? 4 : 2)
                              : ((GROUP == 128 && MT == 1 && NT == 1) ? 4 : ((GROUP == 128 && MT == 1 && NT == 2) ? 3 : 2));
   typedef SplitKLds<MT, NT, WAVES, XC> Lds;
