@@ -146,6 +146,14 @@ int ksq_w4a16_gemm(void* y, const void* x, const void* w_packed, const void* sca
                    void* workspace, size_t workspace_bytes, size_t m, size_t n, size_t k, size_t group, int dtype,
                    void* stream);
 
+/* The same call - same kernels, same plan, same workspace - with the fp32 sums stored as they are: y is [m, n] float
+ * (16-byte aligned) and nothing is rounded to T.  For verification: what separates a result from the fp32-accumulated
+ * dequantize-then-GEMM reference before the output type's own rounding is added.  The reference keeps the same notion
+ * in Marlin's fp32 reduce buffer (c_tmp, K/gptq_marlin/gptq_marlin.cu:610-638), without an entry point for it. */
+int ksq_w4a16_gemm_f32(float* y, const void* x, const void* w_packed, const void* scales_packed, const void* zeros_packed,
+                       void* workspace, size_t workspace_bytes, size_t m, size_t n, size_t k, size_t group, int dtype,
+                       void* stream);
+
 /* The same GEMM without a workspace argument, for callers that cannot allocate or hold device memory of their own at
  * the call site: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
  * counterpart in the reference.  The fp32 partial sums of launches that cut K go through a buffer of
@@ -179,6 +187,11 @@ int ksq_fp8_group_quant(const void* x, void* q, void* s, size_t m, size_t k, siz
 size_t ksq_fp8_blockwise_workspace_size(size_t max_m, size_t n, size_t k);
 int ksq_fp8_blockwise_gemm(const void* a_q, const void* a_s, const void* b, const void* b_s, void* out, size_t m,
                            size_t n, size_t k, int out_dtype, void* workspace, size_t workspace_bytes, void* stream);
+/* The same call with the fp32 sums stored as they are (out [m, n] float, 16-byte aligned): for verification, as
+ * ksq_w4a16_gemm_f32.  The reference's own check of this GEMM compares against a host loop that keeps fp32 throughout
+ * (K/blockwise_gemm/blockwise_gemm_test.cu:138-177). */
+int ksq_fp8_blockwise_gemm_f32(const void* a_q, const void* a_s, const void* b, const void* b_s, float* out, size_t m,
+                               size_t n, size_t k, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------------------------------------------------
  * Per-tensor / per-channel FP8: x [channels, size] T -> q e4m3 with one fp32 scale per channel (channels = 1: per tensor).

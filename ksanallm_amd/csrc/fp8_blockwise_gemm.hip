@@ -26,6 +26,7 @@ struct Fp8Params {
   const float* b_s;   // [ceil(n/128), k/128]
   void* out;          // [m, n]
   uint32_t M, N, K;
+  float* out32;       // dense form, verification only: the fp32 sums go here, [m, n], and nothing is rounded to TO
   uint32_t as_row_stride, as_kb_stride;  // a_s[row * as_row_stride + kb * as_kb_stride]: (1, M) in the dense form
   // grouped (MoE) form: row block b holds the slots sorted_ids[b*16*MT ..] of expert expert_ids[b]
   const int32_t* sorted_ids;
@@ -182,7 +183,9 @@ __global__ void __launch_bounds__(WAVES * 64) fp8_splitk_kernel(Fp8Params p) {
       row = sid;
       v *= mt ? erw1 : erw0;
     }
-    if (live) {
+    if (live && !GROUPED && p.out32) {
+      *reinterpret_cast<f32x4*>(p.out32 + static_cast<size_t>(row) * p.N + n0 + nt * 16 + 4 * (l >> 4)) = v;
+    } else if (live) {
       u32x2 o;
       o.x = pack2(TO::from_float(v[0]), TO::from_float(v[1]));
       o.y = pack2(TO::from_float(v[2]), TO::from_float(v[3]));
@@ -252,6 +255,7 @@ int launch_fp8_tile(const Fp8Params& q, const TilePlan& plan, float* partial, hi
   p.b = q.b;
   p.b_s = q.b_s;
   p.out = q.out;
+  p.out32 = q.out32;
   p.partial = partial;
   p.M = q.M;
   p.N = q.N;
@@ -267,7 +271,7 @@ int launch_fp8_tile(const Fp8Params& q, const TilePlan& plan, float* partial, hi
   if (plan.splits > 1) {
     const unsigned cut = plan.tiles_m * plan.tiles_n - plan.main_items;
     splitk_reduce_kernel<TO, 32 * WM><<<cut * (4 * WM), 256, 0, s>>>(partial, static_cast<uint16_t*>(p.out), p.M, p.N, p.tiles_m,
-                                                                    p.tiles_n, p.main_items, p.splits);
+                                                                    p.tiles_n, p.main_items, p.splits, p.out32);
   }
   return KSQ_OK;
 }
@@ -338,10 +342,13 @@ KSQ_EXPORT size_t ksq_fp8_blockwise_workspace_size(size_t max_m, size_t n, size_
   return need;
 }
 
-KSQ_EXPORT int ksq_fp8_blockwise_gemm(const void* a_q, const void* a_s, const void* b, const void* b_s, void* out,
-                                      size_t m, size_t n, size_t k, int out_dtype, void* workspace,
-                                      size_t workspace_bytes, void* stream) {
-  const char* fn = "ksq_fp8_blockwise_gemm";
+namespace {
+// out32 given (verification entry point): the same kernels under the same plan, with the fp32 sums stored to out32
+// [m, n] instead of rounded into out (which is then not touched)
+int fp8_blockwise_gemm_impl(const char* fn, const void* a_q, const void* a_s, const void* b, const void* b_s, void* out,
+                            size_t m, size_t n, size_t k, int out_dtype, void* workspace, size_t workspace_bytes,
+                            void* stream, float* out32) {
+  if (out32) out = out32;
   if (!a_q || !a_s || !b || !b_s || !out) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: null pointer", fn);
   if (!aligned16(a_q) || !aligned16(b) || !aligned16(out) || (reinterpret_cast<uintptr_t>(a_s) & 3u) ||
       (reinterpret_cast<uintptr_t>(b_s) & 3u))
@@ -357,6 +364,7 @@ KSQ_EXPORT int ksq_fp8_blockwise_gemm(const void* a_q, const void* a_s, const vo
   Fp8Params p{static_cast<const uint8_t*>(a_q), static_cast<const float*>(a_s), static_cast<const uint8_t*>(b),
               static_cast<const float*>(b_s), out, static_cast<uint32_t>(m), static_cast<uint32_t>(n),
               static_cast<uint32_t>(k)};
+  p.out32 = out32;
   p.as_row_stride = 1;
   p.as_kb_stride = static_cast<uint32_t>(m);
   int rc;
@@ -378,6 +386,21 @@ KSQ_EXPORT int ksq_fp8_blockwise_gemm(const void* a_q, const void* a_s, const vo
   }
   if (rc) return rc;
   return check_launch(fn);
+}
+}  // namespace
+
+KSQ_EXPORT int ksq_fp8_blockwise_gemm(const void* a_q, const void* a_s, const void* b, const void* b_s, void* out,
+                                      size_t m, size_t n, size_t k, int out_dtype, void* workspace,
+                                      size_t workspace_bytes, void* stream) {
+  return fp8_blockwise_gemm_impl("ksq_fp8_blockwise_gemm", a_q, a_s, b, b_s, out, m, n, k, out_dtype, workspace,
+                                 workspace_bytes, stream, nullptr);
+}
+
+KSQ_EXPORT int ksq_fp8_blockwise_gemm_f32(const void* a_q, const void* a_s, const void* b, const void* b_s, float* out,
+                                          size_t m, size_t n, size_t k, void* workspace, size_t workspace_bytes,
+                                          void* stream) {
+  return fp8_blockwise_gemm_impl("ksq_fp8_blockwise_gemm_f32", a_q, a_s, b, b_s, nullptr, m, n, k, KSQ_BF16, workspace,
+                                 workspace_bytes, stream, out);
 }
 
 KSQ_EXPORT int ksq_moe_fp8_blockwise_gemm(void* out, const void* a_q, const void* a_s, int a_s_column_major, size_t a_rows, const void* b,

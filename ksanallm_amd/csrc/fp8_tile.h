@@ -28,6 +28,7 @@ struct Fp8TileParams {
   const uint8_t* b;   // [n, k] in packed 2 KiB fragments (ksq_fp8_repack_weight)
   const float* b_s;   // [ceil(n/128), k/128]
   void* out;          // [m, n]
+  float* out32;       // dense form, verification only: the fp32 sums go here, [m, n], and nothing is rounded to TO
   float* partial;     // [slot][part][256][256] fp32 tiles of the workgroups that compute a part of K
   uint32_t M, N, K;
   uint32_t tiles_m, tiles_n;
@@ -391,7 +392,9 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
       for (int t = 0; t < WN; ++t) {
         const uint32_t ncol = n_wave + t * 16 + 4 * lq;
         if (ncol < p.N) {
-          if (GROUPED || direct) {
+          if (!GROUPED && direct && p.out32) {
+            *reinterpret_cast<f32x4*>(p.out32 + static_cast<size_t>(row) * p.N + ncol) = acc[t][i];
+          } else if (GROUPED || direct) {
             f32x4 v = acc[t][i];
             if (GROUPED) v *= rw;
             u32x2 o;

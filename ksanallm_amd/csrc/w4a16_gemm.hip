@@ -147,9 +147,9 @@ int dispatch_mfma_tile(TileParams p, const TilePlan& plan, size_t group, hipStre
     const unsigned cut = plan.tiles_m * plan.tiles_n - plan.main_items;
     uint16_t* y = static_cast<uint16_t*>(p.y);
     if (plan.block_m == 128)
-      splitk_reduce_kernel<T, 128><<<cut * 16, 256, 0, s>>>(p.partial, y, p.M, p.N, p.tiles_m, p.tiles_n, p.main_items, p.splits);
+      splitk_reduce_kernel<T, 128><<<cut * 16, 256, 0, s>>>(p.partial, y, p.M, p.N, p.tiles_m, p.tiles_n, p.main_items, p.splits, p.y32);
     else
-      splitk_reduce_kernel<T, 256><<<cut * 32, 256, 0, s>>>(p.partial, y, p.M, p.N, p.tiles_m, p.tiles_n, p.main_items, p.splits);
+      splitk_reduce_kernel<T, 256><<<cut * 32, 256, 0, s>>>(p.partial, y, p.M, p.N, p.tiles_m, p.tiles_n, p.main_items, p.splits, p.y32);
   }
   return KSQ_OK;
 }
@@ -199,10 +199,12 @@ KSQ_EXPORT size_t ksq_w4a16_workspace_size(size_t max_m, size_t n, size_t k, siz
 }
 
 namespace {
+// y32 given (verification entry point): the same kernels under the same plan, with the fp32 sums stored to y32 [m, n]
+// instead of rounded to T into y (which is then not touched and may be null)
 int w4a16_gemm_impl(const char* fn, void* y, const void* x, const void* w_packed, const void* scales_packed,
                     const void* zeros_packed, void* workspace, size_t workspace_bytes, size_t m, size_t n, size_t k,
-                    size_t group, int dtype, void* stream) {
-  if (int rc = check_common(fn, y, x, w_packed, scales_packed, n, k, group, dtype)) return rc;
+                    size_t group, int dtype, void* stream, float* y32 = nullptr) {
+  if (int rc = check_common(fn, y32 ? static_cast<void*>(y32) : y, x, w_packed, scales_packed, n, k, group, dtype)) return rc;
   if (m == 0) return KSQ_OK;
   if (m > 0x7fffffffull) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: m too large", fn);
   if (!use_mfma_tile(m, n, k, group) && m * k * 2 >= 0x40000000ull)
@@ -227,6 +229,7 @@ int w4a16_gemm_impl(const char* fn, void* y, const void* x, const void* w_packed
     tp.M = static_cast<uint32_t>(m);
     tp.N = static_cast<uint32_t>(n);
     tp.K = static_cast<uint32_t>(k);
+    tp.y32 = y32;
     const TilePlan plan = plan_mfma_tile(m, n, k);
     if (plan.splits > 1) {
       if (!workspace || workspace_bytes < plan.workspace_bytes || !aligned16(workspace))
@@ -253,17 +256,19 @@ int w4a16_gemm_impl(const char* fn, void* y, const void* x, const void* w_packed
     p.partial = static_cast<float*>(workspace);
     p.kt_per_part = static_cast<uint32_t>(div_up(k / 128, c.parts));
   }
+  const bool one_part_f32 = y32 && !p.partial;  // the kernel's partial-sum store with a single part is the fp32 output
+  if (one_part_f32) p.partial = y32;
   int rc = dtype == KSQ_F16 ? dispatch_tile<F16, false>(p, c, static_cast<uint32_t>(m_blocks), group, as_stream(stream))
                             : dispatch_tile<BF16, false>(p, c, static_cast<uint32_t>(m_blocks), group, as_stream(stream));
   if (rc) return rc;
-  if (p.partial) {
+  if (p.partial && !one_part_f32) {
     const size_t mn = m * n;
     const uint32_t parts = static_cast<uint32_t>(div_up(k / 128, p.kt_per_part));
     const unsigned blocks = static_cast<unsigned>(div_up(mn, 256 * 4));
     if (dtype == KSQ_F16)
-      parts_reduce_kernel<F16><<<blocks, 256, 0, as_stream(stream)>>>(p.partial, static_cast<uint16_t*>(y), mn, parts);
+      parts_reduce_kernel<F16><<<blocks, 256, 0, as_stream(stream)>>>(p.partial, static_cast<uint16_t*>(y), mn, parts, y32);
     else
-      parts_reduce_kernel<BF16><<<blocks, 256, 0, as_stream(stream)>>>(p.partial, static_cast<uint16_t*>(y), mn, parts);
+      parts_reduce_kernel<BF16><<<blocks, 256, 0, as_stream(stream)>>>(p.partial, static_cast<uint16_t*>(y), mn, parts, y32);
   }
   return check_launch(fn);
 }
@@ -274,6 +279,13 @@ KSQ_EXPORT int ksq_w4a16_gemm(void* y, const void* x, const void* w_packed, cons
                               size_t k, size_t group, int dtype, void* stream) {
   return w4a16_gemm_impl("ksq_w4a16_gemm", y, x, w_packed, scales_packed, zeros_packed, workspace, workspace_bytes, m, n, k,
                          group, dtype, stream);
+}
+
+KSQ_EXPORT int ksq_w4a16_gemm_f32(float* y, const void* x, const void* w_packed, const void* scales_packed,
+                                  const void* zeros_packed, void* workspace, size_t workspace_bytes, size_t m, size_t n,
+                                  size_t k, size_t group, int dtype, void* stream) {
+  return w4a16_gemm_impl("ksq_w4a16_gemm_f32", nullptr, x, w_packed, scales_packed, zeros_packed, workspace, workspace_bytes, m,
+                         n, k, group, dtype, stream, y);
 }
 
 // ---- the same GEMM for callers that cannot hand over a workspace --------------------------------------------------

@@ -40,6 +40,7 @@ struct TileParams {
   const void* scales;
   const void* zeros;
   float* partial;  // [slot][part][BM][256] fp32 tiles of the workgroups that compute a part of K
+  float* y32;      // dense form, verification only: the fp32 sums go here, [M, N], and nothing is rounded to T
   uint32_t M, N, K;
   uint32_t tiles_m, tiles_n;
   uint32_t main_items, splits, kt_per_split;  // tile_work.h
@@ -537,7 +538,9 @@ __global__ void __launch_bounds__(512, 1) w4a16_tile_kernel(TileParams p) {
       for (int t = 0; t < WN; ++t) {
         if (nt0 + t < n_tiles) {
           const size_t col = static_cast<size_t>(nt0 + t) * 16 + 4 * lq;
-          if (GROUPED || direct) {
+          if (!GROUPED && direct && p.y32) {
+            *reinterpret_cast<f32x4*>(p.y32 + static_cast<size_t>(row) * p.N + col) = acc[t][i];
+          } else if (GROUPED || direct) {
             f32x4 v = acc[t][i];
             if (GROUPED) v *= rw;
             u32x2 o;

@@ -38,11 +38,13 @@ SIGNATURES = {
     "ksq_w4a16_unpack_zeros": (c_i, [c_p, c_i, c_p, c_sz, c_sz, c_sz, c_p]),
     "ksq_w4a16_workspace_size": (c_sz, [c_sz, c_sz, c_sz, c_sz, c_i]),
     "ksq_w4a16_gemm": (c_i, [c_p, c_p, c_p, c_p, c_p, c_p, c_sz, c_sz, c_sz, c_sz, c_sz, c_i, c_p]),
+    "ksq_w4a16_gemm_f32": (c_i, [c_p, c_p, c_p, c_p, c_p, c_p, c_sz, c_sz, c_sz, c_sz, c_sz, c_i, c_p]),
     "ksq_w4a16_static_workspace_bytes": (c_sz, []),
     "ksq_w4a16_gemm_static": (c_i, [c_p, c_p, c_p, c_p, c_p, c_sz, c_sz, c_sz, c_sz, c_i, c_p]),
     "ksq_fp8_group_quant": (c_i, [c_p, c_p, c_p, c_sz, c_sz, c_sz, c_i, c_i, c_i, c_p]),
     "ksq_fp8_blockwise_workspace_size": (c_sz, [c_sz, c_sz, c_sz]),
     "ksq_fp8_blockwise_gemm": (c_i, [c_p, c_p, c_p, c_p, c_p, c_sz, c_sz, c_sz, c_i, c_p, c_sz, c_p]),
+    "ksq_fp8_blockwise_gemm_f32": (c_i, [c_p, c_p, c_p, c_p, c_p, c_sz, c_sz, c_sz, c_p, c_sz, c_p]),
     "ksq_moe_align_capacity": (c_sz, [c_sz, c_sz, c_sz]),
     "ksq_moe_align_scratch_bytes": (c_sz, [c_sz, c_sz]),
     "ksq_moe_align": (c_i, [c_p, c_sz, c_sz, c_sz, c_p, c_p, c_p, c_p, c_p]),

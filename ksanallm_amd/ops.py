@@ -137,6 +137,21 @@ def w4a16_gemm(x, w_packed, scales_packed, zeros_packed, n, k, group, out=None, 
     return out
 
 
+def w4a16_gemm_f32(x, w_packed, scales_packed, zeros_packed, n, k, group, workspace=None):
+    """ksq_w4a16_gemm_f32: the same kernels and plan as w4a16_gemm with the fp32 sums stored unrounded (verification)."""
+    m = x.shape[0]
+    _need_bytes(x, m * k * 2, "w4a16_gemm_f32: x")
+    _need_bytes(w_packed, k * n // 2, "w4a16_gemm_f32: packed weight")
+    _need_bytes(scales_packed, (k // group) * n * 2, "w4a16_gemm_f32: scales")
+    out = torch.empty((m, n), dtype=torch.float32, device=x.device)
+    if workspace is None:
+        workspace = _w4a16_workspace(x.device, m, n, k, group, _dt(x))
+    ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    _l.check(_lib.ksq_w4a16_gemm_f32(_ptr(out), _ptr(x), _ptr(w_packed), _ptr(scales_packed), _ptr(zeros_packed),
+                                     _ptr(workspace), ws_bytes, m, n, k, group, _dt(x), _stream()))
+    return out
+
+
 # ----------------------------------------------------------------------------------------------- FP8
 def per_token_group_quant_fp8(x, k, group=128, column_major=True, fuse_silu_mul=False, q=None, s=None):
     """InvokePerTokenGroupQuantFp8E4m3: returns (codes uint8 [m,k], scales fp32 [k/group,m] or [m,k/group])."""
@@ -169,6 +184,26 @@ def fp8_blockwise_gemm(a_q, a_s, b, b_s, out_dtype=torch.bfloat16, out=None, wor
     ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
     _l.check(_lib.ksq_fp8_blockwise_gemm(_ptr(a_q), _ptr(a_s), _ptr(b), _ptr(b_s), _ptr(out), m, n, k, _dt(out),
                                          _ptr(workspace), ws_bytes, _stream()))
+    return out
+
+
+def fp8_blockwise_gemm_f32(a_q, a_s, b, b_s, workspace=None):
+    """ksq_fp8_blockwise_gemm_f32: the same kernels and plan as fp8_blockwise_gemm with the fp32 sums stored unrounded."""
+    m, k = a_q.shape
+    n = b.shape[0]
+    _need_bytes(a_s, (k // 128) * m * 4, "fp8_blockwise_gemm_f32: activation scales")
+    _need_bytes(b, n * k, "fp8_blockwise_gemm_f32: weight")
+    _need_bytes(b_s, ((n + 127) // 128) * (k // 128) * 4, "fp8_blockwise_gemm_f32: weight scales")
+    out = torch.empty((m, n), dtype=torch.float32, device=a_q.device)
+    if workspace is None:
+        need = _lib.ksq_fp8_blockwise_workspace_size(m, n, k)
+        if need:
+            workspace = _WORKSPACES.get(a_q.device)
+            if workspace is None or workspace.numel() < need:
+                workspace = _WORKSPACES[a_q.device] = torch.empty(need, dtype=torch.uint8, device=a_q.device)
+    ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    _l.check(_lib.ksq_fp8_blockwise_gemm_f32(_ptr(a_q), _ptr(a_s), _ptr(b), _ptr(b_s), _ptr(out), m, n, k,
+                                             _ptr(workspace), ws_bytes, _stream()))
     return out
 
 

@@ -78,3 +78,16 @@ def check_gemm(y_gpu, ref_f32, dtype, what="", weights_rounded=False, rel_l2_max
         excess = np.maximum(err - 0.5 * ulp(ref, dtype), 0.0).max()
         assert excess <= 2e-2, "%s max-abs beyond output rounding %.3e (raw %.3e)" % (what, excess, err.max())
     return rel_l2, err.max()
+
+
+def check_gemm_f32(y32_gpu, ref_f32, what=""):
+    """The parity bar as it is written, on the sums before they are rounded to the output type (the fp32 entry points):
+    rel-L2 <= 5e-3 and max-abs <= 2e-2 against the fp32-accumulated dequant reference, raw, nothing normalised."""
+    y = y32_gpu.cpu().numpy().astype(np.float64)
+    ref = ref_f32.astype(np.float64)
+    assert y.shape == ref.shape and np.all(np.isfinite(y)), what
+    rel_l2 = np.linalg.norm(y - ref) / max(np.linalg.norm(ref), 1e-30)
+    max_abs = np.abs(y - ref).max()
+    assert rel_l2 <= 5e-3, "%s rel-L2 before rounding %.3e" % (what, rel_l2)
+    assert max_abs <= 2e-2, "%s max-abs before rounding %.3e" % (what, max_abs)
+    return rel_l2, max_abs

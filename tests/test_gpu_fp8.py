@@ -295,3 +295,18 @@ def test_blockwise_gemm_full_size_properties(ops, oracle, n, k):
     perm = torch.randperm(m, generator=g).cuda()
     qp, sp = ops.per_token_group_quant_fp8(x[perm].contiguous(), k, 128, True)
     assert torch.equal(ops.fp8_blockwise_gemm(qp, sp, bp, bs, torch.bfloat16), y[perm])
+
+
+# the sums before they are rounded to bf16 (ksq_fp8_blockwise_gemm_f32: same kernels, same plan): the parity bar as
+# written, raw - streaming kernel, tile kernel with whole tiles, tile kernel with tiles cut along K
+@pytest.mark.parametrize("m,n,k", [(1, 18432, 7168), (16, 7168, 18432), (128, 7168, 18432), (128, 18432, 7168),
+                                   (300, 2320, 1152), (1024, 2304, 384)])
+def test_blockwise_gemm_sums_before_output_rounding(ops, oracle, m, n, k):
+    x, bq, bs = make_fp8_problem(oracle, 4800 + m + n, m, n, k)
+    q, s = ops.per_token_group_quant_fp8(x.cuda(), k, 128, True)
+    bp, bsd = packed(ops, bq), torch.from_numpy(bs).cuda()
+    y32 = ops.fp8_blockwise_gemm_f32(q, s, bp, bsd)
+    y = ops.fp8_blockwise_gemm(q, s, bp, bsd, torch.bfloat16)
+    assert torch.equal(y32.to(torch.bfloat16).view(torch.int16), y.view(torch.int16))
+    ref = oracle.fp8_blockwise_gemm(q.cpu().numpy(), s.cpu().numpy(), bq, bs, True)
+    H.check_gemm_f32(y32, ref, "fp8 before rounding m=%d n=%d k=%d" % (m, n, k))
