@@ -160,7 +160,9 @@ int ksq_w4a16_gemm_f32(float* y, const void* x, const void* w_packed, const void
  * KSQ_W4A16_STATIC_WORKSPACE_BYTES that is part of the library's code object (each GPU the library runs on holds it
  * until the process ends); a call whose plan needs more returns KSQ_ERR_WORKSPACE and leaves y untouched - use
  * ksq_w4a16_gemm with a workspace then.  The call allocates nothing and frees nothing.  All calls on one GPU share the
- * buffer: two of them that overlap in time (different streams) race on it; calls on one stream do not. */
+ * buffer: two of them that overlap in time (different streams) race on it; calls on one stream do not.
+ * The first call on a device also looks up the buffer's address there and sets the large-LDS attribute of the kernels
+ * it launches: make one call per device and kernel variant outside graph capture before capturing any. */
 #define KSQ_W4A16_STATIC_WORKSPACE_BYTES (32u << 20)
 size_t ksq_w4a16_static_workspace_bytes(void);
 int ksq_w4a16_gemm_static(void* y, const void* x, const void* w_packed, const void* scales_packed,
@@ -360,6 +362,9 @@ typedef struct ksq_tile_desc {
   int32_t x_chunk;  /* split-K wavefront kernel: k-tiles of activations staged through LDS at a time; 0 = through registers */
 } ksq_tile_desc;
 
+/* The descriptor describes group size 128.  Other group sizes of W4A16 keep the kernel and block shape but carry more
+ * scales per k-tile; W4A8 with group 64 runs 128-token tiles whose K range is not cut (split_k and grid then differ
+ * from what is reported here). */
 int ksq_select_tile(int kind, size_t m, size_t n, size_t k, int dtype, ksq_tile_desc* out_desc);
 
 #ifdef __cplusplus

@@ -67,8 +67,9 @@ __global__ void __launch_bounds__(BLOCK) fp8_group_quant_kernel(const uint16_t* 
                        static_cast<uint16_t>(r2.w), static_cast<uint16_t>(r2.w >> 16)};
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        float g = v[j];
-        float act = g / (1.0f + __expf(-g)) * T::to_float(u[j]);
+        // the one definition of silu * mul every kernel here uses (ksq_common.h), so that the int4 and the block-fp8
+        // expert paths apply the same activation
+        const float act = silu_mul_f32(v[j], T::to_float(u[j]));
         v[j] = T::to_float(T::from_float(act));  // the reference rounds silu*mul to T before quantizing
       }
     }

@@ -1,7 +1,5 @@
 // Per-shape tile selection: closed-form rules of (kind, m, n, k, dtype) for a 256-CU, 8-XCD MI355X.
 // Host code only; no timing and no device queries, so the answer is the same at load time and at run time.
-#include <cstdlib>
-#include <cstdio>
 #include "ksq_common.h"
 #include "tile_select.h"
 
@@ -62,10 +60,6 @@ SplitKChoice select_splitk(size_t m, size_t n, size_t k) {
       c.waves = 8;
       c.xc = 8;
     }
-  }
-  if (const char* f = getenv("KSQ_FORCE_SPLITK")) {  // DEV SWITCH
-    int nt, waves, parts, xc;
-    if (sscanf(f, "%d,%d,%d,%d", &nt, &waves, &parts, &xc) == 4) { c.nt = nt; c.waves = waves; c.parts = parts; c.xc = xc; }
   }
   return c;
 }

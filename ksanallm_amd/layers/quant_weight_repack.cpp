@@ -1,6 +1,7 @@
 #include "quant_weight_repack.h"
 
 #include <algorithm>
+#include <cstring>
 #include <vector>
 
 namespace ksana_llm {
@@ -44,13 +45,24 @@ Tensor PackActOrderSlice(const Tensor& qweight, const Tensor& scales, const std:
     KLLM_THROW("PackGroupQuantWeight: cannot upload perm");
   }
   KsqCheck(ksq_w4a16_repack_rows(qweight.GetPtr<void>(), packed.perm->GetPtr<void>(), packed.GetPtr<void>(), K, Kp, N, stream), who);
-  // scale row of every 32 packed rows, then the packed scale layout for group size 32
+  // scale row of every 32 packed rows, then the packed scale layout for group size 32.  The table is expanded on the
+  // host (one copy down, one up: a device copy per 32 packed rows would be more than a thousand tiny copies per weight)
   const size_t row_bytes = N * GetTypeSize(scales.dtype);
   Tensor expanded(MemoryLocation::LOCATION_DEVICE, scales.dtype, {Kp / 32, N}, rank);
-  for (size_t b = 0; b < Kp / 32; ++b) {
-    if (hipMemcpyAsync(expanded.GetPtr<char>() + b * row_bytes, scales.GetPtr<char>() + static_cast<size_t>(block_group[b]) * row_bytes,
-                       row_bytes, hipMemcpyDeviceToDevice, stream) != hipSuccess) {
-      KLLM_THROW("PackGroupQuantWeight: cannot gather the scale rows");
+  {
+    const size_t table_rows = scales.shape[0];
+    std::vector<char> table(table_rows * row_bytes), wide((Kp / 32) * row_bytes);
+    if (hipStreamSynchronize(stream) != hipSuccess ||
+        hipMemcpy(table.data(), scales.GetPtr<void>(), table.size(), hipMemcpyDeviceToHost) != hipSuccess) {
+      KLLM_THROW("PackGroupQuantWeight: cannot read the scales");
+    }
+    for (size_t b = 0; b < Kp / 32; ++b) {
+      const size_t g = static_cast<size_t>(block_group[b]);
+      if (g >= table_rows) KLLM_THROW("PackGroupQuantWeight: g_idx names a group the scales do not hold");
+      std::memcpy(wide.data() + b * row_bytes, table.data() + g * row_bytes, row_bytes);
+    }
+    if (hipMemcpy(expanded.GetPtr<void>(), wide.data(), wide.size(), hipMemcpyHostToDevice) != hipSuccess) {
+      KLLM_THROW("PackGroupQuantWeight: cannot upload the expanded scales");
     }
   }
   packed.scales = std::make_shared<Tensor>(MemoryLocation::LOCATION_DEVICE, scales.dtype, std::vector<size_t>{Kp / 32, N}, rank);
@@ -77,6 +89,8 @@ Tensor PackGroupQuantWeight(const Tensor& qweight, const Tensor& scales, const T
 
   if (k_slice) {
     if (awq) KLLM_THROW("PackGroupQuantWeight: g_idx (act-order) belongs to GPTQ checkpoints");
+    // padding rows take code 8, which is nothing only under the symmetric zero point
+    if (qzeros) KLLM_THROW("PackGroupQuantWeight: a K range of an act-order weight is packed for symmetric GPTQ only (qzeros given)");
     if (g_idx->GetElementNumber() != K) KLLM_THROW("PackGroupQuantWeight: g_idx must have K entries");
     std::vector<int32_t> groups(K);
     if (hipStreamSynchronize(stream) != hipSuccess ||

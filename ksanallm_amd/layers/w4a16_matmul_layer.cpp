@@ -21,6 +21,9 @@ Status W4A16MatMulLayer::Init(const std::vector<std::any>& parameters, const Run
   [[maybe_unused]] bool use_gemv_cuda_core = std::any_cast<const bool>(parameters[parameter_index++]);  // no analogue
   weight_data_type_ = std::any_cast<const DataType>(parameters[parameter_index++]);
   is_k_full_ = is_gptq_desc_ ? is_k_full_ : true;
+  tp_cut_bound_ = std::max({runtime_config.parallel_basic_config.tensor_parallel_size,
+                            runtime_config.parallel_basic_config.attn_tensor_parallel_size,
+                            runtime_config.parallel_basic_config.moe_tensor_para_size});
   if (is_gptq_desc_ && is_awq_) return Status(RET_INVALID_ARGUMENT, std::string(Name()) + ": desc_act belongs to GPTQ, not AWQ");
   return Status();
 }
@@ -37,7 +40,9 @@ size_t W4A16MatMulLayer::GetWorkspaceSize() {
   // for each of the checkpoint's groups - k * ranks / groupsize of them - that has rows in the range)
   size_t permuted_k = max_k_;
   if (is_gptq_desc_ && !is_k_full_) {
-    const size_t ranks = static_cast<size_t>(std::max(1, context_->GetTensorParallelSize()));
+    // the cut the factory applied is one of the tensor-parallel sizes the configuration names (o_proj and the MLA
+    // projections are cut by the attention size, the MLP by the general one): the largest of them bounds the groups
+    const size_t ranks = std::max<size_t>({static_cast<size_t>(std::max(1, context_->GetTensorParallelSize())), tp_cut_bound_, 1});
     const size_t groups = std::min(max_k_, max_k_ * ranks / std::max<size_t>(1, groupsize_));
     permuted_k = (max_k_ + 31 * groups + 127) / 128 * 128;
     // the GEMM then runs over the padded rows with group size 32: its scratch for any padded depth up to the bound

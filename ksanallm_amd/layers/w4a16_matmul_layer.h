@@ -37,6 +37,7 @@ class W4A16MatMulLayer : public BaseLayer {
   bool is_k_full_ = true;
   size_t max_m_ = 0, max_n_ = 0, max_k_ = 0;
   size_t groupsize_ = 0;
+  size_t tp_cut_bound_ = 1;  // the largest tensor-parallel size the runtime configuration names
   size_t workspace_size_ = 0;
   size_t gemm_workspace_size_ = 0, permuted_input_size_ = 0;
 };

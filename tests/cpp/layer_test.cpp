@@ -133,7 +133,10 @@ static int RunW4A16(int argc, char** argv) {
   // rank), or - k_slice - the row-parallel mlp.down_proj of a model with inter size k and hidden size n, whose K is a
   // rank's slice of the checkpoint's
   const bool k_slice = k_range;
-  if (k_slice) context = std::make_shared<Context>(2, stream);  // two tensor-parallel ranks, this is rank 0
+  // two tensor-parallel ranks, this is rank 0.  argv[12]: the size the context reports, where it differs from the cut the
+  // factory applies (which follows the runtime configuration): the layer's workspace bound must not rest on the former
+  const int context_tp = argc > 12 ? std::atoi(argv[12]) : 2;
+  if (k_slice) context = std::make_shared<Context>(context_tp, stream);
   mc.hidden_units = k_slice ? n : k;
   mc.inter_size = k_slice ? 2 * k : n;
   const std::string name = k_slice ? "model.layers.0.mlp.down_proj.weight" : "model.layers.0.mlp.gate_proj.weight";

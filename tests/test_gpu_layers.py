@@ -71,8 +71,9 @@ def test_w4a16_layer_act_order(tmp_path, oracle, dtype, backend, m, n, k):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("context_tp", [2, 1])   # 1: the context reports fewer ranks than the cut the factory applied
 @pytest.mark.parametrize("dtype,backend,m,n,k", [(H.F16, "marlin", 3, 512, 1024), (H.BF16, "marlin", 40, 256, 1536)])
-def test_w4a16_layer_act_order_k_range(tmp_path, oracle, dtype, backend, m, n, k):
+def test_w4a16_layer_act_order_k_range(tmp_path, oracle, dtype, backend, m, n, k, context_tp):
     """is_k_full = false: this rank holds rows [0, k) of an act-order checkpoint with 2k rows (mlp.down_proj under two
     tensor-parallel ranks).  Its rows belong to arbitrary groups of the whole checkpoint; the oracle is the definition
     y = x . ((code - 8) * scale[g_idx[row]]) over the rank's rows."""
@@ -85,7 +86,7 @@ def test_w4a16_layer_act_order_k_range(tmp_path, oracle, dtype, backend, m, n, k
     H.bits_of(full["scales"]).tofile(tmp_path / "scales.bin")
     H.bits_of(x).tofile(tmp_path / "x.bin")
     g_idx.numpy().tofile(tmp_path / "g_idx.bin")
-    run_driver("w4a16", tmp_path, "gptq", TNAME[dtype], backend, m, n, k, 128, 1, 1)
+    run_driver("w4a16", tmp_path, "gptq", TNAME[dtype], backend, m, n, k, 128, 1, 1, context_tp)
     y = read_out(tmp_path / "y.bin", dtype, (m, n))
     ref = oracle.gptq_act_order_gemm(H.bits_of(x), codes, H.bits_of(full["scales"]), g_idx.numpy(), dtype)
     H.check_gemm(y, ref, dtype, "%s act-order K-range layer" % backend, weights_rounded=m > 32)

@@ -9,18 +9,19 @@ from tests import helpers as H
 pytestmark = pytest.mark.gpu
 
 
-def _problem(ops, L, seed, M, N, K, dtype, awq):
-    d = H.make_w4a16(seed, M, N, K, 128, dtype, awq=awq, x_std=0.5, s_lo=0.002, s_hi=0.01, z_lo=0, z_hi=15)
+def _problem(ops, L, seed, M, N, K, dtype, awq, group=128):
+    d = H.make_w4a16(seed, M, N, K, group, dtype, awq=awq, x_std=0.5, s_lo=0.002, s_hi=0.01, z_lo=0, z_hi=15)
     wp = ops.repack_weight(d["qweight"].cuda(), L.SRC_AWQ if awq else L.SRC_GPTQ, 1, K, N)
-    sp = ops.repack_scales(d["scales"].cuda(), L.SCALE_GN, 1, K, N, 128)
-    zp = ops.repack_zeros(d["qzeros"].cuda(), L.ZERO_AWQ_PACKED, K, N, 128) if awq else None
+    sp = ops.repack_scales(d["scales"].cuda(), L.SCALE_GN, 1, K, N, group)
+    zp = ops.repack_zeros(d["qzeros"].cuda(), L.ZERO_AWQ_PACKED, K, N, group) if awq else None
     return d, d["x"].cuda(), wp, sp, zp
 
 
-def _static(L, x, wp, sp, zp, N, K, dtype):
-    y = torch.full((x.shape[0], N), float("nan"), dtype=x.dtype, device=x.device)
+def _static(L, x, wp, sp, zp, N, K, dtype, group=128, y=None):
+    if y is None:
+        y = torch.full((x.shape[0], N), float("nan"), dtype=x.dtype, device=x.device)
     L.check(L.load().ksq_w4a16_gemm_static(y.data_ptr(), x.data_ptr(), wp.data_ptr(), sp.data_ptr(),
-                                           None if zp is None else zp.data_ptr(), x.shape[0], N, K, 128, dtype,
+                                           None if zp is None else zp.data_ptr(), x.shape[0], N, K, group, dtype,
                                            torch.cuda.current_stream().cuda_stream))
     return y
 
@@ -75,3 +76,54 @@ def test_static_scratch_rejects_plans_beyond_its_size():
     if rc == 0:
         pytest.skip("the plan for m=%d alone fits" % M)
     assert rc == 3 and b"scratch" in lib.ksq_last_error_string()
+
+
+def test_static_scratch_allocates_nothing_and_replays_from_a_graph():
+    """What the entry point promises beyond its results: the device's free memory is the same after a run of calls as
+    before the first of them, and a call captured into a HIP graph (after one eager call on the device, which
+    resolves the buffer's address and the kernels' attributes) replays to the eager bits every time, with eager work
+    between the replays.  The plans cut K (tile kernel, group 128 and group 64; decode kernel), so the scratch is in
+    use."""
+    from ksanallm_amd import lib as L
+    from ksanallm_amd import ops
+    lib = L.load()
+    cases = []
+    for i, (M, N, K, group) in enumerate([(128, 4096, 14336, 128), (96, 2048, 8192, 64), (8, 1024, 4096, 128)]):
+        assert 0 < lib.ksq_w4a16_workspace_size(M, N, K, group, H.BF16) <= lib.ksq_w4a16_static_workspace_bytes()
+        d, x, wp, sp, zp = _problem(ops, L, 8200 + i, M, N, K, H.BF16, False, group)
+        ref = ops.w4a16_gemm(x, wp, sp, zp, N, K, group)
+        H.check_gemm(ref, H.w4a16_oracle(d), H.BF16, "M=%d N=%d K=%d group %d" % (M, N, K, group), weights_rounded=M > 32)
+        y = torch.empty_like(ref)
+        cases.append((x, wp, sp, zp, N, K, group, ref, y))
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    for _ in range(3):
+        for (x, wp, sp, zp, N, K, group, ref, y) in cases:
+            _static(L, x, wp, sp, zp, N, K, H.BF16, group, y)
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before
+    for (x, wp, sp, zp, N, K, group, ref, y) in cases:
+        assert torch.equal(y.view(torch.int16), ref.view(torch.int16))
+    # graph: the three calls in one captured sequence
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        for (x, wp, sp, zp, N, K, group, ref, y) in cases:
+            y.zero_()
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            for (x, wp, sp, zp, N, K, group, ref, y) in cases:
+                _static(L, x, wp, sp, zp, N, K, H.BF16, group, y)
+    torch.cuda.current_stream().wait_stream(side)
+    for rep in range(3):
+        for (x, wp, sp, zp, N, K, group, ref, y) in cases:
+            y.fill_(float("nan"))
+        # eager work that uses the same scratch between the replays
+        x, wp, sp, zp, N, K, group, ref, _ = cases[rep % len(cases)]
+        assert torch.equal(_static(L, x, wp, sp, zp, N, K, H.BF16, group).view(torch.int16), ref.view(torch.int16))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for (x, wp, sp, zp, N, K, group, ref, y) in cases:
+            assert torch.equal(y.view(torch.int16), ref.view(torch.int16)), rep
