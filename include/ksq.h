@@ -274,6 +274,10 @@ int ksq_moe_align(const void* topk_ids, size_t numel, size_t E, size_t block_m, 
  * block_m is the block size the permutation was aligned with: 16 or 32 run the streaming (decode) kernel, 128 or 256
  * the MFMA tile kernel (which multiplies only the 16-row tiles of a block that hold rows); ksq_moe_block_m() gives the
  * choice for a problem size.
+ * A handful of slots (numel <= 64, block_m 16) need no aligned permutation: with sorted_ids NULL, expert_ids is the
+ * router's topk_ids [numel] itself, num_post_pad is not read, and every slot is a block of its own (a slot whose id is
+ * outside [0, E) leaves its output row unwritten, as the alignment would have dropped it).  One launch fewer in front
+ * of a GEMM that takes tens of microseconds.
  * Replaces InvokeMoeWna16Gemm (K/moe/moe_wna16/moe_wna16.cu:263-288) and the Triton
  * InvokeFusedMoeGptqAwqKernel (S/kernels/nvidia/triton_wrapper.h:68-75). */
 size_t ksq_moe_block_m(size_t numel, size_t E);
@@ -285,13 +289,27 @@ int ksq_moe_w4a16_gemm(void* out, const void* x, const void* w_packed, const voi
 /* The first MoE GEMM with the activation in its epilogue: w_packed holds [gate | up] rows (n = 2 * inter), and for every
  * valid sorted slot id s   out[s, c] = T(silu(T(g)) * T(u)),  g = x[s / top_k, :] . W[e, c, :],  u = x[s / top_k, :] . W[e, inter + c, :],
  * out [numel, inter] T: bit for bit what ksq_moe_w4a16_gemm into a [numel, 2 * inter] buffer followed by ksq_silu_mul
- * gives, in one launch and without that buffer.  block_m 16, 32, 128 or 256, as for ksq_moe_w4a16_gemm.
+ * gives, in one launch and without that buffer.  block_m 16, 32, 128 or 256, as for ksq_moe_w4a16_gemm (sorted_ids NULL
+ * likewise).
  * Replaces the pair InvokeMoeWna16Gemm + InvokeSiluAndMul of InvokeFusedMoe
  * (S/kernels/nvidia/moe_kernel_wrapper.cpp:616-640). */
 int ksq_moe_w4a16_gate_up_silu(void* out, const void* x, const void* w_packed, const void* scales_packed,
                                const void* zeros_packed, const void* sorted_ids, const void* expert_ids,
                                const void* num_post_pad, size_t numel, size_t top_k, size_t E, size_t n, size_t k,
                                size_t group, size_t block_m, int dtype, void* stream);
+
+/* The second MoE GEMM and the sum over top-k in one launch, for up to 8 tokens:
+ *   out[t, :] = T( sum_j topk_w[t, j] * (x[t * top_k + j, :] . dequant(W[topk_ids[t, j]])) ),  summed in fp32 and rounded once
+ * x [tokens * top_k, k] T (the activation's output, a token's top_k rows one behind the other), out [tokens, n] T,
+ * topk_w fp32 and topk_ids int32 [tokens, top_k] as the router wrote them (an id outside [0, E) contributes nothing).
+ * A token's row block streams its top_k experts' weights as one long K; no aligned permutation, no [numel, n] buffer,
+ * no separate sum (whose per-expert rounding to T this form does not have: it is closer to the fp32 reference).
+ * Replaces InvokeMoeWna16Gemm followed by InvokeMoeSum for the decode steps of a few sequences
+ * (K/moe/moe_wna16/moe_wna16.cu:36-217, which adds its partial results into the output with atomicAdd;
+ * K/moe_utils/moe_utils.cu:789-835). */
+int ksq_moe_w4a16_down_sum(void* out, const void* x, const void* w_packed, const void* scales_packed, const void* topk_w,
+                           const void* topk_ids, size_t tokens, size_t top_k, size_t E, size_t n, size_t k, size_t group,
+                           int dtype, void* stream);
 
 /* Grouped blockwise-FP8 GEMM over the aligned blocks: for every valid sorted slot id s (< numel)
  *   out[s, :] = sum_kb (a_q[s / top_k, kb] . b[e, :, kb]) * a_s[kb, s / top_k] * b_s[e, :/128, kb] * (topk_w ? topk_w[s] : 1)

@@ -288,6 +288,59 @@ KSQ_EXPORT int ksq_w4a16_gemm_f32(float* y, const void* x, const void* w_packed,
                          n, k, group, dtype, stream, y);
 }
 
+namespace {
+template <typename T, int NT>
+int launch_token_sum(const SplitKParams& p, uint32_t tokens, hipStream_t s) {
+  // one row of x per workgroup: the narrow decode instances' ring depths
+  constexpr int LOOK = NT == 1 ? 4 : 3, OCC = NT == 1 ? 4 : 3;
+  typedef SplitKLds<1, NT, 4, 0> Lds;
+  dim3 grid(p.N / 16 / NT, tokens, 1);
+  w4a16_splitk_kernel<T, 1, NT, 4, LOOK, OCC, 128, false, true, 0, 16, true><<<grid, 4 * 64, Lds::kBytes, s>>>(p);
+  return KSQ_OK;
+}
+}  // namespace
+
+KSQ_EXPORT int ksq_moe_w4a16_down_sum(void* out, const void* x, const void* w_packed, const void* scales_packed,
+                                      const void* topk_w, const void* topk_ids, size_t tokens, size_t top_k, size_t E,
+                                      size_t n, size_t k, size_t group, int dtype, void* stream) {
+  const char* fn = "ksq_moe_w4a16_down_sum";
+  if (int rc = check_common(fn, out, x, w_packed, scales_packed, n, k, group, dtype)) return rc;
+  if (!topk_ids) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: null index buffer", fn);
+  if (group != 128) return fail(KSQ_ERR_UNSUPPORTED, "%s: expert weights need group size 128", fn);
+  if (top_k == 0 || top_k > 32 || E == 0) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: top_k must be in 1..32 and E positive", fn);
+  if (tokens == 0) return KSQ_OK;
+  if (tokens > 8) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: at most 8 tokens (every token streams its own experts)", fn);
+  if (tokens * top_k * k * 2 >= 0x40000000ull) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: x too large", fn);
+  SplitKParams p{};
+  p.y = out;
+  p.x = x;
+  p.w = w_packed;
+  p.scales = scales_packed;
+  p.M = static_cast<uint32_t>(tokens);
+  p.N = static_cast<uint32_t>(n);
+  p.K = static_cast<uint32_t>(top_k * k);  // a token's top_k rows of x, one behind the other
+  p.kt_per_expert = static_cast<uint32_t>(k / 128);
+  p.expert_ids = static_cast<const int32_t*>(topk_ids);
+  p.topk_w = static_cast<const float*>(topk_w);
+  p.numel = static_cast<uint32_t>(tokens);  // rows of the output
+  p.top_k = static_cast<uint32_t>(top_k);
+  p.num_experts = static_cast<uint32_t>(E);
+  p.x_bytes = static_cast<uint32_t>(tokens * top_k * k * 2);
+  p.nibble_mask = 0x000f000fu;
+  // two column tiles per workgroup where that still leaves a workgroup for most CUs
+  const bool two = (n / 16) % 2 == 0 && (n / 32) * tokens >= 192;
+  p.magic2 = dtype == KSQ_F16 ? F16::kMagic2 : BF16::kMagic2;
+  int rc;
+  if (dtype == KSQ_F16)
+    rc = two ? launch_token_sum<F16, 2>(p, static_cast<uint32_t>(tokens), as_stream(stream))
+             : launch_token_sum<F16, 1>(p, static_cast<uint32_t>(tokens), as_stream(stream));
+  else
+    rc = two ? launch_token_sum<BF16, 2>(p, static_cast<uint32_t>(tokens), as_stream(stream))
+             : launch_token_sum<BF16, 1>(p, static_cast<uint32_t>(tokens), as_stream(stream));
+  if (rc) return rc;
+  return check_launch(fn);
+}
+
 // ---- the same GEMM for callers that cannot hand over a workspace --------------------------------------------------
 // The fp32 partial sums of launches that cut K go through this array instead of a caller's buffer.  Every GPU the
 // library runs on holds its own copy from the moment the code object is loaded until the process ends.  The name below is
@@ -351,14 +404,18 @@ int moe_w4a16_gemm_impl(const char* fn, bool fuse_silu, void* out, const void* x
   if (fuse_silu) {
     if (n % 32 != 0) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: n = 2 * inter must be a multiple of 32", fn);
   }
-  if (!sorted_ids || !expert_ids || !num_post_pad) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: null index buffer", fn);
+  // sorted_ids == NULL: a handful of slots, one per 16-row block, with the router's ids in expert_ids (w4a16_splitk.h)
+  const bool few = !sorted_ids;
+  if (!expert_ids || (!few && !num_post_pad)) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: null index buffer", fn);
+  if (few && (block_m != 16 || numel > 64))
+    return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: without sorted_ids every slot is a 16-row block of its own: block_m 16, at most 64 slots", fn);
   if (zeros_packed) return fail(KSQ_ERR_UNSUPPORTED, "%s: zero points are not supported for expert weights", fn);
   if (group != 128) return fail(KSQ_ERR_UNSUPPORTED, "%s: expert weights need group size 128", fn);
   if (top_k == 0 || E == 0) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: top_k and E must be positive", fn);
   if (block_m != 16 && block_m != 32 && block_m != 128 && block_m != 256)
     return fail(KSQ_ERR_UNSUPPORTED, "%s: block_m %zu not in {16,32,128,256}", fn, block_m);
   if (numel == 0) return KSQ_OK;
-  const size_t cap_blocks = (numel + E * (block_m - 1)) / block_m;  // upper bound on aligned blocks
+  const size_t cap_blocks = few ? numel : (numel + E * (block_m - 1)) / block_m;  // upper bound on aligned blocks
   if (block_m >= 128) {  // prefill regime: MFMA tile kernel, rows gathered / scattered through the permutation
     if (numel > 0x7fffffffull || (numel / top_k + 1) * k * 2 > 0xffffffffull)
       return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: x too large", fn);
@@ -408,10 +465,11 @@ int moe_w4a16_gemm_impl(const char* fn, bool fuse_silu, void* out, const void* x
   p.topk_w = static_cast<const float*>(topk_w);
   p.numel = static_cast<uint32_t>(numel);
   p.top_k = static_cast<uint32_t>(top_k);
+  p.num_experts = static_cast<uint32_t>(E);
   p.x_bytes = static_cast<uint32_t>(x_rows * k * 2);
   // about numel/block_m + E/2 of the aligned blocks hold rows; K is never split across workgroups here
   SplitKChoice c = select_splitk_blocks(static_cast<int>(block_m / 16),
-                                        std::min(cap_blocks, numel / block_m + E / 2 + 1), n, k);
+                                        few ? numel : std::min(cap_blocks, numel / block_m + E / 2 + 1), n, k);
   if (fuse_silu) {
     if (c.nt < 2) c.nt = 2;  // a workgroup holds gate and up tiles in pairs
     p.pair_tiles = static_cast<uint32_t>(n / 32);

@@ -58,6 +58,15 @@ struct SplitKParams {
   uint32_t pair_tiles;
   uint32_t x_bytes;  // extent of x, below 1 GiB
   uint32_t nibble_mask, magic2;  // 0x000f000f and T::kMagic2, passed in so that they live in registers
+  // Grouped form for a handful of slots (sorted_ids == nullptr): no aligned permutation, expert_ids holds the router's
+  // ids [numel] as they are.  Block b is slot b alone: row b / top_k of x, expert expert_ids[b], output row b; an id
+  // outside [0, num_experts) leaves its row unwritten, as the alignment would have dropped the slot.
+  // TOKSUM instances (the second GEMM with the sum over top-k in it): block b is token b.  Its top_k rows of x
+  // [numel, kt_per_expert * 128] lie one behind the other, one row of K = top_k * kt_per_expert * 128 values; k-tile kt
+  // of that row meets k-tile kt % kt_per_expert of expert expert_ids[b * top_k + kt / kt_per_expert], its scale times
+  // the routing weight topk_w[b * top_k + kt / kt_per_expert]; the fp32 sum over all of K is output row b of [tokens, N].
+  uint32_t num_experts;
+  uint32_t kt_per_expert;
 };
 
 // Eight codes of a packed dword -> MFMA operand holding magic+code (nibble i and i+4 are the pair k=2i, 2i+1).
@@ -95,8 +104,9 @@ struct SplitKLds {
 // of the ring (16 * MT registers per slot), turns them from 64-byte pieces of sixteen rows into whole cache lines, and
 // leaves rows beyond M unfetched.
 template <typename T, int MT, int NT, int WAVES, int LOOK, int OCC, int GROUP, bool HAS_ZP, bool GROUPED, int XC = 0,
-          int XR = 16 * MT>
+          int XR = 16 * MT, bool TOKSUM = false>
 __global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKParams p) {
+  static_assert(!TOKSUM || (GROUPED && MT == 1 && XC == 0 && !HAS_ZP && GROUP == 128), "the token-sum form is a grouped decode form");
   constexpr int GPT = 128 / GROUP;  // groups per k-tile
   constexpr int SPG = GROUP / 32;   // MFMA k-steps per group
   constexpr bool XLDS = XC > 0;
@@ -111,8 +121,9 @@ __global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKPar
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lrow = lane & 15;
   const int lq = lane >> 4;
-  const uint32_t KT = p.K / 128;
-  const uint32_t G = p.K / GROUP;
+  const uint32_t KT = TOKSUM ? p.kt_per_expert : p.K / 128;  // k-tiles of a weight strip
+  const uint32_t KTL = p.K / 128;                            // k-tiles of a row of x
+  const uint32_t G = KT * GPT;
   const bool fused = GROUPED && NT > 1 && p.pair_tiles != 0;
   const uint32_t nt0 = fused ? blockIdx.x * (NT / 2) : blockIdx.x * NT;
   // tiles skipped between the workgroup's column tile NT/2-1 and its column tile NT/2 (0 unless fused)
@@ -128,16 +139,33 @@ __global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKPar
   uint32_t xrow[MT];
   size_t tile_base = 0;  // first weight tile of the expert, in tiles
   size_t sz_base = 0;    // first scale / zero element of the expert
+  const bool few = GROUPED && p.sorted_ids == nullptr;  // a handful of slots: one per block, no aligned permutation
+  __shared__ uint32_t tok_ids[TOKSUM ? 32 : 1];          // token-sum form: the token's expert ids and routing weights
+  __shared__ float tok_w[TOKSUM ? 32 : 1];
   if (GROUPED) {
     const uint32_t pos0 = blockIdx.y * (16 * MT);
-    if (pos0 >= static_cast<uint32_t>(p.num_post_pad[0])) return;
-    const uint32_t e = static_cast<uint32_t>(p.expert_ids[blockIdx.y]);
+    uint32_t e = 0;
+    if (TOKSUM) {
+      if (threadIdx.x < p.top_k) {
+        tok_ids[threadIdx.x] = static_cast<uint32_t>(p.expert_ids[blockIdx.y * p.top_k + threadIdx.x]);
+        tok_w[threadIdx.x] = p.topk_w ? p.topk_w[blockIdx.y * p.top_k + threadIdx.x] : 1.0f;
+      }
+      __syncthreads();
+    } else {
+      if (!few && pos0 >= static_cast<uint32_t>(p.num_post_pad[0])) return;
+      e = static_cast<uint32_t>(p.expert_ids[blockIdx.y]);
+      if (few && e >= p.num_experts) return;
+    }
     tile_base = static_cast<size_t>(e) * (p.N / 16) * KT;
     sz_base = static_cast<size_t>(e) * G * p.N;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-      const uint32_t sid = static_cast<uint32_t>(p.sorted_ids[pos0 + mt * 16 + lrow]);
-      xrow[mt] = sid < p.numel ? sid / p.top_k : kNoRow;
+      if (few || TOKSUM) {
+        xrow[mt] = (mt == 0 && lrow == 0) ? (TOKSUM ? blockIdx.y : blockIdx.y / p.top_k) : kNoRow;
+      } else {
+        const uint32_t sid = static_cast<uint32_t>(p.sorted_ids[pos0 + mt * 16 + lrow]);
+        xrow[mt] = sid < p.numel ? sid / p.top_k : kNoRow;
+      }
     }
   } else {
 #pragma unroll
@@ -179,6 +207,7 @@ __global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKPar
     u32x4 wq;
     uint32_t sc[GPT];  // 16-bit scale and 8-bit zero point, each widened into a register of its own so that no
     uint32_t zp[GPT];  // packing of ring slots ties loads of different groups together
+    float rw;          // token-sum form: the routing weight of the expert this k-tile belongs to
   };
   struct XBuf {
     u32x4 xf[MT][4];
@@ -189,23 +218,44 @@ __global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKPar
   constexpr uint32_t kOutOfRange = 0x40000000u;
   struct KOff {
     uint32_t w, s, z, x;
+    __amdgpu_buffer_rsrc_t wr, sr;  // token-sum form: the weights and scales of the k-tile's expert
+    float rw;
   };
   const uint32_t kt_begin = GROUPED ? 0 : blockIdx.z * p.kt_per_part;
-  const uint32_t kt_end = GROUPED ? KT : ((KT - kt_begin) < p.kt_per_part ? KT : kt_begin + p.kt_per_part);
+  const uint32_t kt_end = GROUPED ? KTL : ((KTL - kt_begin) < p.kt_per_part ? KTL : kt_begin + p.kt_per_part);
   auto koff = [&](uint32_t round) {
     const uint32_t kt = kt_begin + wave + round * WAVES;
-    const bool ok = kt < kt_end;
+    bool ok = kt < kt_end;
     KOff o;
+    uint32_t ktw = kt;  // k-tile inside the weight strip
+    if constexpr (TOKSUM) {
+      // which expert's strip this k-tile of the token's row meets: a resource of its own per expert (the stack of all
+      // experts is larger than one resource's offsets may span)
+      const uint32_t j = ok ? kt / KT : 0;
+      ktw = kt - j * KT;
+      const uint32_t e = __builtin_amdgcn_readfirstlane(tok_ids[j]);
+      o.rw = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(uint32_t, tok_w[j])));
+      ok = ok && e < p.num_experts;
+      const size_t e_ok = e < p.num_experts ? e : 0;
+      o.wr = make_rsrc(static_cast<const char*>(p.w) + ((e_ok * (p.N / 16) + nt0) * KT) * 1024, NT * w_tile_stride);
+      o.sr = make_rsrc(static_cast<const char*>(p.scales) + (e_ok * G * p.N + static_cast<size_t>(nt0) * G * 16) * 2, NT * s_tile_stride);
+    }
     // readfirstlane pins the offsets to scalar registers (a vector offset would make every load a waterfall loop)
-    o.w = __builtin_amdgcn_readfirstlane(ok ? kt * 1024u : kOutOfRange);
-    o.s = __builtin_amdgcn_readfirstlane(ok ? kt * (GPT * 32u) : kOutOfRange);
-    o.z = __builtin_amdgcn_readfirstlane(ok ? kt * (GPT * 16u) : kOutOfRange);
+    o.w = __builtin_amdgcn_readfirstlane(ok ? ktw * 1024u : kOutOfRange);
+    o.s = __builtin_amdgcn_readfirstlane(ok ? ktw * (GPT * 32u) : kOutOfRange);
+    o.z = __builtin_amdgcn_readfirstlane(ok ? ktw * (GPT * 16u) : kOutOfRange);
     o.x = __builtin_amdgcn_readfirstlane(ok ? kt * 256u : kOutOfRange);
     return o;
   };
 
   auto load_slot = [&](Slot& s, int t, const KOff& o) {
     const bool upper = NT > 1 && t >= NT / 2;  // the up tiles of a fused gate_up workgroup lie pair_extra tiles further
+    if constexpr (TOKSUM) {
+      s.wq = __builtin_amdgcn_raw_buffer_load_b128(o.wr, w_off, t * w_tile_stride + o.w, 2);
+      s.sc[0] = __builtin_amdgcn_raw_buffer_load_b16(o.sr, s_off, t * s_tile_stride + o.s, 0);
+      s.rw = o.rw;
+      return;
+    }
     s.wq = __builtin_amdgcn_raw_buffer_load_b128(wr, w_off, t * w_tile_stride + (upper ? pair_w : 0) + o.w, 2);
 #pragma unroll
     for (int gi = 0; gi < GPT; ++gi) {
@@ -243,7 +293,7 @@ __global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKPar
   auto compute = [&](const Slot& s, const XBuf& b, const f32x4 (&sx)[GPT][MT], int t) {
 #pragma unroll
     for (int gi = 0; gi < GPT; ++gi) {
-      const float sc = T::lo_to_float(s.sc[gi]);
+      const float sc = TOKSUM ? T::lo_to_float(s.sc[gi]) * s.rw : T::lo_to_float(s.sc[gi]);
       const float ncz = HAS_ZP ? -(T::kMagic + static_cast<float>(s.zp[gi])) : -(T::kMagic + 8.0f);
       typename T::frag wf[SPG];
 #pragma unroll
@@ -422,12 +472,13 @@ __global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKPar
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        esid[mt][i] = static_cast<uint32_t>(p.sorted_ids[blockIdx.y * (16 * MT) + mt * 16 + 4 * lq + i]);
+        esid[mt][i] = (few || TOKSUM) ? ((mt == 0 && 4 * lq + i == 0) ? blockIdx.y : kNoRow)
+                                      : static_cast<uint32_t>(p.sorted_ids[blockIdx.y * (16 * MT) + mt * 16 + 4 * lq + i]);
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        erw[mt][i] = (!fused && esid[mt][i] < p.numel && p.topk_w) ? p.topk_w[esid[mt][i]] : 1.0f;
+        erw[mt][i] = (!TOKSUM && !fused && esid[mt][i] < p.numel && p.topk_w) ? p.topk_w[esid[mt][i]] : 1.0f;
   }
 
   if (GROUPED && NT > 1 && fused) {

@@ -207,7 +207,9 @@ Status MoeLayer::Forward(const std::vector<Tensor>& input_tensors, std::vector<T
     const int32_t* ids = topk_ids + begin * topk;
     const float* weights = topk_weights + begin * topk;
 
-    KsqCheck(ksq_moe_align(ids, numel, E, block_m, sorted_ids, expert_ids, num_post_pad, align_scratch, stream), "MoeLayer");
+    const bool few = !IsFp8() && tokens <= kFewTokens && !input_tensors[2].perm && !input_tensors[3].perm &&
+                     (2 * inter) % 32 == 0 && topk <= 32;
+    if (!few) KsqCheck(ksq_moe_align(ids, numel, E, block_m, sorted_ids, expert_ids, num_post_pad, align_scratch, stream), "MoeLayer");
     if (IsFp8()) {
       // InvokeFusedMoeKernelFunc with compute_dtype TYPE_BLOCK_FP8_E4M3 (moe_kernel_wrapper.cpp:435-456): activations
       // are quantized per token and 128 channels (scales [rows, k/128]) in front of each GEMM, silu*mul fused into
@@ -224,6 +226,17 @@ Status MoeLayer::Forward(const std::vector<Tensor>& input_tensors, std::vector<T
                                           num_post_pad, numel, 1, E, hidden_size, inter, block_m, dtype, stream),
                "MoeLayer");
       KsqCheck(ksq_moe_sum(cache3, out + begin * hidden_size * elem, tokens, topk, hidden_size, dtype, stream), "MoeLayer");
+      continue;
+    }
+    // A few decode tokens: two launches.  Every slot is a block of its own (no aligned permutation) in the first GEMM,
+    // which applies the activation in its epilogue; the second GEMM carries the sum over top-k.
+    if (few) {
+      KsqCheck(ksq_moe_w4a16_gate_up_silu(cache2, hidden + begin * hidden_size * elem, w1, w1_scale, nullptr, nullptr, ids,
+                                          nullptr, numel, topk, E, 2 * inter, hidden_size, group_size_, 16, dtype, stream),
+               "MoeLayer");
+      KsqCheck(ksq_moe_w4a16_down_sum(out + begin * hidden_size * elem, cache2, w2, w2_scale, weights, ids, tokens, topk, E,
+                                      hidden_size, inter, group_size_, dtype, stream),
+               "MoeLayer");
       continue;
     }
     // gate_up: every (token, slot) row reads hidden[token]; with act-order experts the row of a slot is gathered

@@ -52,6 +52,7 @@ SIGNATURES = {
                                  c_sz, c_i, c_p]),
     "ksq_moe_w4a16_gate_up_silu": (c_i, [c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_sz, c_sz, c_sz, c_sz, c_sz, c_sz, c_sz,
                                          c_i, c_p]),
+    "ksq_moe_w4a16_down_sum": (c_i, [c_p, c_p, c_p, c_p, c_p, c_p, c_sz, c_sz, c_sz, c_sz, c_sz, c_sz, c_i, c_p]),
     "ksq_w4a16_repack_act_order": (c_i, [c_p, c_p, c_p, c_sz, c_sz, c_p]),
     "ksq_permute_columns": (c_i, [c_p, c_p, c_p, c_sz, c_sz, c_i, c_p]),
     "ksq_w4a16_repack_rows": (c_i, [c_p, c_p, c_p, c_sz, c_sz, c_sz, c_p]),

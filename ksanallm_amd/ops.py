@@ -299,16 +299,30 @@ def moe_sum(x, out=None):
     return out
 
 
+FEW_TOKENS = 2   # up to this many tokens the int4 MoE block runs its two-launch form (ksq_moe_w4a16_down_sum)
+
+
 def fused_moe_w4a16(x, w13_packed, s13_packed, w2_packed, s2_packed, topk_ids, topk_w, E, hidden, inter, group,
                     block_m=None):
     """InvokeFusedMoe<T,false> for int4 weights (S/kernels/nvidia/moe_kernel_wrapper.cpp:463-654):
     align -> GEMM1 -> silu*mul -> GEMM2 (* routed weight) -> sum over top-k."""
     T, topk = topk_ids.shape
     numel = T * topk
+    tw = topk_w.reshape(-1).to(torch.float32).contiguous()
+    if block_m is None and T <= FEW_TOKENS and (2 * inter) % 32 == 0:
+        # a few decode tokens: two launches - the first GEMM with every slot a block of its own (no aligned
+        # permutation) and the activation in its epilogue, the second with the sum over top-k in it
+        ids = topk_ids.reshape(-1).to(torch.int32).contiguous()
+        c2 = torch.empty((numel, inter), dtype=x.dtype, device=x.device)
+        _l.check(_lib.ksq_moe_w4a16_gate_up_silu(_ptr(c2), _ptr(x), _ptr(w13_packed), _ptr(s13_packed), None, None, _ptr(ids),
+                                                 None, numel, topk, E, 2 * inter, hidden, group, 16, _dt(x), _stream()))
+        out = torch.empty((T, hidden), dtype=x.dtype, device=x.device)
+        _l.check(_lib.ksq_moe_w4a16_down_sum(_ptr(out), _ptr(c2), _ptr(w2_packed), _ptr(s2_packed), _ptr(tw), _ptr(ids), T,
+                                             topk, E, hidden, inter, group, _dt(x), _stream()))
+        return out
     if block_m is None:
         block_m = _lib.ksq_moe_block_m(numel, E)
     sorted_ids, expert_ids, npp = moe_align_block_size(topk_ids, E, block_m)
-    tw = topk_w.reshape(-1).to(torch.float32).contiguous()
     # the activation runs in the first GEMM's epilogue, except with 128-row blocks (a size ksq_moe_block_m no longer
     # picks but a caller may ask for), where the two launches measured faster (64 rows per expert: 1.75 against 1.87 ms)
     if block_m != 128 and (2 * inter) % 32 == 0:

@@ -335,6 +335,97 @@ def test_moe_block_benchmark_token_counts(ops, oracle, T):
                      weights_rounded=rounded, rel_l2_max=5e-3 * (2 ** 0.5 if rounded else 1.0))
 
 
+@pytest.mark.parametrize("dtype", [H.F16, H.BF16])
+@pytest.mark.parametrize("T,E,topk,hidden,inter", [(1, 16, 4, 256, 128), (2, 16, 8, 512, 256), (3, 8, 2, 384, 128), (8, 16, 4, 256, 384),
+                                                   (1, 256, 8, 7168, 2048)])
+def test_few_tokens_without_alignment_and_with_the_sum_in_the_second_gemm(ops, oracle, dtype, T, E, topk, hidden, inter):
+    """A handful of slots: the first GEMM with every slot a block of its own (sorted_ids NULL, the router's ids as they
+    are) gives the bits of the aligned form; the second GEMM with the sum over top-k in it agrees with the oracle's
+    block (its fp32 sum is rounded once where the reference rounds every expert's share first)."""
+    from ksanallm_amd import lib as L
+    distinct = min(E, 8)
+    base = make_moe(oracle, 5300 + T + hidden, distinct, hidden, inter, T, topk, 128, dtype)
+    d = dict(base)
+    d["E"] = E
+    for k in ("w13", "w2", "s13", "s2"):
+        d[k] = base[k].repeat((E // distinct, 1, 1))
+    logits = torch.randn((T, E), generator=H.gen(79 + T))
+    tw, ids = torch.topk(torch.softmax(logits, -1), topk, dim=-1)
+    d["ids"], d["tw"] = ids.to(torch.int32).contiguous(), tw.float().contiguous()
+    w13p, s13p, w2p, s2p = pack_moe(ops, d)
+    numel = T * topk
+    x, idf, twf = d["x"].cuda(), d["ids"].cuda().reshape(-1), d["tw"].cuda().reshape(-1)
+    lib = L.load()
+    stream = torch.cuda.current_stream().cuda_stream
+    td = H.TORCH_DT[dtype]
+    # first GEMM + activation: every slot its own block, against the aligned form
+    s, e, npp = ops.moe_align_block_size(d["ids"].cuda(), E, 16)
+    want = ops.moe_w4a16_gate_up_silu(x, w13p, s13p, s, e, npp, numel, topk, E, 2 * inter, hidden, 128, 16)
+    c2 = torch.full((numel, inter), float("nan"), dtype=td, device="cuda")
+    L.check(lib.ksq_moe_w4a16_gate_up_silu(c2.data_ptr(), x.data_ptr(), w13p.data_ptr(), s13p.data_ptr(), None, None,
+                                           idf.data_ptr(), None, numel, topk, E, 2 * inter, hidden, 128, 16, dtype, stream))
+    assert torch.equal(c2.view(torch.int16), want.view(torch.int16))
+    # plain grouped GEMM in the same form (second GEMM without the sum)
+    want3 = ops.moe_w4a16_gemm(c2, w2p, s2p, twf, s, e, npp, numel, 1, E, hidden, inter, 128, 16)
+    c3 = torch.full((numel, hidden), float("nan"), dtype=td, device="cuda")
+    L.check(lib.ksq_moe_w4a16_gemm(c3.data_ptr(), c2.data_ptr(), w2p.data_ptr(), s2p.data_ptr(), None, twf.data_ptr(), None,
+                                   idf.data_ptr(), None, numel, 1, E, hidden, inter, 128, 16, dtype, stream))
+    assert torch.equal(c3.view(torch.int16), want3.view(torch.int16))
+    # second GEMM with the sum in it, and the whole block through the wrapper, against the oracle
+    out = torch.full((T, hidden), float("nan"), dtype=td, device="cuda")
+    L.check(lib.ksq_moe_w4a16_down_sum(out.data_ptr(), c2.data_ptr(), w2p.data_ptr(), s2p.data_ptr(), twf.data_ptr(),
+                                       idf.data_ptr(), T, topk, E, hidden, inter, 128, dtype, stream))
+    # the oracle of this launch: the second GEMM's fp32 rows (routing weight applied) of the same activations, summed
+    # over top-k without the rounding to T in between
+    rows = oracle.moe_w4a16_gemm(H.bits_of(c2.cpu()), d["w2"].numpy(), H.bits_of(d["s2"]), d["ids"].numpy(), d["tw"].numpy(),
+                                 1, 128, True, dtype)
+    H.check_gemm(out, rows.reshape(T, topk, hidden).astype(np.float64).sum(1).astype(np.float32), dtype, "down + sum T=%d" % T)
+    # and the reference's own sequence (every expert's share rounded to T, then summed in T): the block's rel-L2 bar
+    ref = oracle.from_bits(oracle.moe_forward(H.bits_of(d["x"]), d["w13"].numpy(), H.bits_of(d["s13"]), d["w2"].numpy(),
+                                              H.bits_of(d["s2"]), d["ids"].numpy(), d["tw"].numpy(), 128, dtype), dtype)
+    H.check_gemm(out, ref, dtype, "few-token block T=%d" % T, weights_rounded=True)
+    if T <= 2:
+        whole = ops.fused_moe_w4a16(x, w13p, s13p, w2p, s2p, d["ids"].cuda(), d["tw"].cuda(), E, hidden, inter, 128)
+        assert torch.equal(whole.view(torch.int16), out.view(torch.int16))
+
+
+def test_few_tokens_form_drops_ids_outside_the_experts_and_rejects_what_it_cannot_do(ops, oracle):
+    from ksanallm_amd import lib as L
+    E, topk, hidden, inter, T = 8, 4, 256, 128, 2
+    d = make_moe(oracle, 5350, E, hidden, inter, T, topk, 128, H.BF16)
+    w13p, s13p, w2p, s2p = pack_moe(ops, d)
+    ids = d["ids"].clone()
+    ids[0, 1] = E + 3              # an id the alignment would drop
+    ids[1, 2] = -1
+    idf, twf = ids.cuda().reshape(-1), d["tw"].cuda().reshape(-1)
+    lib, stream = L.load(), torch.cuda.current_stream().cuda_stream
+    numel = T * topk
+    c2 = torch.full((numel, inter), 7.0, dtype=torch.bfloat16, device="cuda")
+    xd = d["x"].cuda()
+    L.check(lib.ksq_moe_w4a16_gate_up_silu(c2.data_ptr(), xd.data_ptr(), w13p.data_ptr(), s13p.data_ptr(), None,
+                                           None, idf.data_ptr(), None, numel, topk, E, 2 * inter, hidden, 128, 16, H.BF16, stream))
+    assert torch.all(c2[1] == 7.0) and torch.all(c2[6] == 7.0)          # untouched rows
+    out = torch.empty((T, hidden), dtype=torch.bfloat16, device="cuda")
+    L.check(lib.ksq_moe_w4a16_down_sum(out.data_ptr(), c2.data_ptr(), w2p.data_ptr(), s2p.data_ptr(), twf.data_ptr(),
+                                       idf.data_ptr(), T, topk, E, hidden, inter, 128, H.BF16, stream))
+    # the same with the two slots routed to a real expert at weight zero
+    ids2, tw2 = ids.clone(), d["tw"].clone()
+    ids2[0, 1], ids2[1, 2] = 0, 0
+    tw2[0, 1], tw2[1, 2] = 0.0, 0.0
+    out2 = torch.empty_like(out)
+    c2b = c2.clone()
+    c2b[1], c2b[6] = 0, 0
+    tw2f, ids2f = tw2.cuda().reshape(-1), ids2.cuda().reshape(-1)
+    L.check(lib.ksq_moe_w4a16_down_sum(out2.data_ptr(), c2b.data_ptr(), w2p.data_ptr(), s2p.data_ptr(), tw2f.data_ptr(),
+                                       ids2f.data_ptr(), T, topk, E, hidden, inter, 128, H.BF16, stream))
+    torch.cuda.synchronize()
+    assert torch.equal(out.view(torch.int16), out2.view(torch.int16))
+    assert lib.ksq_moe_w4a16_down_sum(out.data_ptr(), c2.data_ptr(), w2p.data_ptr(), s2p.data_ptr(), twf.data_ptr(),
+                                      idf.data_ptr(), 9, topk, E, hidden, inter, 128, H.BF16, stream) == 1
+    assert lib.ksq_moe_w4a16_gemm(out.data_ptr(), c2.data_ptr(), w2p.data_ptr(), s2p.data_ptr(), None, None, None,
+                                  idf.data_ptr(), None, numel, 1, E, hidden, inter, 128, 32, H.BF16, stream) == 1
+
+
 # ---- block-quantized fp8 experts -------------------------------------------------------------------------------------
 
 def _fp8_experts(oracle, seed, E, n, k):
