@@ -483,14 +483,19 @@ def cpu_baseline(keeps, L, ops):
                 for T in sorted(k["x"]):
                     rows = min(T, 4)            # per-expert dequantization dominates: a few tokens already touch 30 experts
                     ids = (k["ids"][T][:rows] % d).contiguous().numpy().astype(np.int32)   # expert e holds slab e % distinct
+                    # a few tokens run the second GEMM with the sum over top-k in it (fp32, rounded once): held against
+                    # the same sum in fp32; otherwise every expert's share is rounded to T and summed in T, as the
+                    # reference's kernels do
+                    few = T <= ops.FEW_TOKENS
                     t0 = time.perf_counter()
-                    ref = orc.moe_forward(_bits(k["x"][T][:rows]), w13, s13, w2, s2, ids, k["tw"][T][:rows].numpy(), 128, orc.BF16)
+                    ref = orc.moe_forward(_bits(k["x"][T][:rows]), w13, s13, w2, s2, ids, k["tw"][T][:rows].numpy(), 128, orc.BF16,
+                                          sum_fp32=few)
                     t += time.perf_counter() - t0
                     flops += 2 * rows * k["topk"] * 3 * k["hidden"] * k["inter"]
                     sample.append("moe:T=%d%s" % (T, "" if rows == T else "[tokens 0..%d]" % (rows - 1)))
                     if T in k["out"]:
                         # the oracle hands back the block's output as bit patterns of T, like the kernel's buffer
-                        ref_f = orc.from_bits(np.asarray(ref).reshape(rows, -1), orc.BF16)
+                        ref_f = ref if few else orc.from_bits(np.asarray(ref).reshape(rows, -1), orc.BF16)
                         # two GEMMs in a row: where both run on the tile kernel, which rounds every dequantized weight
                         # to T, two independent rounding errors compound
                         tiled = L.load().ksq_moe_block_m(T * k["topk"], k["E"]) >= 128

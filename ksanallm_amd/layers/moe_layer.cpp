@@ -207,7 +207,7 @@ Status MoeLayer::Forward(const std::vector<Tensor>& input_tensors, std::vector<T
     const int32_t* ids = topk_ids + begin * topk;
     const float* weights = topk_weights + begin * topk;
 
-    const bool few = !IsFp8() && tokens <= kFewTokens && !input_tensors[2].perm && !input_tensors[3].perm &&
+    const bool few = !IsFp8() && tokens <= kFewTokens && numel <= 64 && !input_tensors[2].perm && !input_tensors[3].perm &&
                      (2 * inter) % 32 == 0 && topk <= 32;
     if (!few) KsqCheck(ksq_moe_align(ids, numel, E, block_m, sorted_ids, expert_ids, num_post_pad, align_scratch, stream), "MoeLayer");
     if (IsFp8()) {

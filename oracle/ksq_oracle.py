@@ -395,14 +395,18 @@ def moe_sum(x_bits, dtype):
     return out
 
 
-def moe_forward(x_bits, w13, s13, w2, s2, topk_ids, topk_w, group, dtype):
+def moe_forward(x_bits, w13, s13, w2, s2, topk_ids, topk_w, group, dtype, sum_fp32=False):
     """Whole int4 MoE block as S/kernels/nvidia/moe_kernel_wrapper.cpp:616-652 sequences it:
-    GEMM1 (no routed weight) -> T, silu*mul -> T, GEMM2 (* routed weight) -> T, sum over top-k in T."""
+    GEMM1 (no routed weight) -> T, silu*mul -> T, GEMM2 (* routed weight) -> T, sum over top-k in T (bit patterns of T).
+    sum_fp32: the last two steps without their roundings - the second GEMM's fp32 rows summed over top-k, returned as
+    fp32 values: the fp32-accumulated reference of a second GEMM that carries the sum."""
     T, topk = np.asarray(topk_ids).shape
     c1 = moe_w4a16_gemm(x_bits, w13, s13, topk_ids, topk_w, topk, group, False, dtype)
     c1b = to_bits(c1, dtype)
     c2b = silu_mul(c1b, dtype)
     c3 = moe_w4a16_gemm(c2b, w2, s2, topk_ids, topk_w, 1, group, True, dtype)
+    if sum_fp32:
+        return np.asarray(c3, np.float64).reshape(T, topk, -1).sum(1).astype(np.float32)
     c3b = to_bits(c3, dtype).reshape(T, topk, -1)
     return moe_sum(c3b, dtype)
 
