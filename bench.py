@@ -86,6 +86,7 @@ def kernel_label(L, kind, prefix, M, N, K, dt):
 
 # ------------------------------------------------------------------------------------------------ workloads
 CONSTANT_DATA = ""   # --constant-data: "all", "weights" or "activations" hold one value each (configs 1-4)
+FP8_SHAPE = None     # --fp8-shape M,N,K: config 4 becomes one GEMM of that shape
 
 
 def w4a16_cases(ops, L, cfg, shapes, Ms, dtype, awq, x_std, s_lo, s_hi):
@@ -349,6 +350,9 @@ def build(cfg, ops, L):
         return w4a16_cases(ops, L, 3, [("up", 25600, 5120), ("down", 5120, 25600)], [2048, 4096, 8192], "f16", False, 0.5,
                            0.002, 0.01)
     if cfg == 4:
+        if FP8_SHAPE:   # --fp8-shape: one GEMM of a shape of the caller's choice (clock and tile-count experiments)
+            m, n, k = FP8_SHAPE
+            return fp8_cases(ops, L, 4, [("shape", n, k)], [m])
         return fp8_cases(ops, L, 4, [("up", 18432, 7168), ("down", 7168, 18432)], [1, 16, 128, 1024, 4096])
     if cfg == 5:
         return moe_cases(ops, L, 5, [1, 64, 512, 4096])
@@ -400,6 +404,47 @@ def time_case(c, use_graph):
         end.record()
     torch.cuda.synchronize()
     return start.elapsed_time(end) / reps
+
+
+def sample_clock(c, seconds):
+    """Launches case c back to back for `seconds` while a thread reads the shader clock from rocm-smi every 50 ms:
+    the clock the power management grants this kernel on this data, and the launch time at that clock."""
+    import re
+    import subprocess
+    import threading
+    samples, stop = [], []
+
+    def reader():
+        while not stop:
+            try:
+                out = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True, timeout=5).stdout
+                samples.extend(int(m) for m in re.findall(r"sclk clock level: \d+: \((\d+)Mhz\)", out))
+            except Exception:
+                pass
+            time.sleep(0.05)
+
+    for _ in range(3):
+        c.launch()
+    torch.cuda.synchronize()
+    th = threading.Thread(target=reader)
+    th.start()
+    beg, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    n, t0 = 0, time.time()
+    beg.record()
+    while time.time() - t0 < seconds:
+        for _ in range(10):
+            c.launch()
+        torch.cuda.synchronize()
+        n += 10
+    end.record()
+    torch.cuda.synchronize()
+    stop.append(1)
+    th.join()
+    row = {"case": c.name, "kernel": c.kernel, "us": round(beg.elapsed_time(end) / n * 1e3, 2), "launches": n,
+           "sclk_samples": len(samples)}
+    if samples:
+        row.update(sclk_mhz_mean=round(sum(samples) / len(samples), 1), sclk_mhz_min=min(samples), sclk_mhz_max=max(samples))
+    return row
 
 
 # ------------------------------------------------------------------------------------------------ CPU baseline
@@ -576,6 +621,11 @@ def main():
                     help="dense W4A16 and block-fp8 cases: every weight code and scale, every activation, or both (the "
                     "default) hold one value (a valid GEMM on operands that never toggle), to show how much of the "
                     "kernel's time is the clock the data allows; not a benchmark figure")
+    ap.add_argument("--fp8-shape", default="", help="M,N,K: configuration 4 becomes one blockwise-FP8 GEMM of that shape "
+                    "(a side measurement, e.g. tile counts that fill all CUs or three quarters of them)")
+    ap.add_argument("--sample-clock", type=float, default=0.0, metavar="SECONDS", help="instead of the benchmark: loop "
+                    "every selected case for that long while reading the shader clock from rocm-smi every 50 ms, and "
+                    "print launch time and clock per case (what the power management grants the kernel on this data)")
     ap.add_argument("--library-gemm", action="store_true", help="run only the vendor library's plain GEMMs (torch.matmul "
                     "fp16 / bf16, torch._scaled_mm e4m3; no dequantization, no block scales) at the prefill shapes of "
                     "configurations 3 and 4 and exit: what a dense GEMM reaches on this part, beside the MFMA peak")
@@ -596,8 +646,10 @@ def main():
         print(json.dumps({"copy_bytes_read": n, "copy_bytes_written": n, "launches": 5}))
         return
 
-    global CONSTANT_DATA
+    global CONSTANT_DATA, FP8_SHAPE
     CONSTANT_DATA = args.constant_data
+    if args.fp8_shape:
+        FP8_SHAPE = tuple(int(v) for v in args.fp8_shape.split(","))
     if args.library_gemm:
         library_gemm(args.steps, args.warmup)
         return
@@ -620,6 +672,16 @@ def main():
         cases = [c for c in cases if args.only in c.name]
         if not cases:
             raise SystemExit("--only matched no case")
+
+    if args.sample_clock > 0:
+        rows = [sample_clock(c, args.sample_clock) for c in cases if c.flops > 0 or not whole]
+        for r in rows:
+            print("%-28s %-30s %9.1f us  sclk %s MHz (min %s, max %s, %d samples)" % (
+                r["case"], r["kernel"][:30], r["us"], r.get("sclk_mhz_mean"), r.get("sclk_mhz_min"), r.get("sclk_mhz_max"),
+                r["sclk_samples"]), file=sys.stderr)
+        print(json.dumps({"sample_clock_seconds": args.sample_clock, "data": "synthetic, constant %s" % CONSTANT_DATA if
+                          CONSTANT_DATA else "synthetic", "rows": rows}))
+        return
 
     use_graph = not args.no_graph
     # one captured graph per turn of the weight-copy rotation; step i replays graph i % n_graphs.  The whole metric
