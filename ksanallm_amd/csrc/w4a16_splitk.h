@@ -26,6 +26,8 @@
 // row depends only on its own row of x, and those rows are never stored.
 #pragma once
 
+#include <type_traits>
+
 #include "ksq_common.h"
 #include "splitk_reduce.h"
 
@@ -279,18 +281,21 @@ __global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKPar
   asm volatile("" : "+v"(magic2));  // no instruction: keeps the value in a VGPR so the three-operand form applies
   const uint32_t nmask = p.nibble_mask;
 
-  auto sum_x = [&](const XBuf& b, f32x4 (&sx)[GPT][MT]) {
+  // LIVE: the row tiles that are multiplied (all MT, or one of two when the block's second row tile holds no row)
+  auto sum_x = [&](auto live_c, const XBuf& b, f32x4 (&sx)[GPT][MT]) {
+    constexpr int LIVE = decltype(live_c)::value;
 #pragma unroll
     for (int gi = 0; gi < GPT; ++gi)
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
+      for (int mt = 0; mt < LIVE; ++mt) {
         f32x4 r{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int d = gi * SPG; d < (gi + 1) * SPG; ++d) r = T::mfma(as_frag<T>(b.xf[mt][d]), ones, r);
         sx[gi][mt] = r;
       }
   };
-  auto compute = [&](const Slot& s, const XBuf& b, const f32x4 (&sx)[GPT][MT], int t) {
+  auto compute = [&](auto live_c, const Slot& s, const XBuf& b, const f32x4 (&sx)[GPT][MT], int t) {
+    constexpr int LIVE = decltype(live_c)::value;
 #pragma unroll
     for (int gi = 0; gi < GPT; ++gi) {
       const float sc = TOKSUM ? T::lo_to_float(s.sc[gi]) * s.rw : T::lo_to_float(s.sc[gi]);
@@ -299,7 +304,7 @@ __global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKPar
 #pragma unroll
       for (int d = 0; d < SPG; ++d) wf[d] = dequant_magic_fast<T>(s.wq[gi * SPG + d], nmask, magic2);
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
+      for (int mt = 0; mt < LIVE; ++mt) {
         f32x4 r = HAS_ZP ? f32x4{0.f, 0.f, 0.f, 0.f} : sx[gi][mt];
 #pragma unroll
         for (int d = 0; d < SPG; ++d) r = T::mfma(as_frag<T>(b.xf[mt][gi * SPG + d]), wf[d], r);
@@ -315,6 +320,22 @@ __global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKPar
   // followed, in the register form, by the x fragments; a group is refilled for round cur+LOOK while round cur is
   // consumed, so LOOK-1 whole groups stay in flight behind every wait.  The round count is uniform over the workgroup
   // and a multiple of LOOK (of the rounds of a chunk in the LDS form), the surplus rounds load zeros.
+  // The main loop exists once per number of row tiles that are multiplied.  A 32-row expert block whose second row
+  // tile holds no slot (an expert with at most 16 rows: at 16 rows per expert on average, every second one) runs the
+  // loop over one row tile: the MFMAs, sum-of-x MFMAs and scale FMAs of the empty tile are what puts the two-tile form
+  // over a SIMD's issue slots.  The choice is made once per workgroup, outside the loop.
+  bool second_empty = false;
+  if constexpr (GROUPED && MT == 2) second_empty = __builtin_amdgcn_ballot_w64(xrow[1] != kNoRow) == 0;
+  auto run_live = [&](auto&& loop) {
+    if constexpr (GROUPED && MT == 2) {
+      if (second_empty)
+        loop(std::integral_constant<int, 1>{});
+      else
+        loop(std::integral_constant<int, 2>{});
+    } else {
+      loop(std::integral_constant<int, MT>{});
+    }
+  };
   const uint32_t slice_len = kt_end - kt_begin;
   Slot slot[LOOK][NT];
   if constexpr (!XLDS) {
@@ -328,15 +349,16 @@ __global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKPar
       load_x(xb[j], o);
       __builtin_amdgcn_sched_barrier(0);  // keep the groups in issue order, the waits below count on it
     }
+    auto loop = [&](auto live_c) {
     for (uint32_t it = 0; it < rounds; it += LOOK) {
 #pragma unroll
       for (int h = 0; h < LOOK; ++h) {
         const KOff o = koff(it + h + LOOK);  // past the last round this is out of range by construction
         f32x4 sx[GPT][MT];
-        sum_x(xb[h], sx);
+        sum_x(live_c, xb[h], sx);
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
-          compute(slot[h][t], xb[h], sx, t);
+          compute(live_c, slot[h][t], xb[h], sx, t);
           // the refill must be issued here, not sunk below the remaining math: the barriers pin it in place
           __builtin_amdgcn_sched_barrier(0);
           load_slot(slot[h][t], t, o);
@@ -346,6 +368,8 @@ __global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKPar
         __builtin_amdgcn_sched_barrier(0);
       }
     }
+    };
+    run_live(loop);
   } else {
     // Rows of the block that hold data (they come first: pad slots of an expert's block lie at its end).
     uint32_t nrows;
@@ -420,6 +444,7 @@ __global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKPar
     wait_staged();
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");  // no LDS read may move above the barrier
+    auto loop = [&](auto live_c) {
     for (uint32_t c = 0; c < nchunks; ++c) {
       if (c + 1 < nchunks) stage_chunk(c + 1);  // into the buffer chunk c-1 used: every wavefront is past the barrier behind it
 #pragma unroll
@@ -439,10 +464,10 @@ __global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKPar
             for (int d = 0; d < 4; ++d) xb.xf[mt][d] = u32x4{0u, 0u, 0u, 0u};
         }
         f32x4 sx[GPT][MT];
-        sum_x(xb, sx);
+        sum_x(live_c, xb, sx);
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
-          compute(slot[h][t], xb, sx, t);
+          compute(live_c, slot[h][t], xb, sx, t);
           __builtin_amdgcn_sched_barrier(0);
           load_slot(slot[h][t], t, o);
           __builtin_amdgcn_sched_barrier(0);
@@ -452,6 +477,8 @@ __global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKPar
       __builtin_amdgcn_s_barrier();  // chunk c+1 is in LDS for everyone, and everyone is done with chunk c
       asm volatile("" ::: "memory");
     }
+    };
+    run_live(loop);
   }
 
   // ---- cross-wavefront reduction in wavefront order
