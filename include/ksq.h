@@ -325,6 +325,17 @@ int ksq_moe_fp8_blockwise_gemm(void* out, const void* a_q, const void* a_s, int 
                                const void* b_s, const void* topk_w, const void* sorted_ids, const void* expert_ids,
                                const void* num_post_pad, size_t numel, size_t top_k, size_t E, size_t n, size_t k,
                                size_t block_m, int out_dtype, void* stream);
+/* ksq_moe_w4a16_down_sum for block-quantized fp8 experts: the second GEMM and the sum over top-k in one launch, for up
+ * to 8 tokens.  a_q [tokens * top_k, k] e4m3 with scales a_s [tokens * top_k, k/128] row-major (the second
+ * quantization's output), b / b_s the experts' packed weights and block scales, topk_w / topk_ids [tokens, top_k];
+ * out [tokens, n], the fp32 sum over a token's experts rounded once.  sorted_ids NULL in ksq_moe_fp8_blockwise_gemm is
+ * the matching form of the first GEMM (block_m 16, at most 64 slots, expert_ids = topk_ids).
+ * Replaces the fused_moe_kernel launch + InvokeMoeSum pair of InvokeFusedMoe for the decode steps of a few sequences
+ * (S/kernels/nvidia/moe_kernel_wrapper.cpp:435-456, 640-652). */
+int ksq_moe_fp8_down_sum(void* out, const void* a_q, const void* a_s, const void* b, const void* b_s, const void* topk_w,
+                         const void* topk_ids, size_t tokens, size_t top_k, size_t E, size_t n, size_t k, int out_dtype,
+                         void* stream);
+
 
 /* Router: softmax over the E gating logits of every token in fp32, the top_k largest probabilities in descending
  * order (ties: lower expert id first), weights = probability * routed_scaling_factor, optionally renormalised to

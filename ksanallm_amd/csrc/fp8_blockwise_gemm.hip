@@ -34,6 +34,13 @@ struct Fp8Params {
   const int32_t* num_post_pad;
   const float* topk_w;
   uint32_t numel, top_k, scale_rows;  // scale_rows = ceil(N/128): rows of one expert's b_s
+  // Grouped form for a handful of slots (sorted_ids == nullptr): expert_ids holds the router's ids [numel] as they are
+  // and block b is slot b alone (row b / top_k of a, expert expert_ids[b], output row b; an id outside
+  // [0, num_experts) leaves the row unwritten).  TOKSUM instances: block b is token b, whose top_k rows of a
+  // [numel, kb_per_expert * 128] lie one behind the other as one row of K = top_k * kb_per_expert * 128 values; k-block
+  // kb of it meets k-block kb % kb_per_expert of expert expert_ids[b * top_k + kb / kb_per_expert], the weight scale
+  // times the routing weight topk_w[...]; the fp32 sum over all of K is output row b of [tokens, N].
+  uint32_t num_experts, kb_per_expert;
 };
 
 __device__ __forceinline__ f32x4 mfma_fp8_128(i32x8 a, i32x8 b, f32x4 c) {
@@ -53,22 +60,37 @@ __device__ __forceinline__ i32x8 load32(const uint8_t* p) {
 // GROUPED: the MoE form.  Row block blockIdx.y is one block of the aligned slot permutation: slot s reads activation
 // row s / top_k (pad slots carry s >= numel), the weights and weight scales are those of expert expert_ids[block], the
 // result goes to out[s, :] (times topk_w[s] when given).  Blocks past num_post_pad leave at once.
-template <typename TO, int MT, int NT, int WAVES, int LOOK, bool GROUPED = false>
+template <typename TO, int MT, int NT, int WAVES, int LOOK, bool GROUPED = false, bool TOKSUM = false>
 __global__ void __launch_bounds__(WAVES * 64) fp8_splitk_kernel(Fp8Params p) {
+  static_assert(!TOKSUM || (GROUPED && MT == 1), "the token-sum form is a grouped decode form");
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lrow = lane & 15;
   const int lq = lane >> 4;
-  const uint32_t KB = p.K / 128;
+  const uint32_t KB = TOKSUM ? p.kb_per_expert : p.K / 128;  // k-blocks of a weight strip
+  const uint32_t KBL = p.K / 128;                            // k-blocks of a row of a
   const uint32_t n0 = blockIdx.x * (16 * NT);  // NT strips of 16 weight rows share every activation fragment
   const uint32_t m0 = blockIdx.y * (16 * MT);
 
   __shared__ f32x4 red[WAVES][NT][MT][64];
+  __shared__ uint32_t tok_ids[TOKSUM ? 32 : 1];
+  __shared__ float tok_w[TOKSUM ? 32 : 1];
 
+  const bool few = GROUPED && p.sorted_ids == nullptr;  // a handful of slots: one per block, no aligned permutation
   size_t expert = 0;
   if (GROUPED) {
-    if (m0 >= static_cast<uint32_t>(p.num_post_pad[0])) return;  // uniform: the whole workgroup leaves
-    expert = static_cast<size_t>(p.expert_ids[blockIdx.y]);
+    if (TOKSUM) {
+      if (threadIdx.x < p.top_k) {
+        tok_ids[threadIdx.x] = static_cast<uint32_t>(p.expert_ids[blockIdx.y * p.top_k + threadIdx.x]);
+        tok_w[threadIdx.x] = p.topk_w ? p.topk_w[blockIdx.y * p.top_k + threadIdx.x] : 1.0f;
+      }
+      __syncthreads();
+    } else {
+      if (!few && m0 >= static_cast<uint32_t>(p.num_post_pad[0])) return;  // uniform: the whole workgroup leaves
+      const uint32_t e = static_cast<uint32_t>(p.expert_ids[blockIdx.y]);
+      if (few && e >= p.num_experts) return;
+      expert = e;
+    }
   }
   // fragment (strip, k-block) at ((expert*N/16 + strip)*KB + kb) * 2048; this lane's two 16-byte halves at 16*lane, +1024
   const uint8_t* bptr = p.b + ((expert * (p.N / 16) + n0 / 16) * KB) * 2048 + lane * 16;
@@ -78,7 +100,10 @@ __global__ void __launch_bounds__(WAVES * 64) fp8_splitk_kernel(Fp8Params p) {
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     uint32_t row = m0 + mt * 16 + lrow;
-    if (GROUPED) {
+    if (few || TOKSUM) {
+      // every lane reads the block's one row (their results are not stored)
+      row = TOKSUM ? blockIdx.y : blockIdx.y / p.top_k;
+    } else if (GROUPED) {
       uint32_t sid = static_cast<uint32_t>(p.sorted_ids[row]);
       sid = sid < p.numel ? sid : p.numel - 1;  // pad slots read some valid row; their results are not stored
       row = sid / p.top_k;
@@ -103,15 +128,30 @@ __global__ void __launch_bounds__(WAVES * 64) fp8_splitk_kernel(Fp8Params p) {
   };
   Stage ring[LOOK];
   auto load_stage = [&](Stage& s, uint32_t kb) {
-    const bool live = kb < KB;
-    kb = live ? kb : KB - 1;
+    bool live = kb < KBL;
+    kb = live ? kb : KBL - 1;
+    uint32_t kbw = kb;           // k-block inside the weight strip
+    const uint8_t* wbase = bptr;
+    const float* sbase = bs;
+    float rw = 1.0f;
+    if constexpr (TOKSUM) {
+      // the expert whose strip this k-block of the token's row meets (wave-uniform: scalar address arithmetic)
+      const uint32_t j = kb / KB;
+      kbw = kb - j * KB;
+      const uint32_t e = __builtin_amdgcn_readfirstlane(tok_ids[j]);
+      rw = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(uint32_t, tok_w[j])));
+      live = live && e < p.num_experts;
+      const size_t e_ok = e < p.num_experts ? e : 0;
+      wbase = bptr + (e_ok * (p.N / 16) * KB) * 2048;
+      sbase = bs + e_ok * p.scale_rows * KB;
+    }
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
-      const uint8_t* wp = bptr + (static_cast<size_t>(nt) * KB + kb) * 2048;
+      const uint8_t* wp = wbase + (static_cast<size_t>(nt) * KB + kbw) * 2048;
       s.w0[nt] = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(wp));
       s.w1[nt] = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(wp + 1024));
     }
-    s.ws = live ? bs[kb] : 0.f;
+    s.ws = live ? sbase[kbw] * rw : 0.f;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       const i32x4* ap = reinterpret_cast<const i32x4*>(aptr[mt] + static_cast<size_t>(kb) * 128);
@@ -135,7 +175,7 @@ __global__ void __launch_bounds__(WAVES * 64) fp8_splitk_kernel(Fp8Params p) {
     }
   };
 
-  const uint32_t rounds = (KB + WAVES - 1) / WAVES;  // k-blocks this wavefront may own
+  const uint32_t rounds = (KBL + WAVES - 1) / WAVES;  // k-blocks this wavefront may own
 #pragma unroll
   for (int h = 0; h < LOOK; ++h) {
     load_stage(ring[h], wave + h * WAVES);
@@ -162,7 +202,11 @@ __global__ void __launch_bounds__(WAVES * 64) fp8_splitk_kernel(Fp8Params p) {
   static_assert(MT <= 2, "the epilogue selects between two row tiles");
   uint32_t esid0 = 0, esid1 = 0;
   float erw0 = 1.0f, erw1 = 1.0f;
-  if (GROUPED) {
+  if (few || TOKSUM) {
+    esid0 = (lane & 15) == 0 ? blockIdx.y : 0xffffffffu;  // the block's one row; the others are not stored
+    esid1 = 0xffffffffu;
+    if (!TOKSUM && p.topk_w && esid0 < p.numel) erw0 = p.topk_w[esid0];
+  } else if (GROUPED) {
     esid0 = static_cast<uint32_t>(p.sorted_ids[m0 + (lane & 15)]);
     if (MT > 1) esid1 = static_cast<uint32_t>(p.sorted_ids[m0 + 16 + (lane & 15)]);
     if (p.topk_w) {
@@ -409,7 +453,11 @@ KSQ_EXPORT int ksq_moe_fp8_blockwise_gemm(void* out, const void* a_q, const void
                                           size_t E, size_t n, size_t k, size_t block_m, int out_dtype, void* stream) {
   const char* fn = "ksq_moe_fp8_blockwise_gemm";
   if (!a_q || !a_s || !b || !b_s || !out) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: null pointer", fn);
-  if (!sorted_ids || !expert_ids || !num_post_pad) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: null index buffer", fn);
+  // sorted_ids == NULL: a handful of slots, one per 16-row block, with the router's ids in expert_ids
+  const bool few = !sorted_ids;
+  if (!expert_ids || (!few && !num_post_pad)) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: null index buffer", fn);
+  if (few && (block_m != 16 || numel > 64))
+    return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: without sorted_ids every slot is a 16-row block of its own: block_m 16, at most 64 slots", fn);
   if (!aligned16(a_q) || !aligned16(b) || !aligned16(out) || (reinterpret_cast<uintptr_t>(a_s) & 3u) ||
       (reinterpret_cast<uintptr_t>(b_s) & 3u))
     return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: a_q, b, out must be 16-byte aligned, scales 4-byte aligned", fn);
@@ -425,7 +473,7 @@ KSQ_EXPORT int ksq_moe_fp8_blockwise_gemm(void* out, const void* a_q, const void
     return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: %zu activation rows cannot serve %zu slots of top_k %zu", fn, a_rows, numel, top_k);
   if (numel > 0x7fffffffull || a_rows > 0x7fffffffull || n > 0x7fffffffull || k > 0x7fffffffull)
     return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: dimension too large", fn);
-  const size_t cap_blocks = (numel + E * (block_m - 1)) / block_m;  // upper bound on aligned blocks
+  const size_t cap_blocks = few ? numel : (numel + E * (block_m - 1)) / block_m;  // upper bound on aligned blocks
   if (cap_blocks > 65535) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: too many row blocks (%zu)", fn, cap_blocks);
   Fp8Params p{static_cast<const uint8_t*>(a_q), static_cast<const float*>(a_s), static_cast<const uint8_t*>(b),
               static_cast<const float*>(b_s), out, static_cast<uint32_t>(cap_blocks * block_m), static_cast<uint32_t>(n),
@@ -439,6 +487,7 @@ KSQ_EXPORT int ksq_moe_fp8_blockwise_gemm(void* out, const void* a_q, const void
   p.numel = static_cast<uint32_t>(numel);
   p.top_k = static_cast<uint32_t>(top_k);
   p.scale_rows = static_cast<uint32_t>(div_up(n, 128));
+  p.num_experts = static_cast<uint32_t>(E);
   const int mt = block_m == 16 ? 1 : 2;
   const unsigned blocks = static_cast<unsigned>(cap_blocks);
   int rc;
@@ -456,6 +505,46 @@ KSQ_EXPORT int ksq_moe_fp8_blockwise_gemm(void* out, const void* a_q, const void
                               : dispatch_grouped<BF16>(p, mt, blocks, as_stream(stream));
   }
   if (rc) return rc;
+  return check_launch(fn);
+}
+
+KSQ_EXPORT int ksq_moe_fp8_down_sum(void* out, const void* a_q, const void* a_s, const void* b, const void* b_s,
+                                    const void* topk_w, const void* topk_ids, size_t tokens, size_t top_k, size_t E, size_t n,
+                                    size_t k, int out_dtype, void* stream) {
+  const char* fn = "ksq_moe_fp8_down_sum";
+  if (!a_q || !a_s || !b || !b_s || !out || !topk_ids) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: null pointer", fn);
+  if (!aligned16(a_q) || !aligned16(b) || !aligned16(out) || (reinterpret_cast<uintptr_t>(a_s) & 3u) ||
+      (reinterpret_cast<uintptr_t>(b_s) & 3u))
+    return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: a_q, b, out must be 16-byte aligned, scales 4-byte aligned", fn);
+  if (n == 0 || k == 0 || k % 128 != 0 || n % 16 != 0)
+    return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: need k %% 128 == 0 and n %% 16 == 0 (n=%zu k=%zu)", fn, n, k);
+  if (out_dtype != KSQ_F16 && out_dtype != KSQ_BF16) return fail(KSQ_ERR_UNSUPPORTED, "%s: output dtype must be f16 or bf16", fn);
+  if (top_k == 0 || top_k > 32 || E == 0) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: top_k must be in 1..32 and E positive", fn);
+  if (tokens == 0) return KSQ_OK;
+  if (tokens > 8) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: at most 8 tokens (every token streams its own experts)", fn);
+  if (n > 0x7fffffffull || top_k * k > 0x7fffffffull) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: dimension too large", fn);
+  Fp8Params p{static_cast<const uint8_t*>(a_q), static_cast<const float*>(a_s), static_cast<const uint8_t*>(b),
+              static_cast<const float*>(b_s), out, static_cast<uint32_t>(tokens), static_cast<uint32_t>(n),
+              static_cast<uint32_t>(top_k * k)};  // a token's top_k rows of a, one behind the other
+  p.kb_per_expert = static_cast<uint32_t>(k / 128);
+  p.as_row_stride = static_cast<uint32_t>(top_k * (k / 128));  // scales [numel, k/128] row-major: a token's run on
+  p.as_kb_stride = 1;
+  p.expert_ids = static_cast<const int32_t*>(topk_ids);
+  p.topk_w = static_cast<const float*>(topk_w);
+  p.numel = static_cast<uint32_t>(tokens);  // rows of the output
+  p.top_k = static_cast<uint32_t>(top_k);
+  p.num_experts = static_cast<uint32_t>(E);
+  p.scale_rows = static_cast<uint32_t>(div_up(n, 128));
+  const bool four = n % 64 == 0 && (n / 64) * tokens >= 192;
+  dim3 grid(static_cast<unsigned>(n / (four ? 64 : (n % 32 == 0 ? 32 : 16))), static_cast<unsigned>(tokens), 1);
+  hipStream_t st = as_stream(stream);
+#define KSQ_TOKSUM(TO_, NT_) fp8_splitk_kernel<TO_, 1, NT_, 4, 2, true, true><<<grid, 4 * 64, 0, st>>>(p)
+  if (out_dtype == KSQ_F16) {
+    if (four) KSQ_TOKSUM(F16, 4); else if (n % 32 == 0) KSQ_TOKSUM(F16, 2); else KSQ_TOKSUM(F16, 1);
+  } else {
+    if (four) KSQ_TOKSUM(BF16, 4); else if (n % 32 == 0) KSQ_TOKSUM(BF16, 2); else KSQ_TOKSUM(BF16, 1);
+  }
+#undef KSQ_TOKSUM
   return check_launch(fn);
 }
 

@@ -207,7 +207,7 @@ Status MoeLayer::Forward(const std::vector<Tensor>& input_tensors, std::vector<T
     const int32_t* ids = topk_ids + begin * topk;
     const float* weights = topk_weights + begin * topk;
 
-    const bool few = !IsFp8() && tokens <= kFewTokens && numel <= 64 && !input_tensors[2].perm && !input_tensors[3].perm &&
+    const bool few = tokens <= kFewTokens && numel <= 64 && !input_tensors[2].perm && !input_tensors[3].perm &&
                      (2 * inter) % 32 == 0 && topk <= 32;
     if (!few) KsqCheck(ksq_moe_align(ids, numel, E, block_m, sorted_ids, expert_ids, num_post_pad, align_scratch, stream), "MoeLayer");
     if (IsFp8()) {
@@ -218,6 +218,16 @@ Status MoeLayer::Forward(const std::vector<Tensor>& input_tensors, std::vector<T
       void* a2_s = cache2 + a2_q_size_;
       KsqCheck(ksq_fp8_group_quant(hidden + begin * hidden_size * elem, a1, a1_s, tokens, hidden_size, 128, 0, 0, dtype, stream),
                "MoeLayer");
+      if (few) {  // a few decode tokens: no aligned permutation, the sum over top-k inside the second GEMM
+        KsqCheck(ksq_moe_fp8_blockwise_gemm(cache1, a1, a1_s, 0, tokens, w1, w1_scale, nullptr, nullptr, ids, nullptr, numel,
+                                            topk, E, 2 * inter, hidden_size, 16, dtype, stream),
+                 "MoeLayer");
+        KsqCheck(ksq_fp8_group_quant(cache1, cache2, a2_s, numel, inter, 128, 0, 1, dtype, stream), "MoeLayer");
+        KsqCheck(ksq_moe_fp8_down_sum(out + begin * hidden_size * elem, cache2, a2_s, w2, w2_scale, weights, ids, tokens, topk, E,
+                                      hidden_size, inter, dtype, stream),
+                 "MoeLayer");
+        continue;
+      }
       KsqCheck(ksq_moe_fp8_blockwise_gemm(cache1, a1, a1_s, 0, tokens, w1, w1_scale, nullptr, sorted_ids, expert_ids,
                                           num_post_pad, numel, topk, E, 2 * inter, hidden_size, block_m, dtype, stream),
                "MoeLayer");

@@ -67,6 +67,7 @@ SIGNATURES = {
     "ksq_moe_fp8_block_m": (c_sz, [c_sz, c_sz]),
     "ksq_moe_fp8_blockwise_gemm": (c_i, [c_p, c_p, c_p, c_i, c_sz, c_p, c_p, c_p, c_p, c_p, c_p, c_sz, c_sz, c_sz, c_sz,
                                          c_sz, c_sz, c_i, c_p]),
+    "ksq_moe_fp8_down_sum": (c_i, [c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_sz, c_sz, c_sz, c_sz, c_sz, c_i, c_p]),
     "ksq_moe_topk_softmax": (c_i, [c_p, c_p, c_p, c_sz, c_sz, c_sz, c_i, ctypes.c_float, c_i, c_p]),
     "ksq_moe_grouped_topk": (c_i, [c_p, c_p, c_p, c_p, c_sz, c_sz, c_sz, c_sz, c_sz, c_i, c_i, ctypes.c_float, c_i, c_p]),
     "ksq_moe_silu_mul": (c_i, [c_p, c_p, c_sz, c_sz, c_i, c_p]),

@@ -363,10 +363,20 @@ def fused_moe_fp8_blockwise(x, w13, w13_scale, w2, w2_scale, topk_ids, topk_w, b
     E, two_inter, hidden = w13.shape
     inter = two_inter // 2
     numel = T * topk
+    tw = topk_w.reshape(-1).to(torch.float32).contiguous()
+    if block_m is None and T <= FEW_TOKENS and numel <= 64 and topk <= 32:
+        # a few decode tokens: no aligned permutation, the sum over top-k inside the second GEMM (as fused_moe_w4a16)
+        ids = topk_ids.reshape(-1).to(torch.int32).contiguous()
+        a1_q, a1_s = per_token_group_quant_fp8(x, hidden, 128, False)
+        c1 = moe_fp8_blockwise_gemm(a1_q, a1_s, False, w13, w13_scale, None, None, ids, None, numel, topk, 16, x.dtype)
+        a2_q, a2_s = per_token_group_quant_fp8(c1, inter, 128, False, fuse_silu_mul=True)
+        out = torch.empty((T, hidden), dtype=x.dtype, device=x.device)
+        _l.check(_lib.ksq_moe_fp8_down_sum(_ptr(out), _ptr(a2_q), _ptr(a2_s), _ptr(w2), _ptr(w2_scale), _ptr(tw), _ptr(ids), T,
+                                           topk, E, hidden, inter, _dt(out), _stream()))
+        return out
     if block_m is None:
         block_m = _lib.ksq_moe_fp8_block_m(numel, E)
     sorted_ids, expert_ids, npp = moe_align_block_size(topk_ids, E, block_m)
-    tw = topk_w.reshape(-1).to(torch.float32).contiguous()
     a1_q, a1_s = per_token_group_quant_fp8(x, hidden, 128, False)
     c1 = moe_fp8_blockwise_gemm(a1_q, a1_s, False, w13, w13_scale, None, sorted_ids, expert_ids, npp, numel, topk,
                                 block_m, x.dtype)
