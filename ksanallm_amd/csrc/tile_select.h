@@ -17,8 +17,15 @@ SplitKChoice select_splitk(size_t m, size_t n, size_t k);
 // same rule for a grid of m_blocks row blocks of 16*mt rows each (MoE: one block per aligned expert segment)
 SplitKChoice select_splitk_blocks(int mt, size_t m_blocks, size_t n, size_t k);
 
-// true when the MFMA tile kernel (prefill regime) serves the shape: m above the decode range and group 128
+// The decode-form kernels also serve small problems of more than 32 rows, in blocks of 32 rows; never more than this
+// many rows (the workspace queries walk every m up to it).
+constexpr size_t kRowBlockMaxM = 512;
+
+// true when the MFMA tile kernel (prefill regime) serves the shape: m above the decode range, a group size the tile
+// kernel is built for, and a problem past the size up to which the decode kernel over row blocks is faster
 bool use_mfma_tile(size_t m, size_t n, size_t k, size_t group);
+// the size rule alone (whatever ksq_set_small_problem_rule says): what the workspace queries size the decode form for
+bool small_w4a16_problem(size_t m, size_t n, size_t k, size_t group);
 
 // Grid of the MFMA tile kernel: block_m x 256 output tiles; the first main_items tiles (in the order of tile_work.h)
 // are computed whole, the others in `splits` parts of kt_per_split k-steps whose fp32 partial tiles go through the
@@ -30,7 +37,7 @@ struct TilePlan {
 };
 TilePlan plan_mfma_tile(size_t m, size_t n, size_t k);
 
-// Blockwise FP8: rows of activations above which the 256 x 256 MFMA tile kernel replaces the split-K wavefront kernel,
+// Blockwise FP8: whether the MFMA tile kernel replaces the split-K wavefront kernel (above 32 tokens, but for small problems),
 // and its grid (block_m is always 256; kt_per_split counts 128-deep k-blocks).
 bool use_fp8_tile(size_t m, size_t n, size_t k);
 TilePlan plan_fp8_tile(size_t m, size_t n, size_t k);

@@ -1,11 +1,16 @@
 // Per-shape tile selection: closed-form rules of (kind, m, n, k, dtype) for a 256-CU, 8-XCD MI355X.
 // Host code only; no timing and no device queries, so the answer is the same at load time and at run time.
+#include <atomic>
+
 #include "ksq_common.h"
 #include "tile_select.h"
 
 namespace ksq {
 
 static constexpr int kNumCU = 256;
+
+// ksq_set_small_problem_rule: 1 (default) lets small problems of more than 32 rows run the decode-form kernels
+static std::atomic<int> g_small_problem_rule{1};
 
 // Split-K wavefront kernel (decode regime, HBM-bound).  Measured on MI355X the kernel runs fastest with few, long
 // lived wavefronts, each streaming a deep ring of loads, and with every workgroup resident from the first cycle:
@@ -83,12 +88,21 @@ SplitKChoice select_splitk_blocks(int mt, size_t m_blocks, size_t n, size_t k) {
   return c;
 }
 
-// Regime switch.  W4A16 moves 0.5 byte per weight and 2*m flops: on this part the HBM and MFMA bounds cross near
-// m = 80; the split-K kernel handles up to two 16-row tiles per workgroup, the tile kernel takes over above that.
+// Regime switch.  Up to 32 rows the split-K (decode) kernel; above, the MFMA tile kernel - except while the problem is
+// small: the tile kernel has a floor of 17-22 us (a workgroup's prologue, the fp32 partial tiles of the cut along K and
+// the pass that sums them), and the decode kernel run over blocks of 32 rows, each streaming the weights again (out of
+// the L2: the blocks of one column group run on one XCD at the same time), stays below it while
+// ceil(m / 32) * n * k <= 2^28.  Measured on MI355X, decode / tile kernel in us: n = k = 4096 at 64 rows 10.9 / 19.2, at
+// 128 rows 10.8 / 25.6, at 512 rows 27.0 / 29.5; n = 6144, k = 4096 at 256 rows 24.0 / 27.3, at 384 rows 36.1 / 31.9;
+// n = 14336, k = 4096 at 64 rows 19.2 / 23.0, at 128 rows 28.2 / 29.8, at 256 rows 52.9 / 46.4; n = 25600, k = 5120 at
+// 64 rows 33.6 / 35.0, at 96 rows 48.7 / 43.6.  (Group 128 only: the wide decode instances exist for that group.)
+bool small_w4a16_problem(size_t m, size_t n, size_t k, size_t group) {
+  return group == 128 && m <= kRowBlockMaxM && div_up(m, 32) * n * k <= (size_t(1) << 28);
+}
 bool use_mfma_tile(size_t m, size_t n, size_t k, size_t group) {
-  (void)k;
-  (void)n;
-  return m > 32 && (group == 128 || group == 64 || group == 32);
+  if (m <= 32 || !(group == 128 || group == 64 || group == 32)) return false;
+  if (g_small_problem_rule.load(std::memory_order_relaxed) && small_w4a16_problem(m, n, k, group)) return false;
+  return true;
 }
 
 // 256-row tiles halve the weight traffic per output row, 128-row tiles waste less when m sits just above a multiple
@@ -157,10 +171,15 @@ TilePlan plan_mfma_tile(size_t m, size_t n, size_t k) {
   return t;
 }
 
+// Above two 16-token tiles the MFMA tile kernel (with split-K) - except, as for W4A16, while the problem is small enough
+// for the streaming kernel over blocks of 32 tokens to stay below the tile kernel's floor: ceil(m / 32) * n * k <= 5 * 2^24.
+// Measured on MI355X, streaming / tile kernel in us: n = k = 4096 at 64 tokens 8.4 / 17.7, at 128 tokens 14.6 / 22.3, at
+// 256 tokens 27.9 / 23.1; n = k = 7168 at 64 tokens 24.1 / 21.1; n = 18432, k = 7168 at 48 tokens 54.4 / 32.4.
 bool use_fp8_tile(size_t m, size_t n, size_t k) {
-  (void)n;
-  (void)k;
-  return m > 32;  // above two 16-token tiles the MFMA tile kernel (with split-K) measured faster than the streaming one
+  if (m <= 32) return false;
+  if (g_small_problem_rule.load(std::memory_order_relaxed) && m <= kRowBlockMaxM && div_up(m, 32) * n * k <= (size_t(5) << 24))
+    return false;
+  return true;
 }
 
 TilePlan plan_fp8_tile(size_t m, size_t n, size_t k) {
@@ -243,6 +262,8 @@ KSQ_EXPORT size_t ksq_moe_block_m(size_t numel, size_t E) {
   if (per_expert >= 40) return 256;
   return per_expert < 16 ? 16 : 32;
 }
+
+KSQ_EXPORT int ksq_set_small_problem_rule(int enabled) { return g_small_problem_rule.exchange(enabled ? 1 : 0); }
 
 KSQ_EXPORT int ksq_select_tile(int kind, size_t m, size_t n, size_t k, int dtype, ksq_tile_desc* d) {
   if (!d) return fail(KSQ_ERR_INVALID_ARGUMENT, "ksq_select_tile: null descriptor");

@@ -181,7 +181,8 @@ KSQ_EXPORT size_t ksq_w4a16_workspace_size(size_t max_m, size_t n, size_t k, siz
   size_t need = 0;
   // decode kernel: partial sums when K is cut over workgroups
   if (group == 128) {
-    for (size_t m = 1; m <= max_m && m <= 32; ++m) {
+    for (size_t m = 1; m <= max_m && m <= kRowBlockMaxM; ++m) {
+      if (m > 32 && !small_w4a16_problem(m, n, k, group)) break;  // (monotonic in m: no decode-form call above this m)
       const size_t bytes = splitk_workspace(select_splitk(m, n, k), m, n);
       need = bytes > need ? bytes : need;
     }
@@ -189,7 +190,7 @@ KSQ_EXPORT size_t ksq_w4a16_workspace_size(size_t max_m, size_t n, size_t k, siz
   // the plan is the same for all m of a band of 128 rows
   for (size_t band_end = 128; max_m > 32; band_end += 128) {
     const size_t m = band_end < max_m ? band_end : max_m;
-    if (use_mfma_tile(m, n, k, group)) {
+    if (group == 128 || group == 64 || group == 32) {  // (whether or not the small-problem rule sends this m elsewhere)
       const TilePlan t = plan_mfma_tile(m, n, k);
       need = t.workspace_bytes > need ? t.workspace_bytes : need;
     }

@@ -79,6 +79,7 @@ SIGNATURES = {
     "ksq_w4a8_workspace_size": (c_sz, [c_sz, c_sz, c_sz]),
     "ksq_w4a8_gemm": (c_i, [c_p, c_p, c_p, c_p, ctypes.c_float, c_p, c_sz, c_sz, c_sz, c_sz, c_i, c_p, c_sz, c_p]),
     "ksq_select_tile": (c_i, [c_i, c_sz, c_sz, c_sz, c_i, ctypes.POINTER(TileDesc)]),
+    "ksq_set_small_problem_rule": (c_i, [c_i]),
 }
 
 _lib = None
@@ -108,6 +109,12 @@ def load():
 def check(rc):
     if rc != 0:
         raise KsqError(rc, load().ksq_last_error_string().decode())
+
+
+def set_small_problem_rule(enabled):
+    """Process-wide: whether small problems of more than 32 rows run the decode-form kernels (default) or, like every
+    larger one, the tile kernels.  Returns the previous setting."""
+    return bool(load().ksq_set_small_problem_rule(1 if enabled else 0))
 
 
 def select_tile(kind, m, n, k, dtype):

@@ -45,3 +45,27 @@ def test_size_queries_and_tile_selection_are_host_only():
     for m in (33, 64, 100, 128, 129, 700, 4096):
         assert lib.ksq_w4a8_workspace_size(m, 256, 8192) <= need
     assert lib.ksq_w4a8_workspace_size(64, 256, 100) == 0          # k not a multiple of 128: no kernel, no scratch
+
+
+def test_small_problem_rule_and_its_switch():
+    """Above 32 rows the tile kernels, but for small problems; the switch sends those to the tile kernels too, the
+    descriptor follows it, and the workspace query covers both settings."""
+    from ksanallm_amd import lib as L
+    lib = L.load()
+    small, large = (128, 4096, 4096), (160, 14336, 4096)  # ceil(m/32) * n * k = 2^26 and 5 * 14336 * 4096 > 2^28
+    assert L.select_tile(L.KIND_W4A16, *small, L.BF16)["kernel"] == 0
+    assert L.select_tile(L.KIND_W4A16, *large, L.BF16)["kernel"] == 1
+    assert L.select_tile(L.KIND_W4A16, 513, 256, 256, L.BF16)["kernel"] == 1      # never beyond 512 rows
+    assert L.select_tile(L.KIND_FP8_BLOCKWISE, 128, 4096, 4096, L.BF16)["kernel"] == 0
+    assert L.select_tile(L.KIND_FP8_BLOCKWISE, 64, 7168, 7168, L.BF16)["kernel"] == 1
+    ws_on = lib.ksq_w4a16_workspace_size(128, 4096, 14336, 128, L.BF16)
+    assert L.set_small_problem_rule(False) is True
+    try:
+        assert L.select_tile(L.KIND_W4A16, *small, L.BF16)["kernel"] == 1
+        assert L.select_tile(L.KIND_FP8_BLOCKWISE, 128, 4096, 4096, L.BF16)["kernel"] == 1
+        d = L.select_tile(L.KIND_W4A16, 128, 4096, 14336, L.BF16)
+        assert d["kernel"] == 1 and d["split_k"] > 1
+        assert lib.ksq_w4a16_workspace_size(128, 4096, 14336, 128, L.BF16) == ws_on >= d["split_k"] * 128 * 4096 * 4
+    finally:
+        assert L.set_small_problem_rule(True) is False
+    assert L.select_tile(L.KIND_W4A16, *small, L.BF16)["kernel"] == 0

@@ -171,7 +171,7 @@ def test_blockwise_gemm_benchmark_shapes_prefill_rows(ops, oracle, m, n, k):
                                       (130, 4096, 7168, 128), (128, 7168, 2048, 128), (384, 528, 1024, 128), (100, 272, 384, 128),
                                       (500, 768, 640, 128), (512, 4352, 256, 256), (200, 8704, 256, 256),
                                       (1024, 2304, 384, 256)])
-def test_blockwise_gemm_tile_kernel(ops, oracle, m, n, k, bm):
+def test_blockwise_gemm_tile_kernel(ops, oracle, m, n, k, bm, tile_kernels):
     from ksanallm_amd import lib as L
     desc = L.select_tile(L.KIND_FP8_BLOCKWISE, m, n, k, H.BF16)
     assert desc["kernel"] == 1 and desc["block_m"] == bm
@@ -188,8 +188,23 @@ def test_blockwise_gemm_tile_kernel(ops, oracle, m, n, k, bm):
         assert e.value.code == 3
 
 
+# small problems of more than 32 tokens (ceil(m / 32) * n * k <= 5 * 2^24, m <= 512): the streaming kernel over blocks of
+# 32 tokens, ragged last block included
+@pytest.mark.parametrize("m,n,k", [(65, 256, 128), (100, 272, 384), (128, 4096, 4096), (300, 2320, 1152), (500, 768, 640),
+                                   (33, 7168, 2048)])
+def test_blockwise_gemm_row_blocks_above_32_tokens(ops, oracle, m, n, k):
+    from ksanallm_amd import lib as L
+    desc = L.select_tile(L.KIND_FP8_BLOCKWISE, m, n, k, H.BF16)
+    assert desc["kernel"] == 0
+    x, bq, bs = make_fp8_problem(oracle, 4450 + m + n, m, n, k)
+    q, s = ops.per_token_group_quant_fp8(x.cuda(), k, 128, True)
+    out = ops.fp8_blockwise_gemm(q, s, packed(ops, bq), torch.from_numpy(bs).cuda(), torch.bfloat16)
+    ref = oracle.fp8_blockwise_gemm(q.cpu().numpy(), s.cpu().numpy(), bq, bs, True)
+    H.check_gemm(out, ref, H.BF16, "fp8 row blocks m=%d n=%d k=%d" % (m, n, k))
+
+
 # a little more than one round of tiles: the first 256 tiles are computed whole, the rest cut along K
-def test_blockwise_gemm_whole_and_cut_tiles(ops, oracle):
+def test_blockwise_gemm_whole_and_cut_tiles(ops, oracle, tile_kernels):
     from ksanallm_amd import lib as L
     m, n, k = 1030, 13328, 4096
     desc = L.select_tile(L.KIND_FP8_BLOCKWISE, m, n, k, H.BF16)
@@ -301,7 +316,9 @@ def test_blockwise_gemm_full_size_properties(ops, oracle, n, k):
 # written, raw - streaming kernel, tile kernel with whole tiles, tile kernel with tiles cut along K
 @pytest.mark.parametrize("m,n,k", [(1, 18432, 7168), (16, 7168, 18432), (128, 7168, 18432), (128, 18432, 7168),
                                    (300, 2320, 1152), (1024, 2304, 384)])
-def test_blockwise_gemm_sums_before_output_rounding(ops, oracle, m, n, k):
+def test_blockwise_gemm_sums_before_output_rounding(ops, oracle, both_regimes, m, n, k):
+    if m <= 32 and not both_regimes:
+        pytest.skip("the rule only concerns more than 32 tokens")
     x, bq, bs = make_fp8_problem(oracle, 4800 + m + n, m, n, k)
     q, s = ops.per_token_group_quant_fp8(x.cuda(), k, 128, True)
     bp, bsd = packed(ops, bq), torch.from_numpy(bs).cuda()

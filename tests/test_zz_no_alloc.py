@@ -27,7 +27,7 @@ def _static(L, x, wp, sp, zp, N, K, dtype, group=128, y=None):
 
 
 @pytest.mark.parametrize("dtype,awq", [(H.BF16, True), (H.F16, False)])
-def test_static_scratch_matches_workspace_form(dtype, awq):
+def test_static_scratch_matches_workspace_form(dtype, awq, both_regimes):
     from ksanallm_amd import lib as L
     from ksanallm_amd import ops
     lib = L.load()
@@ -52,7 +52,7 @@ def test_static_scratch_matches_workspace_form(dtype, awq):
                        ops.w4a16_gemm(x, wp, sp, zp, N, K, 128).view(torch.int16))
 
 
-def test_static_scratch_rejects_plans_beyond_its_size():
+def test_static_scratch_rejects_plans_beyond_its_size(tile_kernels):
     from ksanallm_amd import lib as L
     lib = L.load()
     cap = lib.ksq_w4a16_static_workspace_bytes()
@@ -78,7 +78,7 @@ def test_static_scratch_rejects_plans_beyond_its_size():
     assert rc == 3 and b"scratch" in lib.ksq_last_error_string()
 
 
-def test_static_scratch_allocates_nothing_and_replays_from_a_graph():
+def test_static_scratch_allocates_nothing_and_replays_from_a_graph(tile_kernels):
     """What the entry point promises beyond its results: the device's free memory is the same after a run of calls as
     before the first of them, and a call captured into a HIP graph (after one eager call on the device, which
     resolves the buffer's address and the kernels' attributes) replays to the eager bits every time, with eager work
