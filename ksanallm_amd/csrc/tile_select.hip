@@ -28,6 +28,11 @@ SplitKChoice select_splitk(size_t m, size_t n, size_t k) {
   const size_t m_blocks = div_up(m, 16 * mt);
   SplitKChoice c = select_splitk_blocks(mt, m_blocks, n, k);
   const size_t strips = n / 16;
+  // several row blocks, and four column tiles per workgroup would put a second workgroup on some CUs only (those then
+  // finish last): eight column tiles when that still leaves half the CUs a workgroup (n = k = 5120 at 128 rows)
+  if (m_blocks >= 2 && c.nt == 4 && strips % 8 == 0 && strips / 4 * m_blocks > static_cast<size_t>(kNumCU) &&
+      strips / 8 * m_blocks >= static_cast<size_t>(kNumCU) / 2)
+    c.nt = 8;
   if (strips % 4 == 0 && c.nt < 4) {
     const size_t rows = m < static_cast<size_t>(16 * mt) ? m : static_cast<size_t>(16 * mt);
     const size_t x_bytes = rows * k * 2 * (strips / c.nt) * m_blocks;  // what all workgroups together read of x
@@ -36,7 +41,11 @@ SplitKChoice select_splitk(size_t m, size_t n, size_t k) {
     // n = k = 4096 at 8 tokens, 17 MB of re-reads, would go 5.5 -> 7.0 us)
     const bool long_k = k >= 2 * n && (x_bytes > k * n / 2 || k > 16384);
     const bool heavy_x = x_bytes >= (size_t(48) << 20);
-    if (long_k || heavy_x) {
+    if (m_blocks >= 2 && !long_k && heavy_x) {
+      // several row blocks: four column tiles with x through LDS (below) rather than a cut along K - the blocks already
+      // fill the chip (n = k = 5120 at 64 rows: 19.2 -> 12 us; n = k = 4096: 10.7 -> 10.0 us)
+      c.nt = 4;
+    } else if (long_k || heavy_x) {
       int parts = 2;
       while (parts < 8 && strips / 4 * m_blocks * parts < 160) parts *= 2;
       while (parts > 1 && k / 128 / parts < 8) parts /= 2;
@@ -92,12 +101,17 @@ SplitKChoice select_splitk_blocks(int mt, size_t m_blocks, size_t n, size_t k) {
 // small: the tile kernel has a floor of 17-22 us (a workgroup's prologue, the fp32 partial tiles of the cut along K and
 // the pass that sums them), and the decode kernel run over blocks of 32 rows, each streaming the weights again (out of
 // the L2: the blocks of one column group run on one XCD at the same time), stays below it while
-// ceil(m / 32) * n * k <= 2^28.  Measured on MI355X, decode / tile kernel in us: n = k = 4096 at 64 rows 10.9 / 19.2, at
-// 128 rows 10.8 / 25.6, at 512 rows 27.0 / 29.5; n = 6144, k = 4096 at 256 rows 24.0 / 27.3, at 384 rows 36.1 / 31.9;
-// n = 14336, k = 4096 at 64 rows 19.2 / 23.0, at 128 rows 28.2 / 29.8, at 256 rows 52.9 / 46.4; n = 25600, k = 5120 at
-// 64 rows 33.6 / 35.0, at 96 rows 48.7 / 43.6.  (Group 128 only: the wide decode instances exist for that group.)
+// ceil(m / 32) * n * k <= 2^28, or 2^27 when K is the long side by four times or more (every block then re-reads a long
+// row of x per column group).  Measured on MI355X over twelve shapes and 48..512 rows, decode / tile kernel in us:
+// n = k = 4096 at 64 rows 10.9 / 19.2, at 128 rows 10.8 / 25.6, at 512 rows 27.0 / 29.5; n = 8192, k = 2048 at 128 rows
+// 11.3 / 26.4, at 512 rows 29.2 / 40.1; n = k = 8192 at 64 rows 18.1 / 24.1, at 128 rows 30.6 / 32.0, at 192 rows
+// 44.4 / 41.3; n = 14336, k = 4096 at 64 rows 17.9 / 23.1, at 128 rows 26.4 / 30.3, at 384 rows 75.1 / 56.3; n = 4096,
+// k = 14336 at 128 rows 27.9 / 32.1, at 192 rows 48.4 / 38.9; n = 25600, k = 5120 at 64 rows 33.5 / 37.6, at 96 rows
+// 48.6 / 46.1; n = 4096, k = 28672 at 64 rows 35.8 / 34.4; n = 5120, k = 25600 at 64 rows 61.7 / 36.6.
+// (Group 128 only: the wide decode instances exist for that group.)
 bool small_w4a16_problem(size_t m, size_t n, size_t k, size_t group) {
-  return group == 128 && m <= kRowBlockMaxM && div_up(m, 32) * n * k <= (size_t(1) << 28);
+  const size_t limit = k >= 4 * n ? (size_t(1) << 27) : (size_t(1) << 28);
+  return group == 128 && m <= kRowBlockMaxM && div_up(m, 32) * n * k <= limit;
 }
 bool use_mfma_tile(size_t m, size_t n, size_t k, size_t group) {
   if (m <= 32 || !(group == 128 || group == 64 || group == 32)) return false;
@@ -172,12 +186,16 @@ TilePlan plan_mfma_tile(size_t m, size_t n, size_t k) {
 }
 
 // Above two 16-token tiles the MFMA tile kernel (with split-K) - except, as for W4A16, while the problem is small enough
-// for the streaming kernel over blocks of 32 tokens to stay below the tile kernel's floor: ceil(m / 32) * n * k <= 5 * 2^24.
-// Measured on MI355X, streaming / tile kernel in us: n = k = 4096 at 64 tokens 8.4 / 17.7, at 128 tokens 14.6 / 22.3, at
-// 256 tokens 27.9 / 23.1; n = k = 7168 at 64 tokens 24.1 / 21.1; n = 18432, k = 7168 at 48 tokens 54.4 / 32.4.
+// for the streaming kernel over blocks of 32 tokens to stay below the tile kernel's floor (15-22 us): weights of at most
+// 3 * 2^23 elements and ceil(m / 32) * n * k <= 5 * 2^24.  Measured on MI355X over ten shapes and 48..512 tokens,
+// streaming / tile kernel in us: n = k = 4096 at 64 tokens 8.3 / 17.6, at 128 tokens 14.8 / 22.2, at 256 tokens
+// 27.8 / 22.8; n = 2048, k = 7168 at 128 tokens 11.8 / 23.0, at 192 tokens 21.8 / 22.2; n = 7168, k = 2048 at 128 tokens
+// 17.9 / 21.3, at 192 tokens 25.0 / 23.5; n = 1024, k = 4096 at 512 tokens 14.0 / 22.0; n = 4608, k = 7168 at 64 tokens
+// 22.4 / 18.6; n = k = 7168 at 64 tokens 24.3 / 21.0; n = 24576, k = 1536 at 64 tokens 26.8 / 19.6.
 bool use_fp8_tile(size_t m, size_t n, size_t k) {
   if (m <= 32) return false;
-  if (g_small_problem_rule.load(std::memory_order_relaxed) && m <= kRowBlockMaxM && div_up(m, 32) * n * k <= (size_t(5) << 24))
+  if (g_small_problem_rule.load(std::memory_order_relaxed) && m <= kRowBlockMaxM && n * k <= (size_t(3) << 23) &&
+      div_up(m, 32) * n * k <= (size_t(5) << 24))
     return false;
   return true;
 }

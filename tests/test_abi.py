@@ -56,6 +56,9 @@ def test_small_problem_rule_and_its_switch():
     assert L.select_tile(L.KIND_W4A16, *small, L.BF16)["kernel"] == 0
     assert L.select_tile(L.KIND_W4A16, *large, L.BF16)["kernel"] == 1
     assert L.select_tile(L.KIND_W4A16, 513, 256, 256, L.BF16)["kernel"] == 1      # never beyond 512 rows
+    assert L.select_tile(L.KIND_W4A16, 64, 25600, 5120, L.F16)["kernel"] == 0      # 2 * n * k < 2^28
+    assert L.select_tile(L.KIND_W4A16, 64, 5120, 25600, L.F16)["kernel"] == 1      # K the long side by 4x: 2^27
+    assert L.select_tile(L.KIND_FP8_BLOCKWISE, 64, 4608, 7168, L.BF16)["kernel"] == 1  # weights beyond 3 * 2^23 elements
     assert L.select_tile(L.KIND_FP8_BLOCKWISE, 128, 4096, 4096, L.BF16)["kernel"] == 0
     assert L.select_tile(L.KIND_FP8_BLOCKWISE, 64, 7168, 7168, L.BF16)["kernel"] == 1
     ws_on = lib.ksq_w4a16_workspace_size(128, 4096, 14336, 128, L.BF16)
