@@ -11,9 +11,11 @@ its weights in the 256 MB Infinity Cache.
 Prints ONE JSON line.  `value` is the time-weighted fraction of the MI355X roofline over the step, in percent:
 sum over cases of max(bytes / 8 TB/s, flops / MFMA peak) divided by the measured step time.
 
-Two side measurements, neither a benchmark figure: `--library-gemm` times the vendor library's plain GEMMs at the
-prefill shapes, and `--constant-data` gives every operand of the dense cases one value (the same kernels and cycle
-counts at the clock that operands which never toggle allow).
+Side measurements, none a benchmark figure: `--library-gemm` times the vendor library's plain GEMMs at the
+prefill shapes, `--constant-data` gives every operand of the dense cases one value (the same kernels and cycle
+counts at the clock that operands which never toggle allow), and `--mfma-stream` times bare streams of the matrix
+instructions on operands held in registers (what the matrix pipes sustain under the part's power limit with no kernel
+around them).
 """
 import argparse
 import json
@@ -603,6 +605,39 @@ def library_gemm(steps, warmup):
     print(json.dumps({"library_gemm": rows}))
 
 
+def mfma_stream(iters=6000, launches=200):
+    """Bare MFMA streams (ksq_diag_mfma_stream), 2 wavefronts per SIMD on all 256 CUs, launches of about 3 ms timed
+    back to back for about 0.6 s: TFLOP/s on operands with random bits and on operands that are all one value."""
+    from ksanallm_amd import lib as L
+    lib = L.load()
+    kinds = [(0, "v_mfma_f32_16x16x32_f16", "f16"), (1, "v_mfma_f32_16x16x32_bf16", "bf16"),
+             (2, "v_mfma_scale_f32_16x16x128_f8f6f4 (e4m3)", "fp8"), (3, "v_mfma_f32_32x32x16_f16", "f16"),
+             (4, "v_mfma_f32_32x32x16_bf16", "bf16"), (5, "v_mfma_scale_f32_32x32x64_f8f6f4 (e4m3)", "fp8")]
+    sink = torch.zeros(256 * 512, dtype=torch.float32, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    rows = []
+    for kind, name, dt in kinds:
+        row = {"instruction": name, "peak_tflops": MFMA_PEAK[dt] / 1e12}
+        for constant in (0, 1):
+            L.check(lib.ksq_diag_mfma_stream(kind, constant, 200, sink.data_ptr(), stream))
+            torch.cuda.synchronize()
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s.record()
+            for _ in range(launches):
+                L.check(lib.ksq_diag_mfma_stream(kind, constant, iters, sink.data_ptr(), stream))
+            e.record()
+            torch.cuda.synchronize()
+            ms = s.elapsed_time(e) / launches
+            row["constant_tflops" if constant else "random_tflops"] = round(lib.ksq_diag_mfma_stream_flops(kind, iters) / ms / 1e9, 1)
+            row["constant_ms" if constant else "random_ms"] = round(ms, 3)
+        row["random_frac_of_peak"] = round(row["random_tflops"] / row["peak_tflops"], 4)
+        rows.append(row)
+        print("%-44s random operands %7.1f TFLOP/s (%.1f %% of %g)   constant operands %7.1f TFLOP/s" % (
+            name, row["random_tflops"], 100 * row["random_frac_of_peak"], row["peak_tflops"], row["constant_tflops"]),
+            file=sys.stderr)
+    print(json.dumps({"mfma_stream": rows, "wavefronts_per_simd": 2, "launch_iters": iters, "launches": launches}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -626,6 +661,9 @@ def main():
     ap.add_argument("--sample-clock", type=float, default=0.0, metavar="SECONDS", help="instead of the benchmark: loop "
                     "every selected case for that long while reading the shader clock from rocm-smi every 50 ms, and "
                     "print launch time and clock per case (what the power management grants the kernel on this data)")
+    ap.add_argument("--mfma-stream", action="store_true", help="run only streams of independent MFMAs on register "
+                    "operands (the library's ksq_diag_mfma_stream: no memory traffic, no LDS, no other arithmetic), on "
+                    "random and on constant operands, and exit: the rate the matrix pipes sustain under the power limit")
     ap.add_argument("--library-gemm", action="store_true", help="run only the vendor library's plain GEMMs (torch.matmul "
                     "fp16 / bf16, torch._scaled_mm e4m3; no dequantization, no block scales) at the prefill shapes of "
                     "configurations 3 and 4 and exit: what a dense GEMM reaches on this part, beside the MFMA peak")
@@ -652,6 +690,9 @@ def main():
         FP8_SHAPE = tuple(int(v) for v in args.fp8_shape.split(","))
     if args.library_gemm:
         library_gemm(args.steps, args.warmup)
+        return
+    if args.mfma_stream:
+        mfma_stream()
         return
 
     from ksanallm_amd import lib as L

@@ -406,6 +406,17 @@ int ksq_select_tile(int kind, size_t m, size_t n, size_t k, int dtype, ksq_tile_
  * No counterpart in the reference (its Marlin / CUTLASS / DeepGEMM paths have no such switch). */
 int ksq_set_small_problem_rule(int enabled);
 
+/* Measurement aid, no counterpart in the reference: one launch of 256 workgroups x 8 wavefronts, each issuing `iters`
+ * rounds of independent matrix instructions on operands that stay in registers (no memory traffic, no LDS, no other
+ * arithmetic).  kind 0 / 1 / 2: v_mfma_f32_16x16x32_f16 / _bf16 / v_mfma_scale_f32_16x16x128_f8f6f4 on e4m3 bytes, the
+ * forms the GEMM kernels use; 3 / 4 / 5: the 32x32x16 and 32x32x64 forms of the same types.  constant_operands = 0:
+ * every lane's operand bits differ; 1: all operands one value.  Timed by the caller (bench.py --mfma-stream), the rate
+ * it sustains is what the matrix pipes deliver under the part's power limit - the ceiling a GEMM kernel on such data has
+ * below the peak figure.  sink: 256 * 512 floats of device memory (never written for these operands).
+ * ksq_diag_mfma_stream_flops: the floating-point operations of one such launch. */
+int ksq_diag_mfma_stream(int kind, int constant_operands, int iters, void* sink, void* stream);
+double ksq_diag_mfma_stream_flops(int kind, int iters);
+
 #ifdef __cplusplus
 }
 #endif

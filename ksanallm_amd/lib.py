@@ -80,6 +80,8 @@ SIGNATURES = {
     "ksq_w4a8_gemm": (c_i, [c_p, c_p, c_p, c_p, ctypes.c_float, c_p, c_sz, c_sz, c_sz, c_sz, c_i, c_p, c_sz, c_p]),
     "ksq_select_tile": (c_i, [c_i, c_sz, c_sz, c_sz, c_i, ctypes.POINTER(TileDesc)]),
     "ksq_set_small_problem_rule": (c_i, [c_i]),
+    "ksq_diag_mfma_stream": (c_i, [c_i, c_i, c_i, c_p, c_p]),
+    "ksq_diag_mfma_stream_flops": (ctypes.c_double, [c_i, c_i]),
 }
 
 _lib = None
