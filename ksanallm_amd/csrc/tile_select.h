@@ -41,7 +41,8 @@ TilePlan plan_mfma_tile(size_t m, size_t n, size_t k);
 // and its grid (block_m is always 256; kt_per_split counts 128-deep k-blocks).
 bool use_fp8_tile(size_t m, size_t n, size_t k);
 TilePlan plan_fp8_tile(size_t m, size_t n, size_t k);
-// W4A8 (w4a8_tile.h): the same tile shapes with its own costs of a cut along K
+// W4A8 (w4a8_tile.h): the same regime rule with its own size limit, the same tile shapes with its own costs of a cut along K
+bool use_w4a8_tile(size_t m, size_t n, size_t k);
 TilePlan plan_w4a8_tile(size_t m, size_t n, size_t k);
 // W4A8 streaming kernel (up to 32 tokens): column tiles per workgroup and wavefronts that split K (parts is always 1)
 SplitKChoice select_w4a8_splitk(size_t m, size_t n);

@@ -200,6 +200,18 @@ bool use_fp8_tile(size_t m, size_t n, size_t k) {
   return true;
 }
 
+// W4A8: the same, with the limit where its two kernels cross: ceil(m / 32) * n * k <= 5 * 2^24.  Measured on MI355X over
+// six shapes and 48..512 tokens, streaming / tile kernel in us: n = k = 4096 at 64 tokens 8.3 / 17.0, at 128 tokens
+// 14.2 / 24.1, at 256 tokens 25.5 / 24.2; n = k = 5120 at 96 tokens 17.3 / 22.7, at 128 tokens 24.2 / 23.3; n = 8192,
+// k = 2048 at 128 tokens 12.8 / 23.5; n = 2048, k = 7168 at 128 tokens 19.1 / 23.9, at 192 tokens 27.2 / 23.0; n = 1024,
+// k = 4096 at 512 tokens 22.9 / 23.6; n = 25600, k = 5120 at 48 tokens 32.8 / 27.7.
+bool use_w4a8_tile(size_t m, size_t n, size_t k) {
+  if (m <= 32) return false;
+  if (g_small_problem_rule.load(std::memory_order_relaxed) && m <= kRowBlockMaxM && div_up(m, 32) * n * k <= (size_t(5) << 24))
+    return false;
+  return true;
+}
+
 TilePlan plan_fp8_tile(size_t m, size_t n, size_t k) {
   TilePlan t{};
   // 128-token tiles where 256-token ones would be half padding (the weights are then fetched once per 128 tokens);
@@ -341,7 +353,7 @@ KSQ_EXPORT int ksq_select_tile(int kind, size_t m, size_t n, size_t k, int dtype
       return KSQ_OK;
     }
     case KSQ_KIND_W4A8: {
-      if (m > 32) {
+      if (use_w4a8_tile(m, n, k)) {
         const TilePlan t = plan_w4a8_tile(m, n, k);
         d->kernel = KSQ_KERNEL_MFMA_TILE;
         d->block_m = t.block_m;

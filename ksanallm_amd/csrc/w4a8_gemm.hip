@@ -365,9 +365,6 @@ int launch_tile(const W4A8Params& q, const TilePlan& plan, float* partial, hipSt
   return KSQ_OK;
 }
 
-// above two 16-token tiles the tile kernel takes over, as for blockwise FP8
-inline bool use_tile(size_t m) { return m > 32; }
-
 }  // namespace
 }  // namespace ksq
 
@@ -493,7 +490,7 @@ KSQ_EXPORT int ksq_w4a8_gemm(const void* a_q, const void* xsum, const void* w_pa
   int rc;
   if (group == 64) {
     // two scale groups per k-block: the streaming kernel, or 128-token tiles over all of K (no workspace)
-    if (use_tile(m)) {
+    if (use_w4a8_tile(m, n, k)) {
       if (256 * k > 0xffffffffull || 16 * (k / 128) * 1024 > 0xffffffffull) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: k too large", fn);
       TilePlan plan{};
       plan.block_m = 128;
@@ -507,7 +504,7 @@ KSQ_EXPORT int ksq_w4a8_gemm(const void* a_q, const void* xsum, const void* w_pa
     } else {
       rc = out_dtype == KSQ_F16 ? dispatch_splitk<F16, 64>(p, st) : dispatch_splitk<BF16, 64>(p, st);
     }
-  } else if (use_tile(m)) {
+  } else if (use_w4a8_tile(m, n, k)) {
     const TilePlan plan = plan_w4a8_tile(m, n, k);
     if (plan.splits > 1 && (!workspace || workspace_bytes < plan.workspace_bytes || !aligned16(workspace)))
       return fail(KSQ_ERR_WORKSPACE, "%s: m=%zu n=%zu k=%zu needs %zu bytes of 16-byte aligned workspace, got %zu", fn, m,

@@ -31,12 +31,12 @@ def tile_kernels():
     L.set_small_problem_rule(before)
 
 
-@pytest.fixture(params=[True, False], ids=["small-problem-rule", "tile-kernels"])
-def both_regimes(request):
-    """The test runs twice: as the library decides by default, and with every problem of more than 32 rows on the tile
-    kernels."""
+@pytest.fixture(autouse=True)
+def _small_problem_rule_restored():
+    """Whatever a test did with the library's process-wide small-problem rule (helpers.each_regime), the next test
+    starts from the default."""
+    yield
     from ksanallm_amd import lib as L
 
-    before = L.set_small_problem_rule(request.param)
-    yield request.param
-    L.set_small_problem_rule(before)
+    if L._lib is not None:
+        L.set_small_problem_rule(True)

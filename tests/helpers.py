@@ -91,3 +91,15 @@ def check_gemm_f32(y32_gpu, ref_f32, what=""):
     assert rel_l2 <= 5e-3, "%s rel-L2 before rounding %.3e" % (what, rel_l2)
     assert max_abs <= 2e-2, "%s max-abs before rounding %.3e" % (what, max_abs)
     return rel_l2, max_abs
+
+
+def each_regime(m):
+    """Once as the library decides by default and, for more than 32 rows, once more with the small-problem rule off
+    (every such problem on the MFMA tile kernels): `for rule in each_regime(m): ...` runs the body under each setting.
+    conftest restores the default after the test whatever happens inside the loop."""
+    from ksanallm_amd import lib as L
+
+    for rule in ((True, False) if m > 32 else (True,)):
+        L.set_small_problem_rule(rule)
+        yield rule
+    L.set_small_problem_rule(True)

@@ -61,11 +61,14 @@ def test_small_problem_rule_and_its_switch():
     assert L.select_tile(L.KIND_FP8_BLOCKWISE, 64, 4608, 7168, L.BF16)["kernel"] == 1  # weights beyond 3 * 2^23 elements
     assert L.select_tile(L.KIND_FP8_BLOCKWISE, 128, 4096, 4096, L.BF16)["kernel"] == 0
     assert L.select_tile(L.KIND_FP8_BLOCKWISE, 64, 7168, 7168, L.BF16)["kernel"] == 1
+    assert L.select_tile(L.KIND_W4A8, 96, 5120, 5120, L.BF16)["kernel"] == 0
+    assert L.select_tile(L.KIND_W4A8, 128, 5120, 5120, L.BF16)["kernel"] == 1
     ws_on = lib.ksq_w4a16_workspace_size(128, 4096, 14336, 128, L.BF16)
     assert L.set_small_problem_rule(False) is True
     try:
         assert L.select_tile(L.KIND_W4A16, *small, L.BF16)["kernel"] == 1
         assert L.select_tile(L.KIND_FP8_BLOCKWISE, 128, 4096, 4096, L.BF16)["kernel"] == 1
+        assert L.select_tile(L.KIND_W4A8, 96, 5120, 5120, L.BF16)["kernel"] == 1
         d = L.select_tile(L.KIND_W4A16, 128, 4096, 14336, L.BF16)
         assert d["kernel"] == 1 and d["split_k"] > 1
         assert lib.ksq_w4a16_workspace_size(128, 4096, 14336, 128, L.BF16) == ws_on >= d["split_k"] * 128 * 4096 * 4

@@ -316,14 +316,13 @@ def test_blockwise_gemm_full_size_properties(ops, oracle, n, k):
 # written, raw - streaming kernel, tile kernel with whole tiles, tile kernel with tiles cut along K
 @pytest.mark.parametrize("m,n,k", [(1, 18432, 7168), (16, 7168, 18432), (128, 7168, 18432), (128, 18432, 7168),
                                    (300, 2320, 1152), (1024, 2304, 384)])
-def test_blockwise_gemm_sums_before_output_rounding(ops, oracle, both_regimes, m, n, k):
-    if m <= 32 and not both_regimes:
-        pytest.skip("the rule only concerns more than 32 tokens")
+def test_blockwise_gemm_sums_before_output_rounding(ops, oracle, m, n, k):
     x, bq, bs = make_fp8_problem(oracle, 4800 + m + n, m, n, k)
     q, s = ops.per_token_group_quant_fp8(x.cuda(), k, 128, True)
     bp, bsd = packed(ops, bq), torch.from_numpy(bs).cuda()
-    y32 = ops.fp8_blockwise_gemm_f32(q, s, bp, bsd)
-    y = ops.fp8_blockwise_gemm(q, s, bp, bsd, torch.bfloat16)
-    assert torch.equal(y32.to(torch.bfloat16).view(torch.int16), y.view(torch.int16))
     ref = oracle.fp8_blockwise_gemm(q.cpu().numpy(), s.cpu().numpy(), bq, bs, True)
-    H.check_gemm_f32(y32, ref, "fp8 before rounding m=%d n=%d k=%d" % (m, n, k))
+    for rule in H.each_regime(m):
+        y32 = ops.fp8_blockwise_gemm_f32(q, s, bp, bsd)
+        y = ops.fp8_blockwise_gemm(q, s, bp, bsd, torch.bfloat16)
+        assert torch.equal(y32.to(torch.bfloat16).view(torch.int16), y.view(torch.int16))
+        H.check_gemm_f32(y32, ref, "fp8 before rounding m=%d n=%d k=%d, small-problem rule %s" % (m, n, k, rule))

@@ -107,9 +107,10 @@ def test_gemm(ops, oracle, out_dtype, m, n, k):
     alpha = 0.05 * 0.7
     xq, xsum = ops.w4a8_static_quant(x.cuda(), in_scale.cuda(), False)
     wp = ops.w4a8_repack_weight(w.cuda())
-    out = ops.w4a8_gemm(xq, xsum, wp, scales.cuda(), alpha, n, H.TORCH_DT[out_dtype])
     ref = oracle.w4a8_gemm(xq.cpu().numpy(), w.numpy().view(np.int8), H.bits_of(scales), alpha)
-    H.check_gemm(out, ref, out_dtype, "w4a8 m=%d n=%d k=%d" % (m, n, k))
+    for rule in H.each_regime(m):  # above 32 tokens: the streaming kernel over 32-token blocks where the problem is small, and the tile kernel
+        out = ops.w4a8_gemm(xq, xsum, wp, scales.cuda(), alpha, n, H.TORCH_DT[out_dtype])
+        H.check_gemm(out, ref, out_dtype, "w4a8 m=%d n=%d k=%d, small-problem rule %s" % (m, n, k, rule))
 
 
 @pytest.mark.parametrize("m,n,k", [
@@ -125,7 +126,7 @@ def test_gemm(ops, oracle, out_dtype, m, n, k):
     (1024, 2304, 384),
 ])
 @pytest.mark.parametrize("out_dtype", [H.F16, H.BF16])
-def test_gemm_tile_kernel(ops, oracle, out_dtype, m, n, k):
+def test_gemm_tile_kernel(ops, oracle, tile_kernels, out_dtype, m, n, k):
     w, scales = make_weight(n + k + m, k, n)
     x = make_act(m * 3 + n, m, k, H.F16)
     in_scale = torch.tensor([0.04], dtype=torch.float32)
@@ -150,7 +151,7 @@ def test_gemm_streaming_kernel_variants(ops, oracle, m, n, k):
     H.check_gemm(out, ref, H.BF16, "w4a8 streaming m=%d n=%d k=%d" % (m, n, k))
 
 
-def test_gemm_workspace_is_checked(ops):
+def test_gemm_workspace_is_checked(ops, tile_kernels):
     from ksanallm_amd import lib as L
     m, n, k = 64, 256, 8192
     need = L.load().ksq_w4a8_workspace_size(m, n, k)
@@ -247,14 +248,15 @@ def test_gemm_group_64(ops, oracle, out_dtype, m, n, k):
     np.testing.assert_array_equal(xsum.cpu().numpy().T, oracle.w4a8_group_sums(xq.cpu().numpy(), 64))
     np.testing.assert_array_equal(ops.w4a8_group_sums(xq, 64).cpu().numpy(), xsum.cpu().numpy())
     wp = ops.w4a8_repack_weight(w.cuda())
-    out = ops.w4a8_gemm(xq, xsum, wp, s64.cuda(), 0.03, n, H.TORCH_DT[out_dtype], group=64)
     ref = oracle.w4a8_gemm(xq.cpu().numpy(), w.numpy().view(np.int8), H.bits_of(s64), 0.03, group=64)
-    H.check_gemm(out, ref, out_dtype, "w4a8 g64 m=%d n=%d k=%d" % (m, n, k))
     s128 = s64[0::2].contiguous()
     same = s128.repeat_interleave(2, 0).contiguous()
-    a = ops.w4a8_gemm(xq, xsum, wp, same.cuda(), 0.03, n, H.TORCH_DT[out_dtype], group=64)
-    b = ops.w4a8_gemm(xq, ops.w4a8_group_sums(xq), wp, s128.cuda(), 0.03, n, H.TORCH_DT[out_dtype])
-    H.check_gemm(a, b.float().cpu().numpy(), out_dtype, "w4a8 g64 against g128")
+    for rule in H.each_regime(m):
+        out = ops.w4a8_gemm(xq, xsum, wp, s64.cuda(), 0.03, n, H.TORCH_DT[out_dtype], group=64)
+        H.check_gemm(out, ref, out_dtype, "w4a8 g64 m=%d n=%d k=%d, small-problem rule %s" % (m, n, k, rule))
+        a = ops.w4a8_gemm(xq, xsum, wp, same.cuda(), 0.03, n, H.TORCH_DT[out_dtype], group=64)
+        b = ops.w4a8_gemm(xq, ops.w4a8_group_sums(xq), wp, s128.cuda(), 0.03, n, H.TORCH_DT[out_dtype])
+        H.check_gemm(a, b.float().cpu().numpy(), out_dtype, "w4a8 g64 against g128")
 
 
 def test_gemm_rejects_what_it_does_not_do(ops):

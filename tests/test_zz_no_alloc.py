@@ -26,15 +26,17 @@ def _static(L, x, wp, sp, zp, N, K, dtype, group=128, y=None):
     return y
 
 
+@pytest.mark.parametrize("small_problem_rule", [True, False])
 @pytest.mark.parametrize("dtype,awq", [(H.BF16, True), (H.F16, False)])
-def test_static_scratch_matches_workspace_form(dtype, awq, both_regimes):
+def test_static_scratch_matches_workspace_form(dtype, awq, small_problem_rule):
     from ksanallm_amd import lib as L
     from ksanallm_amd import ops
     lib = L.load()
+    L.set_small_problem_rule(small_problem_rule)  # off: the two problems of more than 32 rows run the tile kernel
     cap = lib.ksq_w4a16_static_workspace_bytes()
     assert cap == 32 << 20
-    # tile kernel with K cut over workgroups, then the decode kernel with K cut over workgroups on a smaller problem,
-    # then a plan that needs no scratch at all
+    # a problem of 128 rows with K cut over workgroups (decode form over four row blocks, or the tile kernel), then the
+    # decode kernel with K cut over workgroups on a smaller problem, then a plan that needs no scratch at all
     shapes = [(128, 4096, 14336), (8, 1024, 4096), (64, 512, 2048), (3, 768, 256)]
     for i, (M, N, K) in enumerate(shapes):
         need = lib.ksq_w4a16_workspace_size(M, N, K, 128, dtype)
