@@ -398,8 +398,8 @@ int ksq_select_tile(int kind, size_t m, size_t n, size_t k, int dtype, ksq_tile_
 
 /* Above 32 rows ksq_w4a16_gemm, ksq_fp8_blockwise_gemm and ksq_w4a8_gemm run the MFMA tile kernels, but for small
  * problems of up to 512 rows: while ceil(m / 32) * n * k <= 2^28 (W4A16 with group 128; 2^27 when k >= 4 n), or
- * n * k <= 3 * 2^23 and ceil(m / 32) * n * k <= 5 * 2^24 (block-fp8), or ceil(m / 32) * n * k <= 5 * 2^24 (W4A8), the
- * decode-form kernel over blocks of 32 rows is faster (the tile kernels have a floor of about 20 us) and is what runs.  enabled = 0 switches that rule off for the whole process -
+ * <= 5 * 2^24 (block-fp8, n <= 4 k), or <= 5 * 2^25 (W4A8, n <= 4 k), the decode-form kernel over blocks of 32 rows is
+ * faster (the tile kernels have a floor of about 20 us) and is what runs.  enabled = 0 switches that rule off for the whole process -
  * every m > 32 then runs the tile kernel -, 1 (the default) back on; returns the previous setting.  For tests that
  * must reach the tile kernels at sizes a CPU reference can multiply, and for timing one kernel against the other;
  * ksq_select_tile follows the setting, the workspace queries cover both settings.

@@ -269,10 +269,13 @@ int dispatch(const Fp8Params& p, hipStream_t s) {
   // the activation fragments are as large as the weight fragments: two strips share them once there are several
   // tokens, or when K is the long dimension (few strips, long streams)
   int nt = (p.M > 8 || p.K > p.N) ? 2 : 1;
+  // several blocks of 32 tokens (small problems above 32 tokens): four strips share a block's activation fragments while
+  // the blocks together still give every other CU a workgroup
+  if (p.M > 32 && p.N % 64 == 0 && p.N / 64 * div_up(p.M, 32) >= 128) nt = 4;
   if (p.N % (16 * nt) != 0) nt = 1;
 #define KSQ_CASE(MT_, NT_) \
   if (mt == MT_ && nt == NT_) { launch_splitk<TO, MT_, NT_, 4, 2>(p, s); return KSQ_OK; }
-  KSQ_CASE(1, 1) KSQ_CASE(1, 2) KSQ_CASE(2, 1) KSQ_CASE(2, 2)
+  KSQ_CASE(1, 1) KSQ_CASE(1, 2) KSQ_CASE(2, 1) KSQ_CASE(2, 2) KSQ_CASE(2, 4)
 #undef KSQ_CASE
   return fail(KSQ_ERR_UNSUPPORTED, "no fp8 decode kernel for mt=%d nt=%d", mt, nt);
 }

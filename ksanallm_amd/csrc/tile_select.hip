@@ -186,28 +186,33 @@ TilePlan plan_mfma_tile(size_t m, size_t n, size_t k) {
 }
 
 // Above two 16-token tiles the MFMA tile kernel (with split-K) - except, as for W4A16, while the problem is small enough
-// for the streaming kernel over blocks of 32 tokens to stay below the tile kernel's floor (15-22 us): weights of at most
-// 3 * 2^23 elements and ceil(m / 32) * n * k <= 5 * 2^24.  Measured on MI355X over ten shapes and 48..512 tokens,
-// streaming / tile kernel in us: n = k = 4096 at 64 tokens 8.3 / 17.6, at 128 tokens 14.8 / 22.2, at 256 tokens
-// 27.8 / 22.8; n = 2048, k = 7168 at 128 tokens 11.8 / 23.0, at 192 tokens 21.8 / 22.2; n = 7168, k = 2048 at 128 tokens
-// 17.9 / 21.3, at 192 tokens 25.0 / 23.5; n = 1024, k = 4096 at 512 tokens 14.0 / 22.0; n = 4608, k = 7168 at 64 tokens
-// 22.4 / 18.6; n = k = 7168 at 64 tokens 24.3 / 21.0; n = 24576, k = 1536 at 64 tokens 26.8 / 19.6.
+// for the streaming kernel over blocks of 32 tokens (four strips per workgroup sharing a block's activation fragments)
+// to stay below the tile kernel's floor (15-22 us): ceil(m / 32) * n * k <= 5 * 2^24, and not with a K so short that a
+// workgroup's life is its prologue (n > 4 k).  Measured on MI355X over eleven shapes and 48..512 tokens, streaming / tile
+// kernel in us: n = k = 4096 at 64 tokens 11.3 / 17.5, at 128 tokens 11.2 / 22.4, at 256 tokens 20.1 / 23.0, at 384
+// tokens 28.5 / 23.8; n = 2048, k = 7168 at 128 tokens 16.0 / 23.1, at 256 tokens 16.0 / 22.2, at 384 tokens 29.2 / 23.4;
+// n = 7168, k = 2048 at 192 tokens 18.9 / 23.6, at 256 tokens 24.0 / 23.6; n = 4608, k = 7168 at 64 tokens 17.1 / 18.7, at
+// 128 tokens 31.9 / 22.3; n = 7168, k = 4608 at 64 tokens 13.6 / 18.0, at 96 tokens 25.0 / 20.0; n = k = 7168 at 64 tokens
+// 18.2 / 21.0, at 96 tokens 33.6 / 22.9; n = 24576, k = 1536 at 64 tokens 22.0 / 19.6; n = 18432, k = 7168 at 48 tokens
+// 52.9 / 32.1.
 bool use_fp8_tile(size_t m, size_t n, size_t k) {
   if (m <= 32) return false;
-  if (g_small_problem_rule.load(std::memory_order_relaxed) && m <= kRowBlockMaxM && n * k <= (size_t(3) << 23) &&
+  if (g_small_problem_rule.load(std::memory_order_relaxed) && m <= kRowBlockMaxM && n <= 4 * k &&
       div_up(m, 32) * n * k <= (size_t(5) << 24))
     return false;
   return true;
 }
 
-// W4A8: the same, with the limit where its two kernels cross: ceil(m / 32) * n * k <= 5 * 2^24.  Measured on MI355X over
-// six shapes and 48..512 tokens, streaming / tile kernel in us: n = k = 4096 at 64 tokens 8.3 / 17.0, at 128 tokens
-// 14.2 / 24.1, at 256 tokens 25.5 / 24.2; n = k = 5120 at 96 tokens 17.3 / 22.7, at 128 tokens 24.2 / 23.3; n = 8192,
-// k = 2048 at 128 tokens 12.8 / 23.5; n = 2048, k = 7168 at 128 tokens 19.1 / 23.9, at 192 tokens 27.2 / 23.0; n = 1024,
-// k = 4096 at 512 tokens 22.9 / 23.6; n = 25600, k = 5120 at 48 tokens 32.8 / 27.7.
+// W4A8: the same, with the limit where its two kernels cross: ceil(m / 32) * n * k <= 5 * 2^25 (n <= 4 k).  Measured on
+// MI355X over nine shapes and 48..512 tokens, streaming / tile kernel in us: n = k = 4096 at 64 tokens 9.5 / 16.9, at 128
+// tokens 10.5 / 24.1, at 256 tokens 15.3 / 24.1, at 512 tokens 35.0 / 26.0; n = k = 5120 at 96 tokens 11.7 / 22.8, at 192
+// tokens 18.7 / 23.6, at 256 tokens 28.5 / 24.6; n = 8192, k = 2048 at 128 tokens 10.3 / 23.6; n = 2048, k = 7168 at 256
+// tokens 16.4 / 22.0; n = k = 8192 at 64 tokens 18.1 / 20.0, at 96 tokens 26.1 / 24.7; n = 14336, k = 4096 at 64 tokens
+// 15.6 / 18.7, at 96 tokens 23.7 / 23.7; n = 25600, k = 5120 at 48 tokens 32.8 / 27.1.
 bool use_w4a8_tile(size_t m, size_t n, size_t k) {
   if (m <= 32) return false;
-  if (g_small_problem_rule.load(std::memory_order_relaxed) && m <= kRowBlockMaxM && div_up(m, 32) * n * k <= (size_t(5) << 24))
+  if (g_small_problem_rule.load(std::memory_order_relaxed) && m <= kRowBlockMaxM && n <= 4 * k &&
+      div_up(m, 32) * n * k <= (size_t(5) << 25))
     return false;
   return true;
 }
@@ -247,14 +252,16 @@ TilePlan plan_w4a8_tile(size_t m, size_t n, size_t k) {
   return t;
 }
 
-// W4A8 decode: a workgroup takes as many 16-column strips (up to 4) as still leave 128 workgroups, and splits K over 8
-// wavefronts instead of 4 when fewer than 256 workgroups are left.
+// W4A8 decode: a workgroup takes as many 16-column strips (up to 4) as still leave 128 workgroups - counting the row
+// blocks of a problem of more than 32 tokens: n = k = 5120 at 64 tokens 16.8 -> 11.4 us with four strips instead of
+// two -, and splits K over 8 wavefronts instead of 4 when fewer than 256 workgroups are left.
 SplitKChoice select_w4a8_splitk(size_t m, size_t n) {
   SplitKChoice c{};
   c.mt = m <= 16 ? 1 : 2;
   c.nt = 4;
-  while (c.nt > 1 && (n % (16 * c.nt) != 0 || n / (16 * c.nt) < 128)) c.nt /= 2;
-  c.waves = n / (16 * c.nt) < 256 ? 8 : 4;
+  const size_t m_blocks = div_up(m, 16 * c.mt);
+  while (c.nt > 1 && (n % (16 * c.nt) != 0 || n / (16 * c.nt) * m_blocks < 128)) c.nt /= 2;
+  c.waves = n / (16 * c.nt) * m_blocks < 256 ? 8 : 4;
   c.parts = 1;
   c.xc = 0;
   return c;
@@ -343,7 +350,8 @@ KSQ_EXPORT int ksq_select_tile(int kind, size_t m, size_t n, size_t k, int dtype
       const int mt = m <= 16 ? 1 : 2;
       const int waves = 4;
       d->kernel = KSQ_KERNEL_SPLITK_WAVE;
-      const int nt = ((m > 8 || k > n) && n % 32 == 0) ? 2 : 1;
+      int nt = ((m > 8 || k > n) && n % 32 == 0) ? 2 : 1;
+      if (m > 32 && n % 64 == 0 && n / 64 * div_up(m, 32) >= 128) nt = 4;  // as fp8_blockwise_gemm.hip's dispatch
       d->block_m = 16 * mt;
       d->block_n = 16 * nt;
       d->block_k = 128;

@@ -58,11 +58,13 @@ def test_small_problem_rule_and_its_switch():
     assert L.select_tile(L.KIND_W4A16, 513, 256, 256, L.BF16)["kernel"] == 1      # never beyond 512 rows
     assert L.select_tile(L.KIND_W4A16, 64, 25600, 5120, L.F16)["kernel"] == 0      # 2 * n * k < 2^28
     assert L.select_tile(L.KIND_W4A16, 64, 5120, 25600, L.F16)["kernel"] == 1      # K the long side by 4x: 2^27
-    assert L.select_tile(L.KIND_FP8_BLOCKWISE, 64, 4608, 7168, L.BF16)["kernel"] == 1  # weights beyond 3 * 2^23 elements
+    assert L.select_tile(L.KIND_FP8_BLOCKWISE, 64, 4608, 7168, L.BF16)["kernel"] == 0
+    assert L.select_tile(L.KIND_FP8_BLOCKWISE, 64, 24576, 1536, L.BF16)["kernel"] == 1  # n > 4 k
+    assert L.select_tile(L.KIND_FP8_BLOCKWISE, 96, 7168, 7168, L.BF16)["kernel"] == 1   # 3 * n * k > 5 * 2^24
     assert L.select_tile(L.KIND_FP8_BLOCKWISE, 128, 4096, 4096, L.BF16)["kernel"] == 0
     assert L.select_tile(L.KIND_FP8_BLOCKWISE, 64, 7168, 7168, L.BF16)["kernel"] == 1
     assert L.select_tile(L.KIND_W4A8, 96, 5120, 5120, L.BF16)["kernel"] == 0
-    assert L.select_tile(L.KIND_W4A8, 128, 5120, 5120, L.BF16)["kernel"] == 1
+    assert L.select_tile(L.KIND_W4A8, 256, 5120, 5120, L.BF16)["kernel"] == 1
     ws_on = lib.ksq_w4a16_workspace_size(128, 4096, 14336, 128, L.BF16)
     assert L.set_small_problem_rule(False) is True
     try:
