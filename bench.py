@@ -337,8 +337,10 @@ WORKLOADS = {
     6: "DeepSeek-V3 MoE block-fp8 bf16 E=256 top-8 T in {1,64,512,4096}",
     7: "W4A8 bf16 (5120x5120)+(25600x5120) M in {1,16,64,128,256,4096}",
     8: "W4A16 decode on large weights: GPTQ bf16 (57344x8192), AWQ bf16 (28672x8192), GPTQ fp16 (25600x5120) M in {1,8,16}",
+    9: "small problems of 64..512 rows: W4A16 fp16 (4096x4096)+(5120x5120), blockwise FP8 (4096x4096)+(2048x7168), "
+       "W4A8 (4096x4096)+(5120x5120), M in {64,128,256,512}",
 }
-DTYPES = {1: "f16", 2: "bf16", 3: "f16", 4: "fp8", 5: "bf16", 6: "fp8", 7: "fp8", 8: "bf16"}
+DTYPES = {1: "f16", 2: "bf16", 3: "f16", 4: "fp8", 5: "bf16", 6: "fp8", 7: "fp8", 8: "bf16", 9: "f16"}
 
 
 def build(cfg, ops, L):
@@ -369,6 +371,13 @@ def build(cfg, ops, L):
         c, kc = w4a16_cases(ops, L, 8, [("up", 25600, 5120)], [1, 8, 16], "f16", False, 1.0, 0.004, 0.02)
         for x in c:
             x.peak_key = "f16"
+        return a + b + c, ka + kb + kc
+    if cfg == 9:  # not one of the five benchmark configurations: projections of smaller models at 64..512 rows, where the
+        # decode-form kernels over 32-row blocks run instead of the tile kernels (--tile-kernels: the tile kernels)
+        Ms = [64, 128, 256, 512]
+        a, ka = w4a16_cases(ops, L, 9, [("w4a16_4096", 4096, 4096), ("w4a16_5120", 5120, 5120)], Ms, "f16", False, 1.0, 0.004, 0.02)
+        b, kb = fp8_cases(ops, L, 9, [("fp8_4096", 4096, 4096), ("fp8_2048x7168", 2048, 7168)], Ms)
+        c, kc = w4a8_cases(ops, L, 9, [("w4a8_4096", 4096, 4096), ("w4a8_5120", 5120, 5120)], Ms)
         return a + b + c, ka + kb + kc
     raise SystemExit("unknown --config %d" % cfg)
 
@@ -644,7 +653,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", default="all", help="'all' (default): the five benchmark configurations 1..5 in one "
-                    "step; or one number: 1..5, 6 = block-fp8 MoE on the shapes of 5, 7 = W4A8, 8 = W4A16 decode on large weights")
+                    "step; or one number: 1..5, 6 = block-fp8 MoE on the shapes of 5, 7 = W4A8, 8 = W4A16 decode on large weights, "
+                    "9 = small problems of 64..512 rows in the three formats")
     ap.add_argument("--only", default="", help="substring filter on case names (for profiling one case)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-graph", action="store_true", help="launch every kernel from Python instead of replaying "
@@ -661,6 +671,9 @@ def main():
     ap.add_argument("--sample-clock", type=float, default=0.0, metavar="SECONDS", help="instead of the benchmark: loop "
                     "every selected case for that long while reading the shader clock from rocm-smi every 50 ms, and "
                     "print launch time and clock per case (what the power management grants the kernel on this data)")
+    ap.add_argument("--tile-kernels", action="store_true", help="switch the library's small-problem rule off "
+                    "(ksq_set_small_problem_rule(0)): every case of more than 32 rows runs the MFMA tile kernel, to time "
+                    "it against the decode-form kernel the rule would choose; not a benchmark figure")
     ap.add_argument("--mfma-stream", action="store_true", help="run only streams of independent MFMAs on register "
                     "operands (the library's ksq_diag_mfma_stream: no memory traffic, no LDS, no other arithmetic), on "
                     "random and on constant operands, and exit: the rate the matrix pipes sustain under the power limit")
@@ -698,6 +711,8 @@ def main():
     from ksanallm_amd import lib as L
     from ksanallm_amd import ops
 
+    if args.tile_kernels:
+        L.set_small_problem_rule(False)
     cfgs = [1, 2, 3, 4, 5] if args.config == "all" else [int(args.config)]
     whole = len(cfgs) > 1
     cases, keeps = [], {}
@@ -837,7 +852,8 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16 / bf16 / fp8-e4m3 by configuration, fp32 accumulation" if whole else DTYPES[cfgs[0]],
         "data": "synthetic, constant %s (--constant-data)" % CONSTANT_DATA if CONSTANT_DATA else "synthetic",
-        "config": {"workload": workload, "cases": len(cases), "configs": cfgs},
+        "config": {"workload": workload, "cases": len(cases), "configs": cfgs,
+                   **({"tile_kernels": True} if args.tile_kernels else {})},
         "tflops": round(total_flops / step_s / 1e12, 3), "hbm_gbps": round(total_bytes / step_s / 1e9, 1),
         "wall_ms_per_step": round(wall_ms, 5), "launch": "hip graph replay" if use_graph else "python launches",
         "steps_per_graph": (n_graphs if turn is not None and args.steps >= n_graphs else 1),
