@@ -12,6 +12,8 @@
 #include <cstdlib>
 
 #include "fp8_tile.h"
+#include <algorithm>
+
 #include "ksq_common.h"
 #include "splitk_reduce.h"
 #include "tile_select.h"
@@ -327,7 +329,9 @@ int launch_fp8_tile(const Fp8Params& q, const TilePlan& plan, float* partial, hi
 template <typename TO, int WM>
 int launch_fp8_tile_grouped(const Fp8Params& q, unsigned blocks, hipStream_t s) {
   constexpr int kLdsMax = 160 * 1024;
-  const size_t lds = fp8_tile_lds_bytes(WM, q.K / 128);
+  // (the 256-slot kernel runs half-empty blocks on the 128-token tile's three stages)
+  const size_t lds = WM == 8 ? std::max(fp8_tile_lds_bytes(8, q.K / 128), fp8_tile_lds_bytes(4, q.K / 128))
+                             : fp8_tile_lds_bytes(WM, q.K / 128);
   if (lds > kLdsMax) return fail(KSQ_ERR_UNSUPPORTED, "k range of %u blocks per workgroup does not fit the LDS", q.K / 128);
   // more dynamic LDS than a kernel may use without asking: once per device
   static std::atomic<uint64_t> configured{0};

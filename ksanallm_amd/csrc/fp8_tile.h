@@ -60,9 +60,12 @@ constexpr size_t fp8_tile_lds_bytes(int wm, size_t kb_max) {
   return static_cast<size_t>(fp8_tile_stages(wm)) * (fp8_tile_stage_bytes(wm) + 1024) + 2 * kb_max * 4;
 }
 
-template <typename TO, bool GROUPED = false, int WM = 8>
-__global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
+// BLOCK: slots between consecutive row blocks (tile_m * BLOCK is the block's first slot): the tile's own 32 * WM rows, or
+// - grouped form - 256 for a 128-token tile that serves a 256-slot block of which at most the lower half holds tokens.
+template <typename TO, bool GROUPED, int WM, int BLOCK>
+__device__ __forceinline__ void fp8_tile_body(const Fp8TileParams& p, char* lds) {
   static_assert(WM == 8 || WM == 4, "256- or 128-token tiles");
+  static_assert(BLOCK == 2 * WM * 16 || (GROUPED && WM == 4 && BLOCK == 256), "block stride");
   constexpr int WAVES_N = 4;
   constexpr int WN = 4;  // 16x16 tiles per wavefront: 16*WM tokens x 64 weight rows
   constexpr int BM = 2 * WM * 16, BN = 256;
@@ -72,8 +75,6 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
   constexpr int STAGE_BYTES = fp8_tile_stage_bytes(WM);  // AF activation + 16 weight fragments
   constexpr int W_FRAG0 = AF;                 // first weight fragment of a stage
   constexpr int NS = fp8_tile_stages(WM);     // LDS stages
-
-  extern __shared__ __attribute__((aligned(16))) char lds[];  // fp8_tile_lds_bytes
 
   const int lane = threadIdx.x & 63;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -87,7 +88,7 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
   const uint32_t tile_m = __builtin_amdgcn_readfirstlane(work.tile_m), tile_n = __builtin_amdgcn_readfirstlane(work.tile_n);
   const uint32_t part = __builtin_amdgcn_readfirstlane(work.part), slot = __builtin_amdgcn_readfirstlane(work.slot);
   const bool direct = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(work.direct)) != 0;
-  const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
+  const uint32_t m0 = tile_m * BLOCK, n0 = tile_n * BN;
   const uint32_t kb_begin = direct ? 0 : part * p.kb_per_split;
   const uint32_t kb_count = direct ? KB : ((KB - kb_begin) < p.kb_per_split ? (KB - kb_begin) : p.kb_per_split);
 
@@ -112,13 +113,20 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
     expert = static_cast<size_t>(__builtin_amdgcn_readfirstlane(p.expert_ids[tile_m]));
     uint32_t rows = 0;
 #pragma unroll
-    for (int h = 0; h < BM / 64; ++h) {
+    for (int h = 0; h < BLOCK / 64; ++h) {
       const bool is_row = static_cast<uint32_t>(p.sorted_ids[m0 + h * 64 + lane]) < p.numel;
       rows += static_cast<uint32_t>(__builtin_popcountll(__builtin_amdgcn_ballot_w64(is_row)));
     }
     live_tiles = __builtin_amdgcn_readfirstlane((rows + 15) / 16);
   }
-  const bool idle = live_tiles <= wm * WM;  // none of this wavefront's row tiles wm*WM .. holds a token
+  // The two wavefront rows split the block's row tiles: WM each - or, when at most WM of the 2 * WM hold tokens (a
+  // grouped block at most half full: an expert with half a block's slots), WM / 2 each of the lower WM, so that no SIMD
+  // is left with one working wavefront and one that only takes part in loads and barriers.
+  const bool lower_half = GROUPED && live_tiles <= WM;
+  const uint32_t per_wave = lower_half ? WM / 2 : WM;  // row tiles a wavefront covers
+  const uint32_t rt0 = wm * per_wave;                   // its first row tile
+  const uint32_t mine = live_tiles > rt0 ? (live_tiles - rt0 < per_wave ? live_tiles - rt0 : per_wave) : 0;
+  const bool idle = mine == 0;  // none of this wavefront's row tiles holds a token
   const bool stage_act = wave < 4;
   const uint32_t frag0 = (wave & 3) * (stage_act ? AFW : 4);
   // Weights come as packed 2 KiB fragments (ksq_fp8_repack_weight), fragment (strip, k-block) at (strip*KB + kb)*2048:
@@ -191,7 +199,7 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
     }
   }
   const float* bs_lds = reinterpret_cast<const float*>(lds + BS_BASE) + (wn >> 1) * kb_count;
-  const float* as_lds = reinterpret_cast<const float*>(lds + SCALE_BASE) + wm * (WM * 16) + lrow;
+  const float* as_lds = reinterpret_cast<const float*>(lds + SCALE_BASE) + rt0 * 16 + lrow;
 
   // Every group of loads is one assembly statement opening with `s_nop 4`: its scalar operands are in place before
   // it starts, and the wait states a vector memory instruction needs after a VALU write of a scalar register have
@@ -211,7 +219,11 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
   };
   // operands of k-block `kb` -> LDS slot kb % 2.  The instruction offset of an LDS-targeted load is added to the LDS
   // address as well as to the global one: the second half's 64-byte global offset is taken out of its LDS base.
+  // (a block at most half full: the activation fragments of its upper half are never read and, where every wait is
+  // for all of a wavefront's loads - two stages -, not fetched either)
+  const bool skip_act = NS == 2 && lower_half && stage_act && frag0 >= static_cast<uint32_t>(WM);
   auto load_operands = [&](uint32_t kb) {
+    if (skip_act) return;
     const uint32_t k = kb < kb_count ? kb : kb_count - 1;
     const uint8_t* src = g_tile + static_cast<size_t>(k) * k_step;
     const uint32_t f0 = __builtin_amdgcn_readfirstlane(d_lds + (kb % NS) * STAGE_BYTES);
@@ -298,7 +310,7 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
 #pragma unroll
       for (int i = 0; i < WMV; ++i) sc[i] = as_lds[slot * 256 + i * 16] * bs;
     }
-    const char* act = lds + slot * STAGE_BYTES + (wm * WM) * FRAG;
+    const char* act = lds + slot * STAGE_BYTES + rt0 * FRAG;
     const char* wgt = lds + slot * STAGE_BYTES + (W_FRAG0 + wn * WN) * FRAG;
     i32x8 wf[WN];
     i32x8 af[2];
@@ -354,7 +366,7 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
       __builtin_amdgcn_s_barrier();
     }
   } else {
-    for_tile_count<1, WM>(live_tiles - wm * WM, [&](auto wmv_c) {
+    for_tile_count<1, WM>(mine, [&](auto wmv_c) {
       for (uint32_t c = 0; c < kb_count; ++c) {
         compute(wmv_c, c % NS, c, c + NS - 1);
         wait_stage();  // operands and scales of c+1
@@ -373,17 +385,17 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
   float rws[WM];
   if (GROUPED) {
 #pragma unroll
-    for (int i = 0; i < WM; ++i) sids[i] = static_cast<uint32_t>(p.sorted_ids[m0 + wm * (WM * 16) + i * 16 + lrow]);
+    for (int i = 0; i < WM; ++i) sids[i] = static_cast<uint32_t>(p.sorted_ids[m0 + rt0 * 16 + (i < static_cast<int>(per_wave) ? i : 0) * 16 + lrow]);
 #pragma unroll
     for (int i = 0; i < WM; ++i) rws[i] = (sids[i] < p.numel && p.topk_w) ? p.topk_w[sids[i]] : 1.0f;
   }
 #pragma unroll
   for (int i = 0; i < WM; ++i) {
-    uint32_t row = m0 + wm * (WM * 16) + i * 16 + lrow;
-    bool live = row < p.M;
+    uint32_t row = m0 + rt0 * 16 + i * 16 + lrow;
+    bool live = row < p.M && i < static_cast<int>(per_wave);  // row tiles past this wavefront's share belong to the other row
     float rw = 1.0f;
     if (GROUPED) {
-      live = sids[i] < p.numel;
+      live = sids[i] < p.numel && i < static_cast<int>(per_wave);
       row = sids[i];
       rw = rws[i];
     }
@@ -409,6 +421,30 @@ __global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
       }
     }
   }
+}
+
+// A 256-slot block of the grouped form of which at most 128 slots hold tokens (an expert with half a block's tokens or
+// fewer) runs the 128-token tile's code: three stages of 48 KiB instead of two of 64 - a half-empty stage is over in
+// less time than its successor's loads take to arrive - and every wavefront at work.
+template <typename TO, bool GROUPED = false, int WM = 8>
+__global__ void __launch_bounds__(512, 1) fp8_tile_kernel(Fp8TileParams p) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];  // fp8_tile_lds_bytes (the larger of both forms)
+  if constexpr (GROUPED && WM == 8) {
+    const TileWork work = tile_work(blockIdx.x, p.tiles_m, p.tiles_n, p.main_items, p.splits, true);
+    const uint32_t m0 = __builtin_amdgcn_readfirstlane(work.tile_m) * 256;
+    if (m0 >= static_cast<uint32_t>(p.num_post_pad[0])) return;  // uniform: the whole workgroup leaves
+    uint32_t rows = 0;
+#pragma unroll
+    for (int h = 0; h < 4; ++h) {
+      const bool is_row = static_cast<uint32_t>(p.sorted_ids[m0 + h * 64 + (threadIdx.x & 63)]) < p.numel;
+      rows += static_cast<uint32_t>(__builtin_popcountll(__builtin_amdgcn_ballot_w64(is_row)));
+    }
+    if (__builtin_amdgcn_readfirstlane(rows) <= 128) {
+      fp8_tile_body<TO, true, 4, 256>(p, lds);
+      return;
+    }
+  }
+  fp8_tile_body<TO, GROUPED, WM, 2 * WM * 16>(p, lds);
 }
 
 }  // namespace ksq
