@@ -173,6 +173,8 @@ int ksq_w4a16_gemm_static(void* y, const void* x, const void* w_packed, const vo
  *   amax = max(1e-10, max|x|); s = amax / 448; q = e4m3_rne_satfinite(x / s)   (IEEE fp32 divisions)
  * x [m, k] T (or [m, 2k] when fuse_silu_mul: x = T(silu(x[:, :k]) * x[:, k:])), q [m, k] bytes,
  * s fp32 [m, k/group] or, when column_major, [k/group, m].
+ * dtype KSQ_F16, KSQ_BF16 or KSQ_F32 (x float, no rounding to T in the fused form): the reference instantiates all three
+ * (basic_kernel_wrapper.cpp:1237-1239).
  * Replaces InvokePerTokenGroupQuantFp8E4m3 (S/kernels/nvidia/basic_kernel_wrapper.cpp:1222-1232;
  * K/others/sglang/main/quantization/fp8/per_token_group_quant.cu:275-329).
  * ------------------------------------------------------------------------------------------------------------------ */
@@ -182,7 +184,8 @@ int ksq_fp8_group_quant(const void* x, void* q, void* s, size_t m, size_t k, siz
 /* ------------------------------------------------------------------------------------------------------------------
  * Blockwise FP8 GEMM: out[m,n] = sum_kb (a_q[m,kb] . b[n,kb]) * a_s[kb,m] * b_s[n/128,kb], fp32 accumulate.
  * a_q [m,k] e4m3 row-major, a_s fp32 column-major [k/128, m], b [n,k] e4m3 in the packed fragment layout (ksq_fp8_repack_weight),
- * b_s fp32 [ceil(n/128), k/128], out [m,n] in out_dtype.  k must be a multiple of 128, n of 16.
+ * b_s fp32 [ceil(n/128), k/128], out [m,n] in out_dtype (KSQ_F16, KSQ_BF16, or KSQ_F32 for fp32 activations: the sums
+ * as they are, InvokeBlockGemm<float>, basic_kernel_wrapper.cpp:1096).  k must be a multiple of 128, n of 16.
  * Replaces InvokeBlockGemm / InvokeGetBlockGemmWorkspaceSize (K/blockwise_gemm/blockwise_gemm.cu:17-33) and
  * DeepGEMMWrapper::Gemm / GemmSwapAB (K/gemm/deepgemm/deepgemm_wrapper.cu:33-103).
  * ------------------------------------------------------------------------------------------------------------------ */
@@ -200,6 +203,7 @@ int ksq_fp8_blockwise_gemm_f32(const void* a_q, const void* a_s, const void* b, 
  *   dynamic (is_static = 0): scale[c] = max(amax|x[c,:]| / 448, 1 / (448 * 512)) is computed and written first
  *   static  (is_static = 1): scale[c] is read
  *   q = e4m3(clamp(x / scale, -448, 448)), IEEE division, round to nearest even.
+ * dtype KSQ_F16, KSQ_BF16 or KSQ_F32 (x float).
  * Replaces Fp8E4m3Quantize (S/kernels/nvidia/basic_kernel_wrapper.cpp:1028-1036) = InvokeComputeFP8QuantizeScale +
  * InvokeQuantizeMatrix (3rdparty/LLM_kernels/csrc/utils/nvidia/cuda_fp8_utils.cu:32-266).
  * ------------------------------------------------------------------------------------------------------------------ */
@@ -208,7 +212,8 @@ int ksq_fp8_channel_quant(const void* x, void* q, void* scale, size_t channels, 
 
 /* Per-tensor-scaled FP8 GEMM: out[m,n] = T((sum_k a_q[m,k] . b[n,k]) * a_scale[0] * b_scale[0]), fp32 accumulation.
  * a_q [m,k] e4m3 row-major, b [n,k] e4m3 packed by ksq_fp8_repack_weight; a_scale, b_scale: one fp32 each in device
- * memory.  k % 128 == 0, n % 16 == 0.
+ * memory.  k % 128 == 0, n % 16 == 0.  out_dtype KSQ_F16, KSQ_BF16 or KSQ_F32 (fp32 activations: the scaled sums as
+ * they are).
  * The workspace (256-byte aligned) holds the scales spread into the blockwise layouts and the split-K partials of
  * the blockwise kernels, which do the work.
  * Replaces Fp8QuantizedMatMul (S/kernels/nvidia/basic_kernel_wrapper.cpp:1042-1052, cuBLASLt with scale pointers). */

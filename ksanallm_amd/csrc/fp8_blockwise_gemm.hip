@@ -443,6 +443,9 @@ int fp8_blockwise_gemm_impl(const char* fn, const void* a_q, const void* a_s, co
 KSQ_EXPORT int ksq_fp8_blockwise_gemm(const void* a_q, const void* a_s, const void* b, const void* b_s, void* out,
                                       size_t m, size_t n, size_t k, int out_dtype, void* workspace,
                                       size_t workspace_bytes, void* stream) {
+  if (out_dtype == KSQ_F32)  // fp32 activations: the sums are the output (the reference instantiates InvokeBlockGemm<float>)
+    return fp8_blockwise_gemm_impl("ksq_fp8_blockwise_gemm", a_q, a_s, b, b_s, nullptr, m, n, k, KSQ_BF16, workspace,
+                                   workspace_bytes, stream, static_cast<float*>(out));
   return fp8_blockwise_gemm_impl("ksq_fp8_blockwise_gemm", a_q, a_s, b, b_s, out, m, n, k, out_dtype, workspace,
                                  workspace_bytes, stream, nullptr);
 }

@@ -12,6 +12,8 @@
 // mantissa a 16-bit input can have.  The sign of x is put back afterwards (x = -0 would otherwise come out as +0).
 // Scales outside [2^-80, 2^100] take the division itself; inside, r is exact whenever |x / s| >= 2^-20, and a smaller
 // quotient that is one unit in the last place off still converts to the same signed zero.
+#include <type_traits>
+
 #include "exact_div.h"
 #include "ksq_common.h"
 
@@ -35,12 +37,47 @@ __device__ __forceinline__ uint32_t cvt2_e4m3_in_range(float a, float b, uint32_
             : static_cast<uint32_t>(__builtin_amdgcn_cvt_pk_fp8_f32(a, b, static_cast<int>(old), false));
 }
 
+// fp32 activations (the reference instantiates its quantizer for float as well): the same kernel with 32-byte loads and
+// IEEE divisions throughout - the reciprocal-and-correction form above is proven for inputs of at most 11 significant
+// bits, and this type is not on any model's hot path.
+struct F32 {
+  static constexpr int kTag = KSQ_F32;
+};
+
+// eight consecutive channels of one row as floats
+template <typename T>
+__device__ __forceinline__ void load8(const void* x, size_t e, float (&v)[8]) {
+  if constexpr (std::is_same<T, F32>::value) {
+    const float* src = static_cast<const float*>(x) + e;
+    const f32x4 a = *reinterpret_cast<const f32x4*>(src), b = *reinterpret_cast<const f32x4*>(src + 4);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      v[j] = a[j];
+      v[4 + j] = b[j];
+    }
+  } else {
+    const u32x4 raw = *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(x) + e);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      v[2 * j] = T::to_float(static_cast<uint16_t>(raw[j] & 0xffffu));
+      v[2 * j + 1] = T::to_float(static_cast<uint16_t>(raw[j] >> 16));
+    }
+  }
+}
+
+template <typename T>
+__device__ __forceinline__ float load1(const void* x, size_t e) {
+  if constexpr (std::is_same<T, F32>::value) return static_cast<const float*>(x)[e];
+  else return T::to_float(static_cast<const uint16_t*>(x)[e]);
+}
+
 // Grid: x = chunks of BLOCK*8 channels of a row, y and z = the row (token) as z * gridDim.y + y, so that no index needs
 // an integer division (about fifty instructions on this ISA, more than the rest of the kernel).  Lanes past the end of
 // the row in its last chunk idle; groups never straddle a chunk.
 template <typename T, int GROUP, bool COLMAJOR, bool FUSE, int BLOCK>
-__global__ void __launch_bounds__(BLOCK) fp8_group_quant_kernel(const uint16_t* __restrict__ x, uint8_t* __restrict__ q,
+__global__ void __launch_bounds__(BLOCK) fp8_group_quant_kernel(const void* __restrict__ x, uint8_t* __restrict__ q,
                                                                 float* __restrict__ s, uint32_t m, uint32_t k) {
+  constexpr bool kF32 = std::is_same<T, F32>::value;
   constexpr int LPG = GROUP / 8;  // lanes per group
   const uint32_t row = blockIdx.z * gridDim.y + blockIdx.y;
   const uint32_t col0 = (blockIdx.x * BLOCK + threadIdx.x) * 8;
@@ -51,26 +88,18 @@ __global__ void __launch_bounds__(BLOCK) fp8_group_quant_kernel(const uint16_t* 
 
   float v[8];
   {
-    const uint16_t* src = FUSE ? x + static_cast<size_t>(t) * 2 * k + col : x + e0;
-    u32x4 raw = *reinterpret_cast<const u32x4*>(src);
-    uint16_t h[8] = {static_cast<uint16_t>(raw.x), static_cast<uint16_t>(raw.x >> 16),
-                     static_cast<uint16_t>(raw.y), static_cast<uint16_t>(raw.y >> 16),
-                     static_cast<uint16_t>(raw.z), static_cast<uint16_t>(raw.z >> 16),
-                     static_cast<uint16_t>(raw.w), static_cast<uint16_t>(raw.w >> 16)};
-#pragma unroll
-    for (int j = 0; j < 8; ++j) v[j] = T::to_float(h[j]);
+    const size_t src = FUSE ? static_cast<size_t>(t) * 2 * k + col : e0;
+    load8<T>(x, src, v);
     if (FUSE) {
-      u32x4 r2 = *reinterpret_cast<const u32x4*>(src + k);
-      uint16_t u[8] = {static_cast<uint16_t>(r2.x), static_cast<uint16_t>(r2.x >> 16),
-                       static_cast<uint16_t>(r2.y), static_cast<uint16_t>(r2.y >> 16),
-                       static_cast<uint16_t>(r2.z), static_cast<uint16_t>(r2.z >> 16),
-                       static_cast<uint16_t>(r2.w), static_cast<uint16_t>(r2.w >> 16)};
+      float u[8];
+      load8<T>(x, src + k, u);
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         // the one definition of silu * mul every kernel here uses (ksq_common.h), so that the int4 and the block-fp8
         // expert paths apply the same activation
-        const float act = silu_mul_f32(v[j], T::to_float(u[j]));
-        v[j] = T::to_float(T::from_float(act));  // the reference rounds silu*mul to T before quantizing
+        const float act = silu_mul_f32(v[j], u[j]);
+        if constexpr (kF32) v[j] = act;
+        else v[j] = T::to_float(T::from_float(act));  // the reference rounds silu*mul to T before quantizing
       }
     }
   }
@@ -90,7 +119,7 @@ __global__ void __launch_bounds__(BLOCK) fp8_group_quant_kernel(const uint16_t* 
     const float r = __builtin_fmaf(-q0, 448.0f, amax);
     scale = __builtin_fmaf(r, y448, q0);
     scale = amax == 1e-10f ? 1e-10f / 448.0f : scale;
-    scale = (amax >= 0x1p-60f && amax <= 0x1p100f) ? scale : amax / 448.0f;
+    scale = (!kF32 && amax >= 0x1p-60f && amax <= 0x1p100f) ? scale : amax / 448.0f;
   }
   if (!live) return;
   if ((threadIdx.x % LPG) == 0) {
@@ -100,7 +129,7 @@ __global__ void __launch_bounds__(BLOCK) fp8_group_quant_kernel(const uint16_t* 
   }
   u32x2 out{0u, 0u};
   const ExactDiv div(scale);
-  if (div.fast) {
+  if (!kF32 && div.fast) {
     // every |v| <= amax (an infinite v makes amax, hence the scale, infinite: not this branch), so the quotients stay
     // within 448 * (1 + 2^-23), which the conversion rounds to 448 by itself
     out.x = cvt2_e4m3_in_range(div(v[0]), div(v[1]), out.x, false);
@@ -120,7 +149,7 @@ template <typename T, int GROUP, int BLOCK>
 void launch_block(const void* x, void* q, void* s, uint32_t m, uint32_t k, bool col, bool fuse, hipStream_t st) {
   const unsigned gy = m < 32768u ? m : 32768u;
   const dim3 grid(static_cast<unsigned>(div_up(k, BLOCK * 8)), gy, static_cast<unsigned>(div_up(m, gy)));
-  const uint16_t* xp = static_cast<const uint16_t*>(x);
+  const void* xp = x;
   uint8_t* qp = static_cast<uint8_t*>(q);
   float* sp = static_cast<float*>(s);
   if (col) {
@@ -152,36 +181,38 @@ __global__ void fp8_scale_clear_kernel(float* __restrict__ scale, uint32_t chann
 // scale[c] = max(amax(|x[c, :]|) / 448, 1 / (448 * 512)).  Every workgroup folds its maximum in with an integer
 // atomic max on the float's bits (all candidates are positive, so the orders agree); scale[] starts at 0.
 template <typename T>
-__global__ void __launch_bounds__(256) fp8_channel_scale_kernel(const uint16_t* __restrict__ x, float* __restrict__ scale,
+__global__ void __launch_bounds__(256) fp8_channel_scale_kernel(const void* __restrict__ x, float* __restrict__ scale,
                                                                 size_t size, bool vec) {
-  const uint16_t* row = x + static_cast<size_t>(blockIdx.y) * size;
+  const size_t row = static_cast<size_t>(blockIdx.y) * size;  // first element of this channel
   const size_t tid = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
   const size_t stride = static_cast<size_t>(gridDim.x) * 256;
   float amax = 0.f;
   if (vec) {
-    auto fold = [&](u32x4 raw) {
+    auto fold = [&](const float (&v)[8]) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        amax = fmaxf(amax, fabsf(T::to_float(static_cast<uint16_t>(raw[j] & 0xffffu))));
-        amax = fmaxf(amax, fabsf(T::to_float(static_cast<uint16_t>(raw[j] >> 16))));
-      }
+      for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[j]));
     };
     const size_t n8 = size / 8;
     size_t i = tid;
     // four independent loads in flight per thread: one load per trip leaves the pass waiting on memory latency
     for (; i + 3 * stride < n8; i += 4 * stride) {
-      const u32x4 r0 = *reinterpret_cast<const u32x4*>(row + i * 8);
-      const u32x4 r1 = *reinterpret_cast<const u32x4*>(row + (i + stride) * 8);
-      const u32x4 r2 = *reinterpret_cast<const u32x4*>(row + (i + 2 * stride) * 8);
-      const u32x4 r3 = *reinterpret_cast<const u32x4*>(row + (i + 3 * stride) * 8);
+      float r0[8], r1[8], r2[8], r3[8];
+      load8<T>(x, row + i * 8, r0);
+      load8<T>(x, row + (i + stride) * 8, r1);
+      load8<T>(x, row + (i + 2 * stride) * 8, r2);
+      load8<T>(x, row + (i + 3 * stride) * 8, r3);
       fold(r0);
       fold(r1);
       fold(r2);
       fold(r3);
     }
-    for (; i < n8; i += stride) fold(*reinterpret_cast<const u32x4*>(row + i * 8));
+    for (; i < n8; i += stride) {
+      float r0[8];
+      load8<T>(x, row + i * 8, r0);
+      fold(r0);
+    }
   } else {
-    for (size_t i = tid; i < size; i += stride) amax = fmaxf(amax, fabsf(T::to_float(row[i])));
+    for (size_t i = tid; i < size; i += stride) amax = fmaxf(amax, fabsf(load1<T>(x, row + i)));
   }
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
@@ -199,7 +230,7 @@ __global__ void __launch_bounds__(256) fp8_channel_scale_kernel(const uint16_t* 
 
 // q[c, i] = e4m3(clamp(x[c, i] / scale[c], -448, 448)), IEEE division, round to nearest even
 template <typename T>
-__global__ void __launch_bounds__(256) fp8_channel_quant_kernel(const uint16_t* __restrict__ x, uint8_t* __restrict__ q,
+__global__ void __launch_bounds__(256) fp8_channel_quant_kernel(const void* __restrict__ x, uint8_t* __restrict__ q,
                                                                 const float* __restrict__ scale, size_t size, bool vec) {
   const size_t base = static_cast<size_t>(blockIdx.y) * size;
   const float sc = scale[blockIdx.y];
@@ -208,19 +239,14 @@ __global__ void __launch_bounds__(256) fp8_channel_quant_kernel(const uint16_t* 
   const size_t stride = static_cast<size_t>(gridDim.x) * 256;
   if (vec) {
     for (size_t i = tid; i < size / 8; i += stride) {
-      const u32x4 raw = *reinterpret_cast<const u32x4*>(x + base + i * 8);
       float v[8];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        v[2 * j] = T::to_float(static_cast<uint16_t>(raw[j] & 0xffffu));
-        v[2 * j + 1] = T::to_float(static_cast<uint16_t>(raw[j] >> 16));
-      }
+      load8<T>(x, base + i * 8, v);
       // with a scale handed in by the caller an input may be infinite where the scale is not: such a lane keeps the
       // division (a branch, not a select per element: a select would evaluate the division for every element)
       float mx = 0.f;
 #pragma unroll
       for (int j = 0; j < 8; ++j) mx = fmaxf(mx, __builtin_fabsf(v[j]));
-      if (mx == __builtin_inff()) {
+      if (std::is_same<T, F32>::value || mx == __builtin_inff()) {  // (fp32 inputs: the division, see F32)
 #pragma unroll
         for (int j = 0; j < 8; ++j) v[j] = v[j] / sc;
       } else {
@@ -236,7 +262,7 @@ __global__ void __launch_bounds__(256) fp8_channel_quant_kernel(const uint16_t* 
     }
   } else {
     for (size_t i = tid; i < size; i += stride)
-      q[base + i] = static_cast<uint8_t>(cvt2_e4m3(T::to_float(x[base + i]) / sc, 0.f, 0u, false) & 0xffu);
+      q[base + i] = static_cast<uint8_t>(cvt2_e4m3(load1<T>(x, base + i) / sc, 0.f, 0u, false) & 0xffu);
   }
 }
 
@@ -254,7 +280,8 @@ KSQ_EXPORT int ksq_fp8_group_quant(const void* x, void* q, void* s, size_t m, si
   if (group != 32 && group != 64 && group != 128)
     return fail(KSQ_ERR_UNSUPPORTED, "%s: group size %zu not in {32,64,128}", fn, group);
   if (k == 0 || k % group != 0) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: k must be a positive multiple of group", fn);
-  if (dtype != KSQ_F16 && dtype != KSQ_BF16) return fail(KSQ_ERR_UNSUPPORTED, "%s: dtype must be f16 or bf16", fn);
+  if (dtype != KSQ_F16 && dtype != KSQ_BF16 && dtype != KSQ_F32)
+    return fail(KSQ_ERR_UNSUPPORTED, "%s: dtype must be f16, bf16 or f32", fn);
   if (m == 0) return KSQ_OK;
   if (m > 0x7fffffffull || k > 0x7fffffffull || m * k / 8 / 256 + 1 > 0x7fffffffull)
     return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: tensor too large", fn);
@@ -262,7 +289,9 @@ KSQ_EXPORT int ksq_fp8_group_quant(const void* x, void* q, void* s, size_t m, si
   hipStream_t st = as_stream(stream);
   const bool col = column_major != 0, fuse = fuse_silu_mul != 0;
 #define KSQ_Q(TT, G) launch<TT, G>(x, q, s, mm, kk, col, fuse, st)
-  if (dtype == KSQ_F16) {
+  if (dtype == KSQ_F32) {
+    if (group == 128) KSQ_Q(F32, 128); else if (group == 64) KSQ_Q(F32, 64); else KSQ_Q(F32, 32);
+  } else if (dtype == KSQ_F16) {
     if (group == 128) KSQ_Q(F16, 128); else if (group == 64) KSQ_Q(F16, 64); else KSQ_Q(F16, 32);
   } else {
     if (group == 128) KSQ_Q(BF16, 128); else if (group == 64) KSQ_Q(BF16, 64); else KSQ_Q(BF16, 32);
@@ -275,9 +304,10 @@ KSQ_EXPORT int ksq_fp8_channel_quant(const void* x, void* q, void* scale, size_t
                                      int dtype, void* stream) {
   const char* fn = "ksq_fp8_channel_quant";
   if (!x || !q || !scale) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: null pointer", fn);
-  if ((reinterpret_cast<uintptr_t>(x) & 1u) || (reinterpret_cast<uintptr_t>(scale) & 3u))
-    return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: x must be 2-byte, scale 4-byte aligned", fn);
-  if (dtype != KSQ_F16 && dtype != KSQ_BF16) return fail(KSQ_ERR_UNSUPPORTED, "%s: dtype must be f16 or bf16", fn);
+  if (dtype != KSQ_F16 && dtype != KSQ_BF16 && dtype != KSQ_F32)
+    return fail(KSQ_ERR_UNSUPPORTED, "%s: dtype must be f16, bf16 or f32", fn);
+  if ((reinterpret_cast<uintptr_t>(x) & (dtype == KSQ_F32 ? 3u : 1u)) || (reinterpret_cast<uintptr_t>(scale) & 3u))
+    return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: x must be aligned to its element size, scale to 4 bytes", fn);
   if (channels == 0 || size == 0) return KSQ_OK;
   if (channels > 65535) return fail(KSQ_ERR_INVALID_ARGUMENT, "%s: at most 65535 channels", fn);
   // 16-byte loads and 8-byte stores need rows that start on those boundaries
@@ -287,16 +317,18 @@ KSQ_EXPORT int ksq_fp8_channel_quant(const void* x, void* q, void* scale, size_t
   if (bx > 1024) bx = 1024;
   const dim3 grid(static_cast<unsigned>(bx), static_cast<unsigned>(channels), 1);
   hipStream_t st = as_stream(stream);
-  const uint16_t* xp = static_cast<const uint16_t*>(x);
+  const void* xp = x;
   float* sp = static_cast<float*>(scale);
   if (!is_static) {
     fp8_scale_clear_kernel<<<static_cast<unsigned>(div_up(channels, 256)), 256, 0, st>>>(sp, static_cast<uint32_t>(channels));
     // two workgroups per CU read as fast as more do and keep the atomics few
     const dim3 sgrid(static_cast<unsigned>(bx < 512 ? bx : 512), static_cast<unsigned>(channels), 1);
-    if (dtype == KSQ_F16) fp8_channel_scale_kernel<F16><<<sgrid, 256, 0, st>>>(xp, sp, size, vec);
+    if (dtype == KSQ_F32) fp8_channel_scale_kernel<F32><<<sgrid, 256, 0, st>>>(xp, sp, size, vec);
+    else if (dtype == KSQ_F16) fp8_channel_scale_kernel<F16><<<sgrid, 256, 0, st>>>(xp, sp, size, vec);
     else fp8_channel_scale_kernel<BF16><<<sgrid, 256, 0, st>>>(xp, sp, size, vec);
   }
-  if (dtype == KSQ_F16) fp8_channel_quant_kernel<F16><<<grid, 256, 0, st>>>(xp, static_cast<uint8_t*>(q), sp, size, vec);
+  if (dtype == KSQ_F32) fp8_channel_quant_kernel<F32><<<grid, 256, 0, st>>>(xp, static_cast<uint8_t*>(q), sp, size, vec);
+  else if (dtype == KSQ_F16) fp8_channel_quant_kernel<F16><<<grid, 256, 0, st>>>(xp, static_cast<uint8_t*>(q), sp, size, vec);
   else fp8_channel_quant_kernel<BF16><<<grid, 256, 0, st>>>(xp, static_cast<uint8_t*>(q), sp, size, vec);
   return check_launch(fn);
 }

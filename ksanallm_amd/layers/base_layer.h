@@ -58,12 +58,18 @@ class BaseLayer {
 
 namespace ksana_llm {
 
-// activation type of the reference's template parameter T -> tag of the kernel library; fp32 activations have no
-// quantized kernels here (the reference instantiates them but no shipped model config reaches them)
+// activation type of the reference's template parameter T -> tag of the kernel library; fp32 activations are taken by
+// the fp8 layers only (KsqDtypeOrFp32), the int4 kernels multiply 16-bit activations
 inline int KsqDtype(DataType dtype, const char* who) {
   if (dtype == TYPE_FP16) return KSQ_F16;
   if (dtype == TYPE_BF16) return KSQ_BF16;
   KLLM_THROW(std::string(who) + ": Unsupported Dtype type: " + std::to_string(static_cast<int>(dtype)));
+}
+
+// the same for the layers whose kernels also take fp32 activations (the block-fp8 quantizer and GEMM, which the
+// reference instantiates for float: basic_kernel_wrapper.cpp:1096,1237)
+inline int KsqDtypeOrFp32(DataType dtype, const char* who) {
+  return dtype == TYPE_FP32 ? KSQ_F32 : KsqDtype(dtype, who);
 }
 
 // kernel-library status -> exception, like KLLM_KERNEL_CHECK does for a failed launch

@@ -34,8 +34,8 @@ size_t BlockwiseMatMulLayer::GetWorkspaceSize() {
 
 Status BlockwiseMatMulLayer::Preprocess(const ModelConfig& model_config, const RuntimeConfig& runtime_config) {
   ksq_tile_desc desc;
-  const int dtype = KsqDtype(inter_data_type_, "BlockwiseMatMulLayer");
-  if (ksq_select_tile(KSQ_KIND_FP8_BLOCKWISE, max_m_ ? max_m_ : 1, n_, k_, dtype, &desc) != KSQ_OK) {
+  const int dtype = KsqDtypeOrFp32(inter_data_type_, "BlockwiseMatMulLayer");
+  if (ksq_select_tile(KSQ_KIND_FP8_BLOCKWISE, max_m_ ? max_m_ : 1, n_, k_, dtype == KSQ_F32 ? KSQ_BF16 : dtype, &desc) != KSQ_OK) {
     return Status(RET_INVALID_ARGUMENT, std::string("BlockwiseMatMulLayer: ") + ksq_last_error_string());
   }
   return Status();
@@ -51,7 +51,7 @@ Status BlockwiseMatMulLayer::Forward(const std::vector<Tensor>& input_tensors, s
   if (k != k_ && k != 2 * k_) KLLM_THROW("BlockwiseMatMulLayer: activation inner dimension must be k or 2k");
   if (m > max_m_) KLLM_THROW("BlockwiseMatMulLayer: m exceeds max_m");
   if (!input_tensors[1].weight_scales) KLLM_THROW("BlockwiseMatMulLayer: weight tensor has no weight_scales bound");
-  const int dtype = KsqDtype(inter_data_type_, "BlockwiseMatMulLayer");
+  const int dtype = KsqDtypeOrFp32(inter_data_type_, "BlockwiseMatMulLayer");  // fp32: DISPATCH_BY_3_DTYPE of the reference's Forward
   hipStream_t stream = context_->GetComputeStreams()[rank_].Get();
 
   char* base = workspace_buffer_->GetPtr<char>();

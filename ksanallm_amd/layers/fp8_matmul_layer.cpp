@@ -12,7 +12,7 @@ Status Fp8MatMulLayer::Init(const std::vector<std::any>& parameters, const Runti
   max_m_ = std::any_cast<const size_t>(parameters[parameter_index++]);
   max_k_ = std::any_cast<const size_t>(parameters[parameter_index++]);
   if (max_k_ % 128 != 0) return Status(RET_INVALID_ARGUMENT, "Fp8MatMulLayer: k must be a multiple of 128");
-  KsqDtype(inter_data_type_, "Fp8MatMulLayer");
+  KsqDtypeOrFp32(inter_data_type_, "Fp8MatMulLayer");
   return Status();
 }
 
@@ -42,7 +42,7 @@ Status Fp8MatMulLayer::Forward(const std::vector<Tensor>& input_tensors, std::ve
     KLLM_THROW("Fp8MatMulLayer: GEMM scratch " + std::to_string(gemm_need) + " exceeds the budget " +
                std::to_string(kGemmWorkspaceBytes));
   }
-  const int dtype = KsqDtype(inter_data_type_, "Fp8MatMulLayer");
+  const int dtype = KsqDtypeOrFp32(inter_data_type_, "Fp8MatMulLayer");
   hipStream_t stream = context_->GetComputeStreams()[rank_].Get();
 
   char* gemm_workspace = workspace_buffer_->GetPtr<char>();

@@ -25,6 +25,11 @@ MatMulLayerFactory::MatMulLayerFactory(const ModelConfig& model_config, const Ru
         &MatMulLayerFactory::BuildLayer<BlockwiseMatMulLayer>;
     builder_map_[{TYPE_FP8_E4M3, t, t, QUANT_FP8_E4M3, DEFAULT_LINEAR_BACKEND}] = &MatMulLayerFactory::BuildLayer<Fp8MatMulLayer>;
   }
+  // fp32 activations: the two fp8 layers, as in the reference's map (matmul_layer_factory.cpp:70-71, 77-78)
+  builder_map_[{TYPE_FP8_E4M3, TYPE_FP32, TYPE_FP32, QUANT_BLOCK_FP8_E4M3, DEFAULT_LINEAR_BACKEND}] =
+      &MatMulLayerFactory::BuildLayer<BlockwiseMatMulLayer>;
+  builder_map_[{TYPE_FP8_E4M3, TYPE_FP32, TYPE_FP32, QUANT_FP8_E4M3, DEFAULT_LINEAR_BACKEND}] =
+      &MatMulLayerFactory::BuildLayer<Fp8MatMulLayer>;
 }
 
 std::shared_ptr<BaseLayer> MatMulLayerFactory::CreateLayer(DataType weight_type, DataType input_type,

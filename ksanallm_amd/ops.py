@@ -13,11 +13,13 @@ _lib = _l.load()
 F16, BF16 = _l.F16, _l.BF16
 
 
-def _dt(t):
+def _dt(t, allow_f32=False):
     if t.dtype == torch.float16:
         return F16
     if t.dtype == torch.bfloat16:
         return BF16
+    if allow_f32 and t.dtype == torch.float32:   # the block-fp8 quantizer and GEMM also take / give fp32 activations
+        return _l.F32
     raise TypeError("activation dtype must be float16 or bfloat16, got %s" % t.dtype)
 
 
@@ -161,7 +163,7 @@ def per_token_group_quant_fp8(x, k, group=128, column_major=True, fuse_silu_mul=
     if s is None:
         s = torch.empty((k // group, m) if column_major else (m, k // group), dtype=torch.float32, device=x.device)
     _l.check(_lib.ksq_fp8_group_quant(_ptr(x), _ptr(q), _ptr(s), m, k, group, int(column_major), int(fuse_silu_mul),
-                                      _dt(x), _stream()))
+                                      _dt(x, allow_f32=True), _stream()))
     return q, s
 
 
@@ -182,8 +184,8 @@ def fp8_blockwise_gemm(a_q, a_s, b, b_s, out_dtype=torch.bfloat16, out=None, wor
             if workspace is None or workspace.numel() < need:
                 workspace = _WORKSPACES[a_q.device] = torch.empty(need, dtype=torch.uint8, device=a_q.device)
     ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
-    _l.check(_lib.ksq_fp8_blockwise_gemm(_ptr(a_q), _ptr(a_s), _ptr(b), _ptr(b_s), _ptr(out), m, n, k, _dt(out),
-                                         _ptr(workspace), ws_bytes, _stream()))
+    _l.check(_lib.ksq_fp8_blockwise_gemm(_ptr(a_q), _ptr(a_s), _ptr(b), _ptr(b_s), _ptr(out), m, n, k,
+                                         _dt(out, allow_f32=True), _ptr(workspace), ws_bytes, _stream()))
     return out
 
 
@@ -392,7 +394,7 @@ def fp8_e4m3_quantize(x, scale=None):
     q = torch.empty((channels, size), dtype=torch.uint8, device=x.device)
     static = scale is not None
     s = scale if static else torch.empty(channels, dtype=torch.float32, device=x.device)
-    _l.check(_lib.ksq_fp8_channel_quant(_ptr(x), _ptr(q), _ptr(s), channels, size, int(static), _dt(x), _stream()))
+    _l.check(_lib.ksq_fp8_channel_quant(_ptr(x), _ptr(q), _ptr(s), channels, size, int(static), _dt(x, allow_f32=True), _stream()))
     return q, s
 
 
@@ -404,7 +406,7 @@ def fp8_quantized_matmul(a_q, a_scale, b, b_scale, out_dtype=torch.bfloat16, out
         out = torch.empty((m, n), dtype=out_dtype, device=a_q.device)
     if workspace is None:
         workspace = torch.empty(_lib.ksq_fp8_tensor_gemm_workspace_size(m, n, k), dtype=torch.uint8, device=a_q.device)
-    _l.check(_lib.ksq_fp8_tensor_gemm(_ptr(a_q), _ptr(a_scale), _ptr(b), _ptr(b_scale), _ptr(out), m, n, k, _dt(out),
+    _l.check(_lib.ksq_fp8_tensor_gemm(_ptr(a_q), _ptr(a_scale), _ptr(b), _ptr(b_scale), _ptr(out), m, n, k, _dt(out, allow_f32=True),
                                       _ptr(workspace), workspace.numel(), _stream()))
     return out
 

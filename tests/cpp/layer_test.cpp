@@ -81,7 +81,9 @@ class TestWeights : public BaseWeight {
   std::map<std::string, Tensor> weights;
 };
 
-static DataType ParseT(const char* s) { return std::strcmp(s, "bf16") == 0 ? TYPE_BF16 : TYPE_FP16; }
+static DataType ParseT(const char* s) {
+  return std::strcmp(s, "bf16") == 0 ? TYPE_BF16 : (std::strcmp(s, "f32") == 0 ? TYPE_FP32 : TYPE_FP16);
+}
 
 static void Drive(std::shared_ptr<BaseLayer> layer, const ModelConfig& mc, const RuntimeConfig& rc,
                   const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) {

@@ -51,6 +51,40 @@ def test_quant_bit_exact(ops, oracle, dtype, m, k, group, colmajor):
     np.testing.assert_array_equal(q.cpu().numpy(), qo)
 
 
+@pytest.mark.parametrize("m,k,group", [(1, 7168, 128), (37, 1024, 64), (5, 256, 32), (130, 2048, 128)])
+@pytest.mark.parametrize("colmajor", [False, True])
+def test_quant_fp32_activations_bit_exact(ops, oracle, m, k, group, colmajor):
+    """The float instantiation of the reference's quantizer: 24-bit mantissas in, IEEE divisions throughout."""
+    g = H.gen(4040 + m + k)
+    x = torch.randn((m, k), generator=g)
+    x = torch.where(torch.rand((m, k), generator=g) < 0.01, x * 20, x)
+    if m > 2:
+        x[1, :group] = 0          # all-zero group: scale floor 1e-10/448
+        x[2, :group] *= 1e-30     # values far below the floor's scale: codes of zero
+    q, s = ops.per_token_group_quant_fp8(x.cuda(), k, group, colmajor)
+    qo, so = oracle.fp8_group_quant(x.numpy(), k, group, colmajor, False, oracle.F32)
+    np.testing.assert_array_equal(s.cpu().numpy().view(np.uint32), so.view(np.uint32))
+    np.testing.assert_array_equal(q.cpu().numpy(), qo)
+
+
+def test_blockwise_gemm_fp32_activations(ops, oracle):
+    """fp32 in, fp32 out (InvokeBlockGemm<float>): the quantizer's float form in front of the GEMM whose sums are the
+    output, in both kernel regimes."""
+    for (m, n, k) in [(7, 512, 1024), (130, 2304, 1152)]:
+        g = H.gen(4060 + m)
+        w = (torch.randn((n, k), generator=g) * 0.02).to(torch.bfloat16).float().numpy()
+        bq, bs = oracle.fp8_block_quant_weight(w)
+        x = torch.randn((m, k), generator=g)
+        q, s = ops.per_token_group_quant_fp8(x.cuda(), k, 128, True)
+        qo, so = oracle.fp8_group_quant(x.numpy(), k, 128, True, False, oracle.F32)
+        np.testing.assert_array_equal(q.cpu().numpy(), qo)
+        ref = oracle.fp8_blockwise_gemm(qo, so, bq, bs, True)
+        for rule in H.each_regime(m):
+            out = ops.fp8_blockwise_gemm(q, s, packed(ops, bq), torch.from_numpy(bs).cuda(), torch.float32)
+            assert out.dtype == torch.float32
+            H.check_gemm_f32(out, ref, "fp8 fp32 activations m=%d n=%d k=%d" % (m, n, k))
+
+
 def test_quant_every_e4m3_boundary(ops, oracle):
     """Rows whose amax is exactly 448 make the scale 1, so the codes are the bare float->e4m3 conversion: sweep
     every representable value, every rounding midpoint and their neighbours."""
@@ -243,6 +277,21 @@ def test_channel_quant_bit_exact(ops, oracle, dtype, channels, size):
     given = torch.full((channels,), 0.004, dtype=torch.float32)
     q2, _ = ops.fp8_e4m3_quantize(x.cuda(), given.cuda())
     qo2, _ = oracle.fp8_channel_quant(H.bits_of(x), dtype, scale=given.numpy())
+    np.testing.assert_array_equal(q2.cpu().numpy(), qo2)
+
+
+@pytest.mark.parametrize("channels,size", [(1, 31), (1, 16383), (1, 5120), (64, 5120), (3, 77)])
+def test_channel_quant_fp32_activations_bit_exact(ops, oracle, channels, size):
+    """The float instantiation (Fp8E4m3Quantize<float>): 24-bit mantissas, IEEE divisions throughout."""
+    g = H.gen(70 + channels + size)
+    x = torch.randn((channels, size), generator=g) * 2.5
+    q, s = ops.fp8_e4m3_quantize(x.cuda())
+    qo, so = oracle.fp8_channel_quant(x.numpy(), oracle.F32)
+    np.testing.assert_array_equal(s.cpu().numpy(), so)
+    np.testing.assert_array_equal(q.cpu().numpy(), qo)
+    given = torch.full((channels,), 0.004, dtype=torch.float32)
+    q2, _ = ops.fp8_e4m3_quantize(x.cuda(), given.cuda())
+    qo2, _ = oracle.fp8_channel_quant(x.numpy(), oracle.F32, scale=given.numpy())
     np.testing.assert_array_equal(q2.cpu().numpy(), qo2)
 
 

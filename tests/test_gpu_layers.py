@@ -115,6 +115,24 @@ def test_blockwise_layer(tmp_path, oracle, dtype, m, n, k, fuse, max_m):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("m,n,k", [(5, 512, 1024), (70, 256, 640)])
+def test_blockwise_layer_fp32_activations(tmp_path, oracle, m, n, k):
+    """inter_data_type TYPE_FP32 (DISPATCH_BY_3_DTYPE in the reference's Forward): fp32 in, fp32 out."""
+    g = H.gen(9150 + m)
+    w = (torch.randn((n, k), generator=g) * 0.02).to(torch.bfloat16).float().numpy()
+    bq, bs = oracle.fp8_block_quant_weight(w)
+    x = torch.randn((m, k), generator=g)
+    bq.tofile(tmp_path / "w.bin")
+    bs.astype(np.float32).tofile(tmp_path / "w_scale.bin")
+    x.numpy().tofile(tmp_path / "x.bin")
+    run_driver("blockwise", tmp_path, "f32", m, n, k, 0)
+    y = np.fromfile(tmp_path / "y.bin", dtype=np.float32).reshape(m, n)
+    q, s = oracle.fp8_group_quant(x.numpy(), k, 128, True, False, oracle.F32)
+    ref = oracle.fp8_blockwise_gemm(q, s, bq, bs, True)
+    H.check_gemm_f32(torch.from_numpy(y), ref, "blockwise layer fp32")
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("dtype,tokens,renorm,scaling,routing", [
     (H.BF16, 1, 0, 2.5, None), (H.F16, 24, 1, 1.0, None), (H.BF16, 70, 0, 1.0, None), (H.BF16, 400, 0, 1.0, None),
     # 2: scale-norm mode RE_NORM with norm_topk_prob false - the routers follow norm_topk_prob alone (no renormalization)
@@ -270,6 +288,26 @@ def test_fp8_per_tensor_layer(tmp_path, oracle, dtype, m, n, k, static):
     xq, xs = oracle.fp8_channel_quant(H.bits_of(x).reshape(1, -1), dtype, scale=in_scale if static else None)
     ref = oracle.fp8_tensor_gemm(xq.reshape(m, k), xs[0], wq.reshape(n, k), ws[0])
     H.check_gemm(y, ref, dtype, "fp8 per-tensor layer")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("m,n,k,static", [(3, 512, 1024, 0), (77, 256, 512, 1)])
+def test_fp8_per_tensor_layer_fp32_activations(tmp_path, oracle, m, n, k, static):
+    """inter_data_type TYPE_FP32: fp32 in, fp32 out, as the reference's map registers the layer (matmul_layer_factory.cpp:70)."""
+    g = H.gen(9650 + m)
+    w = (torch.randn((n, k), generator=g) * 0.02).to(torch.bfloat16)
+    wq, ws = oracle.fp8_channel_quant(H.bits_of(w).reshape(1, -1), H.BF16)
+    x = torch.randn((m, k), generator=g)
+    wq.tofile(tmp_path / "w.bin")
+    ws.tofile(tmp_path / "w_scale.bin")
+    x.numpy().tofile(tmp_path / "x.bin")
+    in_scale = np.array([0.012], np.float32)
+    in_scale.tofile(tmp_path / "in_scale.bin")
+    run_driver("fp8_tensor", tmp_path, "f32", m, n, k, static)
+    y = np.fromfile(tmp_path / "y.bin", dtype=np.float32).reshape(m, n)
+    xq, xs = oracle.fp8_channel_quant(x.numpy().reshape(1, -1), oracle.F32, scale=in_scale if static else None)
+    ref = oracle.fp8_tensor_gemm(xq.reshape(m, k), xs[0], wq.reshape(n, k), ws[0])
+    H.check_gemm_f32(torch.from_numpy(y), ref, "fp8 per-tensor layer fp32")
 
 
 @pytest.mark.gpu
