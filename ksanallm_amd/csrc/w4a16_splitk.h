@@ -449,8 +449,6 @@ __global__ void __launch_bounds__(WAVES * 64, OCC) w4a16_splitk_kernel(SplitKPar
       if (c + 1 < nchunks) stage_chunk(c + 1);  // into the buffer chunk c-1 used: every wavefront is past the barrier behind it
 #pragma unroll
       for (int j = 0; j < CI; ++j) {
-        constexpr int kDummy = 0;
-        (void)kDummy;
         const int h = j % LOOK;
         const KOff o = koff(c * CI + j + LOOK);
         XBuf xb;
